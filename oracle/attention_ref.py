@@ -1,0 +1,141 @@
+"""CPU restatements of the parallel-attention and MLA-decode references.
+
+Test infrastructure only (see the package docstring).  All functions take the
+tensor layouts of the operators they check (BSHD for the parallel family),
+up-cast to ``compute_dtype`` (fp32 by default, fp64 for pinning tests) and
+loop over (batch, head) slices so the S x S score matrix of one head is the
+largest temporary.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+
+def _causal_keep(sq: int, skv: int, device) -> torch.Tensor:
+    """keep[i, j] = (i >= j): the lower-triangular ``tril(ones)`` mask of
+    testing/test.py:92-97 as a boolean matrix."""
+    i = torch.arange(sq, device=device).unsqueeze(-1)
+    j = torch.arange(skv, device=device).unsqueeze(0)
+    return i >= j
+
+
+def softmax_attention(q, k, v, causal: bool = True, softmax_scale: Optional[float] = None,
+                      compute_dtype=torch.float32, return_lse: bool = False):
+    """Softmax attention forward.  Follows testing/test.py:79-104 (and the
+    identical attention_engine/benchmark/bench_utils.py:1347-1372): scores
+    = q.k^T, masked with -inf above the diagonal, softmax(scores * scale), times
+    v.  q [B,Sq,H,D], k [B,Skv,H,D], v [B,Skv,H,Dv] -> [B,Sq,H,Dv].
+    ``lse`` ([B,H,Sq], natural log, of the scaled scores) is the final row
+    scale of examples/mha.py:65-71."""
+    B, Sq, H, D = q.shape
+    Skv, Dv = k.shape[1], v.shape[-1]
+    scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+    out = torch.empty(B, Sq, H, Dv, dtype=compute_dtype)
+    lse = torch.empty(B, H, Sq, dtype=compute_dtype)
+    keep = _causal_keep(Sq, Skv, q.device) if causal else None
+    for b in range(B):
+        for h in range(H):
+            s = q[b, :, h].to(compute_dtype) @ k[b, :, h].to(compute_dtype).T
+            if keep is not None:
+                s = s.masked_fill(~keep, float("-inf"))
+            s = s * scale
+            lse[b, h] = torch.logsumexp(s, dim=-1)
+            out[b, :, h] = torch.softmax(s, dim=-1) @ v[b, :, h].to(compute_dtype)
+    return (out, lse) if return_lse else out
+
+
+def sigmoid_attention(q, k, v, bias, causal: bool = True, softmax_scale: float = 1.0,
+                      compute_dtype=torch.float32):
+    """Sigmoid attention forward.  testing/test.py:519-543 is the unscaled
+    form (bias added after the -inf masking, sigmoid written as
+    (tanh(x/2)+1)/2); attention_engine/benchmark/bench_utils.py:806-832 is
+    the scaled form (scores*scale + bias, then sigmoid).  ``bias`` is a python
+    float or a 1-element tensor.  Masked positions contribute exactly 0."""
+    B, Sq, H, D = q.shape
+    Skv, Dv = k.shape[1], v.shape[-1]
+    bias = float(bias.reshape(-1)[0]) if torch.is_tensor(bias) else float(bias)
+    out = torch.empty(B, Sq, H, Dv, dtype=compute_dtype)
+    keep = _causal_keep(Sq, Skv, q.device) if causal else None
+    for b in range(B):
+        for h in range(H):
+            s = q[b, :, h].to(compute_dtype) @ k[b, :, h].to(compute_dtype).T
+            if keep is not None:
+                s = s.masked_fill(~keep, float("-inf"))
+            s = s * softmax_scale + bias
+            p = (torch.tanh(s * 0.5) + 1.0) * 0.5
+            out[b, :, h] = p @ v[b, :, h].to(compute_dtype)
+    return out
+
+
+def relu_attention(q, k, v, softmax_scale: Optional[float] = None, compute_dtype=torch.float32):
+    """ReLU attention forward, testing/test.py:599-604: relu(q.k^T / sqrt(D)) v,
+    no mask, no normalisation."""
+    B, Sq, H, D = q.shape
+    Dv = v.shape[-1]
+    scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+    out = torch.empty(B, Sq, H, Dv, dtype=compute_dtype)
+    for b in range(B):
+        for h in range(H):
+            s = q[b, :, h].to(compute_dtype) @ k[b, :, h].to(compute_dtype).T
+            out[b, :, h] = torch.relu(s * scale) @ v[b, :, h].to(compute_dtype)
+    return out
+
+
+def retention_decay_mask(H: int, S: int, dtype=torch.float32) -> torch.Tensor:
+    """[1,H,S,S] decay mask gamma_h^(i-j) * [i>=j] with gamma_h = 1 - 2^(-5-h),
+    the RetNet head decays of testing/test.py:742-744 (there written in the
+    log2 domain)."""
+    g = 1.0 - torch.exp2(-5.0 - torch.arange(H, dtype=torch.float64))
+    idx = torch.arange(S, dtype=torch.float64)
+    diff = idx.unsqueeze(-1) - idx.unsqueeze(0)
+    keep = diff >= 0
+    m = torch.exp2(diff.clamp(min=0).unsqueeze(0) * torch.log2(g).view(H, 1, 1)) * keep
+    return m.unsqueeze(0).to(dtype)
+
+
+def retention_parallel(q, k, v, mask, compute_dtype=torch.float32, return_r: bool = False):
+    """Normalised parallel retention, attention_engine/benchmark/bench_utils.py:1158-1163
+    (same as testing/benchmark_h100.py:808-813): qkm = (q.k^T) * mask,
+    r = max(sum_j |qkm|, 1), o = (qkm / r) v.  q,k [B,S,H,D], v [B,S,H,Dv],
+    mask [1 or B, H, S, S] -> [B,S,H,Dv]."""
+    B, S, H, D = q.shape
+    Dv = v.shape[-1]
+    out = torch.empty(B, S, H, Dv, dtype=compute_dtype)
+    r_out = torch.empty(B, H, S, dtype=compute_dtype)
+    for b in range(B):
+        mb = mask[b if mask.shape[0] > 1 else 0]
+        for h in range(H):
+            s = q[b, :, h].to(compute_dtype) @ k[b, :, h].to(compute_dtype).T
+            s = s * mb[h].to(compute_dtype)
+            r = s.abs().sum(dim=-1, keepdim=True).clamp(min=1.0)
+            r_out[b, h] = r.squeeze(-1)
+            out[b, :, h] = (s / r) @ v[b, :, h].to(compute_dtype)
+    return (out, r_out) if return_r else out
+
+
+def mla_decode(q, q_pe, kv, k_pe, compute_dtype=torch.float32, return_lse: bool = False):
+    """Absorbed MLA decode, testing/test.py:807-839 (same as
+    attention_engine/core/template/tl_template/attn/mla_decode_tl.py:340-380):
+    scores = (q.kv^T + q_pe.k_pe^T) / sqrt(d + d_pe), softmax over the cache,
+    times kv.  q [B,1,Hq,d], q_pe [B,1,Hq,dpe], kv [B,Skv,Hkv,d],
+    k_pe [B,Skv,Hkv,dpe] -> [B,1,Hq,d].  Query head h uses kv head
+    h // (Hq // Hkv)."""
+    B, _, Hq, d = q.shape
+    dpe = q_pe.shape[-1]
+    Hkv = kv.shape[2]
+    group = Hq // Hkv
+    scale = 1.0 / math.sqrt(d + dpe)
+    out = torch.empty(B, 1, Hq, d, dtype=compute_dtype)
+    lse = torch.empty(B, Hq, dtype=compute_dtype)
+    for b in range(B):
+        for g in range(Hkv):
+            hs = slice(g * group, (g + 1) * group)
+            qq = torch.cat([q[b, 0, hs], q_pe[b, 0, hs]], dim=-1).to(compute_dtype)
+            kk = torch.cat([kv[b, :, g], k_pe[b, :, g]], dim=-1).to(compute_dtype)
+            s = (qq @ kk.T) * scale
+            lse[b, hs] = torch.logsumexp(s, dim=-1)
+            out[b, 0, hs] = torch.softmax(s, dim=-1) @ kv[b, :, g].to(compute_dtype)
+    return (out, lse) if return_lse else out

@@ -1,0 +1,213 @@
+"""Pins every oracle function against something independent of its own
+formula: library routines, closed forms, brute-force loops, or an
+algebraically different evaluation of the same operator."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from oracle import inputs
+
+torch.manual_seed(0)
+F64 = torch.float64
+
+
+def _rand(*shape, seed=0, dtype=F64):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g, dtype=dtype)
+
+
+# ---------------------------------------------------------------- softmax
+@pytest.mark.parametrize("causal", [False, True])
+def test_softmax_vs_sdpa(causal):
+    q, k, v = _rand(2, 33, 3, 16, seed=1), _rand(2, 33, 3, 16, seed=2), _rand(2, 33, 3, 24, seed=3)
+    o, lse = oracle.softmax_attention(q, k, v, causal=causal, compute_dtype=F64, return_lse=True)
+    ref = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
+                                         is_causal=causal).transpose(1, 2)
+    torch.testing.assert_close(o, ref, rtol=1e-10, atol=1e-10)
+    s = torch.einsum("bqhd,bkhd->bhqk", q, k) / math.sqrt(16)
+    if causal:
+        s = s.masked_fill(torch.triu(torch.ones(33, 33, dtype=torch.bool), 1), float("-inf"))
+    torch.testing.assert_close(lse, torch.logsumexp(s, -1), rtol=1e-10, atol=1e-10)
+
+
+def test_softmax_closed_forms():
+    # constant K: every unmasked score is equal -> causal output = running mean of V
+    q, v = _rand(1, 9, 2, 8, seed=4), _rand(1, 9, 2, 5, seed=5)
+    k = torch.ones(1, 9, 2, 8, dtype=F64)
+    o = oracle.softmax_attention(q, k, v, causal=True, compute_dtype=F64)
+    mean = torch.cumsum(v, 1) / torch.arange(1, 10, dtype=F64).view(1, 9, 1, 1)
+    torch.testing.assert_close(o, mean, rtol=1e-12, atol=1e-12)
+    # S = 1: O = V
+    q1, k1, v1 = _rand(2, 1, 2, 8), _rand(2, 1, 2, 8, seed=7), _rand(2, 1, 2, 4, seed=8)
+    torch.testing.assert_close(oracle.softmax_attention(q1, k1, v1, compute_dtype=F64), v1)
+
+
+def test_softmax_bruteforce_tiny():
+    q, k, v = _rand(1, 4, 1, 3, seed=9), _rand(1, 4, 1, 3, seed=10), _rand(1, 4, 1, 2, seed=11)
+    o = oracle.softmax_attention(q, k, v, causal=True, compute_dtype=F64)
+    for i in range(4):
+        w = [math.exp(sum(float(q[0, i, 0, d] * k[0, j, 0, d]) for d in range(3)) / math.sqrt(3)) for j in range(i + 1)]
+        for d in range(2):
+            exp = sum(w[j] * float(v[0, j, 0, d]) for j in range(i + 1)) / sum(w)
+            assert abs(float(o[0, i, 0, d]) - exp) < 1e-12
+
+
+# ---------------------------------------------------------------- sigmoid / relu
+def test_sigmoid_closed_form():
+    q, k, v = _rand(1, 6, 2, 4, seed=12), _rand(1, 6, 2, 4, seed=13), _rand(1, 6, 2, 3, seed=14)
+    for scale, bias in [(1.0, -1.7), (0.5, 0.3)]:
+        o = oracle.sigmoid_attention(q, k, v, torch.tensor([bias], dtype=F64), causal=True, softmax_scale=scale, compute_dtype=F64)
+        for h in range(2):
+            for i in range(6):
+                acc = torch.zeros(3, dtype=F64)
+                for j in range(i + 1):          # masked entries contribute exactly 0
+                    x = float(q[0, i, h] @ k[0, j, h]) * scale + bias
+                    acc += v[0, j, h] / (1.0 + math.exp(-x))
+                torch.testing.assert_close(o[0, i, h], acc, rtol=1e-12, atol=1e-12)
+    # non-causal: every pair contributes
+    o = oracle.sigmoid_attention(q, k, v, 0.0, causal=False, compute_dtype=F64)
+    s = torch.einsum("bqhd,bkhd->bhqk", q, k)
+    torch.testing.assert_close(o, torch.einsum("bhqk,bkhd->bqhd", torch.sigmoid(s), v), rtol=1e-12, atol=1e-12)
+
+
+def test_relu_bruteforce():
+    q, k, v = _rand(1, 5, 2, 4, seed=15), _rand(1, 5, 2, 4, seed=16), _rand(1, 5, 2, 3, seed=17)
+    o = oracle.relu_attention(q, k, v, compute_dtype=F64)
+    for h in range(2):
+        for i in range(5):
+            acc = torch.zeros(3, dtype=F64)
+            for j in range(5):
+                acc += max(float(q[0, i, h] @ k[0, j, h]) / 2.0, 0.0) * v[0, j, h]
+            torch.testing.assert_close(o[0, i, h], acc, rtol=1e-12, atol=1e-12)
+
+
+# ---------------------------------------------------------------- retention (parallel, normalised)
+def test_retention_decay_mask_values():
+    m = oracle.retention_decay_mask(3, 6, F64)[0]
+    for h in range(3):
+        g = 1 - 2.0 ** (-5 - h)
+        for i in range(6):
+            for j in range(6):
+                exp = g ** (i - j) if i >= j else 0.0
+                assert abs(float(m[h, i, j]) - exp) < 1e-14
+
+
+def test_retention_parallel_bruteforce_and_clamp():
+    B, S, H, D, DV = 1, 7, 2, 4, 3
+    q, k, v = _rand(B, S, H, D, seed=18), _rand(B, S, H, D, seed=19), _rand(B, S, H, DV, seed=20)
+    mask = oracle.retention_decay_mask(H, S, F64)
+    for qs in (1.0, 0.01):     # qs=0.01 puts every row sum below 1: clamp active -> un-normalised
+        o, r = oracle.retention_parallel(q * qs, k, v, mask, compute_dtype=F64, return_r=True)
+        for h in range(H):
+            for i in range(S):
+                w = [float((q[0, i, h] * qs) @ k[0, j, h]) * float(mask[0, h, i, j]) for j in range(S)]
+                rr = max(sum(abs(x) for x in w), 1.0)
+                exp = sum((w[j] / rr) * v[0, j, h] for j in range(S))
+                torch.testing.assert_close(o[0, i, h], exp, rtol=1e-12, atol=1e-12)
+                assert abs(float(r[0, h, i]) - rr) < 1e-12
+        if qs == 0.01:
+            assert float(r.max()) == 1.0
+    # all-ones causal mask: plain causal linear attention / max(sum|qk|,1)
+    ones = torch.tril(torch.ones(S, S, dtype=F64)).expand(1, H, S, S)
+    o = oracle.retention_parallel(q, k, v, ones, compute_dtype=F64)
+    s = torch.einsum("bqhd,bkhd->bhqk", q, k).tril()
+    ref = torch.einsum("bhqk,bkhd->bqhd", s / s.abs().sum(-1, keepdim=True).clamp(min=1), v)
+    torch.testing.assert_close(o, ref, rtol=1e-12, atol=1e-12)
+
+
+# ---------------------------------------------------------------- RetNet chunked
+def test_retnet_three_way():
+    B, H, T, Dk, Dv = 1, 3, 64, 8, 6
+    q, k, v = _rand(B, H, T, Dk, seed=21), _rand(B, H, T, Dk, seed=22), _rand(B, H, T, Dv, seed=23)
+    quad = oracle.retnet_quadratic(q, k, v, compute_dtype=F64)
+    rec = oracle.retnet_recurrence(q, k, v, compute_dtype=F64)
+    torch.testing.assert_close(quad, rec, rtol=1e-10, atol=1e-10)
+    gam = (1 - torch.exp2(-5.0 - torch.arange(H, dtype=F64))).view(1, H, 1).expand(B, H, T)
+    for chunk in (8, 16, 64):
+        ch = oracle.linear_attention_chunked(q, k, v, torch.log(gam), chunk=chunk, q_scale=Dk ** -0.5, compute_dtype=F64)
+        torch.testing.assert_close(ch, rec, rtol=1e-10, atol=1e-10)
+
+
+# ---------------------------------------------------------------- Mamba2
+def test_ssd_three_way():
+    b, l, h, p, n = 2, 64, 4, 5, 6
+    x = _rand(b, l, h, p, seed=24)
+    Bm, Cm = _rand(b, l, 1, n, seed=25), _rand(b, l, 1, n, seed=26)
+    dt = F.softplus(_rand(b, l, h, seed=27) - 2)
+    A = -torch.exp(torch.rand(h, dtype=F64) * math.log(16))
+    seq = oracle.ssd_sequential(x, dt, A, Bm, Cm)
+    for chunk in (8, 16, 64):
+        ch = oracle.ssd_chunk_scan_combined(x, dt, A, Bm, Cm, chunk_size=chunk, compute_dtype=F64)
+        torch.testing.assert_close(ch, seq, rtol=1e-9, atol=1e-9)
+    # the operator's view of the same computation (q=C, k=B, v=x*dt, log decay = dt*A), BHSD
+    lin = oracle.linear_attention_chunked(
+        Cm.permute(0, 2, 1, 3), Bm.permute(0, 2, 1, 3), x.permute(0, 2, 1, 3),
+        (dt * A).permute(0, 2, 1), chunk=16, v_scale=dt.permute(0, 2, 1), compute_dtype=F64)
+    torch.testing.assert_close(lin.permute(0, 2, 1, 3), seq, rtol=1e-9, atol=1e-9)
+
+
+def test_ssd_two_groups():
+    b, l, h, p, n = 1, 32, 4, 3, 4
+    x, Bm, Cm = _rand(b, l, h, p, seed=28), _rand(b, l, 2, n, seed=29), _rand(b, l, 2, n, seed=30)
+    dt = F.softplus(_rand(b, l, h, seed=31))
+    A = -torch.rand(h, dtype=F64) - 0.5
+    torch.testing.assert_close(oracle.ssd_chunk_scan_combined(x, dt, A, Bm, Cm, 8, F64),
+                               oracle.ssd_sequential(x, dt, A, Bm, Cm), rtol=1e-9, atol=1e-9)
+
+
+# ---------------------------------------------------------------- gated retention
+def test_simple_gla_vs_recurrence():
+    B, H, T, Dk, Dv = 1, 2, 48, 8, 5
+    q, k, v = _rand(B, H, T, Dk, seed=32), _rand(B, H, T, Dk, seed=33), _rand(B, H, T, Dv, seed=34)
+    g = F.logsigmoid(_rand(B, H, T, seed=35)).clamp_min(-5)
+    rec = oracle.simple_gla_recurrence(q, k, v, g)
+    for chunk in (8, 16, 48):
+        torch.testing.assert_close(oracle.simple_gla_chunked(q, k, v, g, chunk, compute_dtype=F64), rec,
+                                   rtol=1e-10, atol=1e-10)
+
+
+# ---------------------------------------------------------------- MLA decode
+def test_mla_vs_sdpa_and_split_invariance():
+    B, Hq, Skv, d, dpe = 2, 6, 40, 16, 4
+    q, q_pe = _rand(B, 1, Hq, d, seed=36), _rand(B, 1, Hq, dpe, seed=37)
+    kv, k_pe = _rand(B, Skv, 1, d, seed=38), _rand(B, Skv, 1, dpe, seed=39)
+    o, lse = oracle.mla_decode(q, q_pe, kv, k_pe, compute_dtype=F64, return_lse=True)
+    qq = torch.cat([q, q_pe], -1).transpose(1, 2)                      # [B,Hq,1,d+dpe]
+    kk = torch.cat([kv, k_pe], -1).transpose(1, 2).expand(B, Hq, Skv, d + dpe)
+    vv = kv.transpose(1, 2).expand(B, Hq, Skv, d)
+    # sdpa's default scale 1/sqrt(E) with E = d + dpe is the scale the operator uses
+    ref = F.scaled_dot_product_attention(qq, kk, vv).transpose(1, 2)
+    torch.testing.assert_close(o, ref, rtol=1e-10, atol=1e-10)
+    # split-KV + log-sum-exp merge reproduces the whole
+    parts = [oracle.mla_decode(q, q_pe, kv[:, s], k_pe[:, s], compute_dtype=F64, return_lse=True)
+             for s in (slice(0, 8), slice(8, 24), slice(24, 40))]
+    lses = torch.stack([p[1] for p in parts])                         # [3,B,Hq]
+    tot = torch.logsumexp(lses, 0)
+    merged = sum(p[0] * torch.exp(p[1] - tot).view(B, 1, Hq, 1) for p in parts)
+    torch.testing.assert_close(merged, o, rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(tot, lse, rtol=1e-10, atol=1e-10)
+
+
+# ---------------------------------------------------------------- helpers
+def test_assert_close_rule():
+    a = torch.zeros(1000)
+    e = torch.zeros(1000)
+    e[:5] = 1.0
+    with pytest.raises(AssertionError):
+        oracle.assert_close(a, e, rtol=1e-2, atol=1e-2)
+    oracle.assert_close(a, e, rtol=1e-2, atol=1e-2, mismatch_ratio=5e-3)
+    with pytest.raises(AssertionError):
+        oracle.assert_close(a, e, rtol=1e-2, atol=1e-2, mismatch_ratio=4e-3)
+
+
+def test_input_generators_are_seeded():
+    a = inputs.softmax_inputs(1, 2, 8, 4, 4, seed=3)
+    b = inputs.softmax_inputs(1, 2, 8, 4, 4, seed=3)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y) and x.dtype == torch.bfloat16
+    Cm, Bm, x, dt, A = inputs.mamba2_inputs(1, 4, 16, 8, 8)
+    assert Cm.shape == (1, 1, 16, 8) and x.shape == (1, 4, 16, 8) and dt.dtype == torch.float32
+    assert (A < 0).all() and (A >= -16).all() and (dt > 0).all()
