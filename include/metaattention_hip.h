@@ -1,0 +1,135 @@
+/*
+ * C ABI of the MI355X (gfx950) attention forward kernel library.
+ *
+ * This is the boundary the Python host side binds with ctypes.  Each entry
+ * point replaces one compiled operator that the reference builds at run time
+ * from a TileLang template; the reference interface it stands in for is cited
+ * per function.  Conventions (all entry points):
+ *   - plain pointers and sizes only; every pointer is a device pointer to
+ *     memory the CALLER owns (inputs, outputs and workspace alike);
+ *   - work is enqueued on the given hipStream_t and the call returns without
+ *     synchronising; the library allocates nothing and keeps no state;
+ *   - return value 0 on success, a negative MA_ERR_* code otherwise, in which
+ *     case ma_last_error() (thread local) describes the problem;
+ *   - strides are in ELEMENTS of the tensor's dtype; the innermost (feature)
+ *     dimension of every tensor must be contiguous.
+ */
+#ifndef METAATTENTION_HIP_H
+#define METAATTENTION_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MA_VERSION 1
+
+enum ma_status {
+  MA_OK = 0,
+  MA_ERR_INVALID_ARG = -1, /* null pointer, non-positive size, bad enum */
+  MA_ERR_UNSUPPORTED = -2, /* shape/dtype/variant outside the kernel library */
+  MA_ERR_WORKSPACE = -3,   /* workspace missing or too small */
+  MA_ERR_LAUNCH = -4       /* HIP reported a launch error */
+};
+
+enum ma_dtype { MA_BF16 = 0, MA_FP16 = 1 };
+
+/* Row function of the parallel family.  The reference expresses these as a
+ * traced score_mod + OnlineFunc pair (attention_engine/attn_engine/attn_engine.py:16-105);
+ * the library holds one hand-written variant per family:
+ *   SOFTMAX   p = exp(s*scale + bias - rowmax) / rowsum, final row scale = lse   (examples/mha.py:21-71)
+ *   SIGMOID   p = sigmoid(s*scale + bias), no row state                           (examples/sigmoid_attn.py:17-52)
+ *   RELU      p = max(s*scale + bias, 0), no row state                            (examples/reluattn.py:15-42)
+ *   RETENTION p = s*scale*mask / max(sum_j |s*scale*mask|, 1), final row scale = r (examples/retention_parallel.py:31-72)
+ */
+enum ma_attn_family { MA_ATTN_SOFTMAX = 0, MA_ATTN_SIGMOID = 1, MA_ATTN_RELU = 2, MA_ATTN_RETENTION = 3 };
+
+/* Structural mask of the parallel family (attn_tl.py:129-151): NONE visits
+ * every kv tile; CAUSAL keeps kv_idx <= q_idx, skips tiles above the diagonal
+ * and (for SOFTMAX/SIGMOID/RELU) sets masked probabilities to exactly 0. */
+enum ma_mask_kind { MA_MASK_NONE = 0, MA_MASK_CAUSAL = 1 };
+
+typedef struct ma_attn_params {
+  int32_t family; /* ma_attn_family */
+  int32_t dtype;  /* ma_dtype of q, k, v, o and of score_mask */
+  int32_t mask;   /* ma_mask_kind */
+  int32_t batch, heads, seqlen_q, seqlen_kv, dim_qk, dim_v;
+  /* q [B,Sq,H,Dqk], k [B,Skv,H,Dqk], v [B,Skv,H,Dv], o [B,Sq,H,Dv]; BSHD is the
+   * layout the reference operator takes (attn_tl.py:69-70) but any strides
+   * with a contiguous last dimension are accepted. */
+  const void* q; int64_t q_stride_b, q_stride_s, q_stride_h;
+  const void* k; int64_t k_stride_b, k_stride_s, k_stride_h;
+  const void* v; int64_t v_stride_b, v_stride_s, v_stride_h;
+  void* o;       int64_t o_stride_b, o_stride_s, o_stride_h;
+  /* optional fp32 [B,H,Sq] final row scale (lse for SOFTMAX, r for
+   * RETENTION; lower.py:386-393); may be NULL */
+  float* row_scale;
+  float scale; /* multiplies q.k^T */
+  float bias;  /* added after scaling ... */
+  const float* bias_ptr; /* ... plus *bias_ptr if not NULL (device fp32[1], sigmoid_attn.py:54-56) */
+  /* RETENTION only: elementwise score multiplier [1 or B, H, Sq, Skv] in
+   * `dtype` (retention_parallel.py:96-98); stride_b may be 0 */
+  const void* score_mask; int64_t sm_stride_b, sm_stride_h, sm_stride_q;
+} ma_attn_params;
+
+/* Chunked linear / stateful attention forward.  Replaces the three launches
+ * of LinearAttention.forward (tl_template/linear/linear_tl.py:1240-1269):
+ * chunk-local cumsum (:36-60), chunk_fwd_h (:146-221), chunk_o (:322-399).
+ *   o_t = q_scale * q_t . sum_{s<=t} exp(G_t - G_s) k_s^T (v_s * v_scale_s),  G = cumsum(log_decay)
+ * q [B,Hq,T,Dk], k [B,Hk,T,Dk], v/o [B,H,T,Dv] (BHSD, contiguous), log_decay
+ * fp32 [B,H,T]; head h reads q head h/(H/Hq) and k head h/(H/Hk) (:172,:351-352).
+ * v_scale (may be NULL) is fp32 [B,H,T]: the fused per-token v modifier
+ * (core/lower/lower_linear.py:211-287). */
+typedef struct ma_linear_params {
+  int32_t dtype;
+  int32_t batch, heads, heads_q, heads_k, seqlen, dim_k, dim_v, chunk;
+  const void* q; const void* k; const void* v; void* o;
+  const float* log_decay;
+  const float* v_scale;
+  float q_scale;
+  void* workspace; size_t workspace_bytes; /* see ma_linear_workspace_bytes */
+} ma_linear_params;
+
+/* Absorbed MLA decode forward.  Replaces flash_attn_split + combine
+ * (tl_template/attn/mla_decode_tl.py:154-290, wrapper :450-459):
+ *   o = softmax((q.kv^T + q_pe.k_pe^T) * scale) . kv
+ * q [B,Hq,D], q_pe [B,Hq,Dpe], kv [B,Skv,D], k_pe [B,Skv,Dpe], o [B,Hq,D]
+ * (one latent kv head, one query token; the [B,1,Hq,.] / [B,Skv,1,.] tensors
+ * of the reference are these with a unit dimension).  Partials are fp32. */
+typedef struct ma_mla_params {
+  int32_t dtype;
+  int32_t batch, heads_q, seqlen_kv, dim, dim_pe;
+  int32_t num_split; /* 0 = let the library choose */
+  const void* q;    int64_t q_stride_b, q_stride_h;
+  const void* q_pe; int64_t qpe_stride_b, qpe_stride_h;
+  const void* kv;   int64_t kv_stride_b, kv_stride_s;
+  const void* k_pe; int64_t kpe_stride_b, kpe_stride_s;
+  void* o;          int64_t o_stride_b, o_stride_h;
+  float* lse;       /* optional fp32 [B,Hq] natural-log lse; may be NULL */
+  float scale;
+  void* workspace; size_t workspace_bytes; /* see ma_mla_workspace_bytes */
+} ma_mla_params;
+
+typedef void* ma_stream_t; /* a hipStream_t */
+
+int ma_version(void);
+const char* ma_last_error(void);
+
+/* attn_tl.py:92-190 (`main`) behind _attention.forward (:654-667) */
+int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream);
+
+/* linear_tl.py:1240-1269 */
+size_t ma_linear_workspace_bytes(const ma_linear_params* p);
+int ma_linear_fwd(const ma_linear_params* p, ma_stream_t stream);
+
+/* mla_decode_tl.py:293-303 (`main_split`) */
+int ma_mla_choose_split(const ma_mla_params* p);
+size_t ma_mla_workspace_bytes(const ma_mla_params* p);
+int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* METAATTENTION_HIP_H */

@@ -1,0 +1,78 @@
+// C ABI entry points (see include/metaattention_hip.h): argument validation,
+// error strings, kernel selection.  No allocation, no synchronisation.
+#include "../../include/metaattention_hip.h"
+#include "attn_fwd.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+namespace {
+thread_local char g_err[512] = "";
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+}  // namespace
+
+extern "C" {
+
+int ma_version(void) { return MA_VERSION; }
+const char* ma_last_error(void) { return g_err; }
+
+int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
+  if (!p) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: params is NULL");
+  if (!p->q || !p->k || !p->v || !p->o) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: q/k/v/o must be non-NULL");
+  if (p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->seqlen_kv <= 0 || p->dim_qk <= 0 || p->dim_v <= 0)
+    return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: sizes must be positive (B=%d H=%d Sq=%d Skv=%d Dqk=%d Dv=%d)", p->batch,
+                p->heads, p->seqlen_q, p->seqlen_kv, p->dim_qk, p->dim_v);
+  if (p->dtype != MA_BF16 && p->dtype != MA_FP16) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: dtype %d", p->dtype);
+  if (p->mask != MA_MASK_NONE && p->mask != MA_MASK_CAUSAL) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: mask kind %d", p->mask);
+  if (p->family < MA_ATTN_SOFTMAX || p->family > MA_ATTN_RETENTION)
+    return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: family %d", p->family);
+  if (!(p->scale > 0.f)) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: scale must be > 0 (got %g)", (double)p->scale);
+  if (p->mask == MA_MASK_CAUSAL && p->seqlen_q != p->seqlen_kv)
+    return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: causal mask needs seqlen_q == seqlen_kv (%d vs %d)", p->seqlen_q, p->seqlen_kv);
+  if (p->family == MA_ATTN_RETENTION && !p->score_mask)
+    return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: RETENTION needs score_mask");
+  const int64_t strides[] = {p->q_stride_s, p->q_stride_h, p->k_stride_s, p->k_stride_h, p->v_stride_s, p->v_stride_h,
+                             p->o_stride_s, p->o_stride_h, p->q_stride_b, p->k_stride_b, p->v_stride_b, p->o_stride_b};
+  for (int64_t s : strides)
+    if (s % 8 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: strides must be multiples of 8 elements (16-byte rows)");
+  const uintptr_t ptrs[] = {(uintptr_t)p->q, (uintptr_t)p->k, (uintptr_t)p->v, (uintptr_t)p->o};
+  for (uintptr_t x : ptrs)
+    if (x % 16 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: q/k/v/o must be 16-byte aligned");
+
+  ma::AttnArgs a{};
+  a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o;
+  a.row_scale = p->row_scale; a.bias_ptr = p->bias_ptr; a.smask = p->score_mask;
+  a.qsb = p->q_stride_b; a.qss = p->q_stride_s; a.qsh = p->q_stride_h;
+  a.ksb = p->k_stride_b; a.kss = p->k_stride_s; a.ksh = p->k_stride_h;
+  a.vsb = p->v_stride_b; a.vss = p->v_stride_s; a.vsh = p->v_stride_h;
+  a.osb = p->o_stride_b; a.oss = p->o_stride_s; a.osh = p->o_stride_h;
+  a.msb = p->sm_stride_b; a.msh = p->sm_stride_h; a.msq = p->sm_stride_q;
+  a.B = p->batch; a.H = p->heads; a.Sq = p->seqlen_q; a.Skv = p->seqlen_kv;
+  a.scale = p->scale; a.bias = p->bias;
+  const int rc = ma::attn_fwd_dispatch(a, p->family, p->mask == MA_MASK_CAUSAL, p->dtype == MA_BF16, p->dim_qk, p->dim_v,
+                                       (hipStream_t)stream);
+  if (rc == -2)
+    return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: no kernel for family %d, Dqk=%d, Dv=%d", p->family, p->dim_qk, p->dim_v);
+  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_attn_fwd: launch failed: %s", hipGetErrorString(hipGetLastError()));
+  return MA_OK;
+}
+
+size_t ma_linear_workspace_bytes(const ma_linear_params* p) { (void)p; return 0; }
+int ma_linear_fwd(const ma_linear_params* p, ma_stream_t stream) {
+  (void)p; (void)stream;
+  return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: not built yet");
+}
+int ma_mla_choose_split(const ma_mla_params* p) { (void)p; return 1; }
+size_t ma_mla_workspace_bytes(const ma_mla_params* p) { (void)p; return 0; }
+int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
+  (void)p; (void)stream;
+  return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: not built yet");
+}
+
+}  // extern "C"

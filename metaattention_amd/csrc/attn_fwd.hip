@@ -1,0 +1,324 @@
+// Parallel (flash-style) attention forward for gfx950.
+//
+// Replaces the operator the reference renders from
+// attention_engine/core/template/tl_template/attn/attn_tl.py:92-190: per Q tile,
+// loop over KV tiles: S = Q K^T, elementwise score function, online row
+// function, O = O * o_scale + P V.  The row functions are the fixed library
+// variants documented in include/metaattention_hip.h.
+//
+// Mapping onto CDNA4 (wave64, v_mfma_f32_32x32x16):
+//   * a workgroup is 4 waves; each wave owns 32 query rows (block_M = 128) and
+//     every wave walks the same 64-row KV tiles staged in LDS (double buffered);
+//   * the score tile is computed TRANSPOSED, S^T = K Q^T (A = K rows from LDS,
+//     B = Q held in registers), so that in the accumulator layout every lane
+//     owns ONE query row: the online row statistics are per-lane scalars, the
+//     row reductions are 31 in-register ops plus one exchange with lane^32, and
+//     the probabilities are already in B-operand layout for O^T += V^T P^T with
+//     no LDS round trip;
+//   * V^T fragments come straight out of the row-major V tile with the
+//     transposing LDS read (ds_read_b64_tr_b16);
+//   * both LDS tiles are XOR-swizzled at 16-byte granularity so the 128-bit K
+//     reads and the transposing V reads are bank-conflict free without padding.
+#include "attn_fwd.h"
+
+namespace ma {
+
+enum { FAM_SOFTMAX = 0, FAM_SIGMOID = 1, FAM_RELU = 2 };
+
+template <int CPR>
+__device__ __forceinline__ int swz_k(int row) {
+  // 16 consecutive rows reading the same logical 16-byte chunk must land in 16
+  // different bank groups.
+  return CPR >= 16 ? (row & 15) : ((row >> 1) & 7);
+}
+template <int CPR>
+__device__ __forceinline__ int swz_v(int row) {
+  // a transposing read touches 8 consecutive rows x 4 consecutive chunks; spread
+  // the 4 rows of each lane block over the high chunk bits.
+  return CPR >= 16 ? (((row & 3) << 2) | ((row >> 2) & 3)) : (((row & 3) << 1) | ((row >> 2) & 1));
+}
+
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
+__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
+  using E = Elem<T>;
+  using x8 = typename E::x8;
+  using x4 = typename E::x4;
+  constexpr int BM = 128, BN = 64, NB = BN / 32;
+  constexpr int KS = DQK / 16;   // k-slices of the QK^T contraction
+  constexpr int DB = DV / 32;    // 32-wide output column blocks
+  constexpr int CPRK = DQK / 8, CPRV = DV / 8;  // 16-byte chunks per row
+  constexpr int KROW = DQK * 2, VROW = DV * 2;
+  constexpr int KTILE = BN * KROW, VTILE = BN * VROW;
+  constexpr int KCH = BN * CPRK / 256, VCH = BN * CPRV / 256;
+  static_assert(KCH >= 1 && VCH >= 1, "tile too small for 256 threads");
+
+  extern __shared__ __align__(16) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
+  // [K buf0][K buf1][V buf0][V buf1]
+  const uint32_t lds_k = lds0, lds_v = lds0 + 2 * KTILE;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
+
+  // workgroup -> (batch*head, q block).  Consecutive workgroup ids are dealt
+  // round-robin to the 8 XCDs, so all q blocks of one (batch, head) are kept on
+  // one XCD (shared K/V stays in that XCD's L2); causal q blocks run heaviest first.
+  const int nmb = a.num_m_blocks, BH = a.B * a.H;
+  int bh, mb;
+  if ((BH & 7) == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    bh = (slot / nmb) * 8 + xcd;
+    mb = slot % nmb;
+  } else {
+    bh = blockIdx.x / nmb;
+    mb = blockIdx.x % nmb;
+  }
+  if (CAUSAL) mb = nmb - 1 - mb;
+  const int b = bh / a.H, h = bh % a.H;
+  const int m_wave = mb * BM + wave * 32;  // first query row of this wave
+  const int m_lane = m_wave + r;
+
+  // ---- Q fragments (B operand of S^T = K Q^T), kept in registers
+  x8 qf[KS];
+  {
+    const int qrow = min(m_lane, a.Sq - 1);
+    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)qrow * a.qss + (int64_t)h * a.qsh + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 16 * ks);
+  }
+
+  const T* kbase = (const T*)a.k + (int64_t)b * a.ksb + (int64_t)h * a.ksh;
+  const T* vbase = (const T*)a.v + (int64_t)b * a.vsb + (int64_t)h * a.vsh;
+
+  int n_tiles = (a.Skv + BN - 1) / BN;
+  if (CAUSAL) n_tiles = min(n_tiles, (mb * BM + BM + BN - 1) / BN);
+
+  // ---- global -> register -> LDS staging of one KV tile
+  u32x4 kreg[KCH], vreg[VCH];
+  auto load_tile = [&](int n0) {
+#pragma unroll
+    for (int i = 0; i < KCH; i++) {
+      const int ci = tid + 256 * i, row = ci / CPRK, c = ci % CPRK;
+      const int nrow = min(n0 + row, a.Skv - 1);
+      kreg[i] = *(const u32x4*)(kbase + (int64_t)nrow * a.kss + c * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < VCH; i++) {
+      const int ci = tid + 256 * i, row = ci / CPRV, c = ci % CPRV;
+      const int nrow = min(n0 + row, a.Skv - 1);
+      vreg[i] = *(const u32x4*)(vbase + (int64_t)nrow * a.vss + c * 8);
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < KCH; i++) {
+      const int ci = tid + 256 * i, row = ci / CPRK, c = ci % CPRK;
+      lds_write<u32x4>(lds_k + buf * KTILE + row * KROW + ((c ^ swz_k<CPRK>(row)) << 4), kreg[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < VCH; i++) {
+      const int ci = tid + 256 * i, row = ci / CPRV, c = ci % CPRV;
+      lds_write<u32x4>(lds_v + buf * VTILE + row * VROW + ((c ^ swz_v<CPRV>(row)) << 4), vreg[i]);
+    }
+  };
+
+  // ---- per-lane LDS read addresses
+  // K (A operand of S^T): row 32nb + r, logical chunk 2ks + g
+  const uint32_t k_row_off = r * KROW;
+  const int k_chunk0 = g ^ swz_k<CPRK>(r);
+  // V (A operand of O^T, through the transposing read): lane block = lane/16,
+  // row nbase + 8*half + 4g + jr, logical chunk 4db + lc
+  const int jr = (lane & 15) >> 2;
+  const int lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
+  const uint32_t v_row_off = (4 * g + jr) * VROW + (lane & 1) * 8;
+  const int v_swz_lane = swz_v<CPRV>(4 * g + jr);  // rows nbase + 8*half keep (row & 3) and flip bit 1 of (row >> 2)
+  const int v_chunk0 = lc ^ v_swz_lane;
+  constexpr int V_HALF_XOR = CPRV >= 16 ? 2 : 0;  // swz_v(row + 8) ^ swz_v(row)
+  static_assert(CPRV >= 16, "DV < 128 needs its own swizzle");
+
+  // ---- accumulators and row state
+  f32x16 o[DB];
+#pragma unroll
+  for (int i = 0; i < DB; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) o[i][j] = 0.f;
+  const float bias = a.bias + (a.bias_ptr ? *a.bias_ptr : 0.f);
+  const float c_scale = a.scale * kLog2e;  // scores are handled in the log2 domain
+  const float c_bias = bias * kLog2e;
+  float row_max = -1e30f;  // running max of (scale*s + bias) * log2e
+  float row_sum = 0.f;     // this lane's share of the running sum (the other half lives in lane^32)
+
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+
+  for (int jt = 0; jt < n_tiles; jt++) {
+    const int buf = jt & 1, n0 = jt * BN;
+    if (jt + 1 < n_tiles) load_tile(n0 + BN);
+
+    // ---- S^T = K Q^T : lane holds query row r, kv rows 32nb + 8(j/4) + 4g + j%4
+    f32x16 s[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+      for (int j = 0; j < 16; j++) s[nb][j] = 0.f;
+    const uint32_t kb = lds_k + buf * KTILE + k_row_off;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      const uint32_t coff = (uint32_t)((k_chunk0 ^ (2 * ks)) << 4);
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+        x8 kf = lds_read<x8>(kb + nb * 32 * KROW + coff);
+        s[nb] = E::mfma32(kf, qf[ks], s[nb]);
+      }
+    }
+
+    // ---- structural mask: exact -inf above the diagonal / beyond the cache
+    const bool need_mask = (CAUSAL && (n0 + BN - 1 > m_wave)) || (n0 + BN > a.Skv);
+    if (need_mask) {
+      const int lim = CAUSAL ? min(m_lane, a.Skv - 1) : a.Skv - 1;  // keep n <= lim
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+          const int n = n0 + 32 * nb + 8 * (j >> 2) + 4 * g + (j & 3);
+          if (n > lim) s[nb][j] = -INFINITY;
+        }
+    }
+
+    // ---- row function
+    if constexpr (FAMILY == FAM_SOFTMAX) {
+      float mx = s[0][0];
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) mx = fmaxf(mx, s[nb][j]);
+      mx = fmaxf(mx, xhalf(mx));
+      const float new_max = fmaxf(row_max, mx * c_scale + c_bias);
+      const float corr = fast_exp2(row_max - new_max);
+      row_max = new_max;
+      const float sub = c_bias - new_max;
+      float part = 0.f;
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+          const float p = fast_exp2(s[nb][j] * c_scale + sub);
+          s[nb][j] = p;
+          part += p;
+        }
+      row_sum = row_sum * corr + part;
+      if (__any(corr != 1.f)) {
+#pragma unroll
+        for (int i = 0; i < DB; i++)
+#pragma unroll
+          for (int j = 0; j < 16; j++) o[i][j] *= corr;
+      }
+    } else if constexpr (FAMILY == FAM_SIGMOID) {
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int j = 0; j < 16; j++)  // sigmoid(x) = 1 / (1 + 2^(-x log2e)); s = -inf gives exactly 0
+          s[nb][j] = fast_rcp(1.f + fast_exp2(-(s[nb][j] * c_scale + c_bias)));
+    } else {
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) s[nb][j] = fmaxf(s[nb][j] * a.scale + bias, 0.f);
+    }
+
+    // ---- O^T += V^T P^T ; the k index of MFMA slice (nb, t), lane half g, slot i is
+    //      kv row 32nb + 16t + 8(i/4) + 4g + i%4 on both operands
+    const uint32_t vb = lds_v + buf * VTILE + v_row_off;
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        x8 pf;
+#pragma unroll
+        for (int i = 0; i < 8; i++) pf[i] = (T)s[nb][8 * t + i];
+        const uint32_t rb = vb + (32 * nb + 16 * t) * VROW;
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+          x4 lo = lds_read_tr4<T>(rb + (uint32_t)((v_chunk0 ^ (4 * db)) << 4));
+          x4 hi = lds_read_tr4<T>(rb + 8 * VROW + (uint32_t)((v_chunk0 ^ (4 * db) ^ V_HALF_XOR) << 4));
+          x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          o[db] = E::mfma32(vf, pf, o[db]);
+        }
+      }
+
+    if (jt + 1 < n_tiles) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: normalise, stage O through LDS (wave-private), coalesced 16-byte stores
+  float inv = 1.f, lse = 0.f;
+  if constexpr (FAMILY == FAM_SOFTMAX) {
+    const float tot = row_sum + xhalf(row_sum);
+    inv = 1.f / tot;
+    lse = (row_max + fast_log2(tot)) * kLn2;
+  }
+  constexpr int OROW = DV * 2 + 16;  // padded staging row
+  const uint32_t ob = lds0 + wave * 32 * OROW;
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; q4++) {
+      x4 w;
+#pragma unroll
+      for (int i = 0; i < 4; i++) w[i] = (T)(o[db][4 * q4 + i] * inv);
+      lds_write<x4>(ob + r * OROW + (32 * db + 8 * q4 + 4 * g) * 2, w);
+    }
+  T* obase = (T*)a.o + (int64_t)b * a.osb + (int64_t)h * a.osh;
+#pragma unroll
+  for (int it = 0; it < 32 * CPRV / 64; it++) {
+    const int ci = lane + 64 * it, row = ci / CPRV, c = ci % CPRV;
+    u32x4 w = lds_read<u32x4>(ob + row * OROW + c * 16);
+    if (m_wave + row < a.Sq) *(u32x4*)(obase + (int64_t)(m_wave + row) * a.oss + c * 8) = w;
+  }
+  if constexpr (FAMILY == FAM_SOFTMAX) {
+    if (a.row_scale && g == 0 && m_lane < a.Sq) a.row_scale[((int64_t)b * a.H + h) * a.Sq + m_lane] = lse;
+  }
+}
+
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
+static int launch(const AttnArgs& a, hipStream_t stream) {
+  constexpr int BM = 128, BN = 64;
+  constexpr size_t tiles = 2 * (size_t)BN * (DQK + DV) * 2;
+  constexpr size_t ostage = 4 * 32 * (size_t)(DV * 2 + 16);
+  constexpr size_t lds = tiles > ostage ? tiles : ostage;
+  auto kern = attn_fwd_kernel<T, DQK, DV, FAMILY, CAUSAL>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
+    attr_set = true;
+  }
+  AttnArgs args = a;
+  args.num_m_blocks = (a.Sq + BM - 1) / BM;
+  const unsigned grid = (unsigned)(args.num_m_blocks * a.B * a.H);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, args);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+template <typename T, int DQK, int DV>
+static int dispatch_family(const AttnArgs& a, int family, bool causal, hipStream_t stream) {
+  switch (family) {
+    case FAM_SOFTMAX:
+      return causal ? launch<T, DQK, DV, FAM_SOFTMAX, true>(a, stream) : launch<T, DQK, DV, FAM_SOFTMAX, false>(a, stream);
+    case FAM_SIGMOID:
+      return causal ? launch<T, DQK, DV, FAM_SIGMOID, true>(a, stream) : launch<T, DQK, DV, FAM_SIGMOID, false>(a, stream);
+    case FAM_RELU:
+      return causal ? launch<T, DQK, DV, FAM_RELU, true>(a, stream) : launch<T, DQK, DV, FAM_RELU, false>(a, stream);
+  }
+  return -2;
+}
+
+// returns 0 ok, -1 launch failure, -2 unsupported
+int attn_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream) {
+  if (dqk == 128 && dv == 128) {
+    return is_bf16 ? dispatch_family<__bf16, 128, 128>(a, family, causal, stream)
+                   : dispatch_family<_Float16, 128, 128>(a, family, causal, stream);
+  }
+  return -2;
+}
+
+}  // namespace ma

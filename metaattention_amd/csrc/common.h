@@ -1,0 +1,82 @@
+// Shared device helpers for the gfx950 kernels: 64-lane MFMA fragments,
+// LDS swizzles, cross-half exchange.  gfx950 only; there is no other target.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ma {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define MA_LDS __attribute__((address_space(3)))
+
+// Element traits.  Fragment conventions of v_mfma_f32_32x32x16_{bf16,f16}
+// (lane l, r = l % 32, g = l / 32), verified on hardware:
+//   A[32 x 16]: lane holds row r, k = 8g .. 8g+7
+//   B[16 x 32]: lane holds column r, k = 8g .. 8g+7
+//   C[32 x 32]: lane holds column r, element j (0..15) is row 8(j/4) + 4g + j%4
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> {
+  using x8 = bf16x8; using x4 = bf16x4; using x2 = bf16x2;
+  static __device__ __forceinline__ f32x16 mfma32(x8 a, x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(x8 a, x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Elem<_Float16> {
+  using x8 = f16x8; using x4 = f16x4; using x2 = f16x2;
+  static __device__ __forceinline__ f32x16 mfma32(x8 a, x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(x8 a, x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// Transposing LDS read (ds_read_b64_tr_b16).  Within each block of 16 lanes,
+// lane j supplies the address of 4 consecutive 16-bit elements; result lane i
+// receives element (i % 4) of lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4.  With
+// lanes 4r..4r+3 pointing at 16 consecutive columns of row r (r = 0..3), lane
+// i ends up with column i of rows 0..3: a 4-deep column read of a row-major
+// tile, which is the K-major operand MFMA wants.  (Mapping verified on hardware.)
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::x4 lds_read_tr4(uint32_t lds_byte_addr) {
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((MA_LDS s16x4*)(uintptr_t)lds_byte_addr);
+  return __builtin_bit_cast(typename Elem<T>::x4, v);
+}
+
+template <typename V>
+__device__ __forceinline__ V lds_read(uint32_t lds_byte_addr) {
+  return *(const MA_LDS V*)(uintptr_t)lds_byte_addr;
+}
+template <typename V>
+__device__ __forceinline__ void lds_write(uint32_t lds_byte_addr, V v) {
+  *(MA_LDS V*)(uintptr_t)lds_byte_addr = v;
+}
+
+// value held by lane (l ^ 32)
+__device__ __forceinline__ float xhalf(float x) {
+  return __shfl_xor(x, 32, 64);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+}  // namespace ma

@@ -1,0 +1,166 @@
+"""ctypes binding of the gfx950 kernel library (``include/metaattention_hip.h``).
+
+The structures below mirror the C header field by field.  The wrappers take
+torch tensors that already live on the GPU, pass raw pointers, strides and the
+current HIP stream, and raise ``MetaAttentionError`` carrying the library's
+error string when a call is rejected.  There is no fallback: if the shared
+library has not been built, loading it raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libmetaattention_hip.so")
+
+MA_BF16, MA_FP16 = 0, 1
+MA_ATTN_SOFTMAX, MA_ATTN_SIGMOID, MA_ATTN_RELU, MA_ATTN_RETENTION = 0, 1, 2, 3
+MA_MASK_NONE, MA_MASK_CAUSAL = 0, 1
+
+EXPORTED_SYMBOLS = (
+    "ma_version", "ma_last_error", "ma_attn_fwd",
+    "ma_linear_workspace_bytes", "ma_linear_fwd",
+    "ma_mla_choose_split", "ma_mla_workspace_bytes", "ma_mla_decode",
+)
+
+
+class MetaAttentionError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"[{code}] {message}")
+        self.code = code
+
+
+class AttnParams(Structure):
+    _fields_ = [
+        ("family", c_int32), ("dtype", c_int32), ("mask", c_int32),
+        ("batch", c_int32), ("heads", c_int32), ("seqlen_q", c_int32), ("seqlen_kv", c_int32),
+        ("dim_qk", c_int32), ("dim_v", c_int32),
+        ("q", c_void_p), ("q_stride_b", c_int64), ("q_stride_s", c_int64), ("q_stride_h", c_int64),
+        ("k", c_void_p), ("k_stride_b", c_int64), ("k_stride_s", c_int64), ("k_stride_h", c_int64),
+        ("v", c_void_p), ("v_stride_b", c_int64), ("v_stride_s", c_int64), ("v_stride_h", c_int64),
+        ("o", c_void_p), ("o_stride_b", c_int64), ("o_stride_s", c_int64), ("o_stride_h", c_int64),
+        ("row_scale", c_void_p),
+        ("scale", c_float), ("bias", c_float), ("bias_ptr", c_void_p),
+        ("score_mask", c_void_p), ("sm_stride_b", c_int64), ("sm_stride_h", c_int64), ("sm_stride_q", c_int64),
+    ]
+
+
+class LinearParams(Structure):
+    _fields_ = [
+        ("dtype", c_int32),
+        ("batch", c_int32), ("heads", c_int32), ("heads_q", c_int32), ("heads_k", c_int32),
+        ("seqlen", c_int32), ("dim_k", c_int32), ("dim_v", c_int32), ("chunk", c_int32),
+        ("q", c_void_p), ("k", c_void_p), ("v", c_void_p), ("o", c_void_p),
+        ("log_decay", c_void_p), ("v_scale", c_void_p),
+        ("q_scale", c_float),
+        ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+    ]
+
+
+class MlaParams(Structure):
+    _fields_ = [
+        ("dtype", c_int32),
+        ("batch", c_int32), ("heads_q", c_int32), ("seqlen_kv", c_int32), ("dim", c_int32), ("dim_pe", c_int32),
+        ("num_split", c_int32),
+        ("q", c_void_p), ("q_stride_b", c_int64), ("q_stride_h", c_int64),
+        ("q_pe", c_void_p), ("qpe_stride_b", c_int64), ("qpe_stride_h", c_int64),
+        ("kv", c_void_p), ("kv_stride_b", c_int64), ("kv_stride_s", c_int64),
+        ("k_pe", c_void_p), ("kpe_stride_b", c_int64), ("kpe_stride_s", c_int64),
+        ("o", c_void_p), ("o_stride_b", c_int64), ("o_stride_h", c_int64),
+        ("lse", c_void_p),
+        ("scale", c_float),
+        ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+    ]
+
+
+_lib = None
+
+
+def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
+    """Loads the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(path):
+        raise MetaAttentionError(
+            -100, f"{path} not found: build it with `python -m metaattention_amd.build` (there is no CPU fallback)")
+    lib = ctypes.CDLL(path)
+    lib.ma_version.restype = c_int
+    lib.ma_last_error.restype = c_char_p
+    lib.ma_attn_fwd.argtypes = [POINTER(AttnParams), c_void_p]
+    lib.ma_attn_fwd.restype = c_int
+    lib.ma_linear_workspace_bytes.argtypes = [POINTER(LinearParams)]
+    lib.ma_linear_workspace_bytes.restype = c_size_t
+    lib.ma_linear_fwd.argtypes = [POINTER(LinearParams), c_void_p]
+    lib.ma_linear_fwd.restype = c_int
+    lib.ma_mla_choose_split.argtypes = [POINTER(MlaParams)]
+    lib.ma_mla_choose_split.restype = c_int
+    lib.ma_mla_workspace_bytes.argtypes = [POINTER(MlaParams)]
+    lib.ma_mla_workspace_bytes.restype = c_size_t
+    lib.ma_mla_decode.argtypes = [POINTER(MlaParams), c_void_p]
+    lib.ma_mla_decode.restype = c_int
+    _lib = lib
+    return lib
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise MetaAttentionError(rc, load_library().ma_last_error().decode())
+
+
+def _dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.bfloat16:
+        return MA_BF16
+    if dt == torch.float16:
+        return MA_FP16
+    raise KeyError(dt)  # same failure mode as the reference's dtype map (attn_engine.py:234-237)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise MetaAttentionError(-101, "tensors must live on the GPU (there is no CPU path)")
+
+
+def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None,
+             score_mask=None, out=None, row_scale=None):
+    """Parallel attention forward on BSHD tensors.  Returns ``out`` ([B,Sq,H,Dv])."""
+    _require_gpu(q, k, v, bias_tensor, score_mask, out, row_scale)
+    B, Sq, H, Dqk = q.shape
+    Skv, Dv = k.shape[1], v.shape[-1]
+    assert k.shape == (B, Skv, H, Dqk) and v.shape == (B, Skv, H, Dv), "q/k/v shapes disagree"
+    for t in (q, k, v):
+        assert t.stride(-1) == 1, "last dimension must be contiguous"
+    if out is None:
+        out = torch.empty(B, Sq, H, Dv, dtype=q.dtype, device=q.device)
+    p = AttnParams()
+    p.family, p.dtype, p.mask = family, _dtype_code(q.dtype), MA_MASK_CAUSAL if causal else MA_MASK_NONE
+    p.batch, p.heads, p.seqlen_q, p.seqlen_kv, p.dim_qk, p.dim_v = B, H, Sq, Skv, Dqk, Dv
+    for name, t in (("q", q), ("k", k), ("v", v), ("o", out)):
+        setattr(p, name, t.data_ptr())
+        setattr(p, f"{name}_stride_b", t.stride(0))
+        setattr(p, f"{name}_stride_s", t.stride(1))
+        setattr(p, f"{name}_stride_h", t.stride(2))
+    if row_scale is not None:
+        assert row_scale.dtype == torch.float32 and row_scale.shape == (B, H, Sq) and row_scale.is_contiguous()
+        p.row_scale = row_scale.data_ptr()
+    p.scale, p.bias = float(scale), float(bias)
+    if bias_tensor is not None:
+        assert bias_tensor.dtype == torch.float32 and bias_tensor.numel() == 1
+        p.bias_ptr = bias_tensor.data_ptr()
+    if score_mask is not None:
+        assert score_mask.dtype == q.dtype and score_mask.dim() == 4 and score_mask.stride(-1) == 1
+        assert score_mask.shape[1:] == (H, Sq, Skv) and score_mask.shape[0] in (1, B)
+        p.score_mask = score_mask.data_ptr()
+        p.sm_stride_b = score_mask.stride(0) if score_mask.shape[0] > 1 else 0
+        p.sm_stride_h, p.sm_stride_q = score_mask.stride(1), score_mask.stride(2)
+    _check(load_library().ma_attn_fwd(ctypes.byref(p), _stream()))
+    return out
