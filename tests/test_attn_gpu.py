@@ -1,0 +1,119 @@
+"""Parity of the HIP parallel-attention forward (through the C ABI) with the
+CPU oracle on identical seeded inputs.  Tolerance: atol 2e-2, rtol 1e-2 on
+fp32-accumulated bf16 results; masking checked exactly."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from oracle import inputs
+
+pytestmark = pytest.mark.gpu
+ATOL, RTOL = 2e-2, 1e-2
+
+
+def _hb():
+    from metaattention_amd import hip_backend as hb
+    hb.load_library()
+    return hb
+
+
+@pytest.mark.parametrize("B,H,S,causal", [
+    (1, 2, 128, True), (2, 3, 256, True), (1, 2, 512, False), (1, 1, 64, True),
+    (1, 2, 200, True), (1, 2, 333, False), (1, 1, 1, True), (1, 2, 129, True), (1, 1, 1000, False),
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_softmax_forward(B, H, S, causal, dtype):
+    hb = _hb()
+    D = 128
+    q, k, v = inputs.softmax_inputs(B, H, S, D, D, dtype=dtype, seed=S)
+    ref, lse_ref = oracle.softmax_attention(q, k, v, causal=causal, return_lse=True)
+    lse = torch.full((B, H, S), float("nan"), device="cuda")
+    print(f"softmax B{B} H{H} S{S} causal={causal} {dtype}", flush=True)
+    o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_SOFTMAX, causal=causal,
+                    scale=1 / math.sqrt(D), row_scale=lse)
+    torch.cuda.synchronize()
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(lse.cpu(), lse_ref, rtol=1e-4, atol=1e-4)
+
+
+def test_softmax_full_size_property():
+    """Full benchmark shape: compare a few (batch, head) slices against the oracle
+    and check that lse is finite everywhere and the first row reproduces V
+    (row 0 of a causal softmax attends only to kv 0)."""
+    hb = _hb()
+    B, H, S, D = 8, 32, 4096, 128
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q, k, v = (torch.randn(B, S, H, D, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(3))
+    lse = torch.empty(B, H, S, device="cuda")
+    o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=1 / math.sqrt(D), row_scale=lse)
+    torch.cuda.synchronize()
+    assert torch.isfinite(lse).all() and torch.isfinite(o.float()).all()
+    assert torch.equal(o[:, 0], v[:, 0])
+    for b, h in [(0, 0), (7, 31), (3, 17)]:
+        ref = oracle.softmax_attention(q[b:b + 1, :, h:h + 1].cpu(), k[b:b + 1, :, h:h + 1].cpu(),
+                                       v[b:b + 1, :, h:h + 1].cpu(), causal=True)
+        oracle.assert_close(o[b:b + 1, :, h:h + 1].float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_causal_mask_is_exact():
+    """Future keys must have exactly zero influence: poisoning k/v at positions
+    > i must not change row i bit-for-bit."""
+    hb = _hb()
+    B, H, S, D = 1, 2, 256, 128
+    q, k, v = (t.cuda() for t in inputs.softmax_inputs(B, H, S, D, D, seed=5))
+    o1 = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=0.1)
+    cut = 100
+    k2, v2 = k.clone(), v.clone()
+    k2[:, cut:] = 1e4
+    v2[:, cut:] = -1e4
+    for fam in (hb.MA_ATTN_SOFTMAX, hb.MA_ATTN_SIGMOID, hb.MA_ATTN_RELU):
+        oa = hb.attn_fwd(q, k, v, family=fam, causal=True, scale=0.1)
+        ob = hb.attn_fwd(q, k2, v2, family=fam, causal=True, scale=0.1)
+        torch.cuda.synchronize()
+        assert torch.equal(oa[:, :cut], ob[:, :cut])
+    assert torch.isfinite(o1.float()).all()
+
+
+@pytest.mark.parametrize("S,causal,scale,bias", [(256, True, 1.0, -3.0), (192, False, 0.088, -5.5), (130, True, 0.088, 0.5)])
+def test_sigmoid_forward(S, causal, scale, bias):
+    hb = _hb()
+    B, H, D = 1, 2, 128
+    q, k, v = inputs.softmax_inputs(B, H, S, D, D, seed=7)
+    if scale == 1.0:   # the unscaled spec is used with small-norm inputs
+        q = (q.float() * 0.3).bfloat16()
+    ref = oracle.sigmoid_attention(q, k, v, bias, causal=causal, softmax_scale=scale)
+    bt = torch.tensor([bias], device="cuda")
+    o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_SIGMOID, causal=causal, scale=scale, bias_tensor=bt)
+    o2 = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_SIGMOID, causal=causal, scale=scale, bias=bias)
+    torch.cuda.synchronize()
+    assert torch.equal(o, o2)
+    # sums of S un-normalised probabilities: tolerance as a fraction of elements, like the reference's own check
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=2e-3)
+
+
+def test_relu_forward():
+    hb = _hb()
+    B, H, S, D = 1, 2, 256, 128
+    q, k, v = inputs.softmax_inputs(B, H, S, D, D, seed=9)
+    k, v = (k.float() * 0.5).bfloat16(), (v.float() * 0.5).bfloat16()   # input scaling of testing/test.py:609-610
+    ref = oracle.relu_attention(q, k, v)
+    o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_RELU, causal=False, scale=1 / math.sqrt(D))
+    torch.cuda.synchronize()
+    # reference acceptance for this family: rtol=atol=1e-1, 1e-3 of elements may miss (testing/test.py:623)
+    oracle.assert_close(o.float().cpu(), ref, rtol=1e-1, atol=1e-1, mismatch_ratio=1e-3)
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=5e-2)
+
+
+def test_rejects_bad_arguments():
+    hb = _hb()
+    q = torch.zeros(1, 64, 1, 128, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(hb.MetaAttentionError):
+        hb.attn_fwd(q, q, q, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=-1.0)
+    q96 = torch.zeros(1, 64, 1, 96, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(hb.MetaAttentionError) as ei:
+        hb.attn_fwd(q96, q96, q96, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=1.0)
+    assert "no kernel" in str(ei.value)
+    with pytest.raises(hb.MetaAttentionError):
+        hb.attn_fwd(q.cpu(), q.cpu(), q.cpu(), family=hb.MA_ATTN_SOFTMAX, causal=True, scale=1.0)
