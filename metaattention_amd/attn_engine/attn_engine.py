@@ -1,0 +1,191 @@
+"""``AttentionEngine`` / ``OnlineFunc``: the public spec API of the parallel,
+decode and MLA operators (attention_engine/attn_engine/attn_engine.py:16-408),
+backed by the pre-built gfx950 kernel library instead of run-time code
+generation.
+
+Construction traces the user's spec, canonicalises it (core/canonical.py) and
+picks a kernel variant; nothing is compiled, tuned or cached on disk.  The
+call takes GPU tensors in the reference's layouts and enqueues the kernels on
+the current stream.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from core.canonical import canonicalize_score_mod, classify_mask, identify_online_func
+from core.transform.core import CustomIO, SymbolicArray, SymbolScalar, Var
+from autotuner.arch import MI355X
+
+
+class OnlineFunc:
+    """Row function of an online (tiled) attention forward.
+
+    ``online_rowscales``: running per-row statistics, each a
+    ``SymbolScalar(name, Var(init))`` with init "-inf", "0.0" or "1";
+    ``final_rowscales``: what is kept after the last tile.
+    ``online_fwd(scores, online_rowscales, b, h, q_idx)`` returns
+    ``(scores', online_rowscales', o_scale)``: the probabilities of this tile,
+    the updated statistics and the factor the output accumulator is rescaled
+    by.  ``online_fwd_epilogue(o, online_rowscales, b, h, q_idx)`` returns
+    ``(o', final_rowscales)``.  ``forward`` / ``backward`` describe the
+    recompute for a backward pass and ``combine`` the split-KV merge; they are
+    part of the contract but unused by the forward kernels here.
+    """
+
+    def __init__(self, online_rowscales: dict, final_rowscales: dict, external_fwd_tensors: CustomIO):
+        self.online_rowscales = online_rowscales
+        self.final_rowscales = final_rowscales
+        self.vars = {"scores": SymbolicArray(), "o_scale": None}
+        self.external_fwd_tensors = external_fwd_tensors
+        self.doosum_rowscales = SymbolicArray("doosum", Var("doosum"), shape_idx=["block_M"])
+
+    @staticmethod
+    def online_fwd(scores, online_rowscales, b, h, q_idx):
+        return scores, online_rowscales, SymbolScalar("o_scale", Var("o_scale"))
+
+    @staticmethod
+    def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+        return o, online_rowscales
+
+    @staticmethod
+    def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
+        return scores
+
+    @staticmethod
+    def backward(dp, scores, final_rowscales, b, h, q_idx, kv_idx):
+        return dp
+
+    @staticmethod
+    def combine(final_rowscales):
+        return SymbolScalar("o_scale", Var("o_scale"))
+
+
+_FAMILY = {
+    ("identity", "softmax"): "softmax",
+    ("sigmoid", "identity"): "sigmoid",
+    ("relu", "identity"): "relu",
+    ("identity", "retention"): "retention",
+}
+
+
+class _ForwardOnly(torch.autograd.Function):
+    """Gives outputs a grad_fn whose backward fails loudly: the library holds
+    forward kernels only."""
+
+    @staticmethod
+    def forward(ctx, run, *tensors):
+        return run(*tensors)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("this operator is forward-only: backward kernels are not part of the gfx950 kernel library")
+
+
+class AttentionEngine:
+    def __init__(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func,
+                 mask_value="-inf", device=None, backend="tl",
+                 tune=False, tune_file="", tune_bwd=False, tune_file_bwd="",
+                 infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=128,
+                 extern_block_mask=False, use_varlen=False, kv_shared=False):
+        # `backend`, `tune*`, `infer_mask*` select code generators / tuners in the
+        # reference; here there is one pre-built backend and fixed tile tables, so
+        # they are accepted and ignored.
+        self.device = device if device is not None else MI355X()
+        self.use_varlen = use_varlen
+        self.block_mask = None
+        self.tl_code = ""     # no source is generated
+        if use_varlen or extern_block_mask:
+            raise NotImplementedError("varlen / external block masks are not in the kernel library")
+        dtype = qkv_meta[0].dtype
+        if dtype not in (torch.float16, torch.bfloat16):
+            raise KeyError(dtype)      # the reference's dtype map has only these two (attn_engine.py:234-237)
+        self.dtype = dtype
+        B, Hq, Sq, Dqk = qkv_meta[0].shape
+        Hkv, Skv, Dv = qkv_meta[2].shape[1], qkv_meta[2].shape[2], qkv_meta[2].shape[3]
+        self.meta = dict(B=B, Hq=Hq, Hkv=Hkv, Sq=Sq, Skv=Skv, Dqk=Dqk, Dv=Dv)
+        self.custom_fwd_inputs = custom_fwd_inputs if custom_fwd_inputs is not None else CustomIO()
+
+        # dispatch by shape, as attn_engine.py:227-343
+        if kv_shared:
+            self._init_mla()
+        elif Sq != Skv:
+            raise NotImplementedError("decode (seq_len_q != seq_len_kv) operators other than MLA are not in the kernel library")
+        elif Hq != Hkv:
+            raise NotImplementedError("grouped-query prefill is not in the kernel library")
+        else:
+            self._init_prefill(score_mod, mask_mod, online_func, mask_value)
+
+    # ------------------------------------------------------------------ prefill
+    def _init_prefill(self, score_mod, mask_mod, online_func, mask_value):
+        m = self.meta
+        form = canonicalize_score_mod(score_mod, self.custom_fwd_inputs)
+        row = identify_online_func(online_func)
+        fam = _FAMILY.get((form.activation, row))
+        if fam is None:
+            raise NotImplementedError(f"no library kernel for score activation '{form.activation}' with row function '{row}'")
+        if fam == "retention" and form.mask_tensor is None:
+            raise NotImplementedError("retention row function without an element-wise score multiplier tensor")
+        if fam != "retention" and form.mask_tensor is not None:
+            raise NotImplementedError("element-wise score multiplier tensors are only in the retention kernel")
+        if not form.scale > 0:
+            raise NotImplementedError("score scale must be positive")
+        if mask_value not in ("-inf", "0"):
+            raise NotImplementedError(f"mask_value {mask_value!r}")
+        self.mask_kind = classify_mask(mask_mod, m["B"], m["Hq"], m["Sq"], m["Skv"])
+        # mask_value "0": the reference applies no element-wise mask in forward, only causal
+        # tile skipping (lower.py:638, attn_tl.py:140-151); the retention kernel does the same.
+        if mask_value == "0" and fam != "retention" and self.mask_kind != "none":
+            raise NotImplementedError("mask_value '0' is only in the retention kernel")
+        self.family, self.score_form = fam, form
+        self.names = list(self.custom_fwd_inputs.input_tensors)
+        self.final_rowscales = None
+        self.attention = self._call_prefill
+
+    def _call_prefill(self, q, k, v, *custom):
+        from hip_backend import attn_fwd, MA_ATTN_SOFTMAX, MA_ATTN_SIGMOID, MA_ATTN_RELU, MA_ATTN_RETENTION
+        fam_code = {"softmax": MA_ATTN_SOFTMAX, "sigmoid": MA_ATTN_SIGMOID, "relu": MA_ATTN_RELU,
+                    "retention": MA_ATTN_RETENTION}[self.family]
+        if len(custom) != len(self.names):
+            raise TypeError(f"expected {len(self.names)} custom tensor(s) {self.names} after q, k, v; got {len(custom)}")
+        given = dict(zip(self.names, custom))
+        form = self.score_form
+
+        def run(q, k, v):
+            B, Sq, H, _ = q.shape
+            rs = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if self.family in ("softmax", "retention") else None
+            bias_t = given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None
+            mask_t = given[form.mask_tensor] if form.mask_tensor else None
+            if mask_t is not None and mask_t.dtype != q.dtype:
+                mask_t = mask_t.to(q.dtype)
+            out = attn_fwd(q, k, v, family=fam_code, causal=self.mask_kind == "causal", scale=form.scale, bias=form.bias,
+                           bias_tensor=bias_t, score_mask=mask_t, row_scale=rs)
+            self.final_rowscales = rs     # kept for a backward pass, not returned (attn_tl.py:661-667)
+            return out
+
+        if any(t.requires_grad for t in (q, k, v)):
+            return _ForwardOnly.apply(run, q, k, v)
+        return run(q, k, v)
+
+    # ------------------------------------------------------------------ MLA decode
+    def _init_mla(self):
+        m = self.meta
+        if m["Hkv"] != 1:
+            raise AssertionError("MLA decode needs a single latent kv head")   # mla_decode_tl.py:58
+        if m["Sq"] != 1:
+            raise NotImplementedError("MLA decode takes one query token")
+        self.mla_dim, self.mla_pe = m["Dv"], m["Dqk"] - m["Dv"]
+        # the spec's score_mod / online_func are not consumed on this path
+        # (core/lower/lower_decode_mla.py:25-38): fixed softmax, scale (d + d_pe)^-0.5
+        self.mla_scale = 1.0 / math.sqrt(m["Dqk"])
+        self.attention = self._call_mla
+
+    def _call_mla(self, q, q_pe, kv, k_pe):
+        from hip_backend import mla_decode
+        return mla_decode(q, q_pe, kv, k_pe, scale=self.mla_scale)
+
+    def __call__(self, *args, **kargs):
+        if kargs.get("block_mask") is not None:
+            raise NotImplementedError("block masks are not in the kernel library")
+        return self.attention(*args)

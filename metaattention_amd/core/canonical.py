@@ -1,0 +1,435 @@
+"""Canonicaliser: traced spec -> kernel selection.
+
+The reference prints every traced spec as kernel source
+(attention_engine/core/lower/lower.py:319-559, lower_linear.py:138-409).  This
+package ships a fixed kernel library instead, so a traced spec is reduced to a
+small normal form and matched against the library:
+
+* ``score_mod`` is reduced algebraically to ``act(a * score [* T] + b + t)``
+  with ``act`` in {identity, sigmoid, relu}, ``a``/``b`` python constants, ``t``
+  an optional one-element custom tensor and ``T`` an optional
+  [.., seq_len, seq_len_kv] custom tensor (an element-wise score multiplier);
+* the ``OnlineFunc`` is identified behaviourally: its traced ``online_fwd`` /
+  ``online_fwd_epilogue`` are run by the spec interpreter on random tiles and
+  compared with each library row function, so algebraically equivalent
+  spellings of the same row function are accepted;
+* the linear-attention mods are reduced to a q scale, a per-token v scale and
+  a traced decay function.
+
+Anything outside the library raises ``NotImplementedError`` naming what was not
+recognised; nothing is silently approximated.
+"""
+from __future__ import annotations
+
+import itertools
+import math
+from dataclasses import dataclass, field
+from typing import Dict, Optional
+
+import torch
+
+from .eager import evaluate, leaves
+from .transform.core import SymbolicArray, SymbolScalar, Var
+
+SEQ_TOKENS = ("seq_len", "seq_len_kv")
+
+
+# ---------------------------------------------------------------------------
+# score_mod: algebraic reduction
+# ---------------------------------------------------------------------------
+@dataclass
+class Affine:
+    """a * score * [mask] + sum_t coef_t * t + c   (t: one-element tensors)"""
+    a: float = 0.0
+    mask: Optional[str] = None
+    tensors: Dict[str, float] = field(default_factory=dict)
+    c: float = 0.0
+    tile: Optional[str] = None   # a bare [.., seq_len, seq_len_kv] tensor (not yet multiplied with the score)
+
+    def is_const(self):
+        return self.a == 0.0 and not self.tensors and self.tile is None
+
+    def scaled(self, f: float):
+        if self.tile is not None:
+            raise NotImplementedError("scaling a bare tile tensor")
+        return Affine(self.a * f, self.mask, {k: v * f for k, v in self.tensors.items()}, self.c * f)
+
+
+@dataclass
+class Activated:
+    """p * fn(inner) + q"""
+    fn: str
+    inner: Affine
+    p: float = 1.0
+    q: float = 0.0
+
+
+@dataclass
+class ScoreForm:
+    activation: str            # "identity" | "sigmoid" | "relu"
+    scale: float
+    bias: float
+    bias_tensor: Optional[str]
+    mask_tensor: Optional[str]
+
+
+def _is_tile_tensor(sym) -> bool:
+    return "seq_len_kv" in sym.shape_idx
+
+
+def _reduce_score(sym: SymbolScalar, score_id: int, custom: dict):
+    t = sym.code.type
+    if id(sym) == score_id:
+        return Affine(a=1.0)
+    if t == "Const":
+        return Affine(c=float(sym.code.value))
+    if t == "Var" and not sym.prev:
+        name = sym.varname
+        if name in custom and custom[name] is sym:
+            if _is_tile_tensor(sym):
+                return Affine(tile=name)
+            numel_tokens = [x for x in sym.shape_idx if x not in ("1",)]
+            if numel_tokens:
+                raise NotImplementedError(
+                    f"score_mod: custom tensor '{name}' of shape {sym.shape_idx} is neither a one-element tensor nor a "
+                    f"[.., seq_len, seq_len_kv] tile")
+            return Affine(tensors={name: 1.0})
+        try:
+            return Affine(c=float(sym.code.name))
+        except ValueError:
+            raise NotImplementedError(f"score_mod uses '{name}', which the kernel library does not provide "
+                                      f"(index-dependent score functions are not in the library)") from None
+    ins = [_reduce_score(p, score_id, custom) for p in sym.prev]
+    if t == "Neg":
+        return _scale(ins[0], -1.0)
+    if t in ("Add", "Sub"):
+        x, y = ins
+        if t == "Sub":
+            y = _scale(y, -1.0)
+        return _add(x, y)
+    if t == "Mul":
+        x, y = ins
+        if isinstance(y, Affine) and y.is_const():
+            return _scale(x, y.c)
+        if isinstance(x, Affine) and x.is_const():
+            return _scale(y, x.c)
+        if isinstance(x, Affine) and isinstance(y, Affine):
+            for u, w in ((x, y), (y, x)):
+                if w.tile is not None and u.tile is None and u.mask is None and not u.tensors and u.c == 0.0 and u.a != 0.0:
+                    return Affine(a=u.a, mask=w.tile)
+        raise NotImplementedError("score_mod: product of two non-constant terms other than score * tile tensor")
+    if t == "Div":
+        x, y = ins
+        if isinstance(y, Affine) and y.is_const():
+            return _scale(x, 1.0 / y.c)
+        if isinstance(x, Affine) and x.is_const() and isinstance(y, Activated) and y.fn == "exp" and y.p == 1.0 and y.q == 1.0:
+            # c / (1 + exp(u)) = c * sigmoid(-u)
+            return Activated("sigmoid", y.inner.scaled(-1.0), p=x.c, q=0.0)
+        raise NotImplementedError("score_mod: division by a non-constant term")
+    if t in ("Tanh", "Exp"):
+        (x,) = ins
+        if not isinstance(x, Affine) or x.tile is not None:
+            raise NotImplementedError(f"score_mod: {t} of a non-affine term")
+        return Activated(t.lower(), x)
+    if t == "Max":
+        x, y = ins
+        if isinstance(y, Affine) and y.is_const() and y.c == 0.0 and isinstance(x, Affine):
+            return Activated("relu", x)
+        if isinstance(x, Affine) and x.is_const() and x.c == 0.0 and isinstance(y, Affine):
+            return Activated("relu", y)
+        raise NotImplementedError("score_mod: max() other than max(affine, 0)")
+    raise NotImplementedError(f"score_mod: op {t} is not in the kernel library")
+
+
+def _scale(x, f: float):
+    if isinstance(x, Affine):
+        return x.scaled(f)
+    return Activated(x.fn, x.inner, x.p * f, x.q * f)
+
+
+def _add(x, y):
+    if isinstance(x, Affine) and isinstance(y, Affine):
+        if x.tile is not None or y.tile is not None:
+            raise NotImplementedError("score_mod: adding a tile tensor to the score (additive bias tiles are not in the library)")
+        if x.a != 0.0 and y.a != 0.0 and x.mask != y.mask:
+            raise NotImplementedError("score_mod: score terms with different multipliers")
+        tensors = dict(x.tensors)
+        for k, v in y.tensors.items():
+            tensors[k] = tensors.get(k, 0.0) + v
+        return Affine(x.a + y.a, x.mask if x.a != 0.0 else y.mask, tensors, x.c + y.c)
+    if isinstance(x, Activated) and isinstance(y, Affine) and y.is_const():
+        return Activated(x.fn, x.inner, x.p, x.q + y.c)
+    if isinstance(y, Activated) and isinstance(x, Affine) and x.is_const():
+        return Activated(y.fn, y.inner, y.p, y.q + x.c)
+    raise NotImplementedError("score_mod: sum of two activated terms")
+
+
+def _close(a: float, b: float) -> bool:
+    return abs(a - b) <= 1e-6 * max(1.0, abs(b))
+
+
+def canonicalize_score_mod(score_mod, custom_fwd_inputs) -> ScoreForm:
+    score = SymbolScalar("scores", Var("scores"), shape_idx=["block_M", "block_N"])
+    idx = [SymbolScalar(n, Var(n)) for n in ("b", "h", "q_idx", "kv_idx")]
+    out = score_mod(score, custom_fwd_inputs, *idx) if score_mod is not None else score
+    form = _reduce_score(out, id(score), custom_fwd_inputs.input_tensors)
+    if isinstance(form, Activated):
+        inner, act = form.inner, None
+        if form.fn == "tanh" and _close(form.p, 0.5) and _close(form.q, 0.5):
+            inner, act = inner.scaled(2.0), "sigmoid"      # (tanh(x)+1)/2 = sigmoid(2x)
+        elif form.fn == "sigmoid" and _close(form.p, 1.0) and _close(form.q, 0.0):
+            act = "sigmoid"
+        elif form.fn == "relu" and _close(form.q, 0.0) and form.p > 0:
+            inner, act = inner.scaled(form.p), "relu"      # p*max(x,0) = max(p*x,0) for p>0
+        if act is None:
+            raise NotImplementedError(f"score_mod: {form.p}*{form.fn}(.)+{form.q} is not a library activation")
+    else:
+        inner, act = form, "identity"
+    if inner.tile is not None or inner.a == 0.0:
+        raise NotImplementedError("score_mod does not depend linearly on the score")
+    bias_tensor = None
+    if inner.tensors:
+        if len(inner.tensors) > 1:
+            raise NotImplementedError("score_mod: more than one bias tensor")
+        (bias_tensor, coef), = inner.tensors.items()
+        if not _close(coef, 1.0):
+            raise NotImplementedError("score_mod: bias tensor with a coefficient other than 1")
+    if act != "identity" and inner.mask is not None:
+        raise NotImplementedError("score_mod: activation of a tile-multiplied score")
+    return ScoreForm(act, inner.a, inner.c, bias_tensor, inner.mask)
+
+
+# ---------------------------------------------------------------------------
+# OnlineFunc: behavioural identification
+# ---------------------------------------------------------------------------
+def _lib_softmax(s, st):
+    m, r = st
+    m_new = torch.maximum(m, s.amax(-1, keepdim=True))
+    c = torch.exp(m - m_new)
+    p = torch.exp(s - m_new)
+    return p, c, (m_new, r * c + p.sum(-1, keepdim=True))
+
+
+def _lib_identity(s, st):
+    return s, torch.ones_like(s[..., :1]), ()
+
+
+def _lib_retention(s, st):
+    r_wo, r = st
+    r_wo_new = r_wo + s.abs().sum(-1, keepdim=True)
+    r_new = torch.clamp(r_wo_new, min=1.0)
+    return s / r_new, r / r_new, (r_wo_new, r_new)
+
+
+ROW_FUNCTIONS = {
+    # name: (fn, state init values, epilogue(o, state) -> (o', final scale or None))
+    "softmax": (_lib_softmax, (float("-inf"), 0.0), lambda o, st: (o / st[1], torch.log(st[1]) + st[0])),
+    "identity": (_lib_identity, (), lambda o, st: (o, None)),
+    "retention": (_lib_retention, (0.0, 0.0), lambda o, st: (o, st[1])),
+}
+
+
+def _random_state(name, M, gen, magnitude=1.0):
+    """Plausible running statistics; ``magnitude`` scales them with the scores so
+    that both sides of a clamp / max are exercised."""
+    if name == "softmax":
+        return (torch.randn(M, 1, generator=gen, dtype=torch.float64), torch.rand(M, 1, generator=gen, dtype=torch.float64) + 0.5)
+    if name == "retention":
+        r_wo = torch.rand(M, 1, generator=gen, dtype=torch.float64) * 2.0 * min(magnitude, 1.0)
+        return (r_wo, torch.clamp(r_wo, min=1.0))
+    return ()
+
+
+def identify_online_func(online_func) -> str:
+    """Returns the name of the library row function ``online_func`` computes."""
+    idx = [SymbolScalar(n, Var(n)) for n in ("b", "h", "q_idx")]
+    state_syms = dict(online_func.online_rowscales)
+    names = list(state_syms)
+    try:
+        inits = tuple(float(s.code.name) for s in state_syms.values())
+    except ValueError as e:
+        raise NotImplementedError(f"online_rowscales initial value not a literal: {e}") from None
+    tile_in = SymbolicArray("scores_online", Var("scores_online"))
+    tile_out, state_out, o_scale = online_func.online_fwd(tile_in, dict(state_syms), *idx)
+    acc_in = SymbolicArray("acc_o", Var("acc_o"), shape_idx=["block_M", "dimv"])
+    acc_out, finals = online_func.online_fwd_epilogue(acc_in, dict(state_syms), *idx)
+    if set(state_out) != set(names):
+        raise NotImplementedError("online_fwd must return every online_rowscale it was given")
+    for sym in leaves([tile_out, o_scale, acc_out] + list(state_out.values()) + list(finals.values())):
+        if sym.code.type == "Var" and sym is not tile_in and sym is not acc_in and all(sym is not s for s in state_syms.values()):
+            try:
+                float(sym.code.name)
+            except ValueError:
+                raise NotImplementedError(f"online_func reads '{sym.varname}', which the kernel library does not provide") from None
+
+    gen = torch.Generator().manual_seed(1234)
+    M, N, DV = 5, 7, 3
+    tried = []
+    for lib_name, (fn, lib_inits, epi) in ROW_FUNCTIONS.items():
+        if len(lib_inits) != len(names):
+            continue
+        for perm in itertools.permutations(range(len(names))):
+            # perm[i] = index of the user's state variable that plays library role i
+            if any(not _same_init(inits[perm[i]], lib_inits[i]) for i in range(len(lib_inits))):
+                continue
+            ok = True
+            for magnitude in (2.0, 0.02, 0.2):
+                s = torch.randn(M, N, generator=gen, dtype=torch.float64) * magnitude
+                st = _random_state(lib_name, M, gen, magnitude)
+                env = {id(tile_in): s}
+                for i, j in enumerate(perm):
+                    env[id(state_syms[names[j]])] = st[i]
+                got = evaluate([tile_out, o_scale] + [state_out[names[j]] for j in perm], env, s)
+                exp_p, exp_c, exp_st = fn(s, st)
+                ok &= _allclose(got[0], exp_p) and _allclose(got[1], exp_c)
+                ok &= all(_allclose(g, e) for g, e in zip(got[2:], exp_st))
+                o = torch.randn(M, DV, generator=gen, dtype=torch.float64)
+                env = {id(acc_in): o}
+                for i, j in enumerate(perm):
+                    env[id(state_syms[names[j]])] = st[i]
+                got = evaluate([acc_out] + list(finals.values()), env, o)
+                exp_o, exp_final = epi(o, st)
+                ok &= _allclose(got[0], exp_o)
+                if exp_final is None:
+                    ok &= len(got) == 1
+                else:
+                    ok &= len(got) == 2 and _allclose(got[1], exp_final)
+                if not ok:
+                    break
+            if ok:
+                return lib_name
+        tried.append(lib_name)
+    raise NotImplementedError(
+        f"OnlineFunc with row scales {names} (initial values {inits}) matches no library row function "
+        f"(softmax, identity, retention); compared against: {tried or 'none with that many row scales'}")
+
+
+def _same_init(a: float, b: float) -> bool:
+    return (math.isinf(a) and math.isinf(b) and a == b) or a == b
+
+
+def _allclose(a, b) -> bool:
+    if a.shape != b.shape:
+        try:
+            a, b = torch.broadcast_tensors(a, b)
+        except RuntimeError:
+            return False
+    return bool(torch.allclose(a, b, rtol=1e-9, atol=1e-11, equal_nan=False))
+
+
+# ---------------------------------------------------------------------------
+# mask_mod
+# ---------------------------------------------------------------------------
+def classify_mask(mask_mod, B, H, Sq, Skv, block_M=128, block_N=128) -> str:
+    """"none" | "causal".  Evaluates ``mask_mod`` densely on index grids on
+    the CPU (as the reference does at block granularity, lower.py:723-740) and
+    compares with the exact causal pattern; every (batch, head) must agree."""
+    from .transform.core import create_mask
+    if mask_mod is None:
+        return "none"
+    qi = torch.arange(Sq).view(Sq, 1)
+    kj = torch.arange(Skv).view(1, Skv)
+    causal = qi >= kj
+    kinds = set()
+    for b in sorted({0, B - 1}):
+        for h in sorted({0, H // 2, H - 1}):
+            m = mask_mod(torch.tensor(b), torch.tensor(h), qi, kj)
+            m = m if torch.is_tensor(m) else torch.full((Sq, Skv), bool(m))
+            m = m.expand(Sq, Skv)
+            if torch.equal(m, causal):
+                kinds.add("causal")
+            elif bool(m.all()):
+                kinds.add("none")
+            else:
+                kinds.add("other")
+    if kinds == {"causal"}:
+        return "causal"
+    if kinds == {"none"}:
+        return "none"
+    raise NotImplementedError(
+        "mask_mod is neither the causal mask (q_idx >= kv_idx) nor all-true; block-sparse and shifted masks are not "
+        "in the kernel library")
+
+
+# ---------------------------------------------------------------------------
+# linear-attention mods
+# ---------------------------------------------------------------------------
+@dataclass
+class LinearPlan:
+    q_scale: float = 1.0
+    v_scale_tensor: Optional[str] = None      # custom tensor ("batch","heads","seq_len") multiplying v per token
+    decay_sym: Optional[SymbolScalar] = None  # traced decay_mod output (None: decay is already the log decay)
+    decay_in: Optional[SymbolScalar] = None
+    decay_kind: str = "identity"              # "identity" | "log" | "mul_head" | "traced"
+    decay_head_tensor: Optional[str] = None
+
+
+def _reduce_linear(sym, x_id, custom):
+    """-> (coef, token_scale_tensor|None) with out = coef * x [* tensor]"""
+    t = sym.code.type
+    if id(sym) == x_id:
+        return (1.0, None)
+    if t == "Const":
+        return ("const", float(sym.code.value))
+    if t == "Var" and not sym.prev:
+        if sym.varname in custom and custom[sym.varname] is sym:
+            return ("tensor", sym.varname)
+        raise NotImplementedError(f"mod uses unknown symbol '{sym.varname}'")
+    ins = [_reduce_linear(p, x_id, custom) for p in sym.prev]
+    if t in ("Mul", "Div"):
+        a, b = ins
+        if t == "Div":
+            if b[0] != "const":
+                raise NotImplementedError("mod: division by a non-constant")
+            b = ("const", 1.0 / b[1])
+        for u, w in ((a, b), (b, a)):
+            if isinstance(u[0], float):
+                if w[0] == "const":
+                    return (u[0] * w[1], u[1])
+                if w[0] == "tensor" and u[1] is None:
+                    return (u[0], w[1])
+        if a[0] == "const" and b[0] == "const":
+            return ("const", a[1] * b[1])
+    if t == "Neg" and isinstance(ins[0][0], float):
+        return (-ins[0][0], ins[0][1])
+    raise NotImplementedError(f"mod: op {t} is not a scaling of its input")
+
+
+def canonicalize_linear_mods(q_mod, k_mod, v_mod, decay_mod, custom_io) -> LinearPlan:
+    custom = custom_io.input_tensors if custom_io is not None else {}
+    plan = LinearPlan()
+
+    def trace(mod, name, shape):
+        x = SymbolScalar(name, Var(name), shape_idx=shape)
+        return x, mod(x, custom_io)
+
+    for mod, name in ((q_mod, "q"), (k_mod, "k")):
+        if mod is None:
+            continue
+        x, out = trace(mod, name, ["batch", "heads", "seq_len", "dim"])
+        coef, tensor = _reduce_linear(out, id(x), custom)
+        if tensor is not None:
+            raise NotImplementedError(f"{name}_mod: multiplying by a tensor is not in the kernel library")
+        plan.q_scale *= coef       # the operator is bilinear in q and k: a k scale folds into the q scale
+    if v_mod is not None:
+        x, out = trace(v_mod, "v", ["batch", "heads", "seq_len", "dimv"])
+        coef, tensor = _reduce_linear(out, id(x), custom)
+        plan.q_scale *= coef
+        if tensor is not None:
+            shp = custom[tensor].shape_idx
+            if shp != ["batch", "heads", "seq_len"]:
+                raise NotImplementedError(f"v_mod: tensor '{tensor}' must have shape (batch, heads, seq_len), got {shp}")
+            plan.v_scale_tensor = tensor
+    if decay_mod is not None:
+        x, out = trace(decay_mod, "decay", ["batch", "heads", "seq_len"])
+        plan.decay_sym, plan.decay_in = out, x
+        plan.decay_kind = "traced"
+        if out.code.type == "Log" and out.prev[0] is x:
+            plan.decay_kind = "log"
+        elif out.code.type == "Mul":
+            a, b = out.prev
+            other = b if a is x else a if b is x else None
+            if other is not None and other.code.type == "Var" and other.varname in custom \
+                    and custom[other.varname].shape_idx == ["1", "heads"]:
+                plan.decay_kind, plan.decay_head_tensor = "mul_head", other.varname
+    return plan
