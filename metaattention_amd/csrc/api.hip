@@ -2,6 +2,7 @@
 // error strings, kernel selection.  No allocation, no synchronisation.
 #include "../../include/metaattention_hip.h"
 #include "attn_fwd.h"
+#include "mla_decode.h"
 
 #include <cstdarg>
 #include <cstdio>
@@ -68,11 +69,66 @@ int ma_linear_fwd(const ma_linear_params* p, ma_stream_t stream) {
   (void)p; (void)stream;
   return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: not built yet");
 }
-int ma_mla_choose_split(const ma_mla_params* p) { (void)p; return 1; }
-size_t ma_mla_workspace_bytes(const ma_mla_params* p) { (void)p; return 0; }
+// Split count: enough workgroups to fill the 256 CUs once, each split a whole
+// number of 64-row tiles, and never more splits than tiles.
+int ma_mla_choose_split(const ma_mla_params* p) {
+  if (!p || p->batch <= 0 || p->heads_q <= 0 || p->seqlen_kv <= 0) return 1;
+  const int head_blocks = (p->heads_q + 63) / 64;
+  const int tiles = (p->seqlen_kv + 63) / 64;
+  int split = 256 / (p->batch * head_blocks);
+  if (split < 1) split = 1;
+  if (split > tiles) split = tiles;
+  if (split > 64) split = 64;
+  return split;
+}
+
+static int mla_split_of(const ma_mla_params* p) { return p->num_split > 0 ? p->num_split : ma_mla_choose_split(p); }
+
+size_t ma_mla_workspace_bytes(const ma_mla_params* p) {
+  if (!p) return 0;
+  const int ns = mla_split_of(p);
+  if (ns <= 1) return 0;
+  return (size_t)p->batch * ns * p->heads_q * ((size_t)p->dim + 1) * sizeof(float);
+}
+
 int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
-  (void)p; (void)stream;
-  return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: not built yet");
+  if (!p) return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: params is NULL");
+  if (!p->q || !p->q_pe || !p->kv || !p->k_pe || !p->o) return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: q/q_pe/kv/k_pe/o must be non-NULL");
+  if (p->batch <= 0 || p->heads_q <= 0 || p->seqlen_kv <= 0)
+    return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: sizes must be positive (B=%d Hq=%d Skv=%d)", p->batch, p->heads_q, p->seqlen_kv);
+  if (p->dtype != MA_BF16 && p->dtype != MA_FP16) return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: dtype %d", p->dtype);
+  if (!(p->scale > 0.f)) return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: scale must be > 0");
+  if (p->batch > 65535) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: batch > 65535");
+  const int64_t strides[] = {p->q_stride_b, p->q_stride_h, p->qpe_stride_b, p->qpe_stride_h, p->kv_stride_b, p->kv_stride_s,
+                             p->kpe_stride_b, p->kpe_stride_s, p->o_stride_b, p->o_stride_h};
+  for (int64_t s : strides)
+    if (s % 8 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: strides must be multiples of 8 elements");
+  const uintptr_t ptrs[] = {(uintptr_t)p->q, (uintptr_t)p->q_pe, (uintptr_t)p->kv, (uintptr_t)p->k_pe, (uintptr_t)p->o};
+  for (uintptr_t x : ptrs)
+    if (x % 16 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: tensors must be 16-byte aligned");
+  const int ns = mla_split_of(p);
+  const int tiles = (p->seqlen_kv + 63) / 64;
+  if (ns > tiles || ns > 64) return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: num_split %d exceeds min(kv tiles=%d, 64)", ns, tiles);
+  ma::MlaArgs a{};
+  a.q = p->q; a.q_pe = p->q_pe; a.kv = p->kv; a.k_pe = p->k_pe; a.o = p->o; a.lse = p->lse;
+  a.qsb = p->q_stride_b; a.qsh = p->q_stride_h; a.qpsb = p->qpe_stride_b; a.qpsh = p->qpe_stride_h;
+  a.kvsb = p->kv_stride_b; a.kvss = p->kv_stride_s; a.kpsb = p->kpe_stride_b; a.kpss = p->kpe_stride_s;
+  a.osb = p->o_stride_b; a.osh = p->o_stride_h;
+  a.B = p->batch; a.Hq = p->heads_q; a.Skv = p->seqlen_kv; a.scale = p->scale;
+  a.num_split = ns;
+  a.split_len = ((tiles + ns - 1) / ns) * 64;
+  if (ns > 1) {
+    const size_t need = ma_mla_workspace_bytes(p);
+    if (!p->workspace || p->workspace_bytes < need)
+      return fail(MA_ERR_WORKSPACE, "ma_mla_decode: workspace of %zu bytes needed for %d splits, got %zu", need, ns, p->workspace_bytes);
+    if ((uintptr_t)p->workspace % 16 != 0) return fail(MA_ERR_WORKSPACE, "ma_mla_decode: workspace must be 16-byte aligned");
+    a.o_part = (float*)p->workspace;
+    a.lse_part = a.o_part + (size_t)p->batch * ns * p->heads_q * p->dim;
+  }
+  const int rc = ma::mla_decode_dispatch(a, p->dtype == MA_BF16, p->dim, p->dim_pe, (hipStream_t)stream);
+  if (rc == -2) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: only dim=512, dim_pe=64 is in the kernel library (got %d, %d)", p->dim, p->dim_pe);
+  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_mla_decode: launch failed: %s", hipGetErrorString(hipGetLastError()));
+  return MA_OK;
 }
 
 }  // extern "C"

@@ -1,0 +1,302 @@
+// Absorbed MLA decode (one query token, shared latent KV cache) for gfx950.
+//
+// Replaces flash_attn_split + combine of
+// attention_engine/core/template/tl_template/attn/mla_decode_tl.py:154-290:
+//   o[b,h,:] = softmax((q[b,h].kv[b,n] + q_pe[b,h].k_pe[b,n]) * scale) . kv[b,n]
+//
+// Split kernel.  A workgroup (4 waves) owns one (batch, kv split, block of 64
+// query heads); wave w owns heads 16w..16w+15 and all four waves consume the
+// same 64-row latent tile from LDS.  The two head blocks of one (batch, split)
+// are given workgroup ids that land on the same XCD, so the second read of a
+// tile is served by that XCD's L2 and the cache leaves HBM once.  Tiles arrive
+// by direct-to-LDS DMA (global_load_lds_dwordx4: no staging registers; the
+// registers hold the 576-wide Q fragments and the 512 x 16 fp32 output
+// accumulator), double buffered.  v_mfma_f32_16x16x32 is used throughout:
+//   A[16 x 32]: lane holds row l%16, k = 8(l/16) .. +7
+//   B[32 x 16]: lane holds column l%16, k = 8(l/16) .. +7
+//   C[16 x 16]: lane holds column l%16, element j is row 4(l/16) + j
+// Scores are computed transposed (S^T = KV Q^T) so each lane owns one head's
+// row statistics and the probabilities feed O^T += KV^T P^T straight from the
+// accumulator registers; KV^T comes out of the same row-major LDS tile through
+// the transposing read, so V is never loaded separately.
+// Combine kernel: log-sum-exp merge of the fp32 partials.
+#include "mla_decode.h"
+
+namespace ma {
+
+namespace {
+constexpr int BN = 64;         // kv rows per tile
+constexpr int HB = 64;         // heads per workgroup
+constexpr int D = 512, DPE = 64;
+constexpr int KV_ROW = D * 2;      // bytes
+constexpr int PE_ROW = DPE * 2;
+constexpr int KV_TILE = BN * KV_ROW;   // 64 KB
+constexpr int PE_TILE = BN * PE_ROW;   // 8 KB
+constexpr int STAGE = KV_TILE + PE_TILE;
+
+__device__ __forceinline__ int swz_kv(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+__device__ __forceinline__ int swz_pe(int row) { return (row >> 1) & 7; }
+
+// Direct-to-LDS load of 64 x 16 bytes: lane i's 16 bytes land at lds_base + 16 i.
+// Issued through inline asm so that the compiler does not serialise later LDS
+// reads behind it; completion is awaited explicitly with vmcnt before the
+// barrier that publishes the tile.
+__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, off\n\t"
+      :
+      : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr)
+      : "memory");
+}
+__device__ __forceinline__ void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ float xlane(float x, int mask) { return __shfl_xor(x, mask, 64); }
+}  // namespace
+
+template <typename T>
+__global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
+  using E = Elem<T>;
+  using x8 = typename E::x8;
+  using x4 = typename E::x4;
+  constexpr int KS = D / 32, KSPE = DPE / 32, DB = D / 16, NB = BN / 16;
+
+  extern __shared__ __align__(16) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, q = lane >> 4;
+  // workgroup id -> (batch, split, head block); head blocks of one (batch, split) share id % 8 (one XCD)
+  const int n_bs = a.B * a.num_split;
+  int bs, hblk;
+  if ((n_bs & 7) == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    hblk = slot % a.head_blocks;
+    bs = (slot / a.head_blocks) * 8 + xcd;
+  } else {
+    hblk = blockIdx.x % a.head_blocks;
+    bs = blockIdx.x / a.head_blocks;
+  }
+  const int b = bs / a.num_split, split = bs % a.num_split;
+  const int head = hblk * HB + wave * 16 + r;
+  const int head_ld = min(head, a.Hq - 1);
+
+  const int n_begin = split * a.split_len;
+  const int n_end = min(n_begin + a.split_len, a.Skv);
+  const int n_tiles = n_end > n_begin ? (n_end - n_begin + BN - 1) / BN : 0;
+
+  // ---- Q fragments: B operand of S^T = KV Q^T
+  x8 qf[KS + KSPE];
+  {
+    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)head_ld * a.qsh + 8 * q;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 32 * ks);
+    const T* qpe = (const T*)a.q_pe + (int64_t)b * a.qpsb + (int64_t)head_ld * a.qpsh + 8 * q;
+#pragma unroll
+    for (int ks = 0; ks < KSPE; ks++) qf[KS + ks] = *(const x8*)(qpe + 32 * ks);
+  }
+
+  const char* kvb = (const char*)a.kv + (int64_t)b * a.kvsb * 2;
+  const char* peb = (const char*)a.k_pe + (int64_t)b * a.kpsb * 2;
+  const int64_t kv_row_bytes = a.kvss * 2, pe_row_bytes = a.kpss * 2;
+
+  // wave w streams tile rows 16w..16w+15: one DMA per latent row (64 lanes x 16 B = 1 KB),
+  // one DMA per 8 rope rows.  Lane i fetches the chunk that belongs at physical chunk i.
+  auto issue_tile = [&](int n0, int buf) {
+    const uint32_t base = lds0 + buf * STAGE;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const int row = wave * 16 + i;
+      const int nrow = min(n0 + row, a.Skv - 1);
+      dma16(kvb + nrow * kv_row_bytes + ((lane ^ swz_kv(row)) << 4), base + row * KV_ROW);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const int row = wave * 16 + i * 8 + (lane >> 3);
+      const int nrow = min(n0 + row, a.Skv - 1);
+      dma16(peb + nrow * pe_row_bytes + (((lane & 7) ^ swz_pe(row)) << 4), base + KV_TILE + (wave * 16 + i * 8) * PE_ROW);
+    }
+  };
+
+  // ---- per-lane LDS read addresses
+  // K side (A operand): row 16nb + r, logical 16-byte chunk 4ks + q
+  const uint32_t k_row_off = r * KV_ROW;
+  const int k_chunk0 = q ^ swz_kv(r);
+  const uint32_t pe_row_off = KV_TILE + r * PE_ROW;
+  const int pe_chunk0 = q ^ swz_pe(r);
+  // V side (transposing read): lane block q reads rows nbase + 4q + jr, columns 16db + 4(l%4)..+3
+  const int jr = r >> 2;
+  const uint32_t v_row_off = (4 * q + jr) * KV_ROW + (lane & 1) * 8;
+  const int v_chunk0 = ((lane & 3) >> 1) ^ swz_kv(4 * q + jr);
+
+  f32x4 o[DB];
+#pragma unroll
+  for (int i = 0; i < DB; i++) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const float c_scale = a.scale * kLog2e;
+  float row_max = -1e30f, row_sum = 0.f;
+
+  if (n_tiles > 0) {
+    issue_tile(n_begin, 0);
+    wait_dma();
+  }
+  __syncthreads();
+
+  for (int jt = 0; jt < n_tiles; jt++) {
+    const int buf = jt & 1, n0 = n_begin + jt * BN;
+    if (jt + 1 < n_tiles) issue_tile(n0 + BN, buf ^ 1);
+    const uint32_t base = lds0 + buf * STAGE;
+
+    // ---- S^T = KV Q^T + K_pe Q_pe^T : lane holds head r, kv rows 16nb + 4q + j
+    f32x4 s[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) s[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      const uint32_t coff = (uint32_t)((k_chunk0 ^ (4 * ks)) << 4);
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+        s[nb] = E::mfma16(lds_read<x8>(base + k_row_off + nb * 16 * KV_ROW + coff), qf[ks], s[nb]);
+    }
+#pragma unroll
+    for (int ks = 0; ks < KSPE; ks++) {
+      const uint32_t coff = (uint32_t)((pe_chunk0 ^ (4 * ks)) << 4);
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+        s[nb] = E::mfma16(lds_read<x8>(base + pe_row_off + nb * 16 * PE_ROW + coff), qf[KS + ks], s[nb]);
+    }
+
+    if (n0 + BN > n_end) {
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          if (n0 + 16 * nb + 4 * q + j >= n_end) s[nb][j] = -INFINITY;
+    }
+
+    // ---- online softmax in the log2 domain (the 4 lanes l%16 == r own one head)
+    float mx = s[0][0];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) mx = fmaxf(mx, s[nb][j]);
+    mx = fmaxf(mx, xlane(mx, 16));
+    mx = fmaxf(mx, xlane(mx, 32));
+    const float new_max = fmaxf(row_max, mx * c_scale);
+    const float corr = fast_exp2(row_max - new_max);
+    row_max = new_max;
+    float part = 0.f;
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const float p = fast_exp2(s[nb][j] * c_scale - new_max);
+        s[nb][j] = p;
+        part += p;
+      }
+    row_sum = row_sum * corr + part;
+    if (__any(corr != 1.f)) {
+#pragma unroll
+      for (int i = 0; i < DB; i++) o[i] *= corr;
+    }
+
+    // ---- O^T += KV^T P^T ; MFMA slice t covers kv rows 32t..32t+31, lane block q, slot i is
+    //      row 32t + 16(i/4) + 4q + i%4 on both operands
+#pragma unroll
+    for (int t = 0; t < BN / 32; t++) {
+      x8 pf;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        pf[i] = (T)s[2 * t][i];
+        pf[4 + i] = (T)s[2 * t + 1][i];
+      }
+      const uint32_t rb = base + v_row_off + 32 * t * KV_ROW;
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        x4 lo = lds_read_tr4<T>(rb + (uint32_t)((v_chunk0 ^ (2 * db)) << 4));
+        x4 hi = lds_read_tr4<T>(rb + 16 * KV_ROW + (uint32_t)((v_chunk0 ^ (2 * db)) << 4));
+        x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        o[db] = E::mfma16(vf, pf, o[db]);
+      }
+    }
+
+    wait_dma();
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane holds head r, output columns 16db + 4q + j
+  float tot = row_sum + xlane(row_sum, 16);
+  tot += xlane(tot, 32);
+  const bool empty = n_tiles == 0;
+  const float inv = empty ? 0.f : 1.f / tot;
+  const float lse2 = empty ? -INFINITY : row_max + fast_log2(tot);   // log2 domain
+  if (head < a.Hq) {
+    if (a.num_split == 1) {
+      T* op = (T*)a.o + (int64_t)b * a.osb + (int64_t)head * a.osh + 4 * q;
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (T)(o[db][i] * inv);
+        *(x4*)(op + 16 * db) = w;
+      }
+      if (a.lse && q == 0) a.lse[(int64_t)b * a.Hq + head] = lse2 * kLn2;
+    } else {
+      float* op = a.o_part + (((int64_t)b * a.num_split + split) * a.Hq + head) * D + 4 * q;
+#pragma unroll
+      for (int db = 0; db < DB; db++) *(f32x4*)(op + 16 * db) = o[db] * inv;
+      if (q == 0) a.lse_part[((int64_t)b * a.num_split + split) * a.Hq + head] = lse2;
+    }
+  }
+}
+
+// One workgroup per (batch, head): 128 threads x 4 output columns.
+template <typename T>
+__global__ __launch_bounds__(128) void mla_combine_kernel(const MlaArgs a) {
+  const int head = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int ns = a.num_split;
+  const float* lp = a.lse_part + (int64_t)b * ns * a.Hq + head;
+  float mx = -INFINITY;
+  for (int s = 0; s < ns; s++) mx = fmaxf(mx, lp[(int64_t)s * a.Hq]);
+  float sum = 0.f;
+  for (int s = 0; s < ns; s++) sum += fast_exp2(lp[(int64_t)s * a.Hq] - mx);
+  const float inv = 1.f / sum;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < ns; s++) {
+    const float w = fast_exp2(lp[(int64_t)s * a.Hq] - mx) * inv;
+    const f32x4 v = *(const f32x4*)(a.o_part + (((int64_t)b * ns + s) * a.Hq + head) * D + tid * 4);
+    acc += v * w;
+  }
+  typename Elem<T>::x4 w;
+#pragma unroll
+  for (int i = 0; i < 4; i++) w[i] = (T)acc[i];
+  *(typename Elem<T>::x4*)((T*)a.o + (int64_t)b * a.osb + (int64_t)head * a.osh + tid * 4) = w;
+  if (a.lse && tid == 0) a.lse[(int64_t)b * a.Hq + head] = (mx + fast_log2(sum)) * kLn2;
+}
+
+template <typename T>
+static int launch_t(const MlaArgs& a, hipStream_t stream) {
+  constexpr size_t lds = 2 * (size_t)STAGE;
+  auto kern = mla_split_kernel<T>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
+    attr_set = true;
+  }
+  MlaArgs args = a;
+  args.head_blocks = (a.Hq + HB - 1) / HB;
+  const unsigned grid = (unsigned)(a.B * a.num_split * args.head_blocks);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, args);
+  if (hipGetLastError() != hipSuccess) return -1;
+  if (a.num_split > 1) {
+    hipLaunchKernelGGL(mla_combine_kernel<T>, dim3(a.Hq, a.B), dim3(128), 0, stream, a);
+    if (hipGetLastError() != hipSuccess) return -1;
+  }
+  return 0;
+}
+
+int mla_decode_dispatch(const MlaArgs& a, bool is_bf16, int dim, int dim_pe, hipStream_t stream) {
+  if (dim != D || dim_pe != DPE) return -2;
+  return is_bf16 ? launch_t<__bf16>(a, stream) : launch_t<_Float16>(a, stream);
+}
+
+}  // namespace ma

@@ -164,3 +164,43 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
         p.sm_stride_h, p.sm_stride_q = score_mask.stride(1), score_mask.stride(2)
     _check(load_library().ma_attn_fwd(ctypes.byref(p), _stream()))
     return out
+
+
+def mla_decode(q, q_pe, kv, k_pe, *, scale: float, num_split: int = 0, out=None, lse=None, workspace=None):
+    """Absorbed MLA decode.  q [B,1,Hq,D], q_pe [B,1,Hq,Dpe], kv [B,Skv,1,D],
+    k_pe [B,Skv,1,Dpe] (the reference operator's layouts) -> [B,1,Hq,D]."""
+    _require_gpu(q, q_pe, kv, k_pe, out, lse, workspace)
+    B, one, Hq, D = q.shape
+    Skv, Dpe = kv.shape[1], q_pe.shape[-1]
+    assert one == 1 and kv.shape[2] == 1 and k_pe.shape == (B, Skv, 1, Dpe) and q_pe.shape == (B, 1, Hq, Dpe)
+    for t in (q, q_pe, kv, k_pe):
+        assert t.stride(-1) == 1, "last dimension must be contiguous"
+    if out is None:
+        out = torch.empty(B, 1, Hq, D, dtype=q.dtype, device=q.device)
+    p = MlaParams()
+    p.dtype = _dtype_code(q.dtype)
+    p.batch, p.heads_q, p.seqlen_kv, p.dim, p.dim_pe, p.num_split = B, Hq, Skv, D, Dpe, num_split
+    p.q, p.q_stride_b, p.q_stride_h = q.data_ptr(), q.stride(0), q.stride(2)
+    p.q_pe, p.qpe_stride_b, p.qpe_stride_h = q_pe.data_ptr(), q_pe.stride(0), q_pe.stride(2)
+    p.kv, p.kv_stride_b, p.kv_stride_s = kv.data_ptr(), kv.stride(0), kv.stride(1)
+    p.k_pe, p.kpe_stride_b, p.kpe_stride_s = k_pe.data_ptr(), k_pe.stride(0), k_pe.stride(1)
+    p.o, p.o_stride_b, p.o_stride_h = out.data_ptr(), out.stride(0), out.stride(2)
+    if lse is not None:
+        assert lse.dtype == torch.float32 and lse.shape == (B, Hq) and lse.is_contiguous()
+        p.lse = lse.data_ptr()
+    p.scale = float(scale)
+    lib = load_library()
+    need = lib.ma_mla_workspace_bytes(ctypes.byref(p))
+    if need:
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        assert workspace.numel() * workspace.element_size() >= need
+        p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    _check(lib.ma_mla_decode(ctypes.byref(p), _stream()))
+    return out
+
+
+def mla_workspace_bytes(B, Hq, Skv, D=512, Dpe=64, num_split=0) -> int:
+    p = MlaParams()
+    p.batch, p.heads_q, p.seqlen_kv, p.dim, p.dim_pe, p.num_split = B, Hq, Skv, D, Dpe, num_split
+    return load_library().ma_mla_workspace_bytes(ctypes.byref(p))
