@@ -28,13 +28,18 @@ namespace {
 constexpr int BN = 64;         // kv rows per tile
 constexpr int HB = 64;         // heads per workgroup
 constexpr int D = 512, DPE = 64;
-constexpr int KV_ROW = D * 2;      // bytes
-constexpr int PE_ROW = DPE * 2;
-constexpr int KV_TILE = BN * KV_ROW;   // 64 KB
+constexpr int KV_ROW = D * 2 + 32;  // bytes; each latent row is its own DMA, so rows can be padded: with a
+                                   // 32 B pad consecutive rows start 8 banks apart (the transposing reads of
+                                   // 8 rows x 32 B tile the 64 banks exactly) and rows 8..15 of a 16-row group
+                                   // additionally swap their 16-byte chunk pairs (kv_flip) so that the 128-bit
+                                   // reads of 16 rows x one chunk hit 16 different bank groups.  Every LDS
+                                   // read address is then lane base + compile-time offset.
+constexpr int PE_ROW = DPE * 2;    // rope rows share a DMA (8 rows per KB): XOR-swizzled instead
+constexpr int KV_TILE = BN * KV_ROW;   // 65 KB
 constexpr int PE_TILE = BN * PE_ROW;   // 8 KB
 constexpr int STAGE = KV_TILE + PE_TILE;
 
-__device__ __forceinline__ int swz_kv(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+__device__ __forceinline__ int kv_flip(int row) { return (row >> 3) & 1; }
 __device__ __forceinline__ int swz_pe(int row) { return (row >> 1) & 7; }
 
 // Direct-to-LDS load of 64 x 16 bytes: lane i's 16 bytes land at lds_base + 16 i.
@@ -50,7 +55,9 @@ __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
       : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr)
       : "memory");
 }
-__device__ __forceinline__ void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// vmcnt(0), other counters untouched.  The builtin (rather than asm) also tells the compiler's own
+// wait-count bookkeeping that no vector-memory load is pending any more.
+__device__ __forceinline__ void wait_dma() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 __device__ __forceinline__ float xlane(float x, int mask) { return __shfl_xor(x, mask, 64); }
 }  // namespace
 
@@ -108,7 +115,7 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
     for (int i = 0; i < 16; i++) {
       const int row = wave * 16 + i;
       const int nrow = min(n0 + row, a.Skv - 1);
-      dma16(kvb + nrow * kv_row_bytes + ((lane ^ swz_kv(row)) << 4), base + row * KV_ROW);
+      dma16(kvb + nrow * kv_row_bytes + ((lane ^ kv_flip(row)) << 4), base + row * KV_ROW);
     }
 #pragma unroll
     for (int i = 0; i < 2; i++) {
@@ -120,14 +127,12 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
 
   // ---- per-lane LDS read addresses
   // K side (A operand): row 16nb + r, logical 16-byte chunk 4ks + q
-  const uint32_t k_row_off = r * KV_ROW;
-  const int k_chunk0 = q ^ swz_kv(r);
+  const uint32_t k_row_off = r * KV_ROW + (q ^ kv_flip(r)) * 16;
   const uint32_t pe_row_off = KV_TILE + r * PE_ROW;
   const int pe_chunk0 = q ^ swz_pe(r);
   // V side (transposing read): lane block q reads rows nbase + 4q + jr, columns 16db + 4(l%4)..+3
   const int jr = r >> 2;
-  const uint32_t v_row_off = (4 * q + jr) * KV_ROW + (lane & 1) * 8;
-  const int v_chunk0 = ((lane & 3) >> 1) ^ swz_kv(4 * q + jr);
+  const uint32_t v_row_off = (4 * q + jr) * KV_ROW + ((((lane & 3) >> 1) ^ kv_flip(4 * q + jr)) << 4) + (lane & 1) * 8;
 
   f32x4 o[DB];
 #pragma unroll
@@ -135,10 +140,8 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
   const float c_scale = a.scale * kLog2e;
   float row_max = -1e30f, row_sum = 0.f;
 
-  if (n_tiles > 0) {
-    issue_tile(n_begin, 0);
-    wait_dma();
-  }
+  if (n_tiles > 0) issue_tile(n_begin, 0);
+  wait_dma();
   __syncthreads();
 
   for (int jt = 0; jt < n_tiles; jt++) {
@@ -150,19 +153,31 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
     f32x4 s[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) s[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    {
+      // fragments are requested two slices ahead of the MFMAs that consume them
+      constexpr int AH = 2, RING = AH + 1, NSL = KS + KSPE;
+      x8 kf[RING][NB];
+      const uint32_t kb = base + k_row_off;
+      auto request = [&](int ks) {
+        if (ks < KS) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      const uint32_t coff = (uint32_t)((k_chunk0 ^ (4 * ks)) << 4);
+          for (int nb = 0; nb < NB; nb++) kf[ks % RING][nb] = lds_read<x8>(kb + nb * 16 * KV_ROW + ks * 64);
+        } else {
+          const uint32_t coff = (uint32_t)((pe_chunk0 ^ (4 * (ks - KS))) << 4);
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++)
-        s[nb] = E::mfma16(lds_read<x8>(base + k_row_off + nb * 16 * KV_ROW + coff), qf[ks], s[nb]);
-    }
+          for (int nb = 0; nb < NB; nb++) kf[ks % RING][nb] = lds_read<x8>(base + pe_row_off + nb * 16 * PE_ROW + coff);
+        }
+      };
 #pragma unroll
-    for (int ks = 0; ks < KSPE; ks++) {
-      const uint32_t coff = (uint32_t)((pe_chunk0 ^ (4 * ks)) << 4);
+      for (int ks = 0; ks < AH; ks++) request(ks);
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++)
-        s[nb] = E::mfma16(lds_read<x8>(base + pe_row_off + nb * 16 * PE_ROW + coff), qf[KS + ks], s[nb]);
+      for (int ks = 0; ks < NSL; ks++) {
+        if (ks + AH < NSL) request(ks + AH);
+        __builtin_amdgcn_sched_barrier(0);   // keep the requests ahead of the MFMAs that hide their latency
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) s[nb] = E::mfma16(kf[ks % RING][nb], qf[ks], s[nb]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
 
     if (n0 + BN > n_end) {
@@ -181,23 +196,27 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
       for (int j = 0; j < 4; j++) mx = fmaxf(mx, s[nb][j]);
     mx = fmaxf(mx, xlane(mx, 16));
     mx = fmaxf(mx, xlane(mx, 32));
-    const float new_max = fmaxf(row_max, mx * c_scale);
-    const float corr = fast_exp2(row_max - new_max);
-    row_max = new_max;
+    // The running max is only moved when some head's max grew by more than 2^8: until then the
+    // probabilities are taken relative to the stale max (at most 256, exact in fp32 / bf16 range) and the
+    // 128 accumulator registers need no rescaling.  The final normalisation by row_sum absorbs the offset.
+    const float cand = fmaxf(row_max, mx * c_scale);
+    if (__any(cand - row_max > 8.f)) {
+      const float corr = fast_exp2(row_max - cand);
+      row_max = cand;
+      row_sum *= corr;
+#pragma unroll
+      for (int i = 0; i < DB; i++) o[i] *= corr;
+    }
     float part = 0.f;
 #pragma unroll
     for (int nb = 0; nb < NB; nb++)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
-        const float p = fast_exp2(s[nb][j] * c_scale - new_max);
+        const float p = fast_exp2(s[nb][j] * c_scale - row_max);
         s[nb][j] = p;
         part += p;
       }
-    row_sum = row_sum * corr + part;
-    if (__any(corr != 1.f)) {
-#pragma unroll
-      for (int i = 0; i < DB; i++) o[i] *= corr;
-    }
+    row_sum += part;
 
     // ---- O^T += KV^T P^T ; MFMA slice t covers kv rows 32t..32t+31, lane block q, slot i is
     //      row 32t + 16(i/4) + 4q + i%4 on both operands
@@ -210,12 +229,23 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
         pf[4 + i] = (T)s[2 * t + 1][i];
       }
       const uint32_t rb = base + v_row_off + 32 * t * KV_ROW;
+      constexpr int PF = 8;   // V fragments in flight
+      x4 lo[PF], hi[PF];
+#pragma unroll
+      for (int i = 0; i < PF - 1; i++) {
+        lo[i] = lds_read_tr4<T>(rb + i * 32);
+        hi[i] = lds_read_tr4<T>(rb + 16 * KV_ROW + i * 32);
+      }
 #pragma unroll
       for (int db = 0; db < DB; db++) {
-        x4 lo = lds_read_tr4<T>(rb + (uint32_t)((v_chunk0 ^ (2 * db)) << 4));
-        x4 hi = lds_read_tr4<T>(rb + 16 * KV_ROW + (uint32_t)((v_chunk0 ^ (2 * db)) << 4));
-        x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        if (db + PF - 1 < DB) {
+          lo[(db + PF - 1) % PF] = lds_read_tr4<T>(rb + (db + PF - 1) * 32);
+          hi[(db + PF - 1) % PF] = lds_read_tr4<T>(rb + 16 * KV_ROW + (db + PF - 1) * 32);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        x8 vf = __builtin_shufflevector(lo[db % PF], hi[db % PF], 0, 1, 2, 3, 4, 5, 6, 7);
         o[db] = E::mfma16(vf, pf, o[db]);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
 
