@@ -76,6 +76,30 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
+// Direct-to-LDS load of 64 x 16 bytes (global_load_lds_dwordx4): lane i's 16 bytes
+// land at lds_base + 16 i; every lane chooses its own global source address.
+// Issued through inline asm so that the compiler does not serialise later LDS
+// reads behind it; completion is awaited explicitly with wait_dma() before the
+// barrier that publishes the data.  lds_base must be wave-uniform.
+__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, off\n\t"
+      :
+      : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr)
+      : "memory");
+}
+// vmcnt(0), other counters untouched.  The builtin (rather than asm) also tells the
+// compiler's own wait-count bookkeeping that no vector-memory load is pending any more.
+__device__ __forceinline__ void wait_dma() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// XOR swizzle (in 16-byte chunks) of a row-major LDS tile with >= 16 chunks per row:
+// a bijection on the low 4 row bits, so 128-bit reads of 16 consecutive rows at one
+// logical chunk hit 16 different bank groups, and the 8 rows x 4 chunks touched by a
+// transposing read spread evenly over the banks.
+__device__ __forceinline__ int swz16(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 

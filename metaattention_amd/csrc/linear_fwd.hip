@@ -1,0 +1,349 @@
+// Chunked linear / stateful attention forward (RetNet retention, Mamba2 SSD,
+// gated retention) for gfx950.
+//
+// Replaces the three launches of LinearAttention.forward in
+// attention_engine/core/template/tl_template/linear/linear_tl.py:1240-1269
+// (chunk_local_cumsum :36-60, chunk_fwd_h :146-221, chunk_o :322-399) with ONE
+// kernel that keeps the inter-chunk state on chip:
+//
+//   o_t = q_scale * q_t . sum_{s<=t} exp(G_t - G_s) k_s^T (v_s * vs_s),   G = cumsum(log_decay)
+//
+// Work split.  A workgroup owns one (batch, head) and a slice of 32*NW value
+// columns; wave w owns 32 of them and the matching DK x 32 block of the fp32
+// state, which lives in its accumulator registers for the whole sequence (the
+// reference writes the state to HBM as bf16 every chunk and reads it back).  The
+// sequence is walked in chunks of 32 tokens; per chunk and wave, with
+// g = chunk-local cumsum of the log decay, everything is computed TRANSPOSED so
+// each lane owns one token column:
+//   A^T = K Q^T                      [32 x 32]   (every wave, redundantly: it is the B operand below)
+//   P^T = A^T * q_scale * exp(g_i - g_j) * vs_j * [j <= i]
+//   O^T = h^T (Q^T) * exp(g_i) q_scale + V^T P^T          [32 dv x 32 tokens]
+//   h   = exp(g_last) h + K^T (V * vs * exp(g_last - g))  [DK x 32 dv]
+// The state accumulator of K^T V (lane = value column, rows = key dims) is,
+// register for register, the A operand of h^T Q^T, so the state never moves.
+// Q/K/V chunk tiles arrive by direct-to-LDS DMA, double buffered, with a single
+// workgroup barrier per chunk.
+#include "linear_fwd.h"
+
+namespace ma {
+
+namespace {
+constexpr int L = 32;  // tokens per chunk
+
+template <int CPR>
+__device__ __forceinline__ int swz_tile(int row) {
+  if constexpr (CPR >= 16) return swz16(row);
+  // 8 chunks per row (128-byte rows): two rows span the banks; see swz16 for the goal
+  return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+}
+
+template <typename X8>
+__device__ __forceinline__ X8 scale_bf16x8(X8 v, const float (&w)[8]) {
+  X8 r;
+#pragma unroll
+  for (int i = 0; i < 8; i++) r[i] = (__bf16)((float)v[i] * w[i]);
+  return r;
+}
+}  // namespace
+
+template <int DK, int NW>
+// second launch-bound argument: minimum waves per SIMD (8 waves of one workgroup need 2)
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(const LinArgs a) {
+  using T = __bf16;
+  using E = Elem<T>;
+  using x8 = typename E::x8;
+  using x4 = typename E::x4;
+  constexpr int DVS = 32 * NW;
+  constexpr int RBQ = DK * 2, RBV = DVS * 2;       // row bytes
+  constexpr int CPRQ = DK / 8, CPRV = DVS / 8;     // 16-byte chunks per row
+  constexpr int QT = L * RBQ, VT = L * RBV;
+  constexpr int STAGE = 2 * QT + VT;
+  constexpr int KB = DK / 32;                      // 32-row blocks of the state
+  constexpr int OROW = 64 + 16;                    // padded row of the per-wave output staging block
+  constexpr int SCAL_BYTES = 3 * L * 4;            // per-wave g / pv*q_scale / w
+  constexpr int NIQ = QT / 1024, NIV = VT / 1024;  // DMA instructions per tile
+  static_assert(CPRQ >= 16, "DK < 128 needs its own Q/K swizzle");
+
+  extern __shared__ __align__(16) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, g = lane >> 5;
+  const uint32_t lds_scal = lds0 + 2 * STAGE + wave * SCAL_BYTES;
+  const uint32_t lds_ost = lds0 + 2 * STAGE + NW * SCAL_BYTES + wave * (L * OROW);
+
+  // workgroup -> (batch*head, value slice); slices of one head share id % 8 (one XCD, shared L2)
+  const int BH = a.B * a.H;
+  int bh, dvb;
+  if ((BH & 7) == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    dvb = slot % a.dv_blocks;
+    bh = (slot / a.dv_blocks) * 8 + xcd;
+  } else {
+    dvb = blockIdx.x % a.dv_blocks;
+    bh = blockIdx.x / a.dv_blocks;
+  }
+  const int b = bh / a.H, h = bh % a.H;
+  const int hq = h / (a.H / a.Hq), hk = h / (a.H / a.Hk);
+  const int Tn = a.T;
+  const char* qb = (const char*)a.q + ((int64_t)(b * a.Hq + hq) * Tn) * RBQ;
+  const char* kb = (const char*)a.k + ((int64_t)(b * a.Hk + hk) * Tn) * RBQ;
+  const char* vb = (const char*)a.v + ((int64_t)bh * Tn * a.Dv + dvb * DVS) * 2;
+  T* ob = (T*)a.o + (int64_t)bh * Tn * a.Dv + dvb * DVS + 32 * wave;
+  const float* ldp = a.log_decay + (int64_t)bh * Tn;
+  const float* vsp = a.v_scale ? a.v_scale + (int64_t)bh * Tn : nullptr;
+  const int64_t v_row_bytes = (int64_t)a.Dv * 2;
+  const int n_chunks = (Tn + L - 1) / L;
+
+  // ---- DMA of one chunk: each instruction moves 1 KB (1024/row_bytes tile rows); lane i fetches
+  //      the 16-byte chunk that belongs at physical position i of that KB.
+  auto issue_chunk = [&](int t0, int buf) {
+    const uint32_t base = lds0 + buf * STAGE;
+    for (int ii = wave; ii < 2 * NIQ + NIV; ii += NW) {
+      if (ii < 2 * NIQ) {
+        const int which = ii >= NIQ, i2 = which ? ii - NIQ : ii;
+        const int row = i2 * (1024 / RBQ) + lane / CPRQ, c = lane % CPRQ;
+        const int trow = min(t0 + row, Tn - 1);
+        const char* src = (which ? kb : qb) + (int64_t)trow * RBQ + ((c ^ swz_tile<CPRQ>(row)) << 4);
+        dma16(src, base + which * QT + i2 * 1024);
+      } else {
+        const int i2 = ii - 2 * NIQ;
+        const int row = i2 * (1024 / RBV) + lane / CPRV, c = lane % CPRV;
+        const int trow = min(t0 + row, Tn - 1);
+        dma16(vb + (int64_t)trow * v_row_bytes + ((c ^ swz_tile<CPRV>(row)) << 4), base + 2 * QT + i2 * 1024);
+      }
+    }
+  };
+
+  // ---- per-lane LDS read offsets
+  // K rows / Q rows as MFMA operands of A^T = K Q^T: row r, logical chunk 2ks + g
+  const uint32_t qk_row = r * RBQ;
+  const int qk_c0 = g ^ swz16(r);
+  // Q^T operand of h^T Q^T: token r, key dims 32b + 16s + 4g + {0..3} and + 8: chunk 4b + 2s (+1), half g
+  const uint32_t qp_row = r * RBQ + g * 8;
+  const int qp_swz = swz16(r);
+  // transposing reads (K^T and V^T): lane block lane/16 -> (row group g, column half), rows 16s + 4g + jr (+8)
+  const int jr = (lane & 15) >> 2;
+  const int lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
+  const uint32_t kt_row = (4 * g + jr) * RBQ + (lane & 1) * 8;
+  const int kt_c0 = lc ^ swz16(4 * g + jr);                      // rows +8 / +16: see HALF_XOR below
+  const uint32_t vt_row = (4 * g + jr) * RBV + (lane & 1) * 8;
+  const int vt_c0 = (4 * wave + lc) ^ swz_tile<CPRV>(4 * g + jr);
+  // swz(row + 8) ^ swz(row) and swz(row + 16) ^ swz(row) for rows < 8
+  constexpr int Q_X8 = 2, Q_X16 = 0;
+  constexpr int V_X8 = CPRV >= 16 ? 2 : 2, V_X16 = CPRV >= 16 ? 0 : 0;
+
+  f32x16 hst[KB];
+#pragma unroll
+  for (int i = 0; i < KB; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) hst[i][j] = 0.f;
+
+  // scalars of the chunk about to be processed (loaded one chunk ahead)
+  const int ti = r;
+  float ld_next = 0.f, vs_next = 1.f;
+  if (ti < Tn) {
+    ld_next = ldp[ti];
+    if (vsp) vs_next = vsp[ti];
+  }
+  if (n_chunks > 0) issue_chunk(0, 0);
+
+  for (int c = 0; c < n_chunks; c++) {
+    const int buf = c & 1, t0 = c * L;
+    wait_dma();
+    __syncthreads();
+    const float ld = ld_next, vs = vs_next;
+    if (c + 1 < n_chunks) {
+      const int tn = t0 + L + ti;
+      ld_next = 0.f;
+      vs_next = 1.f;
+      if (tn < Tn) {
+        ld_next = ldp[tn];
+        if (vsp) vs_next = vsp[tn];
+      }
+      issue_chunk(t0 + L, buf ^ 1);
+    }
+    const uint32_t base = lds0 + buf * STAGE;
+    const uint32_t qbase = base, kbase = base + QT, vbase = base + 2 * QT;
+
+    // ---- chunk scalars: inclusive scan of the log decay over the 32 tokens (both lane halves hold a copy)
+    const bool valid = t0 + ti < Tn;
+    float gi = valid ? ld : 0.f;
+#pragma unroll
+    for (int d = 1; d < 32; d <<= 1) {
+      const float up = __shfl_up(gi, d, 32);
+      if (ti >= d) gi += up;
+    }
+    const float g_last = __shfl(gi, 31, 32);
+    const float pvq = valid ? vs * a.q_scale : 0.f;               // factor of column j in P
+    const float wl = valid ? vs * fast_exp2((g_last - gi) * kLog2e) : 0.f;   // factor of row l in the state update
+    const float eg = fast_exp2(gi * kLog2e) * a.q_scale;          // factor of token i in the inter-chunk term
+    const float decay_all = fast_exp2(g_last * kLog2e);
+    if (g == 0) {
+      lds_write<float>(lds_scal + ti * 4, gi);
+      lds_write<float>(lds_scal + (L + ti) * 4, pvq);
+      lds_write<float>(lds_scal + (2 * L + ti) * 4, wl);
+    }
+    // rows held by this lane in a 32 x 32 accumulator block: 8q4 + 4g + {0..3}
+    float gj[16], pj[16], wj[16];
+#pragma unroll
+    for (int q4 = 0; q4 < 4; q4++) {
+      const f32x4 tg = lds_read<f32x4>(lds_scal + (8 * q4 + 4 * g) * 4);
+      const f32x4 tp = lds_read<f32x4>(lds_scal + (L + 8 * q4 + 4 * g) * 4);
+      const f32x4 tw = lds_read<f32x4>(lds_scal + (2 * L + 8 * q4 + 4 * g) * 4);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        gj[4 * q4 + i] = tg[i];
+        pj[4 * q4 + i] = tp[i];
+        wj[4 * q4 + i] = tw[i];
+      }
+    }
+
+    // ---- A^T = K Q^T (lane: token i = r, rows j = 8(jj/4) + 4g + jj%4)
+    f32x16 sacc;
+#pragma unroll
+    for (int j = 0; j < 16; j++) sacc[j] = 0.f;
+    {
+      constexpr int NS = DK / 16, AH = 2, RING = 3;
+      x8 kf[RING], qf[RING];
+      auto request = [&](int ks) {
+        const uint32_t off = qk_row + (uint32_t)((qk_c0 ^ (2 * ks)) << 4);
+        kf[ks % RING] = lds_read<x8>(kbase + off);
+        qf[ks % RING] = lds_read<x8>(qbase + off);
+      };
+#pragma unroll
+      for (int ks = 0; ks < AH; ks++) request(ks);
+#pragma unroll
+      for (int ks = 0; ks < NS; ks++) {
+        if (ks + AH < NS) request(ks + AH);
+        __builtin_amdgcn_sched_barrier(0);
+        sacc = E::mfma32(kf[ks % RING], qf[ks % RING], sacc);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // ---- P^T: decay, per-token value scale, causal mask (exact zeros above the diagonal)
+    x8 pf[2];
+#pragma unroll
+    for (int jj = 0; jj < 16; jj++) {
+      const int j = 8 * (jj >> 2) + 4 * g + (jj & 3);
+      const float e = fast_exp2(fminf(gi - gj[jj], 0.f) * kLog2e);
+      const float p = j <= ti ? sacc[jj] * e * pj[jj] : 0.f;
+      pf[jj >> 3][jj & 7] = (T)p;
+    }
+
+    // ---- V^T fragments (rows = this wave's 32 value columns; k-slot i of slice s is token
+    //      16s + 8(i/4) + 4g + i%4, the order P^T comes in)
+    x8 vf[2];
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+      const int cx = s ? V_X16 : 0;
+      x4 lo = lds_read_tr4<T>(vbase + vt_row + 16 * s * RBV + (uint32_t)((vt_c0 ^ cx) << 4));
+      x4 hi = lds_read_tr4<T>(vbase + vt_row + (16 * s + 8) * RBV + (uint32_t)((vt_c0 ^ cx ^ V_X8) << 4));
+      vf[s] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+
+    // ---- O^T = (h^T Q^T) * eg + V^T P^T
+    f32x16 o_inter, o_intra;
+#pragma unroll
+    for (int j = 0; j < 16; j++) { o_inter[j] = 0.f; o_intra[j] = 0.f; }
+    o_intra = E::mfma32(vf[0], pf[0], o_intra);
+    o_intra = E::mfma32(vf[1], pf[1], o_intra);
+    // value-scaled V^T for the state update (k-slot i of slice s is token 16s + 8(i/4) + 4g + i%4 -> wj[8s + i])
+    x8 vsf[2];
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+      float w8[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) w8[i] = wj[8 * s + i];
+      vsf[s] = scale_bf16x8(vf[s], w8);
+    }
+
+    {
+      // per 32-row state block b: inter-chunk product with the OLD state, then the state update
+      constexpr int RING = 2;
+      x4 qlo[RING][2], qhi[RING][2], klo[RING][2], khi[RING][2];
+      auto request = [&](int bb) {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          const int lcq = 4 * bb + 2 * s;
+          qlo[bb % RING][s] = lds_read<x4>(qbase + qp_row + (uint32_t)((lcq ^ qp_swz) << 4));
+          qhi[bb % RING][s] = lds_read<x4>(qbase + qp_row + (uint32_t)(((lcq + 1) ^ qp_swz) << 4));
+          const int cx = s ? Q_X16 : 0;
+          klo[bb % RING][s] = lds_read_tr4<T>(kbase + kt_row + 16 * s * RBQ + (uint32_t)((kt_c0 ^ (4 * bb) ^ cx) << 4));
+          khi[bb % RING][s] = lds_read_tr4<T>(kbase + kt_row + (16 * s + 8) * RBQ + (uint32_t)((kt_c0 ^ (4 * bb) ^ cx ^ Q_X8) << 4));
+        }
+      };
+      request(0);
+#pragma unroll
+      for (int bb = 0; bb < KB; bb++) {
+        if (bb + 1 < KB) request(bb + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          x8 hf;
+#pragma unroll
+          for (int i = 0; i < 8; i++) hf[i] = (T)hst[bb][8 * s + i];
+          x8 qf = __builtin_shufflevector(qlo[bb % RING][s], qhi[bb % RING][s], 0, 1, 2, 3, 4, 5, 6, 7);
+          o_inter = E::mfma32(hf, qf, o_inter);
+        }
+#pragma unroll
+        for (int j = 0; j < 16; j++) hst[bb][j] *= decay_all;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          x8 kf = __builtin_shufflevector(klo[bb % RING][s], khi[bb % RING][s], 0, 1, 2, 3, 4, 5, 6, 7);
+          hst[bb] = E::mfma32(kf, vsf[s], hst[bb]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+
+    // ---- write this wave's [32 tokens x 32 columns] block: stage (wave private), then 16-byte row pieces
+#pragma unroll
+    for (int q4 = 0; q4 < 4; q4++) {
+      x4 w;
+#pragma unroll
+      for (int i = 0; i < 4; i++) w[i] = (T)(o_inter[4 * q4 + i] * eg + o_intra[4 * q4 + i]);
+      lds_write<x4>(lds_ost + r * OROW + (8 * q4 + 4 * g) * 2, w);
+    }
+#pragma unroll
+    for (int it = 0; it < 2; it++) {
+      const int ci = lane + 64 * it, row = ci >> 2, cc = ci & 3;
+      const u32x4 w = lds_read<u32x4>(lds_ost + row * OROW + cc * 16);
+      if (t0 + row < Tn) *(u32x4*)(ob + (int64_t)(t0 + row) * a.Dv + cc * 8) = w;
+    }
+  }
+}
+
+template <int DK, int NW>
+static int launch(const LinArgs& a, hipStream_t stream) {
+  constexpr int DVS = 32 * NW;
+  constexpr size_t stage = (size_t)L * (4 * DK + 2 * DVS);
+  constexpr size_t lds = 2 * stage + NW * (3 * L * 4) + NW * (L * 80);
+  auto kern = linear_fwd_kernel<DK, NW>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
+    attr_set = true;
+  }
+  LinArgs args = a;
+  args.dv_blocks = a.Dv / DVS;
+  const unsigned grid = (unsigned)(a.B * a.H * args.dv_blocks);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, args);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// returns 0 ok, -1 launch failure, -2 unsupported
+int linear_fwd_dispatch(const LinArgs& a, int dk, hipStream_t stream) {
+  const int dv = a.Dv;
+  if (dk == 256) {
+    if (dv % 256 == 0) return launch<256, 8>(a, stream);
+    if (dv % 128 == 0) return launch<256, 4>(a, stream);
+    if (dv % 64 == 0) return launch<256, 2>(a, stream);
+  } else if (dk == 128) {
+    if (dv % 256 == 0) return launch<128, 8>(a, stream);
+    if (dv % 128 == 0) return launch<128, 4>(a, stream);
+    if (dv % 64 == 0) return launch<128, 2>(a, stream);
+  }
+  return -2;
+}
+
+}  // namespace ma

@@ -42,22 +42,6 @@ constexpr int STAGE = KV_TILE + PE_TILE;
 __device__ __forceinline__ int kv_flip(int row) { return (row >> 3) & 1; }
 __device__ __forceinline__ int swz_pe(int row) { return (row >> 1) & 7; }
 
-// Direct-to-LDS load of 64 x 16 bytes: lane i's 16 bytes land at lds_base + 16 i.
-// Issued through inline asm so that the compiler does not serialise later LDS
-// reads behind it; completion is awaited explicitly with vmcnt before the
-// barrier that publishes the tile.
-__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
-  asm volatile(
-      "s_mov_b32 m0, %0\n\t"
-      "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %1, off\n\t"
-      :
-      : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr)
-      : "memory");
-}
-// vmcnt(0), other counters untouched.  The builtin (rather than asm) also tells the compiler's own
-// wait-count bookkeeping that no vector-memory load is pending any more.
-__device__ __forceinline__ void wait_dma() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 __device__ __forceinline__ float xlane(float x, int mask) { return __shfl_xor(x, mask, 64); }
 }  // namespace
 

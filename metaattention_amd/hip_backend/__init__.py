@@ -204,3 +204,32 @@ def mla_workspace_bytes(B, Hq, Skv, D=512, Dpe=64, num_split=0) -> int:
     p = MlaParams()
     p.batch, p.heads_q, p.seqlen_kv, p.dim, p.dim_pe, p.num_split = B, Hq, Skv, D, Dpe, num_split
     return load_library().ma_mla_workspace_bytes(ctypes.byref(p))
+
+
+def linear_fwd(q, k, v, log_decay, *, q_scale: float = 1.0, v_scale=None, chunk=None, out=None):
+    """Chunked linear attention forward on BHSD tensors: q [B,Hq,T,Dk], k [B,Hk,T,Dk],
+    v [B,H,T,Dv] (bf16, contiguous), log_decay fp32 [B,H,T], optional per-token value
+    scale [B,H,T].  ``chunk`` is accepted for API compatibility; the result does not
+    depend on it and the kernel uses its own chunking."""
+    _require_gpu(q, k, v, log_decay, v_scale, out)
+    B, H, T, Dv = v.shape
+    Hq, Hk, Dk = q.shape[1], k.shape[1], q.shape[-1]
+    assert q.shape == (B, Hq, T, Dk) and k.shape == (B, Hk, T, Dk), "q/k/v shapes disagree"
+    assert log_decay.shape == (B, H, T), "log_decay must be [B,H,T]"
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    log_decay = log_decay.to(torch.float32).contiguous()
+    if v_scale is not None:
+        assert v_scale.shape == (B, H, T)
+        v_scale = v_scale.to(torch.float32).contiguous()
+    if out is None:
+        out = torch.empty(B, H, T, Dv, dtype=v.dtype, device=v.device)
+    p = LinearParams()
+    p.dtype = _dtype_code(v.dtype)
+    p.batch, p.heads, p.heads_q, p.heads_k, p.seqlen, p.dim_k, p.dim_v = B, H, Hq, Hk, T, Dk, Dv
+    p.chunk = int(chunk or 0)
+    p.q, p.k, p.v, p.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    p.log_decay = log_decay.data_ptr()
+    p.v_scale = v_scale.data_ptr() if v_scale is not None else None
+    p.q_scale = float(q_scale)
+    _check(load_library().ma_linear_fwd(ctypes.byref(p), _stream()))
+    return out

@@ -1,0 +1,136 @@
+"""Parity of the HIP chunked linear-attention forward (through the C ABI and the
+LinearAttentionEngine operator) with the CPU oracle.  Tolerance atol 2e-2 / rtol 1e-2."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from oracle import inputs
+import specs
+
+pytestmark = pytest.mark.gpu
+ATOL, RTOL = 2e-2, 1e-2
+
+
+def _hb():
+    from metaattention_amd import hip_backend as hb
+    hb.load_library()
+    return hb
+
+
+@pytest.mark.parametrize("B,H,T,Dk,Dv", [
+    (1, 2, 64, 256, 256), (1, 2, 256, 256, 512), (2, 3, 100, 128, 64), (1, 2, 128, 128, 128),
+    (1, 1, 1, 128, 64), (1, 2, 33, 256, 128), (1, 16, 512, 256, 512),
+])
+def test_retnet_chunked(B, H, T, Dk, Dv):
+    hb = _hb()
+    q, k, v, decay = inputs.retnet_inputs(B, H, T, Dk, Dv, seed=T)
+    # un-normalised inputs of testing/test.py:750-756 scale (key * 0.1) keep outputs O(1)
+    q, k = (q.float() * math.sqrt(Dk)).bfloat16(), (k.float() * math.sqrt(Dk) * 0.1).bfloat16()
+    ref = oracle.retnet_quadratic(q, k, v)
+    print(f"retnet B{B} H{H} T{T} Dk{Dk} Dv{Dv}", flush=True)
+    o = hb.linear_fwd(q.cuda(), k.cuda(), v.cuda(), torch.log(decay).cuda(), q_scale=Dk ** -0.5)
+    torch.cuda.synchronize()
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("B,H,T", [(1, 4, 128), (2, 8, 300), (1, 64, 512)])
+def test_mamba2_ssd(B, H, T):
+    hb = _hb()
+    P, N = 64, 128
+    Cm, Bm, x, dt, A = inputs.mamba2_inputs(B, H, T, P, N, seed=T)
+    chunk = 64 if T % 64 == 0 else 60
+    ref = oracle.ssd_chunk_scan_combined(x.permute(0, 2, 1, 3), dt.permute(0, 2, 1), A[0], Bm.permute(0, 2, 1, 3),
+                                         Cm.permute(0, 2, 1, 3), chunk_size=chunk).permute(0, 2, 1, 3)
+    print(f"mamba2 B{B} H{H} T{T}", flush=True)
+    o = hb.linear_fwd(Cm.cuda(), Bm.cuda(), x.cuda(), (dt * A.view(1, H, 1)).cuda(), v_scale=dt.cuda())
+    torch.cuda.synchronize()
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_engine_retnet_recurrent():
+    """Operator built from the spec, called like testing/test.py:749-775."""
+    B, H, T, Dk, Dv = 1, 4, 256, 256, 512
+    mod = specs.retnet_recurrent(B, H, T, Dk, Dv)
+    q = torch.randn(B, H, T, Dk, generator=torch.Generator().manual_seed(1)).bfloat16()
+    k = (0.1 * torch.randn(B, H, T, Dk, generator=torch.Generator().manual_seed(2))).bfloat16()
+    v = torch.randn(B, H, T, Dv, generator=torch.Generator().manual_seed(3)).bfloat16()
+    g = (1 - torch.exp2(-5 - torch.arange(H, dtype=torch.float32)))[None, :, None].expand(B, H, T).contiguous()
+    o = mod(q.cuda(), k.cuda(), v.cuda(), g.cuda())
+    torch.cuda.synchronize()
+    assert o.shape == (B, H, T, Dv) and o.dtype == torch.bfloat16
+    oracle.assert_close(o.float().cpu(), oracle.retnet_quadratic(q, k, v), rtol=RTOL, atol=ATOL)
+
+
+def test_engine_mamba2():
+    """mod(C, B, x, dt_fp32, A[1,H], dt_bf16) as in testing/test.py:198-200 (single B/C group)."""
+    B, H, T, P, N = 1, 16, 256, 64, 128
+    mod = specs.mamba2(B, 1, T, N, P, HK=1, HV=H)
+    Cm, Bm, x, dt, A = inputs.mamba2_inputs(B, H, T, P, N, seed=5)
+    o = mod(Cm.cuda(), Bm.cuda(), x.cuda(), dt.cuda(), A.cuda(), dt.bfloat16().cuda())
+    torch.cuda.synchronize()
+    # the operator multiplies v by the bf16 copy of dt (as the reference's fused v_mod does); the oracle gets the same values
+    ref = oracle.linear_attention_chunked(Cm, Bm, x, dt * A.view(1, H, 1), chunk=64, v_scale=dt.bfloat16().float())
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    ref2 = oracle.ssd_chunk_scan_combined(x.permute(0, 2, 1, 3), dt.permute(0, 2, 1), A[0], Bm.permute(0, 2, 1, 3),
+                                          Cm.permute(0, 2, 1, 3), chunk_size=64).permute(0, 2, 1, 3)
+    oracle.assert_close(o.float().cpu(), ref2, rtol=RTOL, atol=ATOL, mismatch_ratio=1e-3)
+
+
+def test_engine_gated_retention():
+    """Per-token log decay (testing/test.py:400-428); the reference compares at rtol=atol=1e-1."""
+    B, H, T, Dk, Dv = 2, 4, 256, 256, 256
+    mod = specs.gated_retention(B, H, T, Dk, Dv)
+    gen = torch.Generator().manual_seed(7)
+    q = torch.randn(B, H, T, Dk, generator=gen).bfloat16()
+    k = torch.randn(B, H, T, Dk, generator=gen).bfloat16()
+    v = torch.randn(B, H, T, Dv, generator=gen).bfloat16()
+    g = torch.nn.functional.logsigmoid(torch.randn(B, H, T, generator=gen)).clamp_min(-5)
+    o = mod(q.cuda(), k.cuda(), v.cuda(), g.cuda())
+    torch.cuda.synchronize()
+    ref = oracle.simple_gla_chunked(q, k, v, g)
+    oracle.assert_close(o.float().cpu(), ref, rtol=1e-1, atol=1e-1)
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=2e-2)   # outputs are O(10): bf16 output rounding
+
+
+def test_full_size_properties():
+    """Benchmark shapes: (i) linearity in v, (ii) a sequence prefix gives the same outputs
+    (causality), (iii) one (batch, head) of each against the oracle."""
+    hb = _hb()
+    B, H, T, Dk, Dv = 8, 16, 2048, 256, 512
+    q, k, v, decay = (t.cuda() for t in inputs.retnet_inputs(B, H, T, Dk, Dv, seed=0))
+    ld = torch.log(decay)
+    o = hb.linear_fwd(q, k, v, ld, q_scale=Dk ** -0.5)
+    o_half = hb.linear_fwd(q[:, :, :1024].contiguous(), k[:, :, :1024].contiguous(), v[:, :, :1024].contiguous(),
+                           ld[:, :, :1024].contiguous(), q_scale=Dk ** -0.5)
+    torch.cuda.synchronize()
+    assert torch.equal(o[:, :, :1024], o_half)
+    ref = oracle.retnet_quadratic(q[5:6, 9:10].cpu(), k[5:6, 9:10].cpu(), v[5:6, 9:10].cpu())
+    # head 9 of the oracle call is head 0 there: rebuild with the right decay through the generic chunked form
+    ref = oracle.linear_attention_chunked(q[5:6, 9:10].cpu(), k[5:6, 9:10].cpu(), v[5:6, 9:10].cpu(), ld[5:6, 9:10].cpu(),
+                                          chunk=64, q_scale=Dk ** -0.5)
+    oracle.assert_close(o[5:6, 9:10].float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    Bm_, H_, T_, P, N = 8, 64, 2048, 64, 128
+    Cm, Bm, x, dt, A = (t.cuda() for t in inputs.mamba2_inputs(Bm_, H_, T_, P, N, seed=0))
+    ldm = dt * A.view(1, H_, 1)
+    y = hb.linear_fwd(Cm, Bm, x, ldm, v_scale=dt)
+    y2 = hb.linear_fwd(Cm, Bm, (x.float() * 2).bfloat16(), ldm, v_scale=dt)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(y2.float(), 2 * y.float(), rtol=2e-2, atol=2e-2)
+    ref = oracle.ssd_chunk_scan_combined(x[3:4, 40:41].permute(0, 2, 1, 3).cpu(), dt[3:4, 40:41].permute(0, 2, 1).cpu(), A[0, 40:41].cpu(),
+                                         Bm[3:4].permute(0, 2, 1, 3).cpu(), Cm[3:4].permute(0, 2, 1, 3).cpu(), chunk_size=256).permute(0, 2, 1, 3)
+    oracle.assert_close(y[3:4, 40:41].float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_linear_rejects_bad_arguments():
+    hb = _hb()
+    q = torch.zeros(1, 2, 64, 96, device="cuda", dtype=torch.bfloat16)
+    v = torch.zeros(1, 2, 64, 64, device="cuda", dtype=torch.bfloat16)
+    ld = torch.zeros(1, 2, 64, device="cuda")
+    with pytest.raises(hb.MetaAttentionError) as ei:
+        hb.linear_fwd(q, q, v, ld)
+    assert "dim_k" in str(ei.value)
+    q2 = torch.zeros(1, 2, 64, 128, device="cuda", dtype=torch.float16)
+    with pytest.raises(hb.MetaAttentionError):
+        hb.linear_fwd(q2, q2, v.half(), ld)
