@@ -37,8 +37,11 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
   if (!(p->scale > 0.f)) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: scale must be > 0 (got %g)", (double)p->scale);
   if (p->mask == MA_MASK_CAUSAL && p->seqlen_q != p->seqlen_kv)
     return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: causal mask needs seqlen_q == seqlen_kv (%d vs %d)", p->seqlen_q, p->seqlen_kv);
-  if (p->family == MA_ATTN_RETENTION && !p->score_mask)
-    return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: RETENTION needs score_mask");
+  if (p->family == MA_ATTN_RETENTION) {
+    if (!p->score_mask) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: RETENTION needs score_mask");
+    if ((uintptr_t)p->score_mask % 8 != 0 || p->sm_stride_b % 4 != 0 || p->sm_stride_h % 4 != 0 || p->sm_stride_q % 4 != 0)
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: score_mask must be 8-byte aligned with strides that are multiples of 4 elements");
+  }
   const int64_t strides[] = {p->q_stride_s, p->q_stride_h, p->k_stride_s, p->k_stride_h, p->v_stride_s, p->v_stride_h,
                              p->o_stride_s, p->o_stride_h, p->q_stride_b, p->k_stride_b, p->v_stride_b, p->o_stride_b};
   for (int64_t s : strides)
