@@ -4,10 +4,17 @@
 A step is one forward pass of the headline workload: causal softmax MHA, bf16
 in / fp32 accumulate, B=8 H=32 S=4096 D=128 (synthetic N(0,1) inputs already
 resident in HBM).  Prints ONE JSON line; `value` is algorithmic TFLOP/s
-(causal counted at one half, 4*B*H*S^2*D*0.5 FLOP per pass).  The same line
+(causal counted at one half: 0.5 * 4 * B*H*S^2*D FLOP per pass).  The same line
 carries the roofline of the dominant kernel, a CPU baseline (the oracle's
 restated PyTorch reference timed on this box's host cores over a bounded
-sample) and, under "other_workloads", the remaining benchmark configurations.
+sample of the same workload) and, under "other_workloads", the remaining
+benchmark configurations, each with its own roofline fraction:
+
+  c2_sigmoid_causal   same shape, sigmoid(q.k*scale - log S) row function
+  c3_retnet_chunked   RetNet retention, chunked operator, B8 H16 S2048 Dqk256 Dv512
+  c3_retnet_parallel  same shape, normalised parallel operator with a [1,H,S,S] decay mask
+  c4_mamba2_ssd       Mamba2 SSD, B8 H64 S2048 P64 N128, one B/C group
+  c5_mla_decode       absorbed MLA decode, B64 Hq128 KV4096 d512+64 (HBM bound)
 """
 from __future__ import annotations
 
@@ -24,22 +31,46 @@ sys.path.insert(0, os.path.join(ROOT, "metaattention_amd"))
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a
+# 1 GiB copy (profiles/attn_fwd_kernel_c2_softmax_sigmoid.md): 849 MB read + 273 MB written
+ATTN_FWD_HBM_BYTES = 1.122e9
 
 
-def time_gpu(fn, steps, warmup):
+def time_gpu(fn, steps, warmup, flush=None):
+    """Average milliseconds per call over `steps` calls, HIP events on the launch stream.
+    With `flush`, the caches are overwritten before every call and each call is
+    timed on its own (for the HBM-bound workload)."""
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
+    if flush is None:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+    total = 0.0
     for _ in range(steps):
+        flush()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
         fn()
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return e0.elapsed_time(e1) / steps, wall_ms
+        e1.record()
+        torch.cuda.synchronize()
+        total += e0.elapsed_time(e1)
+    return total / steps
+
+
+def _mfma_entry(ms, flops, note=None, **extra):
+    tf = flops / ms / 1e9
+    d = dict(ms=round(ms, 4), tflops=round(tf, 1), frac_of_bf16_peak=round(tf / PEAK_BF16_TFLOPS, 4), algorithmic_flops=flops)
+    if note:
+        d["flop_convention"] = note
+    d.update(extra)
+    return d
 
 
 def bench_softmax(steps, warmup, family="softmax"):
@@ -55,26 +86,104 @@ def bench_softmax(steps, warmup, family="softmax"):
         fn = lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale, out=o, row_scale=lse)
     else:  # sigmoid(q.k*scale - log S)
         fn = lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SIGMOID, causal=True, scale=scale, bias=-math.log(S), out=o)
-    ms, wall_ms = time_gpu(fn, steps, warmup)
+    ms = time_gpu(fn, steps, warmup)
     flops = 0.5 * 4.0 * B * H * S * S * D
-    return dict(ms=ms, wall_ms=wall_ms, flops=flops, tflops=flops / ms / 1e9,
-                shape=dict(B=B, H=H, S=S, D=D, DV=D, causal=True))
+    return dict(ms=ms, flops=flops, tflops=flops / ms / 1e9, shape=dict(B=B, H=H, S=S, D=D, DV=D, causal=True))
+
+
+def bench_retnet_chunked(steps, warmup):
+    import torch
+    from metaattention_amd import hip_backend as hb
+    B, H, T, Dk, Dv = 8, 16, 2048, 256, 512
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 16).bfloat16()
+    k = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 16).bfloat16()
+    v = torch.randn(B, H, T, Dv, device="cuda", generator=g).bfloat16()
+    ld = torch.log(1 - torch.exp2(-5 - torch.arange(H, device="cuda").float())).view(1, H, 1).expand(B, H, T).contiguous()
+    o = torch.empty_like(v)
+    ms = time_gpu(lambda: hb.linear_fwd(q, k, v, ld, q_scale=Dk ** -0.5, out=o), steps, warmup)
+    C = 64
+    flops = B * H * (2.0 * T * C * (Dk + Dv) + 4.0 * T * Dk * Dv)
+    return _mfma_entry(ms, flops, "chunked form, chunk 64: 2*S*C*(Dqk+Dv) + 4*S*Dqk*Dv per (batch, head)")
+
+
+def bench_retnet_parallel(steps, warmup):
+    import torch
+    import oracle
+    from metaattention_amd import hip_backend as hb
+    B, H, S, D, DV = 8, 16, 2048, 256, 512
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q = (torch.randn(B, S, H, D, device="cuda", generator=g) / 16).bfloat16()
+    k = (torch.randn(B, S, H, D, device="cuda", generator=g) / 16).bfloat16()
+    v = torch.randn(B, S, H, DV, device="cuda", generator=g).bfloat16()
+    idx = torch.arange(S, device="cuda", dtype=torch.float32)
+    gam = 1 - torch.exp2(-5 - torch.arange(H, device="cuda").float())
+    diff = (idx.view(S, 1) - idx.view(1, S))
+    mask = (torch.exp2(diff.clamp(min=0).unsqueeze(0) * torch.log2(gam).view(H, 1, 1)) * (diff >= 0)).unsqueeze(0).bfloat16()
+    o = torch.empty_like(v)
+    r = torch.empty(B, H, S, device="cuda")
+    ms = time_gpu(lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mask, out=o,
+                                      row_scale=r), steps, warmup)
+    flops = 0.5 * 2.0 * B * H * S * S * (D + DV)
+    return _mfma_entry(ms, flops, "parallel form, causal counted at one half")
+
+
+def bench_mamba2(steps, warmup):
+    import torch
+    from metaattention_amd import hip_backend as hb
+    B, H, T, P, N = 8, 64, 2048, 64, 128
+    g = torch.Generator(device="cuda").manual_seed(0)
+    Cm = (torch.randn(B, 1, T, N, device="cuda", generator=g) / math.sqrt(N)).bfloat16()
+    Bm = (torch.randn(B, 1, T, N, device="cuda", generator=g) / math.sqrt(N)).bfloat16()
+    x = torch.randn(B, H, T, P, device="cuda", generator=g).bfloat16()
+    dt = torch.nn.functional.softplus(torch.randn(B, H, T, device="cuda", generator=g) - 2)
+    A = -torch.exp(torch.rand(1, H, device="cuda", generator=g) * math.log(16))
+    ld = (dt * A.view(1, H, 1)).contiguous()
+    o = torch.empty_like(x)
+    ms = time_gpu(lambda: hb.linear_fwd(Cm, Bm, x, ld, v_scale=dt, out=o), steps, warmup)
+    Lc = 256
+    flops = B * H * (2.0 * T * Lc * N + 2.0 * T * Lc * P + 4.0 * T * N * P)
+    return _mfma_entry(ms, flops, "chunk 256, C.B^T counted per head: 2*S*L*N + 2*S*L*P + 4*S*N*P per (batch, head); "
+                                  "the kernel itself uses 32-token chunks and executes fewer FLOPs")
+
+
+def bench_mla(steps, warmup):
+    import torch
+    from metaattention_amd import hip_backend as hb
+    B, Hq, Skv, D, Dpe = 64, 128, 4096, 512, 64
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q = torch.randn(B, 1, Hq, D, device="cuda", dtype=torch.bfloat16, generator=g)
+    q_pe = torch.randn(B, 1, Hq, Dpe, device="cuda", dtype=torch.bfloat16, generator=g)
+    kv = torch.randn(B, Skv, 1, D, device="cuda", dtype=torch.bfloat16, generator=g)
+    k_pe = torch.randn(B, Skv, 1, Dpe, device="cuda", dtype=torch.bfloat16, generator=g)
+    o = torch.empty_like(q)
+    ws = torch.empty(max(hb.mla_workspace_bytes(B, Hq, Skv), 16), dtype=torch.uint8, device="cuda")
+    junk = torch.empty(512 * 2 ** 20, dtype=torch.uint8, device="cuda")   # larger than L2 + the 256 MB last-level cache
+    fn = lambda: hb.mla_decode(q, q_pe, kv, k_pe, scale=1 / math.sqrt(D + Dpe), out=o, workspace=ws)
+    ms = time_gpu(fn, steps, warmup, flush=lambda: junk.fill_(1))
+    ms_warm = time_gpu(fn, steps, warmup)
+    nbytes = 2.0 * (kv.numel() + k_pe.numel() + q.numel() + q_pe.numel() + o.numel())
+    flops = 2.0 * B * Hq * Skv * (D + Dpe + D)
+    gbs = nbytes / ms / 1e6
+    return dict(ms=round(ms, 4), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / PEAK_HBM_GBS, 4), algorithmic_bytes=nbytes,
+                tflops=round(flops / ms / 1e9, 1), ms_without_cache_flush=round(ms_warm, 4),
+                note="split-KV kernel + combine kernel per call; caches overwritten before every timed call")
 
 
 def cpu_baseline_softmax():
     """Oracle (restated PyTorch reference, fp32) on the host cores over a bounded
-    sample of the headline workload: full S=4096, D=128, causal, B=1, H=8."""
+    sample: the whole headline workload once (B=8, H=32, S=4096, D=128, causal), about ten seconds."""
     import torch
     import oracle
-    B, H, S, D = 1, 8, 4096, 128
+    B, H, S, D = 8, 32, 4096, 128
     q, k, v = oracle.inputs.softmax_inputs(B, H, S, D, D, dtype=torch.bfloat16, seed=0)
-    oracle.softmax_attention(q[:, :, :1], k[:, :, :1], v[:, :, :1], causal=True)  # warm-up
+    oracle.softmax_attention(q[:1, :, :1], k[:1, :, :1], v[:1, :, :1], causal=True)  # warm-up
     t0 = time.perf_counter()
     oracle.softmax_attention(q, k, v, causal=True)
     dt = time.perf_counter() - t0
     flops = 0.5 * 4.0 * B * H * S * S * D
-    return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
-                sample=f"B={B} H={H} of the B=8 H=32 workload (S={S}, D={D}, causal), fp32 oracle, {dt:.2f} s, "
+    return dict(value=round(flops / dt / 1e12, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"B={B} of 8, H={H}, S={S}, D={D}, causal, fp32 oracle (restated PyTorch reference), {dt:.1f} s, "
                        f"os.cpu_count()={os.cpu_count()}")
 
 
@@ -84,6 +193,10 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run 5 plain device-to-device copies of 1 GiB and exit (reference point for rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--only", default="", help="comma list limiting the other workloads (e.g. 'mla'); 'none' skips them")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -95,10 +208,28 @@ def main():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
 
+    if args.calibrate_copy:
+        src = torch.ones(2 ** 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "5 device-to-device copies", "bytes_read_per_copy": 2 ** 30, "bytes_written_per_copy": 2 ** 30}))
+        return
+
     main_res = bench_softmax(args.steps, args.warmup, "softmax")
     others = {}
-    sig = bench_softmax(args.steps, args.warmup, "sigmoid")
-    others = {"c2_sigmoid_causal": dict(tflops=sig["tflops"], ms=sig["ms"], frac_of_bf16_peak=sig["tflops"] / PEAK_BF16_TFLOPS), **others}
+    want = [w for w in args.only.split(",") if w]
+    table = [("c2_sigmoid_causal", "sigmoid", lambda: (lambda r: _mfma_entry(r["ms"], r["flops"]))(bench_softmax(args.steps, args.warmup, "sigmoid"))),
+             ("c3_retnet_chunked", "retnet", lambda: bench_retnet_chunked(args.steps, args.warmup)),
+             ("c3_retnet_parallel", "retention", lambda: bench_retnet_parallel(args.steps, args.warmup)),
+             ("c4_mamba2_ssd", "mamba", lambda: bench_mamba2(args.steps, args.warmup)),
+             ("c5_mla_decode", "mla", lambda: bench_mla(args.steps, args.warmup))]
+    for name, key, fn in table:
+        if want and (want == ["none"] or not any(key.startswith(w) or w in name for w in want)):
+            continue
+        others[name] = fn()
+        torch.cuda.empty_cache()
 
     line = {
         "metric": "fwd TFLOP/s + % bf16 MFMA peak (prefill/chunked); decode HBM GB/s % peak",
@@ -111,8 +242,8 @@ def main():
         "config": {"workload": "causal softmax MHA forward, bf16 in / fp32 accumulate, B=8 H=32 S=4096 D=128",
                    **main_res["shape"]},
         "roofline": {"bound": "mfma", "achieved": round(main_res["tflops"], 2), "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(main_res["tflops"] / PEAK_BF16_TFLOPS, 4), "traffic": None,
-                     "kernel": "attn_fwd_kernel<bf16,128,128,softmax,causal>",
+                     "unit": "TFLOP/s", "frac": round(main_res["tflops"] / PEAK_BF16_TFLOPS, 4), "traffic": ATTN_FWD_HBM_BYTES,
+                     "kernel": "ma::attn_fwd_kernel<bf16, 128, 128, softmax, causal>",
                      "flops_per_launch": main_res["flops"]},
         "cpu_baseline": None,
         "other_workloads": others,
