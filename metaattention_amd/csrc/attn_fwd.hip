@@ -8,7 +8,8 @@
 //
 // Mapping onto CDNA4 (wave64, v_mfma_f32_32x32x16):
 //   * a workgroup is 4 waves; each wave owns 32 query rows (block_M = 128) and
-//     every wave walks the same 64-row KV tiles staged in LDS (double buffered);
+//     every wave walks the same 64-row KV tiles, which arrive in LDS by
+//     direct-to-LDS DMA (double buffered, one barrier per tile, no staging registers);
 //   * the score tile is computed TRANSPOSED, S^T = K Q^T (A = K rows from LDS,
 //     B = Q held in registers), so that in the accumulator layout every lane
 //     owns ONE query row: the online row statistics are per-lane scalars, the
@@ -18,25 +19,17 @@
 //   * V^T fragments come straight out of the row-major V tile with the
 //     transposing LDS read (ds_read_b64_tr_b16);
 //   * both LDS tiles are XOR-swizzled at 16-byte granularity so the 128-bit K
-//     reads and the transposing V reads are bank-conflict free without padding.
+//     reads and the transposing V reads are bank-conflict free without padding;
+//   * LDS fragment reads are requested a few MFMAs ahead of their use (explicit
+//     rings + scheduling barriers), and the output accumulator is only rescaled
+//     when a row maximum has grown by more than 2^8 (see below).
 #include "attn_fwd.h"
+
+#include <type_traits>
 
 namespace ma {
 
 enum { FAM_SOFTMAX = 0, FAM_SIGMOID = 1, FAM_RELU = 2 };
-
-template <int CPR>
-__device__ __forceinline__ int swz_k(int row) {
-  // 16 consecutive rows reading the same logical 16-byte chunk must land in 16
-  // different bank groups.
-  return CPR >= 16 ? (row & 15) : ((row >> 1) & 7);
-}
-template <int CPR>
-__device__ __forceinline__ int swz_v(int row) {
-  // a transposing read touches 8 consecutive rows x 4 consecutive chunks; spread
-  // the 4 rows of each lane block over the high chunk bits.
-  return CPR >= 16 ? (((row & 3) << 2) | ((row >> 2) & 3)) : (((row & 3) << 1) | ((row >> 2) & 1));
-}
 
 template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
@@ -49,15 +42,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
   constexpr int CPRK = DQK / 8, CPRV = DV / 8;  // 16-byte chunks per row
   constexpr int KROW = DQK * 2, VROW = DV * 2;
   constexpr int KTILE = BN * KROW, VTILE = BN * VROW;
-  constexpr int KCH = BN * CPRK / 256, VCH = BN * CPRV / 256;
-  static_assert(KCH >= 1 && VCH >= 1, "tile too small for 256 threads");
+  constexpr int NIK = KTILE / 1024, NIV = VTILE / 1024;  // DMA instructions (1 KB each) per tile
+  static_assert(CPRK >= 16 && CPRV >= 16 && NIK % 4 == 0 && NIV % 4 == 0, "tile shape");
 
   extern __shared__ __align__(16) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
   // [K buf0][K buf1][V buf0][V buf1]
   const uint32_t lds_k = lds0, lds_v = lds0 + 2 * KTILE;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), r = lane & 31, g = lane >> 5;
 
   // workgroup -> (batch*head, q block).  Consecutive workgroup ids are dealt
   // round-robin to the 8 XCDs, so all q blocks of one (batch, head) are kept on
@@ -86,54 +79,60 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 16 * ks);
   }
 
-  const T* kbase = (const T*)a.k + (int64_t)b * a.ksb + (int64_t)h * a.ksh;
-  const T* vbase = (const T*)a.v + (int64_t)b * a.vsb + (int64_t)h * a.vsh;
+  const char* kbase = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)h * a.ksh);
+  const char* vbase = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)h * a.vsh);
+  const int64_t k_row_bytes = a.kss * 2, v_row_bytes = a.vss * 2;
 
   int n_tiles = (a.Skv + BN - 1) / BN;
   if (CAUSAL) n_tiles = min(n_tiles, (mb * BM + BM + BN - 1) / BN);
 
-  // ---- global -> register -> LDS staging of one KV tile
-  u32x4 kreg[KCH], vreg[VCH];
-  auto load_tile = [&](int n0) {
+  // ---- DMA of one KV tile: each instruction moves 1 KB (1024/row_bytes tile rows); lane i fetches the
+  //      16-byte chunk that belongs at physical position i of that KB.  Wave w issues every 4th
+  //      instruction; its rows are 4 ii + lane/16 with ii = w + 4t, so the swizzle term
+  //      swz16(row) = ((lane/16) << 2) | w is the same for all of them and one per-lane 32-bit offset
+  //      serves every instruction (scalar base + vector offset addressing).
+  const uint32_t k_lane_off = (uint32_t)((lane / CPRK) * k_row_bytes) + (uint32_t)((((lane % CPRK) ^ swz16((lane / CPRK) | 0)) ^ (wave & 3)) << 4);
+  const uint32_t v_lane_off = (uint32_t)((lane / CPRV) * v_row_bytes) + (uint32_t)((((lane % CPRV) ^ swz16((lane / CPRV) | 0)) ^ (wave & 3)) << 4);
+  static_assert(1024 / KROW == 4 && 1024 / VROW == 4, "the shared lane offset assumes 4 tile rows per DMA instruction");
+  auto issue_tile = [&](int n0, int buf) {
+    if (n0 + BN <= a.Skv) {
 #pragma unroll
-    for (int i = 0; i < KCH; i++) {
-      const int ci = tid + 256 * i, row = ci / CPRK, c = ci % CPRK;
-      const int nrow = min(n0 + row, a.Skv - 1);
-      kreg[i] = *(const u32x4*)(kbase + (int64_t)nrow * a.kss + c * 8);
-    }
+      for (int t = 0; t < NIK / 4; t++) {
+        const int ii = wave + 4 * t;
+        dma16_so(kbase + (int64_t)(n0 + 4 * ii) * k_row_bytes, k_lane_off, lds_k + buf * KTILE + ii * 1024);
+      }
 #pragma unroll
-    for (int i = 0; i < VCH; i++) {
-      const int ci = tid + 256 * i, row = ci / CPRV, c = ci % CPRV;
-      const int nrow = min(n0 + row, a.Skv - 1);
-      vreg[i] = *(const u32x4*)(vbase + (int64_t)nrow * a.vss + c * 8);
-    }
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < KCH; i++) {
-      const int ci = tid + 256 * i, row = ci / CPRK, c = ci % CPRK;
-      lds_write<u32x4>(lds_k + buf * KTILE + row * KROW + ((c ^ swz_k<CPRK>(row)) << 4), kreg[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < VCH; i++) {
-      const int ci = tid + 256 * i, row = ci / CPRV, c = ci % CPRV;
-      lds_write<u32x4>(lds_v + buf * VTILE + row * VROW + ((c ^ swz_v<CPRV>(row)) << 4), vreg[i]);
+      for (int t = 0; t < NIV / 4; t++) {
+        const int ii = wave + 4 * t;
+        dma16_so(vbase + (int64_t)(n0 + 4 * ii) * v_row_bytes, v_lane_off, lds_v + buf * VTILE + ii * 1024);
+      }
+    } else {   // last, partial tile: rows beyond the sequence are clamped (their scores are masked)
+      for (int t = 0; t < NIK / 4; t++) {
+        const int ii = wave + 4 * t;
+        const int row = ii * 4 + lane / CPRK, c = lane % CPRK;
+        const int nrow = min(n0 + row, a.Skv - 1);
+        dma16(kbase + nrow * k_row_bytes + ((c ^ swz16(row)) << 4), lds_k + buf * KTILE + ii * 1024);
+      }
+      for (int t = 0; t < NIV / 4; t++) {
+        const int ii = wave + 4 * t;
+        const int row = ii * 4 + lane / CPRV, c = lane % CPRV;
+        const int nrow = min(n0 + row, a.Skv - 1);
+        dma16(vbase + nrow * v_row_bytes + ((c ^ swz16(row)) << 4), lds_v + buf * VTILE + ii * 1024);
+      }
     }
   };
 
   // ---- per-lane LDS read addresses
   // K (A operand of S^T): row 32nb + r, logical chunk 2ks + g
   const uint32_t k_row_off = r * KROW;
-  const int k_chunk0 = g ^ swz_k<CPRK>(r);
+  const int k_chunk0 = g ^ swz16(r);
   // V (A operand of O^T, through the transposing read): lane block = lane/16,
   // row nbase + 8*half + 4g + jr, logical chunk 4db + lc
   const int jr = (lane & 15) >> 2;
   const int lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
   const uint32_t v_row_off = (4 * g + jr) * VROW + (lane & 1) * 8;
-  const int v_swz_lane = swz_v<CPRV>(4 * g + jr);  // rows nbase + 8*half keep (row & 3) and flip bit 1 of (row >> 2)
-  const int v_chunk0 = lc ^ v_swz_lane;
-  constexpr int V_HALF_XOR = CPRV >= 16 ? 2 : 0;  // swz_v(row + 8) ^ swz_v(row)
-  static_assert(CPRV >= 16, "DV < 128 needs its own swizzle");
+  const int v_chunk0 = lc ^ swz16(4 * g + jr);
+  constexpr int V_HALF_XOR = 2;  // swz16(row + 8) ^ swz16(row) for row < 8; swz16(row + 16) == swz16(row)
 
   // ---- accumulators and row state
   f32x16 o[DB];
@@ -147,108 +146,157 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
   float row_max = -1e30f;  // running max of (scale*s + bias) * log2e
   float row_sum = 0.f;     // this lane's share of the running sum (the other half lives in lane^32)
 
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
-
-  for (int jt = 0; jt < n_tiles; jt++) {
-    const int buf = jt & 1, n0 = jt * BN;
-    if (jt + 1 < n_tiles) load_tile(n0 + BN);
-
-    // ---- S^T = K Q^T : lane holds query row r, kv rows 32nb + 8(j/4) + 4g + j%4
-    f32x16 s[NB];
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-      for (int j = 0; j < 16; j++) s[nb][j] = 0.f;
-    const uint32_t kb = lds_k + buf * KTILE + k_row_off;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      const uint32_t coff = (uint32_t)((k_chunk0 ^ (2 * ks)) << 4);
-#pragma unroll
-      for (int nb = 0; nb < NB; nb++) {
-        x8 kf = lds_read<x8>(kb + nb * 32 * KROW + coff);
-        s[nb] = E::mfma32(kf, qf[ks], s[nb]);
-      }
-    }
-
-    // ---- structural mask: exact -inf above the diagonal / beyond the cache
-    const bool need_mask = (CAUSAL && (n0 + BN - 1 > m_wave)) || (n0 + BN > a.Skv);
-    if (need_mask) {
-      const int lim = CAUSAL ? min(m_lane, a.Skv - 1) : a.Skv - 1;  // keep n <= lim
-#pragma unroll
+  // One KV tile.  BUF (LDS buffer) and MASKED are compile-time so that every LDS address is a lane
+  // register plus an immediate and the unmasked tiles carry no mask code.
+  auto do_tile = [&](auto buf_c, auto masked_c, const int buf_rt, const int n0) {
+    constexpr bool MASKED = decltype(masked_c)::value;          // may this tile need the structural mask?
+    const int BUF = decltype(buf_c)::value >= 0 ? decltype(buf_c)::value : buf_rt;   // compile-time unless -1
+      // ---- S^T = K Q^T : lane holds query row r, kv rows 32nb + 8(j/4) + 4g + j%4
+      f32x16 s[NB];
+  #pragma unroll
       for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-          const int n = n0 + 32 * nb + 8 * (j >> 2) + 4 * g + (j & 3);
-          if (n > lim) s[nb][j] = -INFINITY;
-        }
-    }
-
-    // ---- row function
-    if constexpr (FAMILY == FAM_SOFTMAX) {
-      float mx = s[0][0];
-#pragma unroll
-      for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-        for (int j = 0; j < 16; j++) mx = fmaxf(mx, s[nb][j]);
-      mx = fmaxf(mx, xhalf(mx));
-      const float new_max = fmaxf(row_max, mx * c_scale + c_bias);
-      const float corr = fast_exp2(row_max - new_max);
-      row_max = new_max;
-      const float sub = c_bias - new_max;
-      float part = 0.f;
-#pragma unroll
-      for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-          const float p = fast_exp2(s[nb][j] * c_scale + sub);
-          s[nb][j] = p;
-          part += p;
-        }
-      row_sum = row_sum * corr + part;
-      if (__any(corr != 1.f)) {
-#pragma unroll
-        for (int i = 0; i < DB; i++)
-#pragma unroll
-          for (int j = 0; j < 16; j++) o[i][j] *= corr;
-      }
-    } else if constexpr (FAMILY == FAM_SIGMOID) {
-#pragma unroll
-      for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-        for (int j = 0; j < 16; j++)  // sigmoid(x) = 1 / (1 + 2^(-x log2e)); s = -inf gives exactly 0
-          s[nb][j] = fast_rcp(1.f + fast_exp2(-(s[nb][j] * c_scale + c_bias)));
-    } else {
-#pragma unroll
-      for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-        for (int j = 0; j < 16; j++) s[nb][j] = fmaxf(s[nb][j] * a.scale + bias, 0.f);
-    }
-
-    // ---- O^T += V^T P^T ; the k index of MFMA slice (nb, t), lane half g, slot i is
-    //      kv row 32nb + 16t + 8(i/4) + 4g + i%4 on both operands
-    const uint32_t vb = lds_v + buf * VTILE + v_row_off;
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-      for (int t = 0; t < 2; t++) {
-        x8 pf;
-#pragma unroll
-        for (int i = 0; i < 8; i++) pf[i] = (T)s[nb][8 * t + i];
-        const uint32_t rb = vb + (32 * nb + 16 * t) * VROW;
-#pragma unroll
-        for (int db = 0; db < DB; db++) {
-          x4 lo = lds_read_tr4<T>(rb + (uint32_t)((v_chunk0 ^ (4 * db)) << 4));
-          x4 hi = lds_read_tr4<T>(rb + 8 * VROW + (uint32_t)((v_chunk0 ^ (4 * db) ^ V_HALF_XOR) << 4));
-          x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          o[db] = E::mfma32(vf, pf, o[db]);
+  #pragma unroll
+        for (int j = 0; j < 16; j++) s[nb][j] = 0.f;
+      {
+        constexpr int AH = 2, RING = 3;   // K fragments are requested AH slices ahead of their MFMAs
+        x8 kf[RING][NB];
+        const uint32_t kb = lds_k + BUF * KTILE + k_row_off;
+        auto request = [&](int ks) {
+          const uint32_t coff = (uint32_t)((k_chunk0 ^ (2 * ks)) << 4);
+  #pragma unroll
+          for (int nb = 0; nb < NB; nb++) kf[ks % RING][nb] = lds_read<x8>(kb + nb * 32 * KROW + coff);
+        };
+  #pragma unroll
+        for (int ks = 0; ks < AH; ks++) request(ks);
+  #pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          if (ks + AH < KS) request(ks + AH);
+          __builtin_amdgcn_sched_barrier(0);
+  #pragma unroll
+          for (int nb = 0; nb < NB; nb++) s[nb] = E::mfma32(kf[ks % RING][nb], qf[ks], s[nb]);
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
 
-    if (jt + 1 < n_tiles) store_tile(buf ^ 1);
+      // ---- structural mask: exact -inf above the diagonal / beyond the cache
+      if (MASKED && ((CAUSAL && (n0 + BN - 1 > m_wave)) || (n0 + BN > a.Skv))) {   // exact -inf above the diagonal / beyond the cache
+        const int lim = CAUSAL ? min(m_lane, a.Skv - 1) : a.Skv - 1;  // keep n <= lim
+  #pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+  #pragma unroll
+          for (int j = 0; j < 16; j++) {
+            const int n = n0 + 32 * nb + 8 * (j >> 2) + 4 * g + (j & 3);
+            if (n > lim) s[nb][j] = -INFINITY;
+          }
+      }
+
+      // ---- row function
+      if constexpr (FAMILY == FAM_SOFTMAX) {
+        float mx = s[0][0];
+  #pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+  #pragma unroll
+          for (int j = 0; j < 16; j++) mx = fmaxf(mx, s[nb][j]);
+        mx = fmaxf(mx, xhalf(mx));
+        // The running max only moves when some row's max grew by more than 2^8: until then probabilities
+        // are taken relative to the stale max (at most 256: exact in fp32, in range for bf16/fp16) and the
+        // accumulator needs no rescaling; the final division by row_sum absorbs the offset.
+        // Each row decides for itself (rows that stay multiply by exactly 1), so a row's result never
+        // depends on what other rows of its wave see.
+        const float cand = fmaxf(row_max, mx * c_scale + c_bias);
+        const bool move = cand - row_max > 8.f;
+        if (__any(move)) {
+          const float corr = move ? fast_exp2(row_max - cand) : 1.f;
+          row_max = move ? cand : row_max;
+          row_sum *= corr;
+  #pragma unroll
+          for (int i = 0; i < DB; i++)
+  #pragma unroll
+            for (int j = 0; j < 16; j++) o[i][j] *= corr;
+        }
+        const float sub = c_bias - row_max;
+        float part = 0.f;
+  #pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+  #pragma unroll
+          for (int j = 0; j < 16; j++) {
+            const float p = fast_exp2(s[nb][j] * c_scale + sub);
+            s[nb][j] = p;
+            part += p;
+          }
+        row_sum += part;
+      } else if constexpr (FAMILY == FAM_SIGMOID) {
+  #pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+  #pragma unroll
+          for (int j = 0; j < 16; j++)  // sigmoid(x) = 1 / (1 + 2^(-x log2e)); s = -inf gives exactly 0
+            s[nb][j] = fast_rcp(1.f + fast_exp2(-(s[nb][j] * c_scale + c_bias)));
+      } else {
+  #pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+  #pragma unroll
+          for (int j = 0; j < 16; j++) s[nb][j] = fmaxf(s[nb][j] * a.scale + bias, 0.f);
+      }
+
+      // ---- O^T += V^T P^T ; the k index of MFMA slice (nb, t), lane half g, slot i is
+      //      kv row 32nb + 16t + 8(i/4) + 4g + i%4 on both operands
+      {
+        x8 pf[2 * NB];
+  #pragma unroll
+        for (int sl = 0; sl < 2 * NB; sl++)
+  #pragma unroll
+          for (int i = 0; i < 8; i++) pf[sl][i] = (T)s[sl >> 1][8 * (sl & 1) + i];
+        const uint32_t vb = lds_v + BUF * VTILE + v_row_off;
+        constexpr int PF = 4, NIT = 2 * NB * DB;   // V fragments in flight; idx = sl * DB + db
+        x4 lo[PF], hi[PF];
+        auto request = [&](int idx) {
+          const int sl = idx / DB, db = idx % DB;
+          const uint32_t rb = vb + 16 * sl * VROW;
+          lo[idx % PF] = lds_read_tr4<T>(rb + (uint32_t)((v_chunk0 ^ (4 * db)) << 4));
+          hi[idx % PF] = lds_read_tr4<T>(rb + 8 * VROW + (uint32_t)((v_chunk0 ^ (4 * db) ^ V_HALF_XOR) << 4));
+        };
+  #pragma unroll
+        for (int i = 0; i < PF - 1; i++) request(i);
+  #pragma unroll
+        for (int idx = 0; idx < NIT; idx++) {
+          if (idx + PF - 1 < NIT) request(idx + PF - 1);
+          __builtin_amdgcn_sched_barrier(0);
+          x8 vf = __builtin_shufflevector(lo[idx % PF], hi[idx % PF], 0, 1, 2, 3, 4, 5, 6, 7);
+          o[idx % DB] = E::mfma32(vf, pf[idx / DB], o[idx % DB]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+  };
+
+  issue_tile(0, 0);
+
+  // Tiles [0, n_fast) need no mask in any wave: they run two per iteration with compile-time buffers.
+  // The remaining ones (the diagonal block of a causal workgroup, a partial last tile) take the generic path.
+  using std::integral_constant;
+  int n_fast = a.Skv / BN;
+  if (CAUSAL) n_fast = min(n_fast, mb * BM / BN);
+  n_fast &= ~1;
+  int jt = 0;
+  for (; jt < n_fast; jt += 2) {
+    wait_dma();
+    __syncthreads();   // tile jt has landed for every wave, and every wave is done reading tile jt-1
+    issue_tile((jt + 1) * BN, 1);
+    do_tile(integral_constant<int, 0>{}, integral_constant<bool, false>{}, 0, jt * BN);
+    wait_dma();
     __syncthreads();
+    if (jt + 2 < n_tiles) issue_tile((jt + 2) * BN, 0);
+    do_tile(integral_constant<int, 1>{}, integral_constant<bool, false>{}, 1, (jt + 1) * BN);
   }
+  for (; jt < n_tiles; jt++) {
+    const int buf = jt & 1, n0 = jt * BN;
+    wait_dma();
+    __syncthreads();
+    if (jt + 1 < n_tiles) issue_tile(n0 + BN, buf ^ 1);
+    // a wave whose 32 rows all lie above this tile's first column has nothing to do in it
+    if (CAUSAL && n0 > m_wave + 31) continue;
+    do_tile(integral_constant<int, -1>{}, integral_constant<bool, true>{}, buf, n0);
+  }
+  __syncthreads();   // every wave is done with the K/V buffers: they become output staging
 
   // ---- epilogue: normalise, stage O through LDS (wave-private), coalesced 16-byte stores
   float inv = 1.f, lse = 0.f;

@@ -184,9 +184,10 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
     // probabilities are taken relative to the stale max (at most 256, exact in fp32 / bf16 range) and the
     // 128 accumulator registers need no rescaling.  The final normalisation by row_sum absorbs the offset.
     const float cand = fmaxf(row_max, mx * c_scale);
-    if (__any(cand - row_max > 8.f)) {
-      const float corr = fast_exp2(row_max - cand);
-      row_max = cand;
+    const bool move = cand - row_max > 8.f;   // per head: heads that stay multiply by exactly 1
+    if (__any(move)) {
+      const float corr = move ? fast_exp2(row_max - cand) : 1.f;
+      row_max = move ? cand : row_max;
       row_sum *= corr;
 #pragma unroll
       for (int i = 0; i < DB; i++) o[i] *= corr;
