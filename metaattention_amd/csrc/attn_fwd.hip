@@ -133,6 +133,16 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
   const uint32_t v_row_off = (4 * g + jr) * VROW + (lane & 1) * 8;
   const int v_chunk0 = lc ^ swz16(4 * g + jr);
   constexpr int V_HALF_XOR = 2;  // swz16(row + 8) ^ swz16(row) for row < 8; swz16(row + 16) == swz16(row)
+  // all lane-dependent parts of the LDS read addresses, one register each; what is added per read
+  // (buffer, 32-row block, 16-row slice) is a compile-time immediate
+  uint32_t k_addr[KS], v_addr[DB][2];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) k_addr[ks] = lds_k + k_row_off + (uint32_t)((k_chunk0 ^ (2 * ks)) << 4);
+#pragma unroll
+  for (int db = 0; db < DB; db++) {
+    v_addr[db][0] = lds_v + v_row_off + (uint32_t)((v_chunk0 ^ (4 * db)) << 4);
+    v_addr[db][1] = lds_v + v_row_off + 8 * VROW + (uint32_t)((v_chunk0 ^ (4 * db) ^ V_HALF_XOR) << 4);
+  }
 
   // ---- accumulators and row state
   f32x16 o[DB];
@@ -246,14 +256,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
         for (int sl = 0; sl < 2 * NB; sl++)
   #pragma unroll
           for (int i = 0; i < 8; i++) pf[sl][i] = (T)s[sl >> 1][8 * (sl & 1) + i];
-        const uint32_t vb = lds_v + BUF * VTILE + v_row_off;
         constexpr int PF = 4, NIT = 2 * NB * DB;   // V fragments in flight; idx = sl * DB + db
         x4 lo[PF], hi[PF];
         auto request = [&](int idx) {
           const int sl = idx / DB, db = idx % DB;
-          const uint32_t rb = vb + 16 * sl * VROW;
-          lo[idx % PF] = lds_read_tr4<T>(rb + (uint32_t)((v_chunk0 ^ (4 * db)) << 4));
-          hi[idx % PF] = lds_read_tr4<T>(rb + 8 * VROW + (uint32_t)((v_chunk0 ^ (4 * db) ^ V_HALF_XOR) << 4));
+          lo[idx % PF] = lds_read_tr4<T>(v_addr[db][0] + BUF * VTILE + 16 * sl * VROW);
+          hi[idx % PF] = lds_read_tr4<T>(v_addr[db][1] + BUF * VTILE + 16 * sl * VROW);
         };
   #pragma unroll
         for (int i = 0; i < PF - 1; i++) request(i);
