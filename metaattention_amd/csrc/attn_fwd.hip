@@ -7,134 +7,121 @@
 // variants documented in include/metaattention_hip.h.
 //
 // Mapping onto CDNA4 (wave64, v_mfma_f32_32x32x16):
-//   * a workgroup is 4 waves; each wave owns 32 query rows (block_M = 128) and
-//     every wave walks the same 64-row KV tiles, which arrive in LDS by
-//     direct-to-LDS DMA (double buffered, one barrier per tile, no staging registers);
+//   * a workgroup is 8 waves (two per SIMD, one workgroup per CU); each wave owns 32 query rows
+//     (block_M = 256) and every wave walks the same 32-row KV sub-tiles, which arrive in LDS by
+//     direct-to-LDS DMA through rings of 8 K and 8 V buffers (loads run 6 sub-tiles ahead, each wave
+//     issues one K and one V instruction per sub-tile, spread between its MFMAs: the CU's vector
+//     memory path moves 64 B/clk and a wave that issues a burst of loads stalls on it);
 //   * the score tile is computed TRANSPOSED, S^T = K Q^T (A = K rows from LDS,
 //     B = Q held in registers), so that in the accumulator layout every lane
 //     owns ONE query row: the online row statistics are per-lane scalars, the
-//     row reductions are 31 in-register ops plus one exchange with lane^32, and
+//     row reductions are in-register ops plus one exchange with lane^32, and
 //     the probabilities are already in B-operand layout for O^T += V^T P^T with
 //     no LDS round trip;
 //   * V^T fragments come straight out of the row-major V tile with the
 //     transposing LDS read (ds_read_b64_tr_b16);
 //   * both LDS tiles are XOR-swizzled at 16-byte granularity so the 128-bit K
 //     reads and the transposing V reads are bank-conflict free without padding;
-//   * LDS fragment reads are requested a few MFMAs ahead of their use (explicit
-//     rings + scheduling barriers), and the output accumulator is only rescaled
-//     when a row maximum has grown by more than 2^8 (see below).
+//   * software pipeline inside each wave, three sub-tiles deep.  Vector-ALU work overlaps matrix work only
+//     when the two are interleaved finely (about four VALU instructions fit behind one MFMA), and a wave
+//     that alternates long MFMA-only and VALU-only phases leaves the matrix pipe idle whenever its SIMD
+//     partner is in the same phase.  So step u of a wave runs, interleaved per MFMA pair,
+//         MFMAs   P(u-1) V(u-1)   and   K(u+2) Q^T
+//         VALU    exp / sum / convert of sub-tile u   and   running row maximum of sub-tile u+1,
+//     with the scores of three and the probabilities of two sub-tiles live in registers: by the time a
+//     sub-tile's exponentials start, its row maximum is already folded into the reference point, so the
+//     exponentials depend on nothing that the step itself computes and every wave's instruction stream
+//     looks the same at all times;
+//   * the reference point of the exponentials follows the running maximum lazily: it (and with it the
+//     accumulator) only moves when a row's maximum has grown by more than 2^8 (see `finish_step`).
 #include "attn_fwd.h"
 
 #include <type_traits>
+#include <utility>
 
 namespace ma {
 
 enum { FAM_SOFTMAX = 0, FAM_SIGMOID = 1, FAM_RELU = 2 };
+constexpr int ATTN_NBUF = 6;   // K and V ring slots (32-row sub-tiles)
+
+namespace {
+template <int B, int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, B + I>{}), ...);
+}
+// f(integral_constant<int, i>) for i in [B, E), fully unrolled with compile-time indices
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl<B>(std::make_integer_sequence<int, E - B>{}, f);
+}
+}  // namespace
 
 template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   using E = Elem<T>;
   using x8 = typename E::x8;
   using x4 = typename E::x4;
-  constexpr int BM = 128, BN = 64, NB = BN / 32;
+  using x2 = typename E::x2;
+  constexpr int NW = 8, BM = 32 * NW, BN = 32, NBUF = ATTN_NBUF;
+  constexpr int DK_AHEAD = 7, DV_AHEAD = 4;   // step u issues the loads of K(u + 7) and V(u + 4)
   constexpr int KS = DQK / 16;   // k-slices of the QK^T contraction
   constexpr int DB = DV / 32;    // 32-wide output column blocks
   constexpr int CPRK = DQK / 8, CPRV = DV / 8;  // 16-byte chunks per row
   constexpr int KROW = DQK * 2, VROW = DV * 2;
   constexpr int KTILE = BN * KROW, VTILE = BN * VROW;
-  constexpr int NIK = KTILE / 1024, NIV = VTILE / 1024;  // DMA instructions (1 KB each) per tile
-  static_assert(CPRK >= 16 && CPRV >= 16 && NIK % 4 == 0 && NIV % 4 == 0, "tile shape");
+  constexpr int NQK = KS, NPV = 2 * DB;                  // MFMAs per sub-tile
+  static_assert(NBUF == 6, "the step bodies are unrolled by ring slot, score buffer (3) and parity (2)");
+  static_assert(CPRK == 16 && CPRV == 16, "one DMA instruction (1 KB) covers 4 tile rows");
+  static_assert(KTILE == NW * 1024 && VTILE == NW * 1024, "one K and one V DMA instruction per wave and sub-tile");
+  static_assert(NQK == NPV && NQK + NPV == 16, "one MFMA pair per two score elements");
+  static_assert(NBUF * KTILE <= 65536, "ring offsets must fit the 16-bit LDS instruction offset");
 
   extern __shared__ __align__(16) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
-  // [K buf0][K buf1][V buf0][V buf1]
-  const uint32_t lds_k = lds0, lds_v = lds0 + 2 * KTILE;
+  const uint32_t lds_k = lds0, lds_v = lds0 + NBUF * KTILE;   // [K ring][V ring]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), r = lane & 31, g = lane >> 5;
+  // Waves w and w + 4 share a SIMD.  Their 32-row blocks are paired as (0,7) (1,6) (2,5) (3,4) so that under
+  // a causal mask, where a block's work grows with its position, every SIMD gets the same amount.
+  const int row_block = wave < 4 ? wave : 11 - wave;
 
-  // workgroup -> (batch*head, q block).  Consecutive workgroup ids are dealt
-  // round-robin to the 8 XCDs, so all q blocks of one (batch, head) are kept on
-  // one XCD (shared K/V stays in that XCD's L2); causal q blocks run heaviest first.
-  const int nmb = a.num_m_blocks, BH = a.B * a.H;
-  int bh, mb;
-  if ((BH & 7) == 0) {
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    bh = (slot / nmb) * 8 + xcd;
-    mb = slot % nmb;
-  } else {
-    bh = blockIdx.x / nmb;
-    mb = blockIdx.x % nmb;
-  }
-  if (CAUSAL) mb = nmb - 1 - mb;
-  const int b = bh / a.H, h = bh % a.H;
-  const int m_wave = mb * BM + wave * 32;  // first query row of this wave
-  const int m_lane = m_wave + r;
+  // ---- per work item (one 256-row q block of one (batch, head)); see the item loop at the bottom
+  int b = 0, h = 0, mb = 0, m_wave = 0, m_lane = 0;
+  x8 qf[KS];                                   // Q fragments (B operand of S^T = K Q^T), kept in registers
+  const char *kbase = nullptr, *vbase = nullptr;
+  int n_sub = 0, last_sub = 0;                 // sub-tiles the workgroup walks; the last one this wave has anything to do in
 
-  // ---- Q fragments (B operand of S^T = K Q^T), kept in registers
-  x8 qf[KS];
-  {
-    const int qrow = min(m_lane, a.Sq - 1);
-    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)qrow * a.qss + (int64_t)h * a.qsh + 8 * g;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 16 * ks);
-  }
-
-  const char* kbase = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)h * a.ksh);
-  const char* vbase = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)h * a.vsh);
-  const int64_t k_row_bytes = a.kss * 2, v_row_bytes = a.vss * 2;
-
-  int n_tiles = (a.Skv + BN - 1) / BN;
-  if (CAUSAL) n_tiles = min(n_tiles, (mb * BM + BM + BN - 1) / BN);
-
-  // ---- DMA of one KV tile: each instruction moves 1 KB (1024/row_bytes tile rows); lane i fetches the
-  //      16-byte chunk that belongs at physical position i of that KB.  Wave w issues every 4th
-  //      instruction; its rows are 4 ii + lane/16 with ii = w + 4t, so the swizzle term
-  //      swz16(row) = ((lane/16) << 2) | w is the same for all of them and one per-lane 32-bit offset
-  //      serves every instruction (scalar base + vector offset addressing).
-  const uint32_t k_lane_off = (uint32_t)((lane / CPRK) * k_row_bytes) + (uint32_t)((((lane % CPRK) ^ swz16((lane / CPRK) | 0)) ^ (wave & 3)) << 4);
-  const uint32_t v_lane_off = (uint32_t)((lane / CPRV) * v_row_bytes) + (uint32_t)((((lane % CPRV) ^ swz16((lane / CPRV) | 0)) ^ (wave & 3)) << 4);
-  static_assert(1024 / KROW == 4 && 1024 / VROW == 4, "the shared lane offset assumes 4 tile rows per DMA instruction");
-  auto issue_tile = [&](int n0, int buf) {
-    if (n0 + BN <= a.Skv) {
-#pragma unroll
-      for (int t = 0; t < NIK / 4; t++) {
-        const int ii = wave + 4 * t;
-        dma16_so(kbase + (int64_t)(n0 + 4 * ii) * k_row_bytes, k_lane_off, lds_k + buf * KTILE + ii * 1024);
-      }
-#pragma unroll
-      for (int t = 0; t < NIV / 4; t++) {
-        const int ii = wave + 4 * t;
-        dma16_so(vbase + (int64_t)(n0 + 4 * ii) * v_row_bytes, v_lane_off, lds_v + buf * VTILE + ii * 1024);
-      }
-    } else {   // last, partial tile: rows beyond the sequence are clamped (their scores are masked)
-      for (int t = 0; t < NIK / 4; t++) {
-        const int ii = wave + 4 * t;
-        const int row = ii * 4 + lane / CPRK, c = lane % CPRK;
-        const int nrow = min(n0 + row, a.Skv - 1);
-        dma16(kbase + nrow * k_row_bytes + ((c ^ swz16(row)) << 4), lds_k + buf * KTILE + ii * 1024);
-      }
-      for (int t = 0; t < NIV / 4; t++) {
-        const int ii = wave + 4 * t;
-        const int row = ii * 4 + lane / CPRV, c = lane % CPRV;
-        const int nrow = min(n0 + row, a.Skv - 1);
-        dma16(vbase + nrow * v_row_bytes + ((c ^ swz16(row)) << 4), lds_v + buf * VTILE + ii * 1024);
-      }
-    }
+  // ---- DMA of one K or V sub-tile: 8 instructions of 1 KB (4 tile rows), one per wave; lane i fetches
+  //      the 16-byte chunk that belongs at physical position i of that KB.  Wave w has tile rows
+  //      4w + lane/16, whose swizzle term swz16(row) = ((lane/16) << 2) | (w & 3).  Rows beyond the
+  //      sequence are clamped to its last row (their scores are masked, their probabilities exactly 0),
+  //      so every step issues the same two instructions without a branch, also past the end.
+  //      Addressing is scalar base + 32-bit lane offset: the host checks that a (batch, head) plane of
+  //      K or V spans less than 4 GB.
+  const uint32_t swz_lane = (uint32_t)((((lane & 15) ^ ((lane >> 4) << 2)) ^ (wave & 3)) << 4);
+  const int tile_row = 4 * wave + (lane >> 4);
+  const uint32_t k_row_bytes = (uint32_t)(a.kss * 2), v_row_bytes = (uint32_t)(a.vss * 2);
+  auto issue_k_rt = [&](int su, uint32_t slot) __attribute__((always_inline)) {
+    const uint32_t row = (uint32_t)min(su * BN + tile_row, a.Skv - 1);
+    dma16_so(kbase, row * k_row_bytes + swz_lane, lds_k + slot * KTILE + wave * 1024);
+  };
+  auto issue_v_rt = [&](int su, uint32_t slot) __attribute__((always_inline)) {
+    const uint32_t row = (uint32_t)min(su * BN + tile_row, a.Skv - 1);
+    dma16_so(vbase, row * v_row_bytes + swz_lane, lds_v + slot * VTILE + wave * 1024);
   };
 
-  // ---- per-lane LDS read addresses
-  // K (A operand of S^T): row 32nb + r, logical chunk 2ks + g
+  // ---- per-lane LDS read addresses: all lane-dependent parts, one register each; what is added per
+  //      read (ring slot, 16-row slice) is a compile-time immediate
+  // K (A operand of S^T): row r, logical chunk 2ks + g
+  // V (A operand of O^T, through the transposing read): lane block = lane/16,
+  //   row 16sl + 8*half + 4g + jr, logical chunk 4db + lc
   const uint32_t k_row_off = r * KROW;
   const int k_chunk0 = g ^ swz16(r);
-  // V (A operand of O^T, through the transposing read): lane block = lane/16,
-  // row nbase + 8*half + 4g + jr, logical chunk 4db + lc
   const int jr = (lane & 15) >> 2;
   const int lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
   const uint32_t v_row_off = (4 * g + jr) * VROW + (lane & 1) * 8;
   const int v_chunk0 = lc ^ swz16(4 * g + jr);
   constexpr int V_HALF_XOR = 2;  // swz16(row + 8) ^ swz16(row) for row < 8; swz16(row + 16) == swz16(row)
-  // all lane-dependent parts of the LDS read addresses, one register each; what is added per read
-  // (buffer, 32-row block, 16-row slice) is a compile-time immediate
   uint32_t k_addr[KS], v_addr[DB][2];
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) k_addr[ks] = lds_k + k_row_off + (uint32_t)((k_chunk0 ^ (2 * ks)) << 4);
@@ -146,201 +133,305 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 
   // ---- accumulators and row state
   f32x16 o[DB];
-#pragma unroll
-  for (int i = 0; i < DB; i++)
-#pragma unroll
-    for (int j = 0; j < 16; j++) o[i][j] = 0.f;
   const float bias = a.bias + (a.bias_ptr ? *a.bias_ptr : 0.f);
   const float c_scale = a.scale * kLog2e;  // scores are handled in the log2 domain
   const float c_bias = bias * kLog2e;
-  float row_max = -1e30f;  // running max of (scale*s + bias) * log2e
+  float row_ref = -1e30f;  // reference point of the exponentials: a running max of (scale*s + bias) * log2e, moved lazily
   float row_sum = 0.f;     // this lane's share of the running sum (the other half lives in lane^32)
 
-  // One KV tile.  BUF (LDS buffer) and MASKED are compile-time so that every LDS address is a lane
-  // register plus an immediate and the unmasked tiles carry no mask code.
-  auto do_tile = [&](auto buf_c, auto masked_c, const int buf_rt, const int n0) {
-    constexpr bool MASKED = decltype(masked_c)::value;          // may this tile need the structural mask?
-    const int BUF = decltype(buf_c)::value >= 0 ? decltype(buf_c)::value : buf_rt;   // compile-time unless -1
-      // ---- S^T = K Q^T : lane holds query row r, kv rows 32nb + 8(j/4) + 4g + j%4
-      f32x16 s[NB];
-  #pragma unroll
-      for (int nb = 0; nb < NB; nb++)
-  #pragma unroll
-        for (int j = 0; j < 16; j++) s[nb][j] = 0.f;
-      {
-        constexpr int AH = 2, RING = 3;   // K fragments are requested AH slices ahead of their MFMAs
-        x8 kf[RING][NB];
-        const uint32_t kb = lds_k + BUF * KTILE + k_row_off;
-        auto request = [&](int ks) {
-          const uint32_t coff = (uint32_t)((k_chunk0 ^ (2 * ks)) << 4);
-  #pragma unroll
-          for (int nb = 0; nb < NB; nb++) kf[ks % RING][nb] = lds_read<x8>(kb + nb * 32 * KROW + coff);
-        };
-  #pragma unroll
-        for (int ks = 0; ks < AH; ks++) request(ks);
-  #pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-          if (ks + AH < KS) request(ks + AH);
-          __builtin_amdgcn_sched_barrier(0);
-  #pragma unroll
-          for (int nb = 0; nb < NB; nb++) s[nb] = E::mfma32(kf[ks % RING][nb], qf[ks], s[nb]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
+  // scores s[u % 3] and probabilities p[u & 1] of sub-tile u.
+  // lane holds query row r; element jj of a sub-tile is kv row 8(jj/4) + 4g + jj%4.
+  // p[par][sl] packs elements 8sl .. 8sl+7: the B operand of PV slice sl (k slot i of lane half g is
+  // kv row 16sl + 8(i/4) + 4g + i%4, matched by the rows the transposing V reads fetch).
+  f32x16 s[3];
+  u32x4 p[2][2];
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-      // ---- structural mask: exact -inf above the diagonal / beyond the cache
-      if (MASKED && ((CAUSAL && (n0 + BN - 1 > m_wave)) || (n0 + BN > a.Skv))) {   // exact -inf above the diagonal / beyond the cache
-        const int lim = CAUSAL ? min(m_lane, a.Skv - 1) : a.Skv - 1;  // keep n <= lim
-  #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-  #pragma unroll
-          for (int j = 0; j < 16; j++) {
-            const int n = n0 + 32 * nb + 8 * (j >> 2) + 4 * g + (j & 3);
-            if (n > lim) s[nb][j] = -INFINITY;
-          }
+  // structural mask of sub-tile su (scores in s[SB]): exact -inf above the diagonal / beyond the cache
+  auto apply_mask = [&](auto sb_c, int su) __attribute__((always_inline)) {
+    constexpr int SB = decltype(sb_c)::value;
+    const int n0 = su * BN;
+    if ((CAUSAL && (n0 + BN - 1 > m_wave)) || (n0 + BN > a.Skv)) {
+      const int lim = CAUSAL ? min(m_lane, a.Skv - 1) : a.Skv - 1;
+#pragma unroll
+      for (int j = 0; j < 16; j++) {
+        const int n = n0 + 8 * (j >> 2) + 4 * g + (j & 3);
+        if (n > lim) s[SB][j] = -INFINITY;
       }
-
-      // ---- row function
-      if constexpr (FAMILY == FAM_SOFTMAX) {
-        float mx = s[0][0];
-  #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-  #pragma unroll
-          for (int j = 0; j < 16; j++) mx = fmaxf(mx, s[nb][j]);
-        mx = fmaxf(mx, xhalf(mx));
-        // The running max only moves when some row's max grew by more than 2^8: until then probabilities
-        // are taken relative to the stale max (at most 256: exact in fp32, in range for bf16/fp16) and the
-        // accumulator needs no rescaling; the final division by row_sum absorbs the offset.
-        // Each row decides for itself (rows that stay multiply by exactly 1), so a row's result never
-        // depends on what other rows of its wave see.
-        const float cand = fmaxf(row_max, mx * c_scale + c_bias);
-        const bool move = cand - row_max > 8.f;
-        if (__any(move)) {
-          const float corr = move ? fast_exp2(row_max - cand) : 1.f;
-          row_max = move ? cand : row_max;
-          row_sum *= corr;
-  #pragma unroll
-          for (int i = 0; i < DB; i++)
-  #pragma unroll
-            for (int j = 0; j < 16; j++) o[i][j] *= corr;
-        }
-        const float sub = c_bias - row_max;
-        float part = 0.f;
-  #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-  #pragma unroll
-          for (int j = 0; j < 16; j++) {
-            const float p = fast_exp2(s[nb][j] * c_scale + sub);
-            s[nb][j] = p;
-            part += p;
-          }
-        row_sum += part;
-      } else if constexpr (FAMILY == FAM_SIGMOID) {
-  #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-  #pragma unroll
-          for (int j = 0; j < 16; j++)  // sigmoid(x) = 1 / (1 + 2^(-x log2e)); s = -inf gives exactly 0
-            s[nb][j] = fast_rcp(1.f + fast_exp2(-(s[nb][j] * c_scale + c_bias)));
-      } else {
-  #pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-  #pragma unroll
-          for (int j = 0; j < 16; j++) s[nb][j] = fmaxf(s[nb][j] * a.scale + bias, 0.f);
-      }
-
-      // ---- O^T += V^T P^T ; the k index of MFMA slice (nb, t), lane half g, slot i is
-      //      kv row 32nb + 16t + 8(i/4) + 4g + i%4 on both operands
-      {
-        x8 pf[2 * NB];
-  #pragma unroll
-        for (int sl = 0; sl < 2 * NB; sl++)
-  #pragma unroll
-          for (int i = 0; i < 8; i++) pf[sl][i] = (T)s[sl >> 1][8 * (sl & 1) + i];
-        constexpr int PF = 4, NIT = 2 * NB * DB;   // V fragments in flight; idx = sl * DB + db
-        x4 lo[PF], hi[PF];
-        auto request = [&](int idx) {
-          const int sl = idx / DB, db = idx % DB;
-          lo[idx % PF] = lds_read_tr4<T>(v_addr[db][0] + BUF * VTILE + 16 * sl * VROW);
-          hi[idx % PF] = lds_read_tr4<T>(v_addr[db][1] + BUF * VTILE + 16 * sl * VROW);
-        };
-  #pragma unroll
-        for (int i = 0; i < PF - 1; i++) request(i);
-  #pragma unroll
-        for (int idx = 0; idx < NIT; idx++) {
-          if (idx + PF - 1 < NIT) request(idx + PF - 1);
-          __builtin_amdgcn_sched_barrier(0);
-          x8 vf = __builtin_shufflevector(lo[idx % PF], hi[idx % PF], 0, 1, 2, 3, 4, 5, 6, 7);
-          o[idx % DB] = E::mfma32(vf, pf[idx / DB], o[idx % DB]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
+    }
   };
 
-  issue_tile(0, 0);
-
-  // Tiles [0, n_fast) need no mask in any wave: they run two per iteration with compile-time buffers.
-  // The remaining ones (the diagonal block of a causal workgroup, a partial last tile) take the generic path.
-  using std::integral_constant;
-  int n_fast = a.Skv / BN;
-  if (CAUSAL) n_fast = min(n_fast, mb * BM / BN);
-  n_fast &= ~1;
-  int jt = 0;
-  for (; jt < n_fast; jt += 2) {
-    wait_dma();
-    __syncthreads();   // tile jt has landed for every wave, and every wave is done reading tile jt-1
-    issue_tile((jt + 1) * BN, 1);
-    do_tile(integral_constant<int, 0>{}, integral_constant<bool, false>{}, 0, jt * BN);
-    wait_dma();
-    __syncthreads();
-    if (jt + 2 < n_tiles) issue_tile((jt + 2) * BN, 0);
-    do_tile(integral_constant<int, 1>{}, integral_constant<bool, false>{}, 1, (jt + 1) * BN);
-  }
-  for (; jt < n_tiles; jt++) {
-    const int buf = jt & 1, n0 = jt * BN;
-    wait_dma();
-    __syncthreads();
-    if (jt + 1 < n_tiles) issue_tile(n0 + BN, buf ^ 1);
-    // a wave whose 32 rows all lie above this tile's first column has nothing to do in it
-    if (CAUSAL && n0 > m_wave + 31) continue;
-    do_tile(integral_constant<int, -1>{}, integral_constant<bool, true>{}, buf, n0);
-  }
-  __syncthreads();   // every wave is done with the K/V buffers: they become output staging
-
-  // ---- epilogue: normalise, stage O through LDS (wave-private), coalesced 16-byte stores
-  float inv = 1.f, lse = 0.f;
-  if constexpr (FAMILY == FAM_SOFTMAX) {
-    const float tot = row_sum + xhalf(row_sum);
-    inv = 1.f / tot;
-    lse = (row_max + fast_log2(tot)) * kLn2;
-  }
-  constexpr int OROW = DV * 2 + 16;  // padded staging row
-  const uint32_t ob = lds0 + wave * 32 * OROW;
+  // elements e0, e0+1 of the sub-tile in s[SB]: score -> probability, row sum, packed into p[PAR]
+  auto prob_pair = [&](auto sb_c, auto par_c, auto e_c, float sub, float& part) __attribute__((always_inline)) {
+#pragma clang fp reassociate(off)   // keep the running sum a chain in element order
+    constexpr int SB = decltype(sb_c)::value, PAR = decltype(par_c)::value, e0 = decltype(e_c)::value;
+    float pe[2];
 #pragma unroll
-  for (int db = 0; db < DB; db++)
-#pragma unroll
-    for (int q4 = 0; q4 < 4; q4++) {
-      x4 w;
-#pragma unroll
-      for (int i = 0; i < 4; i++) w[i] = (T)(o[db][4 * q4 + i] * inv);
-      lds_write<x4>(ob + r * OROW + (32 * db + 8 * q4 + 4 * g) * 2, w);
+    for (int i = 0; i < 2; i++) {
+      const float v = s[SB][e0 + i];
+      if constexpr (FAMILY == FAM_SOFTMAX) {
+        pe[i] = fast_exp2(v * c_scale + sub);
+        part += pe[i];
+      } else if constexpr (FAMILY == FAM_SIGMOID) {   // sigmoid(x) = 1 / (1 + 2^(-x log2e)); s = -inf gives exactly 0
+        pe[i] = fast_rcp(1.f + fast_exp2(-(v * c_scale + c_bias)));
+      } else {
+        pe[i] = fmaxf(v * a.scale + bias, 0.f);
+      }
     }
-  T* obase = (T*)a.o + (int64_t)b * a.osb + (int64_t)h * a.osh;
+    x2 pk;
+    pk[0] = (T)pe[0];
+    pk[1] = (T)pe[1];
+    p[PAR][e0 >> 3][(e0 & 7) >> 1] = __builtin_bit_cast(uint32_t, pk);
+  };
+
+  // Softmax bookkeeping once the raw maximum `mx` of a sub-tile is known, BEFORE that sub-tile's
+  // exponentials: the reference point only moves for rows whose maximum exceeds it by more than 2^8.
+  // Until then probabilities are taken relative to the stale reference (at most 256: exact in fp32, in
+  // range for bf16/fp16) and nothing needs rescaling; the final division by row_sum absorbs the offset.
+  // When rows move, everything accumulated relative to the old reference is rescaled: the accumulator,
+  // the row sum and the probabilities of the previous sub-tile, which are still waiting for their P V.
+  // Each row decides for itself (rows that stay multiply by exactly 1), so a row's result never depends
+  // on what other rows of its wave see.
+  auto fold_max = [&](auto pend_c, float mx) __attribute__((always_inline)) {
+    constexpr int PEND = decltype(pend_c)::value;   // parity of the pending probabilities
+    float m_lo, m_hi;
+    xhalf_pair(mx, m_lo, m_hi);
+    const float cand = fmaxf(m_lo, m_hi) * c_scale + c_bias;
+    const bool move = cand - row_ref > 8.f;
+    if (__builtin_expect(__any(move), 0)) {
+      const float corr = move ? fast_exp2(row_ref - cand) : 1.f;
+      row_ref = move ? cand : row_ref;
+      row_sum *= corr;
+      // In place by construction, and with the wait states that cover the longest MFMA-result-to-VALU
+      // hazard (only the compiler's own instructions get those for free).
+      asm volatile("s_nop 7\n s_nop 7\n s_nop 7");
 #pragma unroll
-  for (int it = 0; it < 32 * CPRV / 64; it++) {
-    const int ci = lane + 64 * it, row = ci / CPRV, c = ci % CPRV;
-    u32x4 w = lds_read<u32x4>(ob + row * OROW + c * 16);
-    if (m_wave + row < a.Sq) *(u32x4*)(obase + (int64_t)(m_wave + row) * a.oss + c * 8) = w;
-  }
-  if constexpr (FAMILY == FAM_SOFTMAX) {
-    if (a.row_scale && g == 0 && m_lane < a.Sq) a.row_scale[((int64_t)b * a.H + h) * a.Sq + m_lane] = lse;
+      for (int i = 0; i < DB; i++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(o[i][j]) : "v"(corr));
+#pragma unroll
+      for (int sl = 0; sl < 2; sl++) {
+        x8 v = __builtin_bit_cast(x8, p[PEND][sl]);
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = (T)((float)v[i] * corr);
+        p[PEND][sl] = __builtin_bit_cast(u32x4, v);
+      }
+    }
+  };
+
+  // K and V fragments travel through small register rings and are requested PF-1 MFMA pairs ahead, across
+  // step boundaries: pair i of a step is PV MFMA i (V slice i / DB, column block i % DB) and QK MFMA i
+  // (k-slice i).
+  constexpr int PF = 3;
+  x4 lo[PF], hi[PF];
+  x8 kf[PF];
+  // pair I of the step whose V is in ring slot VSLOT and whose K is in ring slot KSLOT
+  auto request = [&](auto i_c, auto vslot_c, auto kslot_c) __attribute__((always_inline)) {
+    constexpr int I = decltype(i_c)::value, VS = decltype(vslot_c)::value, KSL = decltype(kslot_c)::value;
+    constexpr int sl = I / DB, db = I % DB;
+    lo[I % PF] = lds_read_tr4<T>(v_addr[db][0] + VS * VTILE + 16 * sl * VROW);
+    hi[I % PF] = lds_read_tr4<T>(v_addr[db][1] + VS * VTILE + 16 * sl * VROW);
+    kf[I % PF] = lds_read<x8>(k_addr[I] + KSL * KTILE);
+  };
+
+  // Step u of the software pipeline; SLOT = u % 6 is compile-time and fixes the ring slots, the score
+  // buffers (u % 3) and the probability buffers (u & 1):
+  //   O^T += V(u-1)^T P(u-1)^T   V ring slot SLOT-1, probabilities p[1-PAR]
+  //   s[(u+2) % 3] = K(u+2) Q^T  K ring slot SLOT+2
+  //   probabilities of sub-tile u from s[u % 3] into p[PAR]          (its maximum is already in row_ref)
+  //   mask and row maximum of sub-tile u+1 in s[(u+1) % 3], folded into row_ref at the end
+  // and, last, the first fragment requests of step u+1 (V(u), K(u+3)).
+  auto step = [&](auto slot_c, int u) __attribute__((always_inline)) {
+    constexpr int SLOT = decltype(slot_c)::value, PAR = SLOT & 1;
+    using ic = std::integral_constant<int, 0>;
+    constexpr auto par_c = std::integral_constant<int, PAR>{};
+    constexpr auto sb_exp_c = std::integral_constant<int, SLOT % 3>{};
+    constexpr auto sb_max_c = std::integral_constant<int, (SLOT + 1) % 3>{};
+    constexpr int SB_MAX = (SLOT + 1) % 3, SB_QK = (SLOT + 2) % 3;
+    constexpr auto vs_c = std::integral_constant<int, (SLOT + NBUF - 1) % NBUF>{};
+    constexpr auto ks_c = std::integral_constant<int, (SLOT + 2) % NBUF>{};
+    constexpr auto vs_next_c = std::integral_constant<int, SLOT>{};
+    constexpr auto ks_next_c = std::integral_constant<int, (SLOT + 3) % NBUF>{};
+    (void)sizeof(ic);
+    if constexpr (FAMILY == FAM_SOFTMAX) apply_mask(sb_max_c, u + 1);
+    else apply_mask(sb_exp_c, u);
+    const float sub = c_bias - row_ref;
+    float part = 0.f, mx = -INFINITY;
+    static_for<0, NPV>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value;
+      if constexpr (i + PF - 1 < NPV) request(std::integral_constant<int, i + PF - 1>{}, vs_c, ks_c);
+      if constexpr (i == 1) issue_k_rt(u + DK_AHEAD, (SLOT + DK_AHEAD) % NBUF);
+      if constexpr (i == 5) issue_v_rt(u + DV_AHEAD, (SLOT + DV_AHEAD) % NBUF);
+      __builtin_amdgcn_sched_barrier(0);
+      x8 vf = __builtin_shufflevector(lo[i % PF], hi[i % PF], 0, 1, 2, 3, 4, 5, 6, 7);
+      o[i % DB] = E::mfma32(vf, __builtin_bit_cast(x8, p[1 - PAR][i / DB]), o[i % DB]);
+      __builtin_amdgcn_sched_barrier(0);
+      s[SB_QK] = E::mfma32(kf[i % PF], qf[i], i == 0 ? zero16 : s[SB_QK]);
+      prob_pair(sb_exp_c, par_c, std::integral_constant<int, 2 * i>{}, sub, part);
+      if constexpr (FAMILY == FAM_SOFTMAX) mx = fmaxf(fmaxf(mx, s[SB_MAX][2 * i]), s[SB_MAX][2 * i + 1]);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    if constexpr (FAMILY == FAM_SOFTMAX) {
+      row_sum += part;
+      fold_max(par_c, mx);
+    }
+    static_for<0, PF - 1>([&](auto i_c) __attribute__((always_inline)) { request(i_c, vs_next_c, ks_next_c); });
+  };
+
+  // ---- work items.  The grid is one workgroup per CU and every workgroup walks its share of the
+  //      (batch*head, q block) items: a workgroup of this size owns its CU, and launching a fresh one per
+  //      item leaves the CU idle for several microseconds between items.  Consecutive workgroup ids are
+  //      dealt round-robin to the 8 XCDs, so XCD x takes the (batch, head) pairs with bh % 8 == x and
+  //      its CUs work on the q blocks of the same few pairs at the same time (their K/V stays in that
+  //      XCD's L2).  Under a causal mask a q block's work grows with its position, so the unit of work
+  //      is a pair of q blocks (k, nmb-1-k) of one (batch, head): every unit weighs the same.
+  const int nmb = a.num_m_blocks, BH = a.B * a.H, G = (int)gridDim.x;
+  const bool paired = CAUSAL && BH * nmb > G;               // (few items: one q block per unit, spread wide)
+  const int upb = paired ? (nmb + 1) >> 1 : nmb;            // units per (batch, head)
+  const bool by_xcd = (BH & 7) == 0 && (G & 7) == 0;
+  const int units = by_xcd ? (BH >> 3) * upb : BH * upb;   // units of this workgroup's stream
+  const int first = by_xcd ? (int)blockIdx.x >> 3 : (int)blockIdx.x, stride = by_xcd ? G >> 3 : G;
+  for (int t = 2 * first; t < 2 * units; t = (t & 1) ? t + 2 * stride - 1 : t + 1) {
+    const int q = t >> 1, k = q % upb;
+    if (paired) {
+      mb = (t & 1) ? k : nmb - 1 - k;
+      if ((t & 1) && k == nmb - 1 - k) continue;   // the middle block of an odd count is its own partner
+    } else {
+      mb = CAUSAL ? nmb - 1 - k : k;
+      if (t & 1) continue;
+    }
+    int bh = q / upb;
+    if (by_xcd) bh = bh * 8 + ((int)blockIdx.x & 7);
+    b = bh / a.H;
+    h = bh % a.H;
+    m_wave = mb * BM + row_block * 32;  // first query row of this wave
+    m_lane = m_wave + r;
+    n_sub = (a.Skv + BN - 1) / BN;
+    if (CAUSAL) n_sub = min(n_sub, (mb * BM + BM) / BN);
+    last_sub = CAUSAL ? min(n_sub - 1, m_wave / BN) : n_sub - 1;
+    kbase = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)h * a.ksh);
+    vbase = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)h * a.vsh);
+    {
+      const int qrow = min(m_lane, a.Sq - 1);
+      const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)qrow * a.qss + (int64_t)h * a.qsh + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 16 * ks);
+    }
+    // V ring slot NBUF-1 is read (times zero probabilities) before anything was loaded into it
+    for (int i = tid; i < VTILE / 16; i += 64 * NW) lds_write<u32x4>(lds_v + (NBUF - 1) * VTILE + i * 16, u32x4{0u, 0u, 0u, 0u});
+#pragma unroll
+    for (int i = 0; i < DB; i++)
+#pragma unroll
+      for (int j = 0; j < 16; j++) o[i][j] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; i++) p[0][i] = p[1][i] = u32x4{0u, 0u, 0u, 0u};
+    row_ref = -1e30f;
+    row_sum = 0.f;
+
+    // ---- schedule.  Step u (u = 0 .. last_sub + 1 for a wave) reads K(u+2), V(u-1) and the first fragments
+    //      of K(u+3), V(u).  The barrier at the top of step u therefore stands for: K(u+3) and V(u) have
+    //      landed for every wave, and every wave is done reading K(<=u+1) and V(<=u-2) -- the ring slots
+    //      that step u refills with K(u+7) and V(u+4).  A wave's loads complete in order and every step
+    //      issues K then V; K(u+3) and V(u) are the pair of step u-4, so at the top of step u the six
+    //      instructions of steps u-3 .. u-1 may still be in flight.
+    static_for<0, NBUF>([&](auto t_c) __attribute__((always_inline)) {   // K(0..5) and V(0..3), plus K(6) below
+      constexpr int t = decltype(t_c)::value;
+      issue_k_rt(t, t);
+      if constexpr (t < DV_AHEAD) issue_v_rt(t, t);
+    });
+    wait_dma();
+    __syncthreads();
+    {   // s[0] = K(0) Q^T with its maximum folded in, s[1] = K(1) Q^T; then K(6) may replace K(0)
+      x8 k0[KS];
+  #pragma unroll
+      for (int ks = 0; ks < KS; ks++) k0[ks] = lds_read<x8>(k_addr[ks]);
+  #pragma unroll
+      for (int ks = 0; ks < KS; ks++) s[0] = E::mfma32(k0[ks], qf[ks], ks == 0 ? zero16 : s[0]);
+  #pragma unroll
+      for (int ks = 0; ks < KS; ks++) k0[ks] = lds_read<x8>(k_addr[ks] + KTILE);
+  #pragma unroll
+      for (int ks = 0; ks < KS; ks++) s[1] = E::mfma32(k0[ks], qf[ks], ks == 0 ? zero16 : s[1]);
+      if constexpr (FAMILY == FAM_SOFTMAX) {
+        apply_mask(std::integral_constant<int, 0>{}, 0);
+        float mx = s[0][0];
+  #pragma unroll
+        for (int j = 1; j < 16; j++) mx = fmaxf(mx, s[0][j]);
+        fold_max(std::integral_constant<int, 1>{}, mx);
+      }
+    }
+    __syncthreads();   // every wave is done reading K(0)
+    issue_k_rt(NBUF, 0);
+    static_for<0, PF - 1>([&](auto i_c) __attribute__((always_inline)) {   // first fragments of step 0: zeros, K(2)
+      request(i_c, std::integral_constant<int, NBUF - 1>{}, std::integral_constant<int, 2>{});
+    });
+    const int my_steps = last_sub + 2;   // steps 0 .. last_sub + 1
+    for (int u0 = 0; u0 < my_steps; u0 += NBUF) {
+      static_for<0, NBUF>([&](auto slot_c) __attribute__((always_inline)) {
+        constexpr int SLOT = decltype(slot_c)::value;
+        const int u = u0 + SLOT;
+        if (u < my_steps) {
+          if (u > 0) {
+            __builtin_amdgcn_s_waitcnt(0x0F70 | 6);   // vmcnt(6)
+            __syncthreads();
+          }
+          step(slot_c, u);
+        }
+      });
+    }
+    // nothing left for this wave: keep feeding the rings and meeting the barriers of the others
+    {
+      uint32_t kslot = (uint32_t)((my_steps + DK_AHEAD) % NBUF), vslot = (uint32_t)((my_steps + DV_AHEAD) % NBUF);
+      for (int u = my_steps; u <= n_sub; u++) {
+        wait_dma();
+        __syncthreads();
+        issue_k_rt(u + DK_AHEAD, kslot);
+        issue_v_rt(u + DV_AHEAD, vslot);
+        kslot = kslot + 1 == NBUF ? 0 : kslot + 1;
+        vslot = vslot + 1 == NBUF ? 0 : vslot + 1;
+      }
+    }
+    wait_dma();
+    __syncthreads();   // every wave is done with the K/V buffers: they become output staging
+
+    // ---- epilogue: normalise, stage O through LDS (wave-private), coalesced 16-byte stores
+    float inv = 1.f, lse = 0.f;
+    if constexpr (FAMILY == FAM_SOFTMAX) {
+      float s_lo, s_hi;
+      xhalf_pair(row_sum, s_lo, s_hi);
+      const float tot = s_lo + s_hi;
+      inv = 1.f / tot;
+      lse = (row_ref + fast_log2(tot)) * kLn2;
+    }
+    constexpr int OROW = DV * 2 + 16;  // padded staging row
+    const uint32_t ob = lds0 + wave * 32 * OROW;
+  #pragma unroll
+    for (int db = 0; db < DB; db++)
+  #pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        x4 w;
+  #pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (T)(o[db][4 * q4 + i] * inv);
+        lds_write<x4>(ob + r * OROW + (32 * db + 8 * q4 + 4 * g) * 2, w);
+      }
+    T* obase = (T*)a.o + (int64_t)b * a.osb + (int64_t)h * a.osh;
+  #pragma unroll
+    for (int it = 0; it < 32 * CPRV / 64; it++) {
+      const int ci = lane + 64 * it, row = ci / CPRV, c = ci % CPRV;
+      u32x4 w = lds_read<u32x4>(ob + row * OROW + c * 16);
+      if (m_wave + row < a.Sq) *(u32x4*)(obase + (int64_t)(m_wave + row) * a.oss + c * 8) = w;
+    }
+    if constexpr (FAMILY == FAM_SOFTMAX) {
+      if (a.row_scale && g == 0 && m_lane < a.Sq) a.row_scale[((int64_t)b * a.H + h) * a.Sq + m_lane] = lse;
+    }
+    __syncthreads();   // the staging area is ring space again
   }
 }
 
 template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
 static int launch(const AttnArgs& a, hipStream_t stream) {
-  constexpr int BM = 128, BN = 64;
-  constexpr size_t tiles = 2 * (size_t)BN * (DQK + DV) * 2;
-  constexpr size_t ostage = 4 * 32 * (size_t)(DV * 2 + 16);
+  constexpr int BM = 256, BN = 32, NBUF = ATTN_NBUF;
+  constexpr size_t tiles = NBUF * (size_t)BN * (DQK + DV) * 2;
+  constexpr size_t ostage = 8 * 32 * (size_t)(DV * 2 + 16);
   constexpr size_t lds = tiles > ostage ? tiles : ostage;
   auto kern = attn_fwd_kernel<T, DQK, DV, FAMILY, CAUSAL>;
   static bool attr_set = false;
@@ -348,10 +439,20 @@ static int launch(const AttnArgs& a, hipStream_t stream) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
     attr_set = true;
   }
+  // the kernel addresses K and V rows with 32-bit byte offsets from the (batch, head) plane
+  if ((uint64_t)a.Skv * (uint64_t)a.kss * 2 >= (1ull << 32) || (uint64_t)a.Skv * (uint64_t)a.vss * 2 >= (1ull << 32)) return -2;
   AttnArgs args = a;
   args.num_m_blocks = (a.Sq + BM - 1) / BM;
-  const unsigned grid = (unsigned)(args.num_m_blocks * a.B * a.H);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, args);
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -1;
+    num_cus = prop.multiProcessorCount;
+  }
+  const int n_items = args.num_m_blocks * a.B * a.H;
+  const unsigned grid = (unsigned)(n_items < num_cus ? n_items : num_cus);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, args);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

@@ -72,6 +72,16 @@ __device__ __forceinline__ float xhalf(float x) {
   return __shfl_xor(x, 32, 64);
 }
 
+// The two halves of the wave exchange x: for every lane, {lo, hi} = {x of the lane's own half, x of lane^32}
+// in an order that is the same for both lanes of a pair -- enough for symmetric combinations (max, sum),
+// and one v_permlane32_swap instead of a trip through the LDS crossbar.
+__device__ __forceinline__ void xhalf_pair(float x, float& lo, float& hi) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, x);
+  const auto rr = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  lo = __builtin_bit_cast(float, (uint32_t)rr[0]);
+  hi = __builtin_bit_cast(float, (uint32_t)rr[1]);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
