@@ -285,21 +285,27 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   //      its CUs work on the q blocks of the same few pairs at the same time (their K/V stays in that
   //      XCD's L2).  Under a causal mask a q block's work grows with its position, so the unit of work
   //      is a pair of q blocks (k, nmb-1-k) of one (batch, head): every unit weighs the same.
+  //      The first loads of an item (its Q rows, K(0..5), V(0..3)) are issued before the output of the
+  //      previous item is written, so their latency hides behind that epilogue.
   const int nmb = a.num_m_blocks, BH = a.B * a.H, G = (int)gridDim.x;
   const bool paired = CAUSAL && BH * nmb > G;               // (few items: one q block per unit, spread wide)
   const int upb = paired ? (nmb + 1) >> 1 : nmb;            // units per (batch, head)
   const bool by_xcd = (BH & 7) == 0 && (G & 7) == 0;
   const int units = by_xcd ? (BH >> 3) * upb : BH * upb;   // units of this workgroup's stream
   const int first = by_xcd ? (int)blockIdx.x >> 3 : (int)blockIdx.x, stride = by_xcd ? G >> 3 : G;
-  for (int t = 2 * first; t < 2 * units; t = (t & 1) ? t + 2 * stride - 1 : t + 1) {
-    const int q = t >> 1, k = q % upb;
-    if (paired) {
-      mb = (t & 1) ? k : nmb - 1 - k;
-      if ((t & 1) && k == nmb - 1 - k) continue;   // the middle block of an odd count is its own partner
-    } else {
-      mb = CAUSAL ? nmb - 1 - k : k;
-      if (t & 1) continue;
+  // item cursor t = 2 * unit + half; returns the next cursor that names an item (or one past the end)
+  auto next_item = [&](int t) -> int {
+    for (;;) {
+      t = (t & 1) ? t + 2 * stride - 1 : t + 1;
+      if (t >= 2 * units) return t;
+      const int k = (t >> 1) % upb;
+      if (paired ? !((t & 1) && k == nmb - 1 - k) : !(t & 1)) return t;   // (the middle block of an odd count is its own partner)
     }
+  };
+  // decode item t into the per-item variables and start its first loads
+  auto open_item = [&](int t) __attribute__((always_inline)) {
+    const int q = t >> 1, k = q % upb;
+    mb = paired ? ((t & 1) ? k : nmb - 1 - k) : (CAUSAL ? nmb - 1 - k : k);
     int bh = q / upb;
     if (by_xcd) bh = bh * 8 + ((int)blockIdx.x & 7);
     b = bh / a.H;
@@ -311,14 +317,24 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
     last_sub = CAUSAL ? min(n_sub - 1, m_wave / BN) : n_sub - 1;
     kbase = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)h * a.ksh);
     vbase = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)h * a.vsh);
-    {
-      const int qrow = min(m_lane, a.Sq - 1);
-      const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)qrow * a.qss + (int64_t)h * a.qsh + 8 * g;
+    // K(0..5) -> slots 0..5, V(0..3) -> slots 0..3; the first step multiplies ring slot NBUF-1 with zero
+    // probabilities: it gets V(0) as well, so that whatever is there belongs to this (batch, head)
+    static_for<0, NBUF>([&](auto t_c) __attribute__((always_inline)) {
+      constexpr int tt = decltype(t_c)::value;
+      issue_k_rt(tt, tt);
+      if constexpr (tt < DV_AHEAD) issue_v_rt(tt, tt);
+    });
+    issue_v_rt(0, NBUF - 1);
+    const int qrow = min(m_lane, a.Sq - 1);
+    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)qrow * a.qss + (int64_t)h * a.qsh + 8 * g;
 #pragma unroll
-      for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 16 * ks);
-    }
-    // V ring slot NBUF-1 is read (times zero probabilities) before anything was loaded into it
-    for (int i = tid; i < VTILE / 16; i += 64 * NW) lds_write<u32x4>(lds_v + (NBUF - 1) * VTILE + i * 16, u32x4{0u, 0u, 0u, 0u});
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 16 * ks);
+  };
+
+  int stores_behind = 0;   // output stores this wave issued after the current item's first loads
+  int t_cur = 2 * first;
+  if (t_cur < 2 * units) open_item(t_cur);
+  while (t_cur < 2 * units) {
 #pragma unroll
     for (int i = 0; i < DB; i++)
 #pragma unroll
@@ -334,12 +350,11 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
     //      that step u refills with K(u+7) and V(u+4).  A wave's loads complete in order and every step
     //      issues K then V; K(u+3) and V(u) are the pair of step u-4, so at the top of step u the six
     //      instructions of steps u-3 .. u-1 may still be in flight.
-    static_for<0, NBUF>([&](auto t_c) __attribute__((always_inline)) {   // K(0..5) and V(0..3), plus K(6) below
-      constexpr int t = decltype(t_c)::value;
-      issue_k_rt(t, t);
-      if constexpr (t < DV_AHEAD) issue_v_rt(t, t);
-    });
-    wait_dma();
+    // the item's first loads (see open_item) must have landed; the previous item's output stores, issued
+    // after them, need not
+    if (stores_behind == 32 * CPRV / 64 + 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (32 * CPRV / 64 + 1));
+    else if (stores_behind == 32 * CPRV / 64) __builtin_amdgcn_s_waitcnt(0x0F70 | (32 * CPRV / 64));
+    else wait_dma();
     __syncthreads();
     {   // s[0] = K(0) Q^T with its maximum folded in, s[1] = K(1) Q^T; then K(6) may replace K(0)
       x8 k0[KS];
@@ -391,9 +406,19 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
       }
     }
     wait_dma();
-    __syncthreads();   // every wave is done with the K/V buffers: they become output staging
+    __syncthreads();   // every wave is done with the K/V rings
 
-    // ---- epilogue: normalise, stage O through LDS (wave-private), coalesced 16-byte stores
+    // ---- what the epilogue needs of this item, then the next item's first loads, then the epilogue
+    T* const obase = (T*)a.o + (int64_t)b * a.osb + (int64_t)h * a.osh + (int64_t)m_wave * a.oss;
+    const int m_out = m_wave;
+    float* const lse_ptr = a.row_scale ? a.row_scale + ((int64_t)b * a.H + h) * a.Sq + m_lane : nullptr;
+    const bool row_ok = m_lane < a.Sq;
+    t_cur = next_item(t_cur);
+    if (t_cur < 2 * units) open_item(t_cur);
+
+    // normalise, stage O through LDS (wave-private rows, 16-byte chunks XOR-swizzled by row so that neither
+    // the 8-byte writes nor the 16-byte reads pile onto one bank group), coalesced 16-byte stores.  The
+    // staging area lies behind the rings, which already receive the next item.
     float inv = 1.f, lse = 0.f;
     if constexpr (FAMILY == FAM_SOFTMAX) {
       float s_lo, s_hi;
@@ -402,28 +427,51 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
       inv = 1.f / tot;
       lse = (row_ref + fast_log2(tot)) * kLn2;
     }
-    constexpr int OROW = DV * 2 + 16;  // padded staging row
-    const uint32_t ob = lds0 + wave * 32 * OROW;
-  #pragma unroll
+    // (the lane id is laundered so that the address arithmetic below is redone per item instead of being
+    // hoisted out of the item loop, where it would occupy registers the main loop has no room for)
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int r_e = lane_e & 31, g_e = lane_e >> 5;
+    const uint32_t ob = lds0 + NBUF * (KTILE + VTILE) + wave * 32 * VROW;
+    const uint32_t ow = ob + r_e * VROW + 8 * g_e;
+#pragma unroll
     for (int db = 0; db < DB; db++)
-  #pragma unroll
+#pragma unroll
       for (int q4 = 0; q4 < 4; q4++) {
         x4 w;
-  #pragma unroll
+#pragma unroll
         for (int i = 0; i < 4; i++) w[i] = (T)(o[db][4 * q4 + i] * inv);
-        lds_write<x4>(ob + r * OROW + (32 * db + 8 * q4 + 4 * g) * 2, w);
+        lds_write<x4>(ow + (((4 * db + q4) ^ (r_e & 15)) << 4), w);
       }
-    T* obase = (T*)a.o + (int64_t)b * a.osb + (int64_t)h * a.osh;
-  #pragma unroll
-    for (int it = 0; it < 32 * CPRV / 64; it++) {
-      const int ci = lane + 64 * it, row = ci / CPRV, c = ci % CPRV;
-      u32x4 w = lds_read<u32x4>(ob + row * OROW + c * 16);
-      if (m_wave + row < a.Sq) *(u32x4*)(obase + (int64_t)(m_wave + row) * a.oss + c * 8) = w;
+    // Stores count in the same in-order counter as the loads that were just started for the next item.
+    // A wave whose 32 rows all exist issues a known number of them, and the next item only waits for what
+    // is older than these stores; otherwise it waits for everything.
+    constexpr int NST = 32 * CPRV / 64;
+    if (m_out + 32 <= a.Sq) {
+#pragma unroll
+      for (int it = 0; it < NST; it++) {
+        const int ci = lane_e + 64 * it, row = ci / CPRV, c = ci % CPRV;
+        u32x4 w = lds_read<u32x4>(ob + row * VROW + ((c ^ (row & 15)) << 4));
+        *(u32x4*)(obase + (int64_t)row * a.oss + c * 8) = w;
+      }
+      if (FAMILY == FAM_SOFTMAX && lse_ptr) {
+        if (g_e == 0) *lse_ptr = lse;
+        stores_behind = NST + 1;
+      } else {
+        stores_behind = NST;
+      }
+    } else {
+#pragma unroll
+      for (int it = 0; it < NST; it++) {
+        const int ci = lane_e + 64 * it, row = ci / CPRV, c = ci % CPRV;
+        u32x4 w = lds_read<u32x4>(ob + row * VROW + ((c ^ (row & 15)) << 4));
+        if (m_out + row < a.Sq) *(u32x4*)(obase + (int64_t)row * a.oss + c * 8) = w;
+      }
+      if constexpr (FAMILY == FAM_SOFTMAX) {
+        if (lse_ptr && g_e == 0 && row_ok) *lse_ptr = lse;
+      }
+      stores_behind = 0;
     }
-    if constexpr (FAMILY == FAM_SOFTMAX) {
-      if (a.row_scale && g == 0 && m_lane < a.Sq) a.row_scale[((int64_t)b * a.H + h) * a.Sq + m_lane] = lse;
-    }
-    __syncthreads();   // the staging area is ring space again
   }
 }
 
@@ -431,8 +479,7 @@ template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
 static int launch(const AttnArgs& a, hipStream_t stream) {
   constexpr int BM = 256, BN = 32, NBUF = ATTN_NBUF;
   constexpr size_t tiles = NBUF * (size_t)BN * (DQK + DV) * 2;
-  constexpr size_t ostage = 8 * 32 * (size_t)(DV * 2 + 16);
-  constexpr size_t lds = tiles > ostage ? tiles : ostage;
+  constexpr size_t lds = tiles + 8 * 32 * (size_t)DV * 2;   // rings + output staging
   auto kern = attn_fwd_kernel<T, DQK, DV, FAMILY, CAUSAL>;
   static bool attr_set = false;
   if (!attr_set) {
