@@ -161,26 +161,27 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
     }
   };
 
-  // elements e0, e0+1 of the sub-tile in s[SB]: score -> probability, row sum, packed into p[PAR]
-  auto prob_pair = [&](auto sb_c, auto par_c, auto e_c, float sub, float& part) __attribute__((always_inline)) {
+  // one element of the sub-tile in s[SB]: score -> probability (and its contribution to the row sum)
+  auto prob_one = [&](auto sb_c, auto e_c, float sub, float& part) __attribute__((always_inline)) -> float {
 #pragma clang fp reassociate(off)   // keep the running sum a chain in element order
-    constexpr int SB = decltype(sb_c)::value, PAR = decltype(par_c)::value, e0 = decltype(e_c)::value;
-    float pe[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-      const float v = s[SB][e0 + i];
-      if constexpr (FAMILY == FAM_SOFTMAX) {
-        pe[i] = fast_exp2(v * c_scale + sub);
-        part += pe[i];
-      } else if constexpr (FAMILY == FAM_SIGMOID) {   // sigmoid(x) = 1 / (1 + 2^(-x log2e)); s = -inf gives exactly 0
-        pe[i] = fast_rcp(1.f + fast_exp2(-(v * c_scale + c_bias)));
-      } else {
-        pe[i] = fmaxf(v * a.scale + bias, 0.f);
-      }
+    constexpr int SB = decltype(sb_c)::value, e = decltype(e_c)::value;
+    const float v = s[SB][e];
+    if constexpr (FAMILY == FAM_SOFTMAX) {
+      const float pe = fast_exp2(v * c_scale + sub);
+      part += pe;
+      return pe;
+    } else if constexpr (FAMILY == FAM_SIGMOID) {   // sigmoid(x) = 1 / (1 + 2^(-x log2e)); s = -inf gives exactly 0
+      return fast_rcp(1.f + fast_exp2(-(v * c_scale + c_bias)));
+    } else {
+      return fmaxf(v * a.scale + bias, 0.f);
     }
+  };
+  // elements e0, e0+1 packed into p[PAR]
+  auto pack_pair = [&](auto par_c, auto e_c, float pe0, float pe1) __attribute__((always_inline)) {
+    constexpr int PAR = decltype(par_c)::value, e0 = decltype(e_c)::value;
     x2 pk;
-    pk[0] = (T)pe[0];
-    pk[1] = (T)pe[1];
+    pk[0] = (T)pe0;
+    pk[1] = (T)pe1;
     p[PAR][e0 >> 3][(e0 & 7) >> 1] = __builtin_bit_cast(uint32_t, pk);
   };
 
@@ -265,10 +266,12 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
       __builtin_amdgcn_sched_barrier(0);
       x8 vf = __builtin_shufflevector(lo[i % PF], hi[i % PF], 0, 1, 2, 3, 4, 5, 6, 7);
       o[i % DB] = E::mfma32(vf, __builtin_bit_cast(x8, p[1 - PAR][i / DB]), o[i % DB]);
+      const float pe0 = prob_one(sb_exp_c, std::integral_constant<int, 2 * i>{}, sub, part);   // behind the PV MFMA
+      if constexpr (FAMILY == FAM_SOFTMAX) mx = fmaxf(fmaxf(mx, s[SB_MAX][2 * i]), s[SB_MAX][2 * i + 1]);
       __builtin_amdgcn_sched_barrier(0);
       s[SB_QK] = E::mfma32(kf[i % PF], qf[i], i == 0 ? zero16 : s[SB_QK]);
-      prob_pair(sb_exp_c, par_c, std::integral_constant<int, 2 * i>{}, sub, part);
-      if constexpr (FAMILY == FAM_SOFTMAX) mx = fmaxf(fmaxf(mx, s[SB_MAX][2 * i]), s[SB_MAX][2 * i + 1]);
+      const float pe1 = prob_one(sb_exp_c, std::integral_constant<int, 2 * i + 1>{}, sub, part);   // behind the QK MFMA
+      pack_pair(par_c, std::integral_constant<int, 2 * i>{}, pe0, pe1);
       __builtin_amdgcn_sched_barrier(0);
     });
     if constexpr (FAMILY == FAM_SOFTMAX) {
