@@ -97,7 +97,8 @@ typedef struct ma_linear_params {
  *   o = softmax((q.kv^T + q_pe.k_pe^T) * scale) . kv
  * q [B,Hq,D], q_pe [B,Hq,Dpe], kv [B,Skv,D], k_pe [B,Skv,Dpe], o [B,Hq,D]
  * (one latent kv head, one query token; the [B,1,Hq,.] / [B,Skv,1,.] tensors
- * of the reference are these with a unit dimension).  Partials are fp32. */
+ * of the reference are these with a unit dimension).  Partial outputs are kept in the tensors' dtype, as Output_partial
+ * of the reference is (mla_decode_tl.py:160); their log-sum-exp is fp32. */
 typedef struct ma_mla_params {
   int32_t dtype;
   int32_t batch, heads_q, seqlen_kv, dim, dim_pe;

@@ -100,7 +100,7 @@ int ma_linear_fwd(const ma_linear_params* p, ma_stream_t stream) {
 // number of 64-row tiles, and never more splits than tiles.
 int ma_mla_choose_split(const ma_mla_params* p) {
   if (!p || p->batch <= 0 || p->heads_q <= 0 || p->seqlen_kv <= 0) return 1;
-  const int head_blocks = (p->heads_q + 63) / 64;
+  const int head_blocks = (p->heads_q + 127) / 128;
   const int tiles = (p->seqlen_kv + 63) / 64;
   int split = 256 / (p->batch * head_blocks);
   if (split < 1) split = 1;
@@ -115,7 +115,7 @@ size_t ma_mla_workspace_bytes(const ma_mla_params* p) {
   if (!p) return 0;
   const int ns = mla_split_of(p);
   if (ns <= 1) return 0;
-  return (size_t)p->batch * ns * p->heads_q * ((size_t)p->dim + 1) * sizeof(float);
+  return (size_t)p->batch * ns * p->heads_q * ((size_t)p->dim * 2 + sizeof(float));   // 2-byte partial outputs + fp32 lse
 }
 
 int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
@@ -149,8 +149,8 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
     if (!p->workspace || p->workspace_bytes < need)
       return fail(MA_ERR_WORKSPACE, "ma_mla_decode: workspace of %zu bytes needed for %d splits, got %zu", need, ns, p->workspace_bytes);
     if ((uintptr_t)p->workspace % 16 != 0) return fail(MA_ERR_WORKSPACE, "ma_mla_decode: workspace must be 16-byte aligned");
-    a.o_part = (float*)p->workspace;
-    a.lse_part = a.o_part + (size_t)p->batch * ns * p->heads_q * p->dim;
+    a.o_part = p->workspace;
+    a.lse_part = (float*)((char*)p->workspace + (size_t)p->batch * ns * p->heads_q * p->dim * 2);
   }
   const int rc = ma::mla_decode_dispatch(a, p->dtype == MA_BF16, p->dim, p->dim_pe, (hipStream_t)stream);
   if (rc == -2) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: only dim=512, dim_pe=64 is in the kernel library (got %d, %d)", p->dim, p->dim_pe);

@@ -4,30 +4,32 @@
 // attention_engine/core/template/tl_template/attn/mla_decode_tl.py:154-290:
 //   o[b,h,:] = softmax((q[b,h].kv[b,n] + q_pe[b,h].k_pe[b,n]) * scale) . kv[b,n]
 //
-// Split kernel.  A workgroup (4 waves) owns one (batch, kv split, block of 64
-// query heads); wave w owns heads 16w..16w+15 and all four waves consume the
-// same 64-row latent tile from LDS.  The two head blocks of one (batch, split)
-// are given workgroup ids that land on the same XCD, so the second read of a
-// tile is served by that XCD's L2 and the cache leaves HBM once.  Tiles arrive
-// by direct-to-LDS DMA (global_load_lds_dwordx4: no staging registers; the
-// registers hold the 576-wide Q fragments and the 512 x 16 fp32 output
-// accumulator), double buffered.  v_mfma_f32_16x16x32 is used throughout:
+// Split kernel.  A workgroup (8 waves, two per SIMD, the whole CU) owns one (batch, kv split, block of
+// 128 query heads); wave w owns heads 16w..16w+15 and all eight waves consume the same 32-row latent
+// sub-tiles from LDS, so the cache leaves HBM exactly once.  Sub-tiles arrive by direct-to-LDS DMA
+// (global_load_lds_dwordx4: no staging registers; the registers hold the 576-wide Q fragments and the
+// 512 x 16 fp32 output accumulator of the wave) through a ring of 4 stages, three sub-tiles ahead of their
+// use, and a wave waits for its own share with a partial vmcnt before the one barrier per sub-tile.
+// v_mfma_f32_16x16x32 is used throughout:
 //   A[16 x 32]: lane holds row l%16, k = 8(l/16) .. +7
 //   B[32 x 16]: lane holds column l%16, k = 8(l/16) .. +7
 //   C[16 x 16]: lane holds column l%16, element j is row 4(l/16) + j
 // Scores are computed transposed (S^T = KV Q^T) so each lane owns one head's
 // row statistics and the probabilities feed O^T += KV^T P^T straight from the
 // accumulator registers; KV^T comes out of the same row-major LDS tile through
-// the transposing read, so V is never loaded separately.
+// the transposing read, so V is never loaded separately.  Within a wave the phases of a sub-tile run one
+// after the other (scores, softmax, P V); the second wave on the SIMD fills the gaps.
 // Combine kernel: log-sum-exp merge of the fp32 partials.
 #include "mla_decode.h"
 
 namespace ma {
 
 namespace {
-constexpr int BN = 64;         // kv rows per tile
-constexpr int HB = 64;         // heads per workgroup
+constexpr int BN = 32;         // kv rows per sub-tile
+constexpr int HB = 128;        // heads per workgroup
+constexpr int NW = 8;          // waves per workgroup
 constexpr int D = 512, DPE = 64;
+constexpr int NSTAGE = 4;
 constexpr int KV_ROW = D * 2 + 32;  // bytes; each latent row is its own DMA, so rows can be padded: with a
                                    // 32 B pad consecutive rows start 8 banks apart (the transposing reads of
                                    // 8 rows x 32 B tile the 64 banks exactly) and rows 8..15 of a 16-row group
@@ -35,8 +37,8 @@ constexpr int KV_ROW = D * 2 + 32;  // bytes; each latent row is its own DMA, so
                                    // reads of 16 rows x one chunk hit 16 different bank groups.  Every LDS
                                    // read address is then lane base + compile-time offset.
 constexpr int PE_ROW = DPE * 2;    // rope rows share a DMA (8 rows per KB): XOR-swizzled instead
-constexpr int KV_TILE = BN * KV_ROW;   // 65 KB
-constexpr int PE_TILE = BN * PE_ROW;   // 8 KB
+constexpr int KV_TILE = BN * KV_ROW;   // 33 KB
+constexpr int PE_TILE = BN * PE_ROW;   // 4 KB
 constexpr int STAGE = KV_TILE + PE_TILE;
 
 __device__ __forceinline__ int kv_flip(int row) { return (row >> 3) & 1; }
@@ -46,7 +48,7 @@ __device__ __forceinline__ float xlane(float x, int mask) { return __shfl_xor(x,
 }  // namespace
 
 template <typename T>
-__global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
+__global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) {
   using E = Elem<T>;
   using x8 = typename E::x8;
   using x4 = typename E::x4;
@@ -57,17 +59,7 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, q = lane >> 4;
-  // workgroup id -> (batch, split, head block); head blocks of one (batch, split) share id % 8 (one XCD)
-  const int n_bs = a.B * a.num_split;
-  int bs, hblk;
-  if ((n_bs & 7) == 0) {
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    hblk = slot % a.head_blocks;
-    bs = (slot / a.head_blocks) * 8 + xcd;
-  } else {
-    hblk = blockIdx.x % a.head_blocks;
-    bs = blockIdx.x / a.head_blocks;
-  }
+  const int hblk = blockIdx.x % a.head_blocks, bs = blockIdx.x / a.head_blocks;
   const int b = bs / a.num_split, split = bs % a.num_split;
   const int head = hblk * HB + wave * 16 + r;
   const int head_ld = min(head, a.Hq - 1);
@@ -91,30 +83,34 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
   const char* peb = (const char*)a.k_pe + (int64_t)b * a.kpsb * 2;
   const int64_t kv_row_bytes = a.kvss * 2, pe_row_bytes = a.kpss * 2;
 
-  // wave w streams tile rows 16w..16w+15: one DMA per latent row (64 lanes x 16 B = 1 KB),
-  // one DMA per 8 rope rows.  Lane i fetches the chunk that belongs at physical chunk i.
-  auto issue_tile = [&](int n0, int buf) {
-    const uint32_t base = lds0 + buf * STAGE;
+  // ---- DMA.  Wave w streams latent rows 4w..4w+3 of a sub-tile, one instruction per row (64 lanes x 16 B =
+  //      the 1 KB row; lane i fetches the chunk that belongs at physical chunk i); waves 0..3 also fetch 8
+  //      rope rows each with one more instruction.  Rows beyond the cache are clamped to its last row
+  //      (their scores are masked).  NDMA is the wave's instruction count per sub-tile.
+  const int NDMA = wave < 4 ? 5 : 4;
+  const uint32_t lane_off = (uint32_t)(lane ^ ((wave >> 1) & 1)) << 4;   // kv_flip(4w + i) = (w >> 1) & 1
+  auto issue_tile = [&](int jt) {
+    const uint32_t sb = lds0 + (jt & (NSTAGE - 1)) * STAGE;
+    const int n0 = n_begin + jt * BN;
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      const int row = wave * 16 + i;
+    for (int i = 0; i < 4; i++) {
+      const int row = wave * 4 + i;
       const int nrow = min(n0 + row, a.Skv - 1);
-      dma16(kvb + nrow * kv_row_bytes + ((lane ^ kv_flip(row)) << 4), base + row * KV_ROW);
+      dma16_so(kvb + nrow * kv_row_bytes, lane_off, sb + row * KV_ROW);
     }
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-      const int row = wave * 16 + i * 8 + (lane >> 3);
+    if (wave < 4) {
+      const int row = wave * 8 + (lane >> 3);
       const int nrow = min(n0 + row, a.Skv - 1);
-      dma16(peb + nrow * pe_row_bytes + (((lane & 7) ^ swz_pe(row)) << 4), base + KV_TILE + (wave * 16 + i * 8) * PE_ROW);
+      dma16(peb + nrow * pe_row_bytes + (((lane & 7) ^ swz_pe(row)) << 4), sb + KV_TILE + wave * 8 * PE_ROW);
     }
   };
 
-  // ---- per-lane LDS read addresses
+  // ---- per-lane LDS read offsets within a stage
   // K side (A operand): row 16nb + r, logical 16-byte chunk 4ks + q
   const uint32_t k_row_off = r * KV_ROW + (q ^ kv_flip(r)) * 16;
   const uint32_t pe_row_off = KV_TILE + r * PE_ROW;
   const int pe_chunk0 = q ^ swz_pe(r);
-  // V side (transposing read): lane block q reads rows nbase + 4q + jr, columns 16db + 4(l%4)..+3
+  // V side (transposing read): lane block q reads rows 4q + jr (and + 16), columns 16db + 4(l%4)..+3
   const int jr = r >> 2;
   const uint32_t v_row_off = (4 * q + jr) * KV_ROW + ((((lane & 3) >> 1) ^ kv_flip(4 * q + jr)) << 4) + (lane & 1) * 8;
 
@@ -124,24 +120,36 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
   const float c_scale = a.scale * kLog2e;
   float row_max = -1e30f, row_sum = 0.f;
 
-  if (n_tiles > 0) issue_tile(n_begin, 0);
-  wait_dma();
-  __syncthreads();
+  if (n_tiles > 0) issue_tile(0);
+  if (n_tiles > 1) issue_tile(1);
+  if (n_tiles > 2) issue_tile(2);
 
   for (int jt = 0; jt < n_tiles; jt++) {
-    const int buf = jt & 1, n0 = n_begin + jt * BN;
-    if (jt + 1 < n_tiles) issue_tile(n0 + BN, buf ^ 1);
-    const uint32_t base = lds0 + buf * STAGE;
+    // Sub-tile jt has landed for every wave (a wave's loads complete in order: only those of the up to two
+    // later sub-tiles may still be in flight) and every wave is done with sub-tile jt-1, whose stage
+    // takes sub-tile jt+3.
+    if (jt + 2 < n_tiles) {
+      if (wave < 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 10); else __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+    } else if (jt + 1 < n_tiles) {
+      if (wave < 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 5); else __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+    } else {
+      wait_dma();
+    }
+    __syncthreads();
+    if (jt + 3 < n_tiles) issue_tile(jt + 3);
+    const int n0 = n_begin + jt * BN;
+    uint32_t base = lds0 + (jt & (NSTAGE - 1)) * STAGE;
 
     // ---- S^T = KV Q^T + K_pe Q_pe^T : lane holds head r, kv rows 16nb + 4q + j
     f32x4 s[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) s[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
     {
-      // fragments are requested two slices ahead of the MFMAs that consume them
+      // fragments are requested AH slices ahead of the MFMAs that consume them
       constexpr int AH = 2, RING = AH + 1, NSL = KS + KSPE;
       x8 kf[RING][NB];
-      const uint32_t kb = base + k_row_off;
+      uint32_t kb = base + k_row_off, pb = base + pe_row_off;
+      asm volatile("" : "+v"(kb), "+v"(pb));   // one address register + immediates for every read below
       auto request = [&](int ks) {
         if (ks < KS) {
 #pragma unroll
@@ -149,7 +157,7 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
         } else {
           const uint32_t coff = (uint32_t)((pe_chunk0 ^ (4 * (ks - KS))) << 4);
 #pragma unroll
-          for (int nb = 0; nb < NB; nb++) kf[ks % RING][nb] = lds_read<x8>(base + pe_row_off + nb * 16 * PE_ROW + coff);
+          for (int nb = 0; nb < NB; nb++) kf[ks % RING][nb] = lds_read<x8>(pb + nb * 16 * PE_ROW + coff);
         }
       };
 #pragma unroll
@@ -190,7 +198,9 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
       row_max = move ? cand : row_max;
       row_sum *= corr;
 #pragma unroll
-      for (int i = 0; i < DB; i++) o[i] *= corr;
+      for (int i = 0; i < DB; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(o[i][j]) : "v"(corr));
     }
     float part = 0.f;
 #pragma unroll
@@ -203,18 +213,17 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
       }
     row_sum += part;
 
-    // ---- O^T += KV^T P^T ; MFMA slice t covers kv rows 32t..32t+31, lane block q, slot i is
-    //      row 32t + 16(i/4) + 4q + i%4 on both operands
-#pragma unroll
-    for (int t = 0; t < BN / 32; t++) {
+    // ---- O^T += KV^T P^T ; lane block q, k slot i is kv row 16(i/4) + 4q + i%4 on both operands
+    {
       x8 pf;
 #pragma unroll
       for (int i = 0; i < 4; i++) {
-        pf[i] = (T)s[2 * t][i];
-        pf[4 + i] = (T)s[2 * t + 1][i];
+        pf[i] = (T)s[0][i];
+        pf[4 + i] = (T)s[1][i];
       }
-      const uint32_t rb = base + v_row_off + 32 * t * KV_ROW;
-      constexpr int PF = 8;   // V fragments in flight
+      uint32_t rb = base + v_row_off;
+      asm volatile("" : "+v"(rb));
+      constexpr int PF = 4;   // V fragments in flight
       x4 lo[PF], hi[PF];
 #pragma unroll
       for (int i = 0; i < PF - 1; i++) {
@@ -233,9 +242,6 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-
-    wait_dma();
-    __syncthreads();
   }
 
   // ---- epilogue: lane holds head r, output columns 16db + 4q + j
@@ -256,41 +262,69 @@ __global__ __launch_bounds__(256, 1) void mla_split_kernel(const MlaArgs a) {
       }
       if (a.lse && q == 0) a.lse[(int64_t)b * a.Hq + head] = lse2 * kLn2;
     } else {
-      float* op = a.o_part + (((int64_t)b * a.num_split + split) * a.Hq + head) * D + 4 * q;
+      T* op = (T*)a.o_part + (((int64_t)b * a.num_split + split) * a.Hq + head) * D + 4 * q;
 #pragma unroll
-      for (int db = 0; db < DB; db++) *(f32x4*)(op + 16 * db) = o[db] * inv;
+      for (int db = 0; db < DB; db++) {
+        x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (T)(o[db][i] * inv);
+        *(x4*)(op + 16 * db) = w;
+      }
       if (q == 0) a.lse_part[((int64_t)b * a.num_split + split) * a.Hq + head] = lse2;
     }
   }
 }
 
-// One workgroup per (batch, head): 128 threads x 4 output columns.
+// Four (batch, head) pairs per workgroup: 64 threads x 8 output columns each.
 template <typename T>
-__global__ __launch_bounds__(128) void mla_combine_kernel(const MlaArgs a) {
-  const int head = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+__global__ __launch_bounds__(256) void mla_combine_kernel(const MlaArgs a) {
+  using x8 = typename Elem<T>::x8;
+  const int tid = threadIdx.x & 63;
+  const int64_t bh = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (bh >= (int64_t)a.B * a.Hq) return;
+  const int b = (int)(bh / a.Hq), head = (int)(bh % a.Hq);
   const int ns = a.num_split;
+  // lane s of the wave holds the log-sum-exp of split s (at most 64 splits): one load, wave reductions
   const float* lp = a.lse_part + (int64_t)b * ns * a.Hq + head;
-  float mx = -INFINITY;
-  for (int s = 0; s < ns; s++) mx = fmaxf(mx, lp[(int64_t)s * a.Hq]);
-  float sum = 0.f;
-  for (int s = 0; s < ns; s++) sum += fast_exp2(lp[(int64_t)s * a.Hq] - mx);
-  const float inv = 1.f / sum;
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < ns; s++) {
-    const float w = fast_exp2(lp[(int64_t)s * a.Hq] - mx) * inv;
-    const f32x4 v = *(const f32x4*)(a.o_part + (((int64_t)b * ns + s) * a.Hq + head) * D + tid * 4);
-    acc += v * w;
-  }
-  typename Elem<T>::x4 w;
+  const float my = tid < ns ? lp[(int64_t)tid * a.Hq] : -INFINITY;
+  float mx = my;
 #pragma unroll
-  for (int i = 0; i < 4; i++) w[i] = (T)acc[i];
-  *(typename Elem<T>::x4*)((T*)a.o + (int64_t)b * a.osb + (int64_t)head * a.osh + tid * 4) = w;
+  for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+  const float e = tid < ns ? fast_exp2(my - mx) : 0.f;
+  float sum = e;
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, 64);
+  const float wgt = e / sum;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const T* pp = (const T*)a.o_part + ((int64_t)b * ns * a.Hq + head) * D + tid * 8;
+  int s0 = 0;
+  for (; s0 + 4 <= ns; s0 += 4) {   // four independent loads in flight
+    x8 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) v[k] = *(const x8*)(pp + (int64_t)(s0 + k) * a.Hq * D);
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const float w = __shfl(wgt, s0 + k, 64);
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc[i] += (float)v[k][i] * w;
+    }
+  }
+  for (; s0 < ns; s0++) {
+    const float w = __shfl(wgt, s0, 64);
+    const x8 v = *(const x8*)(pp + (int64_t)s0 * a.Hq * D);
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] += (float)v[i] * w;
+  }
+  x8 w;
+#pragma unroll
+  for (int i = 0; i < 8; i++) w[i] = (T)acc[i];
+  *(x8*)((T*)a.o + (int64_t)b * a.osb + (int64_t)head * a.osh + tid * 8) = w;
   if (a.lse && tid == 0) a.lse[(int64_t)b * a.Hq + head] = (mx + fast_log2(sum)) * kLn2;
 }
 
 template <typename T>
 static int launch_t(const MlaArgs& a, hipStream_t stream) {
-  constexpr size_t lds = 2 * (size_t)STAGE;
+  constexpr size_t lds = NSTAGE * (size_t)STAGE;
   auto kern = mla_split_kernel<T>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -300,10 +334,10 @@ static int launch_t(const MlaArgs& a, hipStream_t stream) {
   MlaArgs args = a;
   args.head_blocks = (a.Hq + HB - 1) / HB;
   const unsigned grid = (unsigned)(a.B * a.num_split * args.head_blocks);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, args);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, args);
   if (hipGetLastError() != hipSuccess) return -1;
   if (a.num_split > 1) {
-    hipLaunchKernelGGL(mla_combine_kernel<T>, dim3(a.Hq, a.B), dim3(128), 0, stream, a);
+    hipLaunchKernelGGL(mla_combine_kernel<T>, dim3((unsigned)(((int64_t)a.B * a.Hq + 3) / 4)), dim3(256), 0, stream, a);
     if (hipGetLastError() != hipSuccess) return -1;
   }
   return 0;
