@@ -37,6 +37,11 @@ __device__ __forceinline__ int swz_tile(int row) {
   return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
 }
 
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+
 template <typename X8>
 __device__ __forceinline__ X8 scale_bf16x8(X8 v, const float (&w)[8]) {
   X8 r;
@@ -67,7 +72,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
   extern __shared__ __align__(16) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r = lane & 31, g = lane >> 5;
+  const int r0 = lane & 31;
   const uint32_t lds_scal = lds0 + 2 * STAGE + wave * SCAL_BYTES;
   const uint32_t lds_ost = lds0 + 2 * STAGE + NW * SCAL_BYTES + wave * (L * OROW);
 
@@ -98,7 +103,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
   //      the 16-byte chunk that belongs at physical position i of that KB.
   auto issue_chunk = [&](int t0, int buf) {
     const uint32_t base = lds0 + buf * STAGE;
-    for (int ii = wave; ii < 2 * NIQ + NIV; ii += NW) {
+#pragma unroll (DK <= 128 ? 16 : 1)   // (with a 256-wide key the state leaves no registers for an unrolled burst)
+    for (int it = 0; it < (2 * NIQ + NIV + NW - 1) / NW; it++) {
+      const int ii = wave + NW * it;
+      if ((2 * NIQ + NIV) % NW != 0 && ii >= 2 * NIQ + NIV) break;
       if (ii < 2 * NIQ) {
         const int which = ii >= NIQ, i2 = which ? ii - NIQ : ii;
         const int row = i2 * (1024 / RBQ) + lane / CPRQ, c = lane % CPRQ;
@@ -114,24 +122,6 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
     }
   };
 
-  // ---- per-lane LDS read offsets
-  // K rows / Q rows as MFMA operands of A^T = K Q^T: row r, logical chunk 2ks + g
-  const uint32_t qk_row = r * RBQ;
-  const int qk_c0 = g ^ swz16(r);
-  // Q^T operand of h^T Q^T: token r, key dims 32b + 16s + 4g + {0..3} and + 8: chunk 4b + 2s (+1), half g
-  const uint32_t qp_row = r * RBQ + g * 8;
-  const int qp_swz = swz16(r);
-  // transposing reads (K^T and V^T): lane block lane/16 -> (row group g, column half), rows 16s + 4g + jr (+8)
-  const int jr = (lane & 15) >> 2;
-  const int lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
-  const uint32_t kt_row = (4 * g + jr) * RBQ + (lane & 1) * 8;
-  const int kt_c0 = lc ^ swz16(4 * g + jr);                      // rows +8 / +16: see HALF_XOR below
-  const uint32_t vt_row = (4 * g + jr) * RBV + (lane & 1) * 8;
-  const int vt_c0 = (4 * wave + lc) ^ swz_tile<CPRV>(4 * g + jr);
-  // swz(row + 8) ^ swz(row) and swz(row + 16) ^ swz(row) for rows < 8
-  constexpr int Q_X8 = 2, Q_X16 = 0;
-  constexpr int V_X8 = CPRV >= 16 ? 2 : 2, V_X16 = CPRV >= 16 ? 0 : 0;
-
   f32x16 hst[KB];
 #pragma unroll
   for (int i = 0; i < KB; i++)
@@ -139,7 +129,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
     for (int j = 0; j < 16; j++) hst[i][j] = 0.f;
 
   // scalars of the chunk about to be processed (loaded one chunk ahead)
-  const int ti = r;
+  const int ti = r0;
   float ld_next = 0.f, vs_next = 1.f;
   if (ti < Tn) {
     ld_next = ldp[ti];
@@ -165,15 +155,41 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
     const uint32_t base = lds0 + buf * STAGE;
     const uint32_t qbase = base, kbase = base + QT, vbase = base + 2 * QT;
 
+    // ---- per-lane LDS read offsets.  They are loop invariant; left outside the loop, they (and every
+    //      swizzled address derived from them, dozens) stay in registers across chunks, which the state
+    //      accumulator leaves no room for.  The lane id is laundered so that they are rebuilt per chunk.
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int r = ln & 31, g = ln >> 5;
+    // K rows / Q rows as MFMA operands of A^T = K Q^T: row r, logical chunk 2ks + g
+    const uint32_t qk_row = r * RBQ;
+    const int qk_c0 = g ^ swz16(r);
+    // Q^T operand of h^T Q^T: token r, key dims 32b + 16s + 4g + {0..3} and + 8: chunk 4b + 2s (+1), half g
+    const uint32_t qp_row = r * RBQ + g * 8;
+    const int qp_swz = swz16(r);
+    // transposing reads (K^T and V^T): lane block lane/16 -> (row group g, column half), rows 16s + 4g + jr (+8)
+    const int jr = (ln & 15) >> 2;
+    const int lc = (((ln >> 4) & 1) << 1) | ((ln & 3) >> 1);
+    const uint32_t kt_row = (4 * g + jr) * RBQ + (ln & 1) * 8;
+    const int kt_c0 = lc ^ swz16(4 * g + jr);                      // rows +8 / +16: see HALF_XOR below
+    const uint32_t vt_row = (4 * g + jr) * RBV + (ln & 1) * 8;
+    const int vt_c0 = (4 * wave + lc) ^ swz_tile<CPRV>(4 * g + jr);
+    // swz(row + 8) ^ swz(row) and swz(row + 16) ^ swz(row) for rows < 8
+    constexpr int Q_X8 = 2, Q_X16 = 0;
+    constexpr int V_X8 = CPRV >= 16 ? 2 : 2, V_X16 = CPRV >= 16 ? 0 : 0;
+
+
     // ---- chunk scalars: inclusive scan of the log decay over the 32 tokens (both lane halves hold a copy)
     const bool valid = t0 + ti < Tn;
+    // (DPP: shifts within rows of 16 lanes, then lane 15 of rows 0 and 2 carried into rows 1 and 3; the
+    // two halves of the wave scan the same 32 values)
     float gi = valid ? ld : 0.f;
-#pragma unroll
-    for (int d = 1; d < 32; d <<= 1) {
-      const float up = __shfl_up(gi, d, 32);
-      if (ti >= d) gi += up;
-    }
-    const float g_last = __shfl(gi, 31, 32);
+    gi += dpp_f32<0x111>(gi);   // row_shr:1, lanes shifted in from outside the row read 0
+    gi += dpp_f32<0x112>(gi);
+    gi += dpp_f32<0x114>(gi);
+    gi += dpp_f32<0x118>(gi);
+    gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, gi), 0x142, 0xa, 0xf, false));   // row_bcast:15
+    const float g_last = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, gi), 31));
     const float pvq = valid ? vs * a.q_scale : 0.f;               // factor of column j in P
     const float wl = valid ? vs * fast_exp2((g_last - gi) * kLog2e) : 0.f;   // factor of row l in the state update
     const float eg = fast_exp2(gi * kLog2e) * a.q_scale;          // factor of token i in the inter-chunk term
@@ -183,25 +199,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
       lds_write<float>(lds_scal + (L + ti) * 4, pvq);
       lds_write<float>(lds_scal + (2 * L + ti) * 4, wl);
     }
-    // rows held by this lane in a 32 x 32 accumulator block: 8q4 + 4g + {0..3}
-    float gj[16], pj[16], wj[16];
-#pragma unroll
-    for (int q4 = 0; q4 < 4; q4++) {
-      const f32x4 tg = lds_read<f32x4>(lds_scal + (8 * q4 + 4 * g) * 4);
-      const f32x4 tp = lds_read<f32x4>(lds_scal + (L + 8 * q4 + 4 * g) * 4);
-      const f32x4 tw = lds_read<f32x4>(lds_scal + (2 * L + 8 * q4 + 4 * g) * 4);
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        gj[4 * q4 + i] = tg[i];
-        pj[4 * q4 + i] = tp[i];
-        wj[4 * q4 + i] = tw[i];
-      }
-    }
-
     // ---- A^T = K Q^T (lane: token i = r, rows j = 8(jj/4) + 4g + jj%4)
-    f32x16 sacc;
+    f32x16 sacc, sacc2;   // two chains, so that consecutive MFMAs do not wait for each other
 #pragma unroll
-    for (int j = 0; j < 16; j++) sacc[j] = 0.f;
+    for (int j = 0; j < 16; j++) { sacc[j] = 0.f; sacc2[j] = 0.f; }
     {
       constexpr int NS = DK / 16, AH = 2, RING = 3;
       x8 kf[RING], qf[RING];
@@ -216,8 +217,21 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
       for (int ks = 0; ks < NS; ks++) {
         if (ks + AH < NS) request(ks + AH);
         __builtin_amdgcn_sched_barrier(0);
-        sacc = E::mfma32(kf[ks % RING], qf[ks % RING], sacc);
+        if (ks & 1) sacc2 = E::mfma32(kf[ks % RING], qf[ks % RING], sacc2);
+        else sacc = E::mfma32(kf[ks % RING], qf[ks % RING], sacc);
         __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // rows held by this lane in a 32 x 32 accumulator block: 8q4 + 4g + {0..3}
+    float gj[16], pj[16];
+#pragma unroll
+    for (int q4 = 0; q4 < 4; q4++) {
+      const f32x4 tg = lds_read<f32x4>(lds_scal + (8 * q4 + 4 * g) * 4);
+      const f32x4 tp = lds_read<f32x4>(lds_scal + (L + 8 * q4 + 4 * g) * 4);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        gj[4 * q4 + i] = tg[i];
+        pj[4 * q4 + i] = tp[i];
       }
     }
     // ---- P^T: decay, per-token value scale, causal mask (exact zeros above the diagonal)
@@ -226,8 +240,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
     for (int jj = 0; jj < 16; jj++) {
       const int j = 8 * (jj >> 2) + 4 * g + (jj & 3);
       const float e = fast_exp2(fminf(gi - gj[jj], 0.f) * kLog2e);
-      const float p = j <= ti ? sacc[jj] * e * pj[jj] : 0.f;
-      pf[jj >> 3][jj & 7] = (T)p;
+      float p = (sacc[jj] + sacc2[jj]) * e * pj[jj];
+      asm volatile("" : "+v"(p));   // computed for every lane, then selected: no branch per element
+      pf[jj >> 3][jj & 7] = (T)(j <= ti ? p : 0.f);
     }
 
     // ---- V^T fragments (rows = this wave's 32 value columns; k-slot i of slice s is token
@@ -242,9 +257,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
     }
 
     // ---- O^T = (h^T Q^T) * eg + V^T P^T
-    f32x16 o_inter, o_intra;
+    f32x16 o_inter, o_inter2, o_intra;
 #pragma unroll
-    for (int j = 0; j < 16; j++) { o_inter[j] = 0.f; o_intra[j] = 0.f; }
+    for (int j = 0; j < 16; j++) { o_inter[j] = 0.f; o_inter2[j] = 0.f; o_intra[j] = 0.f; }
     o_intra = E::mfma32(vf[0], pf[0], o_intra);
     o_intra = E::mfma32(vf[1], pf[1], o_intra);
     // value-scaled V^T for the state update (k-slot i of slice s is token 16s + 8(i/4) + 4g + i%4 -> wj[8s + i])
@@ -253,7 +268,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
     for (int s = 0; s < 2; s++) {
       float w8[8];
 #pragma unroll
-      for (int i = 0; i < 8; i++) w8[i] = wj[8 * s + i];
+      for (int h2 = 0; h2 < 2; h2++) {
+        const f32x4 tw = lds_read<f32x4>(lds_scal + (2 * L + 16 * s + 8 * h2 + 4 * g) * 4);
+#pragma unroll
+        for (int i = 0; i < 4; i++) w8[4 * h2 + i] = tw[i];
+      }
       vsf[s] = scale_bf16x8(vf[s], w8);
     }
 
@@ -283,7 +302,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
 #pragma unroll
           for (int i = 0; i < 8; i++) hf[i] = (T)hst[bb][8 * s + i];
           x8 qf = __builtin_shufflevector(qlo[bb % RING][s], qhi[bb % RING][s], 0, 1, 2, 3, 4, 5, 6, 7);
-          o_inter = E::mfma32(hf, qf, o_inter);
+          if (DK < 256 && s) o_inter2 = E::mfma32(hf, qf, o_inter2);   // (a second chain where registers allow)
+          else o_inter = E::mfma32(hf, qf, o_inter);
         }
 #pragma unroll
         for (int j = 0; j < 16; j++) hst[bb][j] *= decay_all;
@@ -301,7 +321,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
     for (int q4 = 0; q4 < 4; q4++) {
       x4 w;
 #pragma unroll
-      for (int i = 0; i < 4; i++) w[i] = (T)(o_inter[4 * q4 + i] * eg + o_intra[4 * q4 + i]);
+      for (int i = 0; i < 4; i++) w[i] = (T)((o_inter[4 * q4 + i] + o_inter2[4 * q4 + i]) * eg + o_intra[4 * q4 + i]);
       lds_write<x4>(lds_ost + r * OROW + (8 * q4 + 4 * g) * 2, w);
     }
 #pragma unroll
