@@ -76,6 +76,63 @@ def test_causal_mask_is_exact():
     assert torch.isfinite(o1.float()).all()
 
 
+@pytest.mark.parametrize("B,H,S,causal", [(8, 16, 768, True), (3, 30, 1280, True), (2, 24, 1536, False)])
+def test_softmax_work_distribution(B, H, S, causal):
+    """More work items than CUs, odd numbers of q blocks, (batch*head) counts that are and are not
+    multiples of 8: every item must be computed exactly once whatever the item -> workgroup mapping."""
+    hb = _hb()
+    D = 128
+    g = torch.Generator(device="cuda").manual_seed(S)
+    q, k, v = (torch.randn(B, S, H, D, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(3))
+    o = torch.full((B, S, H, D), float("nan"), device="cuda", dtype=torch.bfloat16)
+    lse = torch.full((B, H, S), float("nan"), device="cuda")
+    print(f"work distribution B{B} H{H} S{S} causal={causal}", flush=True)
+    hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=causal, scale=1 / math.sqrt(D), out=o, row_scale=lse)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    if causal:
+        assert torch.equal(o[:, 0], v[:, 0])
+    for b, h in [(0, 0), (B - 1, H - 1), (B // 2, H // 3)]:
+        ref, lse_ref = oracle.softmax_attention(q[b:b + 1, :, h:h + 1].cpu(), k[b:b + 1, :, h:h + 1].cpu(),
+                                                v[b:b + 1, :, h:h + 1].cpu(), causal=causal, return_lse=True)
+        oracle.assert_close(o[b:b + 1, :, h:h + 1].float().cpu(), ref, rtol=RTOL, atol=ATOL)
+        torch.testing.assert_close(lse[b:b + 1, h:h + 1].cpu(), lse_ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_softmax_growing_and_jumping_scores(dtype):
+    """Row maxima that keep growing along the kv axis (the reference point of the exponentials moves
+    many times) and single keys whose score jumps by hundreds (no overflow, no loss of the rest)."""
+    hb = _hb()
+    B, H, S, D = 1, 2, 640, 128
+    q, k, v = inputs.softmax_inputs(B, H, S, D, D, dtype=dtype, seed=11)
+    ramp = (1.0 + torch.arange(S, dtype=torch.float32) / 8.0).view(1, S, 1, 1)
+    q = (q.float().abs() + 0.5).to(dtype)
+    k = (k.float().abs() * ramp).to(dtype)                      # scores grow roughly linearly with the key index
+    k[:, 333] = k[:, 333] * 6                                   # and one key towers over its neighbours
+    for causal in (True, False):
+        ref, lse_ref = oracle.softmax_attention(q, k, v, causal=causal, return_lse=True)
+        lse = torch.full((B, H, S), float("nan"), device="cuda")
+        print(f"growing scores causal={causal} {dtype}", flush=True)
+        o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_SOFTMAX, causal=causal, scale=1 / math.sqrt(D), row_scale=lse)
+        torch.cuda.synchronize()
+        assert torch.isfinite(o.float()).all()
+        oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+        torch.testing.assert_close(lse.cpu(), lse_ref, rtol=1e-4, atol=1e-3)
+
+
+def test_softmax_cross_lengths():
+    """Different query and key lengths without a mask."""
+    hb = _hb()
+    B, H, Sq, Skv, D = 2, 3, 300, 1000, 128
+    q, _, _ = inputs.softmax_inputs(B, H, Sq, D, D, seed=21)
+    _, k, v = inputs.softmax_inputs(B, H, Skv, D, D, seed=22)
+    ref = oracle.softmax_attention(q, k, v, causal=False)
+    o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_SOFTMAX, causal=False, scale=1 / math.sqrt(D))
+    torch.cuda.synchronize()
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("S,causal,scale,bias", [(256, True, 1.0, -3.0), (192, False, 0.088, -5.5), (130, True, 0.088, 0.5)])
 def test_sigmoid_forward(S, causal, scale, bias):
     hb = _hb()
