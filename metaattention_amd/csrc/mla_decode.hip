@@ -5,21 +5,25 @@
 //   o[b,h,:] = softmax((q[b,h].kv[b,n] + q_pe[b,h].k_pe[b,n]) * scale) . kv[b,n]
 //
 // Split kernel.  A workgroup (8 waves, two per SIMD, the whole CU) owns one (batch, kv split, block of
-// 128 query heads); wave w owns heads 16w..16w+15 and all eight waves consume the same 32-row latent
-// sub-tiles from LDS, so the cache leaves HBM exactly once.  Sub-tiles arrive by direct-to-LDS DMA
-// (global_load_lds_dwordx4: no staging registers; the registers hold the 576-wide Q fragments and the
-// 512 x 16 fp32 output accumulator of the wave) through a ring of 4 stages, three sub-tiles ahead of their
-// use, and a wave waits for its own share with a partial vmcnt before the one barrier per sub-tile.
-// v_mfma_f32_16x16x32 is used throughout:
-//   A[16 x 32]: lane holds row l%16, k = 8(l/16) .. +7
-//   B[32 x 16]: lane holds column l%16, k = 8(l/16) .. +7
-//   C[16 x 16]: lane holds column l%16, element j is row 4(l/16) + j
-// Scores are computed transposed (S^T = KV Q^T) so each lane owns one head's
-// row statistics and the probabilities feed O^T += KV^T P^T straight from the
-// accumulator registers; KV^T comes out of the same row-major LDS tile through
-// the transposing read, so V is never loaded separately.  Within a wave the phases of a sub-tile run one
-// after the other (scores, softmax, P V); the second wave on the SIMD fills the gaps.
-// Combine kernel: log-sum-exp merge of the fp32 partials.
+// 128 query heads) and consumes 32-row latent sub-tiles from LDS, so the cache leaves HBM exactly once.
+// At 128 heads the arithmetic is as dense as the memory stream, and what saturates first is the LDS: every
+// MFMA needs a fresh 1 KB operand from it.  v_mfma_f32_32x32x16 with 32 heads per MFMA halves that
+// traffic per flop, but a wave cannot hold 32 heads x (576 Q + 512 accumulator) columns.  So two waves
+// share a group of 32 heads and split the work along the long axes:
+//   * scores:  each wave takes half of the 576-wide contraction (18 of the 36 k-slices, Q fragments of
+//     its half in 72 registers), S^T_half = KV_half Q_half^T; the halves are exchanged through LDS
+//     (4 KB each way) and added, so both waves hold the full 32 x 32 score tile;
+//   * softmax: computed by both (16 scores per lane; the sums a+b and b+a are the same bits);
+//   * output:  each wave takes half of the 512 value columns, O^T_half += KV_half^T P^T (128 registers).
+// Sub-tiles arrive by direct-to-LDS DMA (global_load_lds_dwordx4: no staging registers) through a ring of
+// 3 stages, two sub-tiles ahead of their use, and a wave waits for its own share with a partial vmcnt.
+//   A[32 x 16]: lane holds row l%32, k = 8(l/32) .. +7
+//   B[16 x 32]: lane holds column l%32, k = 8(l/32) .. +7
+//   C[32 x 32]: lane holds column l%32, element j is row 8(j/4) + 4(l/32) + j%4
+// Scores are computed transposed (S^T = KV Q^T) so each lane owns one head's row statistics and the
+// probabilities feed O^T += KV^T P^T straight from the accumulator registers; KV^T comes out of the same
+// row-major LDS tile through the transposing read, so V is never loaded separately.
+// Combine kernel: log-sum-exp merge of the partials.
 #include "mla_decode.h"
 
 namespace ma {
@@ -27,12 +31,12 @@ namespace ma {
 namespace {
 constexpr int BN = 32;         // kv rows per sub-tile
 constexpr int HB = 128;        // heads per workgroup
-constexpr int NW = 8;          // waves per workgroup
+constexpr int NW = 8;          // waves per workgroup: 4 head groups x 2 halves
 constexpr int D = 512, DPE = 64;
-constexpr int NSTAGE = 4;
+constexpr int NSTAGE = 3;
 constexpr int KV_ROW = D * 2 + 32;  // bytes; each latent row is its own DMA, so rows can be padded: with a
                                    // 32 B pad consecutive rows start 8 banks apart (the transposing reads of
-                                   // 8 rows x 32 B tile the 64 banks exactly) and rows 8..15 of a 16-row group
+                                   // 8 rows x 32 B tile the 64 banks exactly) and rows 8..15 of every 16-row group
                                    // additionally swap their 16-byte chunk pairs (kv_flip) so that the 128-bit
                                    // reads of 16 rows x one chunk hit 16 different bank groups.  Every LDS
                                    // read address is then lane base + compile-time offset.
@@ -40,11 +44,10 @@ constexpr int PE_ROW = DPE * 2;    // rope rows share a DMA (8 rows per KB): XOR
 constexpr int KV_TILE = BN * KV_ROW;   // 33 KB
 constexpr int PE_TILE = BN * PE_ROW;   // 4 KB
 constexpr int STAGE = KV_TILE + PE_TILE;
+constexpr int XCHG = 4096;             // one wave's half score tile: 16 fp32 per lane
 
 __device__ __forceinline__ int kv_flip(int row) { return (row >> 3) & 1; }
 __device__ __forceinline__ int swz_pe(int row) { return (row >> 1) & 7; }
-
-__device__ __forceinline__ float xlane(float x, int mask) { return __shfl_xor(x, mask, 64); }
 }  // namespace
 
 template <typename T>
@@ -52,31 +55,37 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
   using E = Elem<T>;
   using x8 = typename E::x8;
   using x4 = typename E::x4;
-  constexpr int KS = D / 32, KSPE = DPE / 32, DB = D / 16, NB = BN / 16;
+  using x2 = typename E::x2;
+  constexpr int NSL = (D + DPE) / 16 / 2;   // 18 k-slices of 16 per wave
+  constexpr int NLAT1 = D / 16 - NSL;       // latent slices of the second half (14); its last 4 slices are the rope columns
+  constexpr int DBH = D / 32 / 2;           // 8 output blocks of 32 columns per wave
 
   extern __shared__ __align__(16) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
+  const uint32_t lds_x = lds0 + NSTAGE * STAGE;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r = lane & 15, q = lane >> 4;
+  const int hg = wave & 3, hf = wave >> 2;   // head group, half
+  const int r = lane & 31, g = lane >> 5;
   const int hblk = blockIdx.x % a.head_blocks, bs = blockIdx.x / a.head_blocks;
   const int b = bs / a.num_split, split = bs % a.num_split;
-  const int head = hblk * HB + wave * 16 + r;
+  const int head = hblk * HB + hg * 32 + r;
   const int head_ld = min(head, a.Hq - 1);
 
   const int n_begin = split * a.split_len;
   const int n_end = min(n_begin + a.split_len, a.Skv);
   const int n_tiles = n_end > n_begin ? (n_end - n_begin + BN - 1) / BN : 0;
 
-  // ---- Q fragments: B operand of S^T = KV Q^T
-  x8 qf[KS + KSPE];
+  // ---- Q fragments of this wave's half of the contraction: B operand (lane: head r, k = 8g .. 8g+7 of a slice)
+  x8 qf[NSL];
   {
-    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)head_ld * a.qsh + 8 * q;
+    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)head_ld * a.qsh + 8 * g + hf * (NSL * 16);
+    const T* qpe = (const T*)a.q_pe + (int64_t)b * a.qpsb + (int64_t)head_ld * a.qpsh + 8 * g;
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 32 * ks);
-    const T* qpe = (const T*)a.q_pe + (int64_t)b * a.qpsb + (int64_t)head_ld * a.qpsh + 8 * q;
-#pragma unroll
-    for (int ks = 0; ks < KSPE; ks++) qf[KS + ks] = *(const x8*)(qpe + 32 * ks);
+    for (int sl = 0; sl < NSL; sl++) {
+      const T* src = (hf == 1 && sl >= NLAT1) ? qpe + 16 * (sl - NLAT1) : qp + 16 * sl;
+      qf[sl] = *(const x8*)src;
+    }
   }
 
   const char* kvb = (const char*)a.kv + (int64_t)b * a.kvsb * 2;
@@ -86,11 +95,10 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
   // ---- DMA.  Wave w streams latent rows 4w..4w+3 of a sub-tile, one instruction per row (64 lanes x 16 B =
   //      the 1 KB row; lane i fetches the chunk that belongs at physical chunk i); waves 0..3 also fetch 8
   //      rope rows each with one more instruction.  Rows beyond the cache are clamped to its last row
-  //      (their scores are masked).  NDMA is the wave's instruction count per sub-tile.
-  const int NDMA = wave < 4 ? 5 : 4;
+  //      (their scores are masked).
   const uint32_t lane_off = (uint32_t)(lane ^ ((wave >> 1) & 1)) << 4;   // kv_flip(4w + i) = (w >> 1) & 1
   auto issue_tile = [&](int jt) {
-    const uint32_t sb = lds0 + (jt & (NSTAGE - 1)) * STAGE;
+    const uint32_t sb = lds0 + (jt % NSTAGE) * STAGE;
     const int n0 = n_begin + jt * BN;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -106,171 +114,171 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
   };
 
   // ---- per-lane LDS read offsets within a stage
-  // K side (A operand): row 16nb + r, logical 16-byte chunk 4ks + q
-  const uint32_t k_row_off = r * KV_ROW + (q ^ kv_flip(r)) * 16;
-  const uint32_t pe_row_off = KV_TILE + r * PE_ROW;
-  const int pe_chunk0 = q ^ swz_pe(r);
-  // V side (transposing read): lane block q reads rows 4q + jr (and + 16), columns 16db + 4(l%4)..+3
-  const int jr = r >> 2;
-  const uint32_t v_row_off = (4 * q + jr) * KV_ROW + ((((lane & 3) >> 1) ^ kv_flip(4 * q + jr)) << 4) + (lane & 1) * 8;
+  // K side (A operand): row r, logical 16-byte chunk 2 * slice + g; this wave's first slice is hf * 18
+  const uint32_t k_off = r * KV_ROW + ((g ^ kv_flip(r)) << 4) + hf * (NSL * 32);
+  const uint32_t pe_off = KV_TILE + r * PE_ROW;
+  const int pe_c0 = g ^ swz_pe(r);
+  // V side (transposing read): the low half of a fragment reads rows 16sl + 4g + jr (chunks not flipped), the
+  // high half rows + 8 (chunk pairs flipped); chunk 4 * block + lc; this wave's first block is hf * 8
+  const int jr = (lane & 15) >> 2;
+  const int lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
+  const uint32_t v_lo_off = (4 * g + jr) * KV_ROW + (lc << 4) + (lane & 1) * 8 + hf * (DBH * 64);
+  const uint32_t v_hi_off = (4 * g + jr + 8) * KV_ROW + ((lc ^ 1) << 4) + (lane & 1) * 8 + hf * (DBH * 64);
+  // exchange of the half score tiles: 4 x 16 bytes per lane, lane-major
+  const uint32_t x_mine = lds_x + wave * XCHG + lane * 16, x_other = lds_x + (wave ^ 4) * XCHG + lane * 16;
 
-  f32x4 o[DB];
+  f32x16 o[DBH];
 #pragma unroll
-  for (int i = 0; i < DB; i++) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < DBH; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) o[i][j] = 0.f;
   const float c_scale = a.scale * kLog2e;
-  float row_max = -1e30f, row_sum = 0.f;
+  float row_ref = -1e30f, row_sum = 0.f;
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   if (n_tiles > 0) issue_tile(0);
   if (n_tiles > 1) issue_tile(1);
-  if (n_tiles > 2) issue_tile(2);
 
   for (int jt = 0; jt < n_tiles; jt++) {
-    // Sub-tile jt has landed for every wave (a wave's loads complete in order: only those of the up to two
-    // later sub-tiles may still be in flight) and every wave is done with sub-tile jt-1, whose stage
-    // takes sub-tile jt+3.
-    if (jt + 2 < n_tiles) {
-      if (wave < 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 10); else __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
-    } else if (jt + 1 < n_tiles) {
+    // Sub-tile jt has landed for every wave (a wave's loads complete in order: only those of sub-tile jt+1
+    // may still be in flight), every wave is done with sub-tile jt-1, whose stage takes sub-tile jt+2, and
+    // every wave has read its partner's half scores of sub-tile jt-1.
+    if (jt + 1 < n_tiles) {
       if (wave < 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 5); else __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
     } else {
       wait_dma();
     }
     __syncthreads();
-    if (jt + 3 < n_tiles) issue_tile(jt + 3);
+    if (jt + 2 < n_tiles) issue_tile(jt + 2);
     const int n0 = n_begin + jt * BN;
-    uint32_t base = lds0 + (jt & (NSTAGE - 1)) * STAGE;
+    const uint32_t base = lds0 + (jt % NSTAGE) * STAGE;
 
-    // ---- S^T = KV Q^T + K_pe Q_pe^T : lane holds head r, kv rows 16nb + 4q + j
-    f32x4 s[NB];
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++) s[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // ---- half scores: S^T_half = KV_half Q_half^T over this wave's 18 k-slices
+    f32x16 sc;
     {
-      // fragments are requested AH slices ahead of the MFMAs that consume them
-      constexpr int AH = 2, RING = AH + 1, NSL = KS + KSPE;
-      x8 kf[RING][NB];
-      uint32_t kb = base + k_row_off, pb = base + pe_row_off;
-      asm volatile("" : "+v"(kb), "+v"(pb));   // one address register + immediates for every read below
-      auto request = [&](int ks) {
-        if (ks < KS) {
+      constexpr int AH = 2, RING = AH + 1;
+      x8 kf[RING];
+      uint32_t kb = base + k_off, pb = base + pe_off;
+      asm volatile("" : "+v"(kb), "+v"(pb));   // one address register + immediates for the reads below
+      // the last four slices of the second half are the rope columns (their own, XOR-swizzled tile)
+      uint32_t tail[NSL - NLAT1];
 #pragma unroll
-          for (int nb = 0; nb < NB; nb++) kf[ks % RING][nb] = lds_read<x8>(kb + nb * 16 * KV_ROW + ks * 64);
-        } else {
-          const uint32_t coff = (uint32_t)((pe_chunk0 ^ (4 * (ks - KS))) << 4);
-#pragma unroll
-          for (int nb = 0; nb < NB; nb++) kf[ks % RING][nb] = lds_read<x8>(pb + nb * 16 * PE_ROW + coff);
-        }
+      for (int j = 0; j < NSL - NLAT1; j++) tail[j] = hf ? pb + (uint32_t)((pe_c0 ^ (2 * j)) << 4) : kb + 32 * (NLAT1 + j);
+      auto request = [&](int sl) {
+        kf[sl % RING] = lds_read<x8>(sl < NLAT1 ? kb + 32 * sl : tail[sl < NLAT1 ? 0 : sl - NLAT1]);
       };
 #pragma unroll
-      for (int ks = 0; ks < AH; ks++) request(ks);
+      for (int sl = 0; sl < AH; sl++) request(sl);
 #pragma unroll
-      for (int ks = 0; ks < NSL; ks++) {
-        if (ks + AH < NSL) request(ks + AH);
+      for (int sl = 0; sl < NSL; sl++) {
+        if (sl + AH < NSL) request(sl + AH);
         __builtin_amdgcn_sched_barrier(0);   // keep the requests ahead of the MFMAs that hide their latency
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) s[nb] = E::mfma16(kf[ks % RING][nb], qf[ks], s[nb]);
+        sc = E::mfma32(kf[sl % RING], qf[sl], sl == 0 ? zero16 : sc);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    // ---- exchange and add the halves
+#pragma unroll
+    for (int j4 = 0; j4 < 4; j4++) lds_write<f32x4>(x_mine + j4 * 1024, f32x4{sc[4 * j4], sc[4 * j4 + 1], sc[4 * j4 + 2], sc[4 * j4 + 3]});
+    __syncthreads();
+#pragma unroll
+    for (int j4 = 0; j4 < 4; j4++) {
+      const f32x4 t = lds_read<f32x4>(x_other + j4 * 1024);
+#pragma unroll
+      for (int i = 0; i < 4; i++) sc[4 * j4 + i] += t[i];
+    }
 
+    // the first fragments of P V are requested before the softmax: their latency hides behind it
+    uint32_t vlo = base + v_lo_off, vhi = base + v_hi_off;
+    asm volatile("" : "+v"(vlo), "+v"(vhi));
+    constexpr int PF = 3, NPV = 2 * DBH;   // fragments in flight; MFMA i: slice i / DBH, block i % DBH
+    x4 lo[PF], hi[PF];
+    auto v_request = [&](int i) {
+      const int sl = i / DBH, db = i % DBH;
+      lo[i % PF] = lds_read_tr4<T>(vlo + 16 * sl * KV_ROW + 64 * db);
+      hi[i % PF] = lds_read_tr4<T>(vhi + 16 * sl * KV_ROW + 64 * db);
+    };
+#pragma unroll
+    for (int i = 0; i < PF - 1; i++) v_request(i);
+
+    // ---- mask, online softmax in the log2 domain: lane holds head r, kv rows 8(j/4) + 4g + j%4
     if (n0 + BN > n_end) {
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-          if (n0 + 16 * nb + 4 * q + j >= n_end) s[nb][j] = -INFINITY;
+      for (int j = 0; j < 16; j++)
+        if (n0 + 8 * (j >> 2) + 4 * g + (j & 3) >= n_end) sc[j] = -INFINITY;
     }
-
-    // ---- online softmax in the log2 domain (the 4 lanes l%16 == r own one head)
-    float mx = s[0][0];
+    float mx = sc[0];
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-      for (int j = 0; j < 4; j++) mx = fmaxf(mx, s[nb][j]);
-    mx = fmaxf(mx, xlane(mx, 16));
-    mx = fmaxf(mx, xlane(mx, 32));
-    // The running max is only moved when some head's max grew by more than 2^8: until then the
-    // probabilities are taken relative to the stale max (at most 256, exact in fp32 / bf16 range) and the
-    // 128 accumulator registers need no rescaling.  The final normalisation by row_sum absorbs the offset.
-    const float cand = fmaxf(row_max, mx * c_scale);
-    const bool move = cand - row_max > 8.f;   // per head: heads that stay multiply by exactly 1
+    for (int j = 1; j < 16; j++) mx = fmaxf(mx, sc[j]);
+    {
+      float m_lo, m_hi;
+      xhalf_pair(mx, m_lo, m_hi);
+      mx = fmaxf(m_lo, m_hi);
+    }
+    // The reference point of the exponentials only moves when some head's max grew by more than 2^8: until
+    // then the probabilities are taken relative to the stale reference (at most 256, exact in fp32 / in
+    // range for bf16 and fp16) and the 128 accumulator registers need no rescaling.  The final
+    // normalisation by row_sum absorbs the offset.  Each head decides for itself.
+    const float cand = fmaxf(row_ref, mx * c_scale);
+    const bool move = cand - row_ref > 8.f;
     if (__any(move)) {
-      const float corr = move ? fast_exp2(row_max - cand) : 1.f;
-      row_max = move ? cand : row_max;
+      const float corr = move ? fast_exp2(row_ref - cand) : 1.f;
+      row_ref = move ? cand : row_ref;
       row_sum *= corr;
 #pragma unroll
-      for (int i = 0; i < DB; i++)
+      for (int i = 0; i < DBH; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(o[i][j]) : "v"(corr));
+        for (int j = 0; j < 16; j++) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(o[i][j]) : "v"(corr));
     }
+    // probabilities, packed as the B operand of P V: p[sl] holds elements 8sl .. 8sl+7 (k slot i of lane
+    // half g is kv row 16sl + 8(i/4) + 4g + i%4, matched by the rows the transposing V reads fetch)
+    x8 p[2];
     float part = 0.f;
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const float p = fast_exp2(s[nb][j] * c_scale - row_max);
-        s[nb][j] = p;
-        part += p;
-      }
+    for (int j = 0; j < 16; j++) {
+      const float pe = fast_exp2(sc[j] * c_scale - row_ref);
+      part += pe;
+      p[j >> 3][j & 7] = (T)pe;
+    }
     row_sum += part;
 
-    // ---- O^T += KV^T P^T ; lane block q, k slot i is kv row 16(i/4) + 4q + i%4 on both operands
-    {
-      x8 pf;
+    // ---- O^T_half += KV_half^T P^T
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        pf[i] = (T)s[0][i];
-        pf[4 + i] = (T)s[1][i];
-      }
-      uint32_t rb = base + v_row_off;
-      asm volatile("" : "+v"(rb));
-      constexpr int PF = 4;   // V fragments in flight
-      x4 lo[PF], hi[PF];
-#pragma unroll
-      for (int i = 0; i < PF - 1; i++) {
-        lo[i] = lds_read_tr4<T>(rb + i * 32);
-        hi[i] = lds_read_tr4<T>(rb + 16 * KV_ROW + i * 32);
-      }
-#pragma unroll
-      for (int db = 0; db < DB; db++) {
-        if (db + PF - 1 < DB) {
-          lo[(db + PF - 1) % PF] = lds_read_tr4<T>(rb + (db + PF - 1) * 32);
-          hi[(db + PF - 1) % PF] = lds_read_tr4<T>(rb + 16 * KV_ROW + (db + PF - 1) * 32);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        x8 vf = __builtin_shufflevector(lo[db % PF], hi[db % PF], 0, 1, 2, 3, 4, 5, 6, 7);
-        o[db] = E::mfma16(vf, pf, o[db]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+    for (int i = 0; i < NPV; i++) {
+      if (i + PF - 1 < NPV) v_request(i + PF - 1);
+      __builtin_amdgcn_sched_barrier(0);
+      x8 vf = __builtin_shufflevector(lo[i % PF], hi[i % PF], 0, 1, 2, 3, 4, 5, 6, 7);
+      o[i % DBH] = E::mfma32(vf, p[i / DBH], o[i % DBH]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
-  // ---- epilogue: lane holds head r, output columns 16db + 4q + j
-  float tot = row_sum + xlane(row_sum, 16);
-  tot += xlane(tot, 32);
+  // ---- epilogue: lane holds head r, output columns 256 hf + 32db + 8(j/4) + 4g + j%4
+  float t_lo, t_hi;
+  xhalf_pair(row_sum, t_lo, t_hi);
+  const float tot = t_lo + t_hi;
   const bool empty = n_tiles == 0;
   const float inv = empty ? 0.f : 1.f / tot;
-  const float lse2 = empty ? -INFINITY : row_max + fast_log2(tot);   // log2 domain
+  const float lse2 = empty ? -INFINITY : row_ref + fast_log2(tot);   // log2 domain
   if (head < a.Hq) {
-    if (a.num_split == 1) {
-      T* op = (T*)a.o + (int64_t)b * a.osb + (int64_t)head * a.osh + 4 * q;
+    T* op = a.num_split == 1 ? (T*)a.o + (int64_t)b * a.osb + (int64_t)head * a.osh
+                             : (T*)a.o_part + (((int64_t)b * a.num_split + split) * a.Hq + head) * D;
+    op += hf * (D / 2) + 4 * g;
 #pragma unroll
-      for (int db = 0; db < DB; db++) {
+    for (int db = 0; db < DBH; db++)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
         x4 w;
 #pragma unroll
-        for (int i = 0; i < 4; i++) w[i] = (T)(o[db][i] * inv);
-        *(x4*)(op + 16 * db) = w;
+        for (int i = 0; i < 4; i++) w[i] = (T)(o[db][4 * q4 + i] * inv);
+        *(x4*)(op + 32 * db + 8 * q4) = w;
       }
-      if (a.lse && q == 0) a.lse[(int64_t)b * a.Hq + head] = lse2 * kLn2;
-    } else {
-      T* op = (T*)a.o_part + (((int64_t)b * a.num_split + split) * a.Hq + head) * D + 4 * q;
-#pragma unroll
-      for (int db = 0; db < DB; db++) {
-        x4 w;
-#pragma unroll
-        for (int i = 0; i < 4; i++) w[i] = (T)(o[db][i] * inv);
-        *(x4*)(op + 16 * db) = w;
+    if (hf == 0 && g == 0) {
+      if (a.num_split == 1) {
+        if (a.lse) a.lse[(int64_t)b * a.Hq + head] = lse2 * kLn2;
+      } else {
+        a.lse_part[((int64_t)b * a.num_split + split) * a.Hq + head] = lse2;
       }
-      if (q == 0) a.lse_part[((int64_t)b * a.num_split + split) * a.Hq + head] = lse2;
     }
   }
 }
@@ -324,7 +332,7 @@ __global__ __launch_bounds__(256) void mla_combine_kernel(const MlaArgs a) {
 
 template <typename T>
 static int launch_t(const MlaArgs& a, hipStream_t stream) {
-  constexpr size_t lds = NSTAGE * (size_t)STAGE;
+  constexpr size_t lds = NSTAGE * (size_t)STAGE + NW * (size_t)XCHG;
   auto kern = mla_split_kernel<T>;
   static bool attr_set = false;
   if (!attr_set) {
