@@ -260,10 +260,13 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
   const bool empty = n_tiles == 0;
   const float inv = empty ? 0.f : 1.f / tot;
   const float lse2 = empty ? -INFINITY : row_ref + fast_log2(tot);   // log2 domain
-  if (head < a.Hq) {
-    T* op = a.num_split == 1 ? (T*)a.o + (int64_t)b * a.osb + (int64_t)head * a.osh
-                             : (T*)a.o_part + (((int64_t)b * a.num_split + split) * a.Hq + head) * D;
-    op += hf * (D / 2) + 4 * g;
+  // Stage the wave's 32 heads x 256 columns through LDS (the stages are free now) so that every head's
+  // half row leaves as 512 contiguous bytes in 16-byte pieces; chunks are XOR-swizzled by head so that
+  // neither the 8-byte writes nor the 16-byte reads pile onto one bank group.
+  __syncthreads();   // every wave is done with the last sub-tile
+  {
+    constexpr int SROW = D;   // bytes: 256 columns of T
+    const uint32_t sb = lds0 + wave * 32 * SROW;
 #pragma unroll
     for (int db = 0; db < DBH; db++)
 #pragma unroll
@@ -271,14 +274,23 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
         x4 w;
 #pragma unroll
         for (int i = 0; i < 4; i++) w[i] = (T)(o[db][4 * q4 + i] * inv);
-        *(x4*)(op + 32 * db + 8 * q4) = w;
+        lds_write<x4>(sb + r * SROW + (((4 * db + q4) ^ (r & 31)) << 4) + 8 * g, w);
       }
-    if (hf == 0 && g == 0) {
-      if (a.num_split == 1) {
-        if (a.lse) a.lse[(int64_t)b * a.Hq + head] = lse2 * kLn2;
-      } else {
-        a.lse_part[((int64_t)b * a.num_split + split) * a.Hq + head] = lse2;
-      }
+    T* obase = a.num_split == 1 ? (T*)a.o + (int64_t)b * a.osb : (T*)a.o_part + ((int64_t)b * a.num_split + split) * a.Hq * D;
+    const int64_t ostride = a.num_split == 1 ? a.osh : D;
+    const int head0 = hblk * HB + hg * 32;
+#pragma unroll
+    for (int it = 0; it < 32 * (SROW / 16) / 64; it++) {
+      const int ci = lane + 64 * it, row = ci / (SROW / 16), c = ci % (SROW / 16);
+      const u32x4 w = lds_read<u32x4>(sb + row * SROW + ((c ^ (row & 31)) << 4));
+      if (head0 + row < a.Hq) *(u32x4*)(obase + (int64_t)(head0 + row) * ostride + hf * (D / 2) + c * 8) = w;
+    }
+  }
+  if (head < a.Hq && hf == 0 && g == 0) {
+    if (a.num_split == 1) {
+      if (a.lse) a.lse[(int64_t)b * a.Hq + head] = lse2 * kLn2;
+    } else {
+      a.lse_part[((int64_t)b * a.num_split + split) * a.Hq + head] = lse2;
     }
   }
 }
