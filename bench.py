@@ -101,7 +101,8 @@ def bench_retnet_chunked(steps, warmup):
     v = torch.randn(B, H, T, Dv, device="cuda", generator=g).bfloat16()
     ld = torch.log(1 - torch.exp2(-5 - torch.arange(H, device="cuda").float())).view(1, H, 1).expand(B, H, T).contiguous()
     o = torch.empty_like(v)
-    ms = time_gpu(lambda: hb.linear_fwd(q, k, v, ld, q_scale=Dk ** -0.5, out=o), steps, warmup)
+    ws = torch.empty(max(hb.linear_workspace_bytes(B, H, H, H, T, Dk, Dv), 16), dtype=torch.uint8, device="cuda")
+    ms = time_gpu(lambda: hb.linear_fwd(q, k, v, ld, q_scale=Dk ** -0.5, out=o, workspace=ws), steps, warmup)
     C = 64
     flops = B * H * (2.0 * T * C * (Dk + Dv) + 4.0 * T * Dk * Dv)
     return _mfma_entry(ms, flops, "chunked form, chunk 64: 2*S*C*(Dqk+Dv) + 4*S*Dqk*Dv per (batch, head)")
@@ -140,7 +141,8 @@ def bench_mamba2(steps, warmup):
     A = -torch.exp(torch.rand(1, H, device="cuda", generator=g) * math.log(16))
     ld = (dt * A.view(1, H, 1)).contiguous()
     o = torch.empty_like(x)
-    ms = time_gpu(lambda: hb.linear_fwd(Cm, Bm, x, ld, v_scale=dt, out=o), steps, warmup)
+    ws = torch.empty(max(hb.linear_workspace_bytes(B, H, 1, 1, T, N, P), 16), dtype=torch.uint8, device="cuda")
+    ms = time_gpu(lambda: hb.linear_fwd(Cm, Bm, x, ld, v_scale=dt, out=o, workspace=ws), steps, warmup)
     Lc = 256
     flops = B * H * (2.0 * T * Lc * N + 2.0 * T * Lc * P + 4.0 * T * N * P)
     return _mfma_entry(ms, flops, "chunk 256, C.B^T counted per head: 2*S*L*N + 2*S*L*P + 4*S*N*P per (batch, head); "

@@ -89,7 +89,8 @@ typedef struct ma_linear_params {
   const float* log_decay;
   const float* v_scale;
   float q_scale;
-  void* workspace; size_t workspace_bytes; /* see ma_linear_workspace_bytes */
+  int32_t segments; /* 0 = let the library choose; 1 = single pass; n = cut the sequence into at most n segments */
+  void* workspace; size_t workspace_bytes; /* see ma_linear_workspace_bytes; may be NULL (then single pass) */
 } ma_linear_params;
 
 /* Absorbed MLA decode forward.  Replaces flash_attn_split + combine

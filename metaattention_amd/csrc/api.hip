@@ -68,28 +68,49 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
   return MA_OK;
 }
 
-// The state stays on chip, so the forward pass needs no workspace; the entry point exists so
-// that callers size buffers through the library rather than assuming that.
-size_t ma_linear_workspace_bytes(const ma_linear_params* p) { (void)p; return 0; }
-
-int ma_linear_fwd(const ma_linear_params* p, ma_stream_t stream) {
-  if (!p) return fail(MA_ERR_INVALID_ARG, "ma_linear_fwd: params is NULL");
-  if (!p->q || !p->k || !p->v || !p->o || !p->log_decay)
-    return fail(MA_ERR_INVALID_ARG, "ma_linear_fwd: q/k/v/o/log_decay must be non-NULL");
+static int check_linear(const ma_linear_params* p, const char* who) {
+  if (!p) return fail(MA_ERR_INVALID_ARG, "%s: params is NULL", who);
   if (p->batch <= 0 || p->heads <= 0 || p->heads_q <= 0 || p->heads_k <= 0 || p->seqlen <= 0 || p->dim_k <= 0 || p->dim_v <= 0)
-    return fail(MA_ERR_INVALID_ARG, "ma_linear_fwd: sizes must be positive");
-  if (p->dtype != MA_BF16) return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: only bf16 (the reference's linear kernels are bf16 only)");
+    return fail(MA_ERR_INVALID_ARG, "%s: sizes must be positive", who);
+  if (p->dtype != MA_BF16) return fail(MA_ERR_UNSUPPORTED, "%s: only bf16 (the reference's linear kernels are bf16 only)", who);
   if (p->heads % p->heads_q != 0 || p->heads % p->heads_k != 0)
-    return fail(MA_ERR_INVALID_ARG, "ma_linear_fwd: heads (%d) must be a multiple of heads_q (%d) and heads_k (%d)", p->heads, p->heads_q, p->heads_k);
-  if ((int64_t)p->batch * p->heads * ((p->dim_v + 63) / 64) > 0x7fffffff) return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: grid too large");
-  const uintptr_t ptrs[] = {(uintptr_t)p->q, (uintptr_t)p->k, (uintptr_t)p->v, (uintptr_t)p->o};
-  for (uintptr_t x : ptrs)
-    if (x % 16 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: q/k/v/o must be 16-byte aligned");
+    return fail(MA_ERR_INVALID_ARG, "%s: heads (%d) must be a multiple of heads_q (%d) and heads_k (%d)", who, p->heads, p->heads_q, p->heads_k);
+  if (p->segments < 0) return fail(MA_ERR_INVALID_ARG, "%s: segments must be >= 0", who);
+  if ((int64_t)p->batch * p->heads * ((p->dim_v + 63) / 64) * (p->segments > 8 ? p->segments : 8) > 0x7fffffff)
+    return fail(MA_ERR_UNSUPPORTED, "%s: grid too large", who);
+  return MA_OK;
+}
+
+static ma::LinArgs linear_args(const ma_linear_params* p) {
   ma::LinArgs a{};
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.log_decay = p->log_decay; a.v_scale = p->v_scale;
   a.q_scale = p->q_scale;
   a.B = p->batch; a.H = p->heads; a.Hq = p->heads_q; a.Hk = p->heads_k; a.T = p->seqlen; a.Dv = p->dim_v;
-  const int rc = ma::linear_fwd_dispatch(a, p->dim_k, (hipStream_t)stream);
+  return a;
+}
+
+// The state of one sequence stays on chip; a workspace is only used when the sequence is cut into
+// segments that run side by side (few batch x heads): it then holds the segments' fp32 end states.
+// Without it (or with segments = 1) the forward pass runs as a single pass.  Returns 0 for
+// arguments ma_linear_fwd would refuse and when no device is present.
+size_t ma_linear_workspace_bytes(const ma_linear_params* p) {
+  if (!p || p->batch <= 0 || p->heads <= 0 || p->heads_q <= 0 || p->heads_k <= 0 || p->seqlen <= 0 || p->dim_k <= 0 || p->dim_v <= 0 ||
+      p->heads % p->heads_q != 0 || p->heads % p->heads_k != 0 || p->segments < 0)
+    return 0;
+  size_t bytes = 0;
+  if (ma::linear_fwd_dispatch(linear_args(p), p->dim_k, p->segments, nullptr, 0, nullptr, &bytes) != 0) return 0;
+  return bytes;
+}
+
+int ma_linear_fwd(const ma_linear_params* p, ma_stream_t stream) {
+  if (const int rc0 = check_linear(p, "ma_linear_fwd")) return rc0;
+  if (!p->q || !p->k || !p->v || !p->o || !p->log_decay)
+    return fail(MA_ERR_INVALID_ARG, "ma_linear_fwd: q/k/v/o/log_decay must be non-NULL");
+  const uintptr_t ptrs[] = {(uintptr_t)p->q, (uintptr_t)p->k, (uintptr_t)p->v, (uintptr_t)p->o};
+  for (uintptr_t x : ptrs)
+    if (x % 16 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: q/k/v/o must be 16-byte aligned");
+  const ma::LinArgs a = linear_args(p);
+  const int rc = ma::linear_fwd_dispatch(a, p->dim_k, p->segments, p->workspace, p->workspace_bytes, (hipStream_t)stream, nullptr);
   if (rc == -2)
     return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: no kernel for dim_k=%d (128 or 256) / dim_v=%d (multiple of 64)", p->dim_k, p->dim_v);
   if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_linear_fwd: launch failed: %s", hipGetErrorString(hipGetLastError()));

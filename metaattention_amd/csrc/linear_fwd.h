@@ -10,8 +10,13 @@ struct LinArgs {
   const float* v_scale;    // [B,H,T] or null
   float q_scale;
   int B, H, Hq, Hk, T, Dv, dv_blocks;
+  // sequence segments (see linear_fwd.hip): nseg segments of seg_chunks 32-token chunks; local end
+  // states [group][segment][wave][registers][lane] fp32 and per-(batch*head, segment) log decays
+  int nseg, seg_chunks;
+  float* ws_state;
+  float* ws_decay;
 };
 
-int linear_fwd_dispatch(const LinArgs& a, int dk, hipStream_t stream);
+int linear_fwd_dispatch(const LinArgs& a, int dk, int want_segments, void* ws, size_t ws_size, hipStream_t stream, size_t* query);
 
 }  // namespace ma

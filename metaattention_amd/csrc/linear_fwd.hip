@@ -23,6 +23,18 @@
 // register for register, the A operand of h^T Q^T, so the state never moves.
 // Q/K/V chunk tiles arrive by direct-to-LDS DMA, double buffered, with a single
 // workgroup barrier per chunk.
+//
+// Heads that share their q and k head (Mamba2: one B/C group for all heads) can be
+// grouped HG to a workgroup, which then shares the Q/K tiles in LDS.
+//
+// Segments.  One (batch, head) is a serial chain of T/32 chunks; when batch x heads
+// is too small to give every SIMD several waves, the sequence is cut into segments
+// that run side by side: a first launch (MODE 1) computes, for every segment but the
+// last, the state it ends in when entered with a zero state and its total log decay;
+// the second launch (MODE 2) enters segment s with
+//   sum_{s' < s} exp(sum_{s' < s'' < s} D[s'']) h_local[s']
+// (states are exchanged in accumulator-register order, fp32, through the workspace)
+// and produces the outputs.  MODE 0 is the single pass.
 #include "linear_fwd.h"
 
 namespace ma {
@@ -51,9 +63,15 @@ __device__ __forceinline__ X8 scale_bf16x8(X8 v, const float (&w)[8]) {
 }
 }  // namespace
 
-template <int DK, int NW>
-// second launch-bound argument: minimum waves per SIMD (8 waves of one workgroup need 2)
-__global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(const LinArgs a) {
+// minimum waves per SIMD asked of the register allocator: 8 waves of one workgroup need 2; the
+// two-heads-per-workgroup configuration is meant to run three workgroups of 4 waves per CU
+template <int DK, int NWH, int HG>
+constexpr int min_waves_per_simd() { return HG > 1 ? 3 : (NWH == 4 ? 1 : 2); }
+
+template <int DK, int NWH, int HG, int MODE>
+__global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>())) void linear_fwd_kernel(const LinArgs a) {
+  constexpr int NW = NWH * HG;
+  constexpr bool ALIAS_OST = HG > 1;     // output staging block inside the wave's own (already consumed) V columns
   using T = __bf16;
   using E = Elem<T>;
   using x8 = typename E::x8;
@@ -74,50 +92,75 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r0 = lane & 31;
   const uint32_t lds_scal = lds0 + 2 * STAGE + wave * SCAL_BYTES;
-  const uint32_t lds_ost = lds0 + 2 * STAGE + NW * SCAL_BYTES + wave * (L * OROW);
+  const uint32_t lds_ost = lds0 + 2 * STAGE + NW * SCAL_BYTES + wave * (L * OROW);   // (unused with ALIAS_OST)
 
-  // workgroup -> (batch*head, value slice); slices of one head share id % 8 (one XCD, shared L2)
-  const int BH = a.B * a.H;
-  int bh, dvb;
-  if ((BH & 7) == 0) {
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    dvb = slot % a.dv_blocks;
-    bh = (slot / a.dv_blocks) * 8 + xcd;
-  } else {
-    dvb = blockIdx.x % a.dv_blocks;
-    bh = blockIdx.x / a.dv_blocks;
+  // workgroup -> (head group, value slice, segment); the workgroups of one head group share
+  // id % 8 (one XCD, shared L2)
+  const int n_seg = MODE == 0 ? 1 : (MODE == 1 ? a.nseg - 1 : a.nseg);
+  const int BG = a.B * a.H / HG;
+  int bg, dvb, seg;
+  {
+    int slot;
+    if ((BG & 7) == 0) {
+      const int xcd = blockIdx.x & 7;
+      slot = blockIdx.x >> 3;
+      seg = slot % n_seg;
+      slot /= n_seg;
+      dvb = slot % a.dv_blocks;
+      bg = (slot / a.dv_blocks) * 8 + xcd;
+    } else {
+      slot = blockIdx.x;
+      seg = slot % n_seg;
+      slot /= n_seg;
+      dvb = slot % a.dv_blocks;
+      bg = slot / a.dv_blocks;
+    }
   }
-  const int b = bh / a.H, h = bh % a.H;
-  const int hq = h / (a.H / a.Hq), hk = h / (a.H / a.Hk);
+  const int hl = wave / NWH;                      // head of the group this wave works for
+  const int bh0 = bg * HG, bh = bh0 + hl;
+  const int b = bh0 / a.H, h0 = bh0 % a.H;        // (HG divides H, and the heads of a group share hq and hk)
+  const int hq = h0 / (a.H / a.Hq), hk = h0 / (a.H / a.Hk);
   const int Tn = a.T;
   const char* qb = (const char*)a.q + ((int64_t)(b * a.Hq + hq) * Tn) * RBQ;
   const char* kb = (const char*)a.k + ((int64_t)(b * a.Hk + hk) * Tn) * RBQ;
-  const char* vb = (const char*)a.v + ((int64_t)bh * Tn * a.Dv + dvb * DVS) * 2;
-  T* ob = (T*)a.o + (int64_t)bh * Tn * a.Dv + dvb * DVS + 32 * wave;
+  const char* vb = (const char*)a.v + ((int64_t)bh0 * Tn * a.Dv + dvb * (32 * NWH)) * 2;
+  const int64_t v_head_bytes = (int64_t)Tn * a.Dv * 2;
+  T* ob = (T*)a.o + (int64_t)bh * Tn * a.Dv + dvb * (32 * NWH) + 32 * (wave % NWH);
   const float* ldp = a.log_decay + (int64_t)bh * Tn;
   const float* vsp = a.v_scale ? a.v_scale + (int64_t)bh * Tn : nullptr;
   const int64_t v_row_bytes = (int64_t)a.Dv * 2;
-  const int n_chunks = (Tn + L - 1) / L;
+  const int n_chunks_all = (Tn + L - 1) / L;
+  const int c_begin = MODE == 0 ? 0 : seg * a.seg_chunks;
+  const int c_end = MODE == 0 ? n_chunks_all : min(c_begin + a.seg_chunks, n_chunks_all);
+  // this wave's block of the exchanged states: [segment][wave][KB*16 registers][64 lanes]
+  float* ws_mine = nullptr;
+  if (MODE != 0)
+    ws_mine = a.ws_state + ((((int64_t)bg * a.dv_blocks + dvb) * (a.nseg - 1)) * NW + wave) * (int64_t)(KB * 16 * 64) + lane;
+  constexpr int64_t WS_SEG = (int64_t)NW * KB * 16 * 64;
 
   // ---- DMA of one chunk: each instruction moves 1 KB (1024/row_bytes tile rows); lane i fetches
   //      the 16-byte chunk that belongs at physical position i of that KB.
   auto issue_chunk = [&](int t0, int buf) {
     const uint32_t base = lds0 + buf * STAGE;
-#pragma unroll (DK <= 128 ? 16 : 1)   // (with a 256-wide key the state leaves no registers for an unrolled burst)
-    for (int it = 0; it < (2 * NIQ + NIV + NW - 1) / NW; it++) {
+    constexpr int NQK = MODE == 1 ? NIQ : 2 * NIQ;      // (the state-only pass needs no Q)
+#pragma unroll (DK <= 128 && HG == 1 ? 16 : 1)   // (unrolled burst only where the state leaves registers for it)
+    for (int it = 0; it < (NQK + NIV + NW - 1) / NW; it++) {
       const int ii = wave + NW * it;
-      if ((2 * NIQ + NIV) % NW != 0 && ii >= 2 * NIQ + NIV) break;
-      if (ii < 2 * NIQ) {
-        const int which = ii >= NIQ, i2 = which ? ii - NIQ : ii;
+      if ((NQK + NIV) % NW != 0 && ii >= NQK + NIV) break;
+      if (ii < NQK) {
+        const int which = MODE == 1 ? 1 : ii >= NIQ, i2 = (MODE != 1 && which) ? ii - NIQ : ii;
         const int row = i2 * (1024 / RBQ) + lane / CPRQ, c = lane % CPRQ;
         const int trow = min(t0 + row, Tn - 1);
         const char* src = (which ? kb : qb) + (int64_t)trow * RBQ + ((c ^ swz_tile<CPRQ>(row)) << 4);
         dma16(src, base + which * QT + i2 * 1024);
       } else {
-        const int i2 = ii - 2 * NIQ;
+        const int i2 = ii - NQK;
         const int row = i2 * (1024 / RBV) + lane / CPRV, c = lane % CPRV;
         const int trow = min(t0 + row, Tn - 1);
-        dma16(vb + (int64_t)trow * v_row_bytes + ((c ^ swz_tile<CPRV>(row)) << 4), base + 2 * QT + i2 * 1024);
+        const int lc = c ^ swz_tile<CPRV>(row);          // logical 16-byte chunk: head lc / (4 NWH), then its columns
+        const char* src = vb + (int64_t)trow * v_row_bytes + ((lc % (4 * NWH)) << 4);
+        if (HG > 1) src += (lc / (4 * NWH)) * v_head_bytes;
+        dma16(src, base + 2 * QT + i2 * 1024);
       }
     }
   };
@@ -131,18 +174,34 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
   // scalars of the chunk about to be processed (loaded one chunk ahead)
   const int ti = r0;
   float ld_next = 0.f, vs_next = 1.f;
-  if (ti < Tn) {
-    ld_next = ldp[ti];
-    if (vsp) vs_next = vsp[ti];
+  if (c_begin * L + ti < Tn) {
+    ld_next = ldp[c_begin * L + ti];
+    if (vsp) vs_next = vsp[c_begin * L + ti];
   }
-  if (n_chunks > 0) issue_chunk(0, 0);
+  if (c_begin < c_end) issue_chunk(c_begin * L, 0);
 
-  for (int c = 0; c < n_chunks; c++) {
-    const int buf = c & 1, t0 = c * L;
+  if (MODE == 2 && seg > 0) {
+    // entering state: the local end states of the earlier segments, each decayed by the segments between
+    const float* dec = a.ws_decay + (int64_t)bh * (a.nseg - 1);
+    float acc_log = 0.f;
+    for (int sp = seg - 1; sp >= 0; sp--) {
+      const float coef = fast_exp2(acc_log * kLog2e);
+      const float* src = ws_mine + sp * WS_SEG;
+#pragma unroll
+      for (int i = 0; i < KB; i++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) hst[i][j] += coef * src[(i * 16 + j) * 64];
+      acc_log += dec[sp];
+    }
+  }
+  float seg_log = 0.f;   // MODE 1: total log decay of the segment
+
+  for (int c = c_begin; c < c_end; c++) {
+    const int buf = (c - c_begin) & 1, t0 = c * L;
     wait_dma();
     __syncthreads();
     const float ld = ld_next, vs = vs_next;
-    if (c + 1 < n_chunks) {
+    if (c + 1 < c_end) {
       const int tn = t0 + L + ti;
       ld_next = 0.f;
       vs_next = 1.f;
@@ -194,16 +253,20 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
     const float wl = valid ? vs * fast_exp2((g_last - gi) * kLog2e) : 0.f;   // factor of row l in the state update
     const float eg = fast_exp2(gi * kLog2e) * a.q_scale;          // factor of token i in the inter-chunk term
     const float decay_all = fast_exp2(g_last * kLog2e);
+    if (MODE == 1) seg_log += g_last;
     if (g == 0) {
       lds_write<float>(lds_scal + ti * 4, gi);
       lds_write<float>(lds_scal + (L + ti) * 4, pvq);
       lds_write<float>(lds_scal + (2 * L + ti) * 4, wl);
     }
     // ---- A^T = K Q^T (lane: token i = r, rows j = 8(jj/4) + 4g + jj%4)
-    f32x16 sacc, sacc2;   // two chains, so that consecutive MFMAs do not wait for each other
+    // two accumulation chains, so that consecutive MFMAs do not wait for each other, where registers
+    // allow (with three waves per SIMD the other waves fill those gaps)
+    constexpr bool TWO_CHAINS = HG == 1;
+    f32x16 sacc, sacc2;
 #pragma unroll
     for (int j = 0; j < 16; j++) { sacc[j] = 0.f; sacc2[j] = 0.f; }
-    {
+    if constexpr (MODE != 1) {
       constexpr int NS = DK / 16, AH = 2, RING = 3;
       x8 kf[RING], qf[RING];
       auto request = [&](int ks) {
@@ -217,13 +280,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
       for (int ks = 0; ks < NS; ks++) {
         if (ks + AH < NS) request(ks + AH);
         __builtin_amdgcn_sched_barrier(0);
-        if (ks & 1) sacc2 = E::mfma32(kf[ks % RING], qf[ks % RING], sacc2);
+        if (TWO_CHAINS && (ks & 1)) sacc2 = E::mfma32(kf[ks % RING], qf[ks % RING], sacc2);
         else sacc = E::mfma32(kf[ks % RING], qf[ks % RING], sacc);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
     // rows held by this lane in a 32 x 32 accumulator block: 8q4 + 4g + {0..3}
     float gj[16], pj[16];
+    if constexpr (MODE != 1) {
 #pragma unroll
     for (int q4 = 0; q4 < 4; q4++) {
       const f32x4 tg = lds_read<f32x4>(lds_scal + (8 * q4 + 4 * g) * 4);
@@ -234,15 +298,18 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
         pj[4 * q4 + i] = tp[i];
       }
     }
+    }
     // ---- P^T: decay, per-token value scale, causal mask (exact zeros above the diagonal)
     x8 pf[2];
+    if constexpr (MODE != 1) {
 #pragma unroll
     for (int jj = 0; jj < 16; jj++) {
       const int j = 8 * (jj >> 2) + 4 * g + (jj & 3);
       const float e = fast_exp2(fminf(gi - gj[jj], 0.f) * kLog2e);
-      float p = (sacc[jj] + sacc2[jj]) * e * pj[jj];
+      float p = (TWO_CHAINS ? sacc[jj] + sacc2[jj] : sacc[jj]) * e * pj[jj];
       asm volatile("" : "+v"(p));   // computed for every lane, then selected: no branch per element
       pf[jj >> 3][jj & 7] = (T)(j <= ti ? p : 0.f);
+    }
     }
 
     // ---- V^T fragments (rows = this wave's 32 value columns; k-slot i of slice s is token
@@ -260,8 +327,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
     f32x16 o_inter, o_inter2, o_intra;
 #pragma unroll
     for (int j = 0; j < 16; j++) { o_inter[j] = 0.f; o_inter2[j] = 0.f; o_intra[j] = 0.f; }
-    o_intra = E::mfma32(vf[0], pf[0], o_intra);
-    o_intra = E::mfma32(vf[1], pf[1], o_intra);
+    if constexpr (MODE != 1) {
+      o_intra = E::mfma32(vf[0], pf[0], o_intra);
+      o_intra = E::mfma32(vf[1], pf[1], o_intra);
+    }
     // value-scaled V^T for the state update (k-slot i of slice s is token 16s + 8(i/4) + 4g + i%4 -> wj[8s + i])
     x8 vsf[2];
 #pragma unroll
@@ -284,26 +353,34 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
 #pragma unroll
         for (int s = 0; s < 2; s++) {
           const int lcq = 4 * bb + 2 * s;
-          qlo[bb % RING][s] = lds_read<x4>(qbase + qp_row + (uint32_t)((lcq ^ qp_swz) << 4));
-          qhi[bb % RING][s] = lds_read<x4>(qbase + qp_row + (uint32_t)(((lcq + 1) ^ qp_swz) << 4));
+          if constexpr (MODE != 1) {
+            qlo[bb % RING][s] = lds_read<x4>(qbase + qp_row + (uint32_t)((lcq ^ qp_swz) << 4));
+            qhi[bb % RING][s] = lds_read<x4>(qbase + qp_row + (uint32_t)(((lcq + 1) ^ qp_swz) << 4));
+          }
           const int cx = s ? Q_X16 : 0;
           klo[bb % RING][s] = lds_read_tr4<T>(kbase + kt_row + 16 * s * RBQ + (uint32_t)((kt_c0 ^ (4 * bb) ^ cx) << 4));
           khi[bb % RING][s] = lds_read_tr4<T>(kbase + kt_row + (16 * s + 8) * RBQ + (uint32_t)((kt_c0 ^ (4 * bb) ^ cx ^ Q_X8) << 4));
         }
       };
-      request(0);
+      // operands are requested one block ahead, except where three waves per SIMD hide the LDS latency
+      // and the registers are needed elsewhere
+      constexpr bool AHEAD = HG == 1;
+      if (AHEAD) request(0);
 #pragma unroll
       for (int bb = 0; bb < KB; bb++) {
-        if (bb + 1 < KB) request(bb + 1);
+        if (!AHEAD) request(bb);
+        else if (bb + 1 < KB) request(bb + 1);
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (MODE != 1) {
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-          x8 hf;
+          for (int s = 0; s < 2; s++) {
+            x8 hf;
 #pragma unroll
-          for (int i = 0; i < 8; i++) hf[i] = (T)hst[bb][8 * s + i];
-          x8 qf = __builtin_shufflevector(qlo[bb % RING][s], qhi[bb % RING][s], 0, 1, 2, 3, 4, 5, 6, 7);
-          if (DK < 256 && s) o_inter2 = E::mfma32(hf, qf, o_inter2);   // (a second chain where registers allow)
-          else o_inter = E::mfma32(hf, qf, o_inter);
+            for (int i = 0; i < 8; i++) hf[i] = (T)hst[bb][8 * s + i];
+            x8 qf = __builtin_shufflevector(qlo[bb % RING][s], qhi[bb % RING][s], 0, 1, 2, 3, 4, 5, 6, 7);
+            if (DK < 256 && HG == 1 && s) o_inter2 = E::mfma32(hf, qf, o_inter2);   // (a second chain where registers allow)
+            else o_inter = E::mfma32(hf, qf, o_inter);
+          }
         }
 #pragma unroll
         for (int j = 0; j < 16; j++) hst[bb][j] *= decay_all;
@@ -316,52 +393,134 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 1 : 2) void linear_fwd_kernel(co
       }
     }
 
-    // ---- write this wave's [32 tokens x 32 columns] block: stage (wave private), then 16-byte row pieces
+    // ---- write this wave's [32 tokens x 32 columns] block: stage (wave private), then 16-byte row pieces.
+    //      With ALIAS_OST the staging block is the wave's own 4 chunks per row of the V tile just consumed
+    //      (only this wave reads them, and the next DMA into this buffer is issued behind the next barrier).
+    if constexpr (MODE != 1) {
+      const int sw_r = swz_tile<CPRV>(r);
 #pragma unroll
-    for (int q4 = 0; q4 < 4; q4++) {
-      x4 w;
+      for (int q4 = 0; q4 < 4; q4++) {
+        x4 w;
 #pragma unroll
-      for (int i = 0; i < 4; i++) w[i] = (T)((o_inter[4 * q4 + i] + o_inter2[4 * q4 + i]) * eg + o_intra[4 * q4 + i]);
-      lds_write<x4>(lds_ost + r * OROW + (8 * q4 + 4 * g) * 2, w);
+        for (int i = 0; i < 4; i++)
+          w[i] = (T)((DK < 256 && HG == 1 ? o_inter[4 * q4 + i] + o_inter2[4 * q4 + i] : o_inter[4 * q4 + i]) * eg + o_intra[4 * q4 + i]);
+        if (ALIAS_OST) lds_write<x4>(vbase + r * RBV + (uint32_t)(((4 * wave + q4) ^ sw_r) << 4) + g * 8, w);
+        else lds_write<x4>(lds_ost + r * OROW + (8 * q4 + 4 * g) * 2, w);
+      }
+#pragma unroll
+      for (int it = 0; it < 2; it++) {
+        const int ci = ln + 64 * it, row = ci >> 2, cc = ci & 3;
+        const u32x4 w = ALIAS_OST ? lds_read<u32x4>(vbase + row * RBV + (uint32_t)(((4 * wave + cc) ^ swz_tile<CPRV>(row)) << 4))
+                                  : lds_read<u32x4>(lds_ost + row * OROW + cc * 16);
+        if (t0 + row < Tn) *(u32x4*)(ob + (int64_t)(t0 + row) * a.Dv + cc * 8) = w;
+      }
     }
+  }
+  if (MODE == 1) {
+    // the state this segment ends in when entered with zeros, and its total log decay
+    float* dst = ws_mine + seg * WS_SEG;
 #pragma unroll
-    for (int it = 0; it < 2; it++) {
-      const int ci = lane + 64 * it, row = ci >> 2, cc = ci & 3;
-      const u32x4 w = lds_read<u32x4>(lds_ost + row * OROW + cc * 16);
-      if (t0 + row < Tn) *(u32x4*)(ob + (int64_t)(t0 + row) * a.Dv + cc * 8) = w;
-    }
+    for (int i = 0; i < KB; i++)
+#pragma unroll
+      for (int j = 0; j < 16; j++) dst[(i * 16 + j) * 64] = hst[i][j];
+    if (dvb == 0 && wave % NWH == 0 && lane == 0) a.ws_decay[(int64_t)bh * (a.nseg - 1) + seg] = seg_log;
   }
 }
 
-template <int DK, int NW>
-static int launch(const LinArgs& a, hipStream_t stream) {
-  constexpr int DVS = 32 * NW;
-  constexpr size_t stage = (size_t)L * (4 * DK + 2 * DVS);
-  constexpr size_t lds = 2 * stage + NW * (3 * L * 4) + NW * (L * 80);
-  auto kern = linear_fwd_kernel<DK, NW>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
-    attr_set = true;
-  }
-  LinArgs args = a;
-  args.dv_blocks = a.Dv / DVS;
-  const unsigned grid = (unsigned)(a.B * a.H * args.dv_blocks);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, args);
-  return hipGetLastError() == hipSuccess ? 0 : -1;
-}
+namespace {
+// Resident workgroups per CU and the CU count, asked of the runtime once per configuration.
+template <int DK, int NWH, int HG>
+struct Config {
+  static constexpr int NW = NWH * HG;
+  static constexpr size_t stage = (size_t)L * (4 * DK + 2 * 32 * NW);
+  static constexpr size_t lds = 2 * stage + NW * (3 * L * 4) + (HG > 1 ? 0 : NW * (L * 80));
+  static constexpr int64_t ws_wave_floats = (int64_t)(DK / 32) * 16 * 64;
 
-// returns 0 ok, -1 launch failure, -2 unsupported
-int linear_fwd_dispatch(const LinArgs& a, int dk, hipStream_t stream) {
+  static bool prepare(int& resident, int& cus) {
+    static int s_resident = -1, s_cus = 0;
+    if (s_resident < 0) {
+      const void* kerns[3] = {(const void*)linear_fwd_kernel<DK, NWH, HG, 0>, (const void*)linear_fwd_kernel<DK, NWH, HG, 1>,
+                              (const void*)linear_fwd_kernel<DK, NWH, HG, 2>};
+      for (const void* kp : kerns)
+        if (hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return false;
+      int dev = 0, n = 0, r = 0;
+      if (hipGetDevice(&dev) != hipSuccess) return false;
+      if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return false;
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, linear_fwd_kernel<DK, NWH, HG, 2>, 64 * NW, lds) != hipSuccess) return false;
+      s_cus = n;
+      s_resident = r < 1 ? 1 : r;
+    }
+    resident = s_resident;
+    cus = s_cus;
+    return true;
+  }
+
+  // Number of segments and chunks per segment for this problem.  want: 0 = choose (as many segments as
+  // keep every CU's resident workgroup slots busy, each at least 4 chunks long), n >= 1 = at most n.
+  static void plan(const LinArgs& a, int want, int resident, int cus, int& nseg, int& seg_chunks) {
+    const int n_chunks = (a.T + L - 1) / L;
+    const int64_t groups = (int64_t)a.B * a.H / HG * (a.Dv / (32 * NWH));
+    int n;
+    if (want >= 1) n = want;
+    else {
+      n = (int)((int64_t)resident * cus / groups);
+      if (n > 8) n = 8;
+      if (n > n_chunks / 4) n = n_chunks / 4;
+    }
+    if (n > n_chunks) n = n_chunks;
+    if (n < 1) n = 1;
+    seg_chunks = (n_chunks + n - 1) / n;
+    nseg = (n_chunks + seg_chunks - 1) / seg_chunks;
+  }
+
+  static size_t ws_bytes(const LinArgs& a, int nseg) {
+    if (nseg <= 1) return 0;
+    const int64_t groups = (int64_t)a.B * a.H / HG * (a.Dv / (32 * NWH));
+    return (size_t)((groups * (nseg - 1) * NW * ws_wave_floats + (int64_t)a.B * a.H * (nseg - 1)) * 4);
+  }
+
+  // query != null: only report the workspace the launch would use
+  static int run(const LinArgs& a, int want_segments, void* ws, size_t ws_size, hipStream_t stream, size_t* query) {
+    int resident = 1, cus = 256;
+    if (!prepare(resident, cus)) {
+      if (query) { *query = 0; return 0; }
+      return -1;
+    }
+    LinArgs args = a;
+    args.dv_blocks = a.Dv / (32 * NWH);
+    plan(a, want_segments, resident, cus, args.nseg, args.seg_chunks);
+    if (query) { *query = ws_bytes(a, args.nseg); return 0; }
+    if (args.nseg > 1 && (!ws || ws_size < ws_bytes(a, args.nseg) || ((uintptr_t)ws & 3) != 0)) args.nseg = 1;   // no workspace: single pass
+    const unsigned groups = (unsigned)((int64_t)a.B * a.H / HG * args.dv_blocks);
+    if (args.nseg <= 1) {
+      args.nseg = 1;
+      hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 0>), dim3(groups), dim3(64 * NW), lds, stream, args);
+    } else {
+      args.ws_state = (float*)ws;
+      args.ws_decay = args.ws_state + (int64_t)groups * (args.nseg - 1) * NW * ws_wave_floats;
+      hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 1>), dim3(groups * (args.nseg - 1)), dim3(64 * NW), lds, stream, args);
+      hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 2>), dim3(groups * args.nseg), dim3(64 * NW), lds, stream, args);
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+  }
+};
+}  // namespace
+
+// returns 0 ok, -1 launch failure, -2 unsupported.  With query != null nothing is launched and *query
+// receives the workspace size the same call would use.
+int linear_fwd_dispatch(const LinArgs& a, int dk, int want_segments, void* ws, size_t ws_size, hipStream_t stream, size_t* query) {
   const int dv = a.Dv;
+  // two heads per workgroup when they share their q and k heads (Mamba2: all heads of a batch entry do)
+  const bool pairable = a.H % 2 == 0 && (a.H / a.Hq) % 2 == 0 && (a.H / a.Hk) % 2 == 0;
   if (dk == 256) {
-    if (dv % 256 == 0) return launch<256, 8>(a, stream);
-    if (dv % 128 == 0) return launch<256, 4>(a, stream);
-    if (dv % 64 == 0) return launch<256, 2>(a, stream);
+    if (dv % 256 == 0) return Config<256, 8, 1>::run(a, want_segments, ws, ws_size, stream, query);
+    if (dv % 128 == 0) return Config<256, 4, 1>::run(a, want_segments, ws, ws_size, stream, query);
+    if (dv % 64 == 0) return Config<256, 2, 1>::run(a, want_segments, ws, ws_size, stream, query);
   } else if (dk == 128) {
-    if (dv % 256 == 0) return launch<128, 8>(a, stream);
-    if (dv % 128 == 0) return launch<128, 4>(a, stream);
-    if (dv % 64 == 0) return launch<128, 2>(a, stream);
+    if (dv % 256 == 0) return Config<128, 8, 1>::run(a, want_segments, ws, ws_size, stream, query);
+    if (dv % 128 == 0) return Config<128, 4, 1>::run(a, want_segments, ws, ws_size, stream, query);
+    if (dv % 64 == 0 && pairable) return Config<128, 2, 2>::run(a, want_segments, ws, ws_size, stream, query);
+    if (dv % 64 == 0) return Config<128, 2, 1>::run(a, want_segments, ws, ws_size, stream, query);
   }
   return -2;
 }

@@ -56,7 +56,7 @@ class LinearParams(Structure):
         ("seqlen", c_int32), ("dim_k", c_int32), ("dim_v", c_int32), ("chunk", c_int32),
         ("q", c_void_p), ("k", c_void_p), ("v", c_void_p), ("o", c_void_p),
         ("log_decay", c_void_p), ("v_scale", c_void_p),
-        ("q_scale", c_float),
+        ("q_scale", c_float), ("segments", c_int32),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
     ]
 
@@ -206,12 +206,16 @@ def mla_workspace_bytes(B, Hq, Skv, D=512, Dpe=64, num_split=0) -> int:
     return load_library().ma_mla_workspace_bytes(ctypes.byref(p))
 
 
-def linear_fwd(q, k, v, log_decay, *, q_scale: float = 1.0, v_scale=None, chunk=None, out=None):
+def linear_fwd(q, k, v, log_decay, *, q_scale: float = 1.0, v_scale=None, chunk=None, out=None, segments: int = 0,
+               workspace=None):
     """Chunked linear attention forward on BHSD tensors: q [B,Hq,T,Dk], k [B,Hk,T,Dk],
     v [B,H,T,Dv] (bf16, contiguous), log_decay fp32 [B,H,T], optional per-token value
     scale [B,H,T].  ``chunk`` is accepted for API compatibility; the result does not
-    depend on it and the kernel uses its own chunking."""
-    _require_gpu(q, k, v, log_decay, v_scale, out)
+    depend on it and the kernel uses its own chunking.  ``segments``: 0 lets the library
+    decide whether to cut the sequence into segments that run side by side (it does when
+    batch x heads is small), 1 forces the single pass, n allows up to n segments; the
+    workspace that needs is allocated here unless one is passed."""
+    _require_gpu(q, k, v, log_decay, v_scale, out, workspace)
     B, H, T, Dv = v.shape
     Hq, Hk, Dk = q.shape[1], k.shape[1], q.shape[-1]
     assert q.shape == (B, Hq, T, Dk) and k.shape == (B, Hk, T, Dk), "q/k/v shapes disagree"
@@ -231,5 +235,19 @@ def linear_fwd(q, k, v, log_decay, *, q_scale: float = 1.0, v_scale=None, chunk=
     p.log_decay = log_decay.data_ptr()
     p.v_scale = v_scale.data_ptr() if v_scale is not None else None
     p.q_scale = float(q_scale)
-    _check(load_library().ma_linear_fwd(ctypes.byref(p), _stream()))
+    p.segments = int(segments)
+    lib = load_library()
+    need = lib.ma_linear_workspace_bytes(ctypes.byref(p))
+    if need > 0:
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=v.device)
+        assert workspace.numel() * workspace.element_size() >= need
+        p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    _check(lib.ma_linear_fwd(ctypes.byref(p), _stream()))
     return out
+
+
+def linear_workspace_bytes(B, H, Hq, Hk, T, Dk, Dv, segments: int = 0) -> int:
+    p = LinearParams()
+    p.dtype, p.batch, p.heads, p.heads_q, p.heads_k, p.seqlen, p.dim_k, p.dim_v, p.segments = MA_BF16, B, H, Hq, Hk, T, Dk, Dv, segments
+    return load_library().ma_linear_workspace_bytes(ctypes.byref(p))

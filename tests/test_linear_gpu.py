@@ -123,6 +123,80 @@ def test_full_size_properties():
     oracle.assert_close(y[3:4, 40:41].float().cpu(), ref, rtol=RTOL, atol=ATOL)
 
 
+def _mamba2_case(B, H, T, seed):
+    P, N = 64, 128
+    Cm, Bm, x, dt, A = inputs.mamba2_inputs(B, H, T, P, N, seed=seed)
+    chunk = 64 if T % 64 == 0 else T
+    ref = oracle.ssd_chunk_scan_combined(x.permute(0, 2, 1, 3), dt.permute(0, 2, 1), A[0], Bm.permute(0, 2, 1, 3),
+                                         Cm.permute(0, 2, 1, 3), chunk_size=chunk).permute(0, 2, 1, 3)
+    return (Cm.cuda(), Bm.cuda(), x.cuda(), (dt * A.view(1, H, 1)).cuda()), dict(v_scale=dt.cuda()), ref
+
+
+def _retnet_case(B, H, T, Dk, Dv, seed):
+    q, k, v, decay = inputs.retnet_inputs(B, H, T, Dk, Dv, seed=seed)
+    q, k = (q.float() * math.sqrt(Dk)).bfloat16(), (k.float() * math.sqrt(Dk) * 0.1).bfloat16()
+    return (q.cuda(), k.cuda(), v.cuda(), torch.log(decay).cuda()), dict(q_scale=Dk ** -0.5), oracle.retnet_quadratic(q, k, v)
+
+
+@pytest.mark.parametrize("case", ["mamba2_pairs", "mamba2_odd_heads", "mamba2_ragged", "retnet_256_512", "retnet_128_128_ragged"])
+@pytest.mark.parametrize("segments", [2, 3, 7])
+def test_sequence_segments(case, segments):
+    """The sequence cut into segments that run side by side (local end states exchanged through the
+    workspace) gives the single pass's result up to the rounding of the entering state, and the oracle's."""
+    hb = _hb()
+    args, kw, ref = {
+        "mamba2_pairs": lambda: _mamba2_case(2, 4, 512, 11),          # two heads per workgroup
+        "mamba2_odd_heads": lambda: _mamba2_case(1, 3, 256, 12),      # heads cannot be paired
+        "mamba2_ragged": lambda: _mamba2_case(1, 2, 300, 13),         # last chunk partial, last segment short
+        "retnet_256_512": lambda: _retnet_case(1, 2, 512, 256, 512, 14),
+        "retnet_128_128_ragged": lambda: _retnet_case(2, 3, 200, 128, 128, 15),
+    }[case]()
+    print(f"segments {case} n={segments}", flush=True)
+    single = hb.linear_fwd(*args, segments=1, **kw)
+    cut = hb.linear_fwd(*args, segments=segments, **kw)
+    torch.cuda.synchronize()
+    oracle.assert_close(single.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    oracle.assert_close(cut.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(cut.float(), single.float(), rtol=1e-2, atol=1e-2)
+    n_first = (((args[2].shape[2] + 31) // 32 + segments - 1) // segments) * 32
+    assert torch.equal(cut[:, :, :n_first], single[:, :, :n_first])            # the first segment is the single pass's prefix
+
+
+def test_segments_need_a_workspace_else_single_pass():
+    """Through the C ABI: segments asked for but no workspace passed -> the single pass runs (bit-identical result);
+    ma_linear_workspace_bytes grows with the number of segments and is 0 for one."""
+    import ctypes
+    hb = _hb()
+    (q, k, v, ld), kw, _ = _mamba2_case(1, 4, 512, 21)
+    single = hb.linear_fwd(q, k, v, ld, segments=1, **kw)
+    out = torch.empty_like(single)
+    p = hb.LinearParams()
+    p.dtype, p.batch, p.heads, p.heads_q, p.heads_k, p.seqlen, p.dim_k, p.dim_v = hb.MA_BF16, 1, 4, 1, 1, 512, 128, 64
+    p.q, p.k, p.v, p.o, p.log_decay, p.v_scale = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), ld.data_ptr(), kw["v_scale"].data_ptr()
+    p.q_scale, p.segments = 1.0, 4
+    lib = hb.load_library()
+    assert lib.ma_linear_fwd(ctypes.byref(p), torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, single)
+    assert hb.linear_workspace_bytes(1, 4, 1, 1, 512, 128, 64, segments=1) == 0
+    b2, b4 = (hb.linear_workspace_bytes(1, 4, 1, 1, 512, 128, 64, segments=n) for n in (2, 4))
+    assert 0 < b2 < b4
+    # per segment but the last: [head pairs 2][waves 4][128/32 * 16 registers][64 lanes] fp32 states + one log decay per head
+    assert b2 == (2 * 4 * 4 * 16 * 64 + 4) * 4 and b4 == 3 * b2
+
+
+def test_full_size_mamba2_auto_segments():
+    """B=8 H=64 S=2048 P=64 N=128: the library's own choice of segments against the single pass."""
+    hb = _hb()
+    Cm, Bm, x, dt, A = (t.cuda() for t in inputs.mamba2_inputs(8, 64, 2048, 64, 128, seed=0))
+    ldm = dt * A.view(1, 64, 1)
+    assert hb.linear_workspace_bytes(8, 64, 1, 1, 2048, 128, 64) > 0
+    y = hb.linear_fwd(Cm, Bm, x, ldm, v_scale=dt)
+    y1 = hb.linear_fwd(Cm, Bm, x, ldm, v_scale=dt, segments=1)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(y.float(), y1.float(), rtol=1e-2, atol=1e-2)
+
+
 def test_linear_rejects_bad_arguments():
     hb = _hb()
     q = torch.zeros(1, 2, 64, 96, device="cuda", dtype=torch.bfloat16)
