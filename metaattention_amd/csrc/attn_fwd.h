@@ -14,7 +14,7 @@ struct AttnArgs {
   float scale, bias;
 };
 
-int retention_fwd_dispatch(const AttnArgs& a, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);
+int attn_wide_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);
 int attn_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);
 
 }  // namespace ma

@@ -1,0 +1,335 @@
+// Parallel attention forward for every head size the fast kernel (attn_fwd.hip, 128/128) does not
+// take, and for the normalised retention family (wide heads: Dqk 256, Dv 512), for gfx950.
+//
+// Same operator as attn_fwd.hip: attention_engine/core/template/tl_template/attn/attn_tl.py:92-190
+// behind _attention.forward (:654-667), with the row functions of examples/mha.py (softmax),
+// examples/sigmoid_attn.py, examples/reluattn.py and examples/retention_parallel.py:
+//   softmax    p = exp(x - m),  o = sum p v / sum p,  lse = m + log sum p      (x = s * scale + bias)
+//   sigmoid    p = 1 / (1 + exp(-x)),  masked p = 0
+//   relu       p = max(x, 0),          masked p = 0
+//   retention  qkm = s * scale * M,  r = max(sum_j |qkm|, 1),  o = (qkm / r) v, M a caller-supplied
+//              [1|B, H, Sq, Skv] multiplier (the decay mask).  As in the reference (mask_value "0") no
+//              element-wise causal mask is applied in forward: with the causal structural mask only kv
+//              tiles above the workgroup's diagonal are skipped and the zeros come from M itself.
+// The head sizes of the reference's own test list are covered (testing/test.py:54-63: 128/256 softmax,
+// 64/64 relu, 256/512 retention) next to 256/256 and, without softmax, 256/512.
+//
+// Structure.  One workgroup of 4 waves owns 128 query rows (32 per wave, Q fragments in registers)
+// and walks the kv sequence in tiles of 32 rows; K and V tiles arrive by direct-to-LDS DMA, double
+// buffered, one barrier per tile.  Scores are computed transposed (S^T = K Q^T) as in attn_fwd.hip, so
+// a lane owns one query row, row statistics stay in the lane pair (l, l ^ 32) and P^T is the B operand
+// of O^T += V^T P^T without a shuffle.  With Dv = 512 the fp32 accumulator takes 256 registers per lane
+// and a wave runs alone on its SIMD.
+//   * softmax rescales the accumulator only on tiles where some row's maximum grew;
+//   * the retention row function is linear up to its final clamp, so the accumulator is kept
+//     un-normalised (O = sum_j P_j V_j, r = sum_j |P_j| in fp32) and divided by max(r, 1) once at the
+//     end; the online form of the reference rescales every tile and gives the same value up to rounding.
+#include "attn_fwd.h"
+
+namespace ma {
+
+namespace {
+enum { WF_SOFTMAX = 0, WF_SIGMOID = 1, WF_RELU = 2, WF_RETENTION = 3 };   // = MA_ATTN_* of the C interface
+}
+
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
+__global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_kernel(const AttnArgs a) {
+  using E = Elem<T>;
+  using x8 = typename E::x8;
+  using x4 = typename E::x4;
+  constexpr int BM = 128, BN = 32;
+  constexpr int KS = DQK / 16, DB = DV / 32;
+  constexpr int KROW = DQK * 2, VROW = DV * 2;
+  constexpr int CPRK = DQK / 8, CPRV = DV / 8;
+  constexpr int KTILE = BN * KROW, VTILE = BN * VROW, STAGE = KTILE + VTILE;
+  constexpr int NIK = KTILE / 1024, NIV = VTILE / 1024;
+  static_assert(CPRK >= 8 && CPRV >= 8 && DQK % 16 == 0 && DV % 64 == 0, "head size");
+
+  extern __shared__ __align__(16) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, g = lane >> 5;
+
+  const int nmb = a.num_m_blocks, BH = a.B * a.H;
+  int bh, mb;
+  if ((BH & 7) == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    bh = (slot / nmb) * 8 + xcd;
+    mb = slot % nmb;
+  } else {
+    bh = blockIdx.x / nmb;
+    mb = blockIdx.x % nmb;
+  }
+  if (CAUSAL) mb = nmb - 1 - mb;
+  const int b = bh / a.H, h = bh % a.H;
+  const int m_wave = mb * BM + wave * 32, m_lane = m_wave + r;
+  const int m_ld = min(m_lane, a.Sq - 1);
+
+  x8 qf[KS];
+  {
+    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)m_ld * a.qss + (int64_t)h * a.qsh + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 16 * ks);
+  }
+  const char* kb = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)h * a.ksh);
+  const char* vb = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)h * a.vsh);
+  const int64_t k_row_bytes = a.kss * 2, v_row_bytes = a.vss * 2;
+  const T* mrow = nullptr;
+  if constexpr (FAMILY == WF_RETENTION) mrow = (const T*)a.smask + (int64_t)b * a.msb + (int64_t)h * a.msh + (int64_t)m_ld * a.msq;
+
+  int n_tiles = (a.Skv + BN - 1) / BN;
+  if (CAUSAL) n_tiles = min(n_tiles, (mb * BM + BM + BN - 1) / BN);
+
+  // DMA of one tile: each instruction moves 1 KB (1024 / row bytes tile rows); lane i fetches the
+  // 16-byte chunk that belongs at physical position i of that KB.  Rows beyond the sequence are clamped
+  // to its last row (their scores are masked, or multiplied by a zero of M).
+  auto issue_tile = [&](int n0, int buf) {
+    const uint32_t base = lds0 + buf * STAGE;
+    for (int ii = wave; ii < NIK + NIV; ii += 4) {
+      if (ii < NIK) {
+        const int row = ii * (1024 / KROW) + lane / CPRK, c = lane % CPRK;
+        const int nrow = min(n0 + row, a.Skv - 1);
+        dma16(kb + nrow * k_row_bytes + ((c ^ swz_tile<CPRK>(row)) << 4), base + ii * 1024);
+      } else {
+        const int i2 = ii - NIK;
+        const int row = i2 * (1024 / VROW) + lane / CPRV, c = lane % CPRV;
+        const int nrow = min(n0 + row, a.Skv - 1);
+        dma16(vb + nrow * v_row_bytes + ((c ^ swz_tile<CPRV>(row)) << 4), base + KTILE + i2 * 1024);
+      }
+    }
+  };
+  // multiplier values of this lane's score elements: row m_lane, columns n0 + 8q4 + 4g + {0..3}
+  auto load_mask = [&](int n0, x4 (&mk)[4]) {
+#pragma unroll
+    for (int q4 = 0; q4 < 4; q4++) {
+      const int n = n0 + 8 * q4 + 4 * g;
+      if (n + 3 < a.Skv) {
+        mk[q4] = *(const x4*)(mrow + n);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) mk[q4][i] = n + i < a.Skv ? mrow[n + i] : (T)0.f;
+      }
+    }
+  };
+
+  const uint32_t k_row_off = r * KROW;
+  const int k_c0 = g ^ swz_tile<CPRK>(r);
+  const int jr = (lane & 15) >> 2;
+  const int lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
+  const uint32_t v_row_off = (4 * g + jr) * VROW + (lane & 1) * 8;
+  const int v_c0 = lc ^ swz_tile<CPRV>(4 * g + jr);
+
+  f32x16 o[DB];
+#pragma unroll
+  for (int i = 0; i < DB; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) o[i][j] = 0.f;
+  float r_part = 0.f;      // this lane's share of the row sum (sum p, or sum |p| for retention)
+  float row_max = -1e30f;  // softmax: running maximum of x * log2(e), the same in both lanes of a row
+  const float bias = a.bias + (a.bias_ptr ? *a.bias_ptr : 0.f);
+  const float c_scale = a.scale * kLog2e, c_bias = bias * kLog2e;
+
+  x4 mk_next[4];
+  if (n_tiles > 0) {
+    issue_tile(0, 0);
+    if constexpr (FAMILY == WF_RETENTION) load_mask(0, mk_next);
+  }
+
+  for (int jt = 0; jt < n_tiles; jt++) {
+    const int buf = jt & 1, n0 = jt * BN;
+    wait_dma();
+    __syncthreads();
+    x4 mk[4];
+    if constexpr (FAMILY == WF_RETENTION) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) mk[q4] = mk_next[q4];
+    }
+    if (jt + 1 < n_tiles) {
+      if constexpr (FAMILY == WF_RETENTION) load_mask(n0 + BN, mk_next);
+      issue_tile(n0 + BN, buf ^ 1);
+    }
+    const uint32_t kbase = lds0 + buf * STAGE, vbase = kbase + KTILE;
+
+    // ---- S^T = K Q^T
+    f32x16 s;
+#pragma unroll
+    for (int j = 0; j < 16; j++) s[j] = 0.f;
+    {
+      constexpr int AH = 2, RING = 3;
+      x8 kf[RING];
+#pragma unroll
+      for (int ks = 0; ks < AH; ks++) kf[ks] = lds_read<x8>(kbase + k_row_off + (uint32_t)((k_c0 ^ (2 * ks)) << 4));
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        if (ks + AH < KS) kf[(ks + AH) % RING] = lds_read<x8>(kbase + k_row_off + (uint32_t)((k_c0 ^ (2 * (ks + AH))) << 4));
+        __builtin_amdgcn_sched_barrier(0);
+        s = E::mfma32(kf[ks % RING], qf[ks], s);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // ---- P^T from S^T (lane: row m_lane, kv rows n0 + 8(jj/4) + 4g + jj%4)
+    x8 pf[2];
+    if constexpr (FAMILY == WF_RETENTION) {
+#pragma unroll
+      for (int jj = 0; jj < 16; jj++) {
+        const float p = s[jj] * a.scale * (float)mk[jj >> 2][jj & 3];
+        r_part += fabsf(p);
+        pf[jj >> 3][jj & 7] = (T)p;
+      }
+    } else {
+      // element-wise mask only on tiles that reach past the diagonal or the end of the sequence
+      const bool edge = (CAUSAL && n0 + BN - 1 > m_wave) || n0 + BN > a.Skv;
+      if (edge) {
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++) {
+          const int n = n0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
+          if ((CAUSAL && n > m_lane) || n >= a.Skv) s[jj] = -INFINITY;
+        }
+      }
+      if constexpr (FAMILY == WF_SOFTMAX) {
+        float mx = s[0];
+#pragma unroll
+        for (int jj = 1; jj < 16; jj++) mx = fmaxf(mx, s[jj]);
+        mx = fmaxf(mx, xhalf(mx)) * c_scale + c_bias;
+        const float m_new = fmaxf(row_max, mx);
+        if (__any(m_new > row_max)) {
+          const float corr = fast_exp2(row_max - m_new);
+          r_part *= corr;
+#pragma unroll
+          for (int i = 0; i < DB; i++)
+#pragma unroll
+            for (int j = 0; j < 16; j++) o[i][j] *= corr;
+        }
+        row_max = m_new;
+        const float sub = c_bias - row_max;
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++) {
+          const float p = fast_exp2(s[jj] * c_scale + sub);
+          r_part += p;
+          pf[jj >> 3][jj & 7] = (T)p;
+        }
+      } else if constexpr (FAMILY == WF_SIGMOID) {
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++)   // sigmoid(x) = 1 / (1 + 2^(-x log2e)); s = -inf gives exactly 0
+          pf[jj >> 3][jj & 7] = (T)fast_rcp(1.f + fast_exp2(-(s[jj] * c_scale + c_bias)));
+      } else {
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++) pf[jj >> 3][jj & 7] = (T)fmaxf(s[jj] * a.scale + bias, 0.f);
+      }
+    }
+    // ---- O^T += V^T P^T
+    {
+      constexpr int PF = DB >= 4 ? 6 : 2 * DB;
+      x4 lo[PF], hi[PF];
+      auto request = [&](int idx) {   // idx = 2 db + s
+        const int db = idx >> 1, sl = idx & 1;
+        const uint32_t rb = vbase + v_row_off + 16 * sl * VROW;
+        lo[idx % PF] = lds_read_tr4<T>(rb + (uint32_t)((v_c0 ^ (4 * db)) << 4));
+        hi[idx % PF] = lds_read_tr4<T>(rb + 8 * VROW + (uint32_t)((v_c0 ^ (4 * db) ^ 2) << 4));
+      };
+#pragma unroll
+      for (int i = 0; i < PF - 1; i++) request(i);
+#pragma unroll
+      for (int idx = 0; idx < 2 * DB; idx++) {
+        if (idx + PF - 1 < 2 * DB) request(idx + PF - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        x8 vf = __builtin_shufflevector(lo[idx % PF], hi[idx % PF], 0, 1, 2, 3, 4, 5, 6, 7);
+        o[idx >> 1] = E::mfma32(vf, pf[idx & 1], o[idx >> 1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  __syncthreads();   // every wave is done with the K/V buffers: they become output staging
+
+  float inv = 1.f;
+  float* const rs_ptr = a.row_scale && g == 0 && m_lane < a.Sq ? a.row_scale + ((int64_t)b * a.H + h) * a.Sq + m_lane : nullptr;
+  if constexpr (FAMILY == WF_RETENTION) {
+    const float r_tot = fmaxf(r_part + xhalf(r_part), 1.f);
+    inv = 1.f / r_tot;
+    if (rs_ptr) *rs_ptr = r_tot;
+  } else if constexpr (FAMILY == WF_SOFTMAX) {
+    const float tot = r_part + xhalf(r_part);
+    inv = 1.f / tot;
+    if (rs_ptr) *rs_ptr = (row_max + fast_log2(tot)) * kLn2;
+  }
+
+  // ---- O: two halves of DV/2 columns through a wave-private LDS block, coalesced 16-byte stores
+  constexpr int HALF = DV / 2, OROW = HALF * 2 + 16;
+  const uint32_t ob = lds0 + wave * 32 * OROW;
+  T* obase = (T*)a.o + (int64_t)b * a.osb + (int64_t)h * a.osh;
+#pragma unroll
+  for (int hf = 0; hf < 2; hf++) {
+#pragma unroll
+    for (int dbl = 0; dbl < DB / 2; dbl++)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (T)(o[hf * (DB / 2) + dbl][4 * q4 + i] * inv);
+        lds_write<x4>(ob + r * OROW + (32 * dbl + 8 * q4 + 4 * g) * 2, w);
+      }
+#pragma unroll
+    for (int it = 0; it < 32 * (HALF / 8) / 64; it++) {
+      const int ci = lane + 64 * it, row = ci / (HALF / 8), c = ci % (HALF / 8);
+      const u32x4 w = lds_read<u32x4>(ob + row * OROW + c * 16);
+      if (m_wave + row < a.Sq) *(u32x4*)(obase + (int64_t)(m_wave + row) * a.oss + hf * HALF + c * 8) = w;
+    }
+  }
+}
+
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
+static int launch_wide(const AttnArgs& a, hipStream_t stream) {
+  constexpr size_t tiles = 2 * (size_t)32 * (DQK + DV) * 2;
+  constexpr size_t ostage = 4 * 32 * (size_t)(DV + 16);
+  constexpr size_t lds = tiles > ostage ? tiles : ostage;
+  auto kern = attn_wide_fwd_kernel<T, DQK, DV, FAMILY, CAUSAL>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
+    attr_set = true;
+  }
+  AttnArgs args = a;
+  args.num_m_blocks = (a.Sq + 127) / 128;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(args.num_m_blocks * a.B * a.H)), dim3(256), lds, stream, args);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+template <typename T, int DQK, int DV>
+static int wide_family(const AttnArgs& a, int family, bool causal, hipStream_t stream) {
+  switch (family) {
+    case WF_SOFTMAX:
+      if constexpr (DV <= 256)
+        return causal ? launch_wide<T, DQK, DV, WF_SOFTMAX, true>(a, stream) : launch_wide<T, DQK, DV, WF_SOFTMAX, false>(a, stream);
+      return -2;
+    case WF_SIGMOID:
+      return causal ? launch_wide<T, DQK, DV, WF_SIGMOID, true>(a, stream) : launch_wide<T, DQK, DV, WF_SIGMOID, false>(a, stream);
+    case WF_RELU:
+      return causal ? launch_wide<T, DQK, DV, WF_RELU, true>(a, stream) : launch_wide<T, DQK, DV, WF_RELU, false>(a, stream);
+  }
+  return -2;
+}
+
+template <typename T>
+static int wide_dims(const AttnArgs& a, int family, bool causal, int dqk, int dv, hipStream_t stream) {
+  if (family == WF_RETENTION) {
+    if (dqk == 256 && dv == 512)
+      return causal ? launch_wide<T, 256, 512, WF_RETENTION, true>(a, stream) : launch_wide<T, 256, 512, WF_RETENTION, false>(a, stream);
+    if (dqk == 128 && dv == 128)
+      return causal ? launch_wide<T, 128, 128, WF_RETENTION, true>(a, stream) : launch_wide<T, 128, 128, WF_RETENTION, false>(a, stream);
+    return -2;
+  }
+  if (dqk == 64 && dv == 64) return wide_family<T, 64, 64>(a, family, causal, stream);
+  if (dqk == 128 && dv == 256) return wide_family<T, 128, 256>(a, family, causal, stream);
+  if (dqk == 256 && dv == 256) return wide_family<T, 256, 256>(a, family, causal, stream);
+  // (softmax is left out at 256/512: rescaling a 256-register accumulator that lives in the MFMA
+  // accumulation registers makes the compiler spill it)
+  if (dqk == 256 && dv == 512 && family != WF_SOFTMAX) return wide_family<T, 256, 512>(a, family, causal, stream);
+  return -2;
+}
+
+// returns 0 ok, -1 launch failure, -2 unsupported
+int attn_wide_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream) {
+  return is_bf16 ? wide_dims<__bf16>(a, family, causal, dqk, dv, stream) : wide_dims<_Float16>(a, family, causal, dqk, dv, stream);
+}
+
+}  // namespace ma

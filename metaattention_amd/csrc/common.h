@@ -123,6 +123,14 @@ __device__ __forceinline__ void wait_dma() { __builtin_amdgcn_s_waitcnt(0x0F70);
 // transposing read spread evenly over the banks.
 __device__ __forceinline__ int swz16(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 
+// The same for any row length: with 8 chunks per row (128-byte rows) two rows span the banks, so the
+// row's bit 1 goes to chunk bit 2 and row bits 2..3 to chunk bits 0..1.
+template <int CPR>
+__device__ __forceinline__ int swz_tile(int row) {
+  if constexpr (CPR >= 16) return swz16(row);
+  return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+}
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 

@@ -42,13 +42,6 @@ namespace ma {
 namespace {
 constexpr int L = 32;  // tokens per chunk
 
-template <int CPR>
-__device__ __forceinline__ int swz_tile(int row) {
-  if constexpr (CPR >= 16) return swz16(row);
-  // 8 chunks per row (128-byte rows): two rows span the banks; see swz16 for the goal
-  return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
-}
-
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float x) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
