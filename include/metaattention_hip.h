@@ -56,7 +56,7 @@ typedef struct ma_attn_params {
   int32_t dtype;  /* ma_dtype of q, k, v, o and of score_mask */
   int32_t mask;   /* ma_mask_kind */
   int32_t batch, heads, seqlen_q, seqlen_kv, dim_qk, dim_v;
-  /* q [B,Sq,H,Dqk], k [B,Skv,H,Dqk], v [B,Skv,H,Dv], o [B,Sq,H,Dv]; BSHD is the
+  /* q [B,Sq,H,Dqk], k [B,Skv,Hkv,Dqk], v [B,Skv,Hkv,Dv], o [B,Sq,H,Dv]; BSHD is the
    * layout the reference operator takes (attn_tl.py:69-70) but any strides
    * with a contiguous last dimension are accepted. */
   const void* q; int64_t q_stride_b, q_stride_s, q_stride_h;
@@ -72,6 +72,9 @@ typedef struct ma_attn_params {
   /* RETENTION only: elementwise score multiplier [1 or B, H, Sq, Skv] in
    * `dtype` (retention_parallel.py:96-98); stride_b may be 0 */
   const void* score_mask; int64_t sm_stride_b, sm_stride_h, sm_stride_q;
+  /* grouped-query attention (attn_gqa_tl.py:21-24, :80, :95): k and v have heads_kv heads and query
+   * head h reads kv head h / (heads / heads_kv); 0 means heads_kv = heads */
+  int32_t heads_kv;
 } ma_attn_params;
 
 /* Chunked linear / stateful attention forward.  Replaces the three launches

@@ -110,11 +110,15 @@ class AttentionEngine:
         # dispatch by shape, as attn_engine.py:227-343
         if kv_shared:
             self._init_mla()
-        elif Sq != Skv:
-            raise NotImplementedError("decode (seq_len_q != seq_len_kv) operators other than MLA are not in the kernel library")
-        elif Hq != Hkv:
-            raise NotImplementedError("grouped-query prefill is not in the kernel library")
+        elif Hq % Hkv != 0:
+            raise NotImplementedError("heads of q must be a multiple of the heads of k and v")
         else:
+            # prefill, multi-head or grouped-query (attn_engine.py:305-343: same kernel family, kv head = head // groups).
+            # Dense decode (seq_len_q != seq_len_kv, attn_engine.py:262-303; the examples pad the declared seq_len_q to
+            # a multiple of 128 and pass the real query, examples/mha_decode.py:104-108) runs through the same kernels
+            # with no structural mask; the reference's split-KV launch and its block-sparse variants have no counterpart.
+            if Sq != Skv and mask_mod is not None:
+                raise NotImplementedError("masked decode (seq_len_q != seq_len_kv with a mask_mod) is not in the kernel library")
             self._init_prefill(score_mod, mask_mod, online_func, mask_value)
 
     # ------------------------------------------------------------------ prefill

@@ -37,6 +37,8 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
   if (!(p->scale > 0.f)) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: scale must be > 0 (got %g)", (double)p->scale);
   if (p->mask == MA_MASK_CAUSAL && p->seqlen_q != p->seqlen_kv)
     return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: causal mask needs seqlen_q == seqlen_kv (%d vs %d)", p->seqlen_q, p->seqlen_kv);
+  if (p->heads_kv < 0 || (p->heads_kv > 0 && p->heads % p->heads_kv != 0))
+    return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: heads (%d) must be a multiple of heads_kv (%d)", p->heads, p->heads_kv);
   if (p->family == MA_ATTN_RETENTION) {
     if (!p->score_mask) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: RETENTION needs score_mask");
     if ((uintptr_t)p->score_mask % 8 != 0 || p->sm_stride_b % 4 != 0 || p->sm_stride_h % 4 != 0 || p->sm_stride_q % 4 != 0)
@@ -59,6 +61,7 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
   a.osb = p->o_stride_b; a.oss = p->o_stride_s; a.osh = p->o_stride_h;
   a.msb = p->sm_stride_b; a.msh = p->sm_stride_h; a.msq = p->sm_stride_q;
   a.B = p->batch; a.H = p->heads; a.Sq = p->seqlen_q; a.Skv = p->seqlen_kv;
+  a.kv_group = p->heads_kv > 0 ? p->heads / p->heads_kv : 1;
   a.scale = p->scale; a.bias = p->bias;
   const int rc = ma::attn_fwd_dispatch(a, p->family, p->mask == MA_MASK_CAUSAL, p->dtype == MA_BF16, p->dim_qk, p->dim_v,
                                        (hipStream_t)stream);

@@ -11,6 +11,7 @@ struct AttnArgs {
   const void* smask;
   int64_t qsb, qss, qsh, ksb, kss, ksh, vsb, vss, vsh, osb, oss, osh, msb, msh, msq;
   int B, H, Sq, Skv, num_m_blocks;
+  int kv_group;   // query heads per kv head (1 unless grouped-query)
   float scale, bias;
 };
 

@@ -318,8 +318,8 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
     n_sub = (a.Skv + BN - 1) / BN;
     if (CAUSAL) n_sub = min(n_sub, (mb * BM + BM) / BN);
     last_sub = CAUSAL ? min(n_sub - 1, m_wave / BN) : n_sub - 1;
-    kbase = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)h * a.ksh);
-    vbase = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)h * a.vsh);
+    kbase = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)(h / a.kv_group) * a.ksh);
+    vbase = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)(h / a.kv_group) * a.vsh);
     // K(0..5) -> slots 0..5, V(0..3) -> slots 0..3; the first step multiplies ring slot NBUF-1 with zero
     // probabilities: it gets V(0) as well, so that whatever is there belongs to this (batch, head)
     static_for<0, NBUF>([&](auto t_c) __attribute__((always_inline)) {

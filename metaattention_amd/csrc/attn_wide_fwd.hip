@@ -71,8 +71,8 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 16 * ks);
   }
-  const char* kb = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)h * a.ksh);
-  const char* vb = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)h * a.vsh);
+  const char* kb = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)(h / a.kv_group) * a.ksh);
+  const char* vb = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)(h / a.kv_group) * a.vsh);
   const int64_t k_row_bytes = a.kss * 2, v_row_bytes = a.vss * 2;
   const T* mrow = nullptr;
   if constexpr (FAMILY == WF_RETENTION) mrow = (const T*)a.smask + (int64_t)b * a.msb + (int64_t)h * a.msh + (int64_t)m_ld * a.msq;

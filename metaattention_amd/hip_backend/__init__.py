@@ -46,6 +46,7 @@ class AttnParams(Structure):
         ("row_scale", c_void_p),
         ("scale", c_float), ("bias", c_float), ("bias_ptr", c_void_p),
         ("score_mask", c_void_p), ("sm_stride_b", c_int64), ("sm_stride_h", c_int64), ("sm_stride_q", c_int64),
+        ("heads_kv", c_int32),
     ]
 
 
@@ -132,11 +133,12 @@ def _require_gpu(*tensors):
 
 def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None,
              score_mask=None, out=None, row_scale=None):
-    """Parallel attention forward on BSHD tensors.  Returns ``out`` ([B,Sq,H,Dv])."""
+    """Parallel attention forward on BSHD tensors.  Returns ``out`` ([B,Sq,H,Dv]).  k and v may
+    have fewer heads than q (grouped-query: query head h reads kv head h // (H // Hkv))."""
     _require_gpu(q, k, v, bias_tensor, score_mask, out, row_scale)
     B, Sq, H, Dqk = q.shape
-    Skv, Dv = k.shape[1], v.shape[-1]
-    assert k.shape == (B, Skv, H, Dqk) and v.shape == (B, Skv, H, Dv), "q/k/v shapes disagree"
+    Skv, Hkv, Dv = k.shape[1], k.shape[2], v.shape[-1]
+    assert k.shape == (B, Skv, Hkv, Dqk) and v.shape == (B, Skv, Hkv, Dv) and H % Hkv == 0, "q/k/v shapes disagree"
     for t in (q, k, v):
         assert t.stride(-1) == 1, "last dimension must be contiguous"
     if out is None:
@@ -144,6 +146,7 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
     p = AttnParams()
     p.family, p.dtype, p.mask = family, _dtype_code(q.dtype), MA_MASK_CAUSAL if causal else MA_MASK_NONE
     p.batch, p.heads, p.seqlen_q, p.seqlen_kv, p.dim_qk, p.dim_v = B, H, Sq, Skv, Dqk, Dv
+    p.heads_kv = Hkv
     for name, t in (("q", q), ("k", k), ("v", v), ("o", out)):
         setattr(p, name, t.data_ptr())
         setattr(p, f"{name}_stride_b", t.stride(0))

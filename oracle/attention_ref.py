@@ -27,7 +27,9 @@ def softmax_attention(q, k, v, causal: bool = True, softmax_scale: Optional[floa
     """Softmax attention forward.  Follows testing/test.py:79-104 (and the
     identical attention_engine/benchmark/bench_utils.py:1347-1372): scores
     = q.k^T, masked with -inf above the diagonal, softmax(scores * scale), times
-    v.  q [B,Sq,H,D], k [B,Skv,H,D], v [B,Skv,H,Dv] -> [B,Sq,H,Dv].
+    v.  q [B,Sq,H,D], k [B,Skv,Hkv,D], v [B,Skv,Hkv,Dv] -> [B,Sq,H,Dv]; with Hkv < H
+    query head h reads kv head h // (H // Hkv), the grouped-query layout of
+    tl_template/attn/attn_gqa_tl.py:21-24, :80, :95 (all functions of this file).
     ``lse`` ([B,H,Sq], natural log, of the scaled scores) is the final row
     scale of examples/mha.py:65-71."""
     B, Sq, H, D = q.shape
@@ -38,12 +40,12 @@ def softmax_attention(q, k, v, causal: bool = True, softmax_scale: Optional[floa
     keep = _causal_keep(Sq, Skv, q.device) if causal else None
     for b in range(B):
         for h in range(H):
-            s = q[b, :, h].to(compute_dtype) @ k[b, :, h].to(compute_dtype).T
+            s = q[b, :, h].to(compute_dtype) @ k[b, :, h // (H // k.shape[2])].to(compute_dtype).T
             if keep is not None:
                 s = s.masked_fill(~keep, float("-inf"))
             s = s * scale
             lse[b, h] = torch.logsumexp(s, dim=-1)
-            out[b, :, h] = torch.softmax(s, dim=-1) @ v[b, :, h].to(compute_dtype)
+            out[b, :, h] = torch.softmax(s, dim=-1) @ v[b, :, h // (H // v.shape[2])].to(compute_dtype)
     return (out, lse) if return_lse else out
 
 
@@ -61,12 +63,12 @@ def sigmoid_attention(q, k, v, bias, causal: bool = True, softmax_scale: float =
     keep = _causal_keep(Sq, Skv, q.device) if causal else None
     for b in range(B):
         for h in range(H):
-            s = q[b, :, h].to(compute_dtype) @ k[b, :, h].to(compute_dtype).T
+            s = q[b, :, h].to(compute_dtype) @ k[b, :, h // (H // k.shape[2])].to(compute_dtype).T
             if keep is not None:
                 s = s.masked_fill(~keep, float("-inf"))
             s = s * softmax_scale + bias
             p = (torch.tanh(s * 0.5) + 1.0) * 0.5
-            out[b, :, h] = p @ v[b, :, h].to(compute_dtype)
+            out[b, :, h] = p @ v[b, :, h // (H // v.shape[2])].to(compute_dtype)
     return out
 
 
@@ -79,8 +81,8 @@ def relu_attention(q, k, v, softmax_scale: Optional[float] = None, compute_dtype
     out = torch.empty(B, Sq, H, Dv, dtype=compute_dtype)
     for b in range(B):
         for h in range(H):
-            s = q[b, :, h].to(compute_dtype) @ k[b, :, h].to(compute_dtype).T
-            out[b, :, h] = torch.relu(s * scale) @ v[b, :, h].to(compute_dtype)
+            s = q[b, :, h].to(compute_dtype) @ k[b, :, h // (H // k.shape[2])].to(compute_dtype).T
+            out[b, :, h] = torch.relu(s * scale) @ v[b, :, h // (H // v.shape[2])].to(compute_dtype)
     return out
 
 
@@ -108,11 +110,11 @@ def retention_parallel(q, k, v, mask, compute_dtype=torch.float32, return_r: boo
     for b in range(B):
         mb = mask[b if mask.shape[0] > 1 else 0]
         for h in range(H):
-            s = q[b, :, h].to(compute_dtype) @ k[b, :, h].to(compute_dtype).T
+            s = q[b, :, h].to(compute_dtype) @ k[b, :, h // (H // k.shape[2])].to(compute_dtype).T
             s = s * mb[h].to(compute_dtype)
             r = s.abs().sum(dim=-1, keepdim=True).clamp(min=1.0)
             r_out[b, h] = r.squeeze(-1)
-            out[b, :, h] = (s / r) @ v[b, :, h].to(compute_dtype)
+            out[b, :, h] = (s / r) @ v[b, :, h // (H // v.shape[2])].to(compute_dtype)
     return (out, r_out) if return_r else out
 
 

@@ -162,3 +162,13 @@ def mamba2(B, HQ, S, D, DV, HK=None, HV=None, dtype=torch.bfloat16, chunk_size=N
     io = CustomIO({"A": (1, "heads"), "dt": ("batch", "heads", "seq_len")})
     return LinearAttentionEngine(meta, decay_mod=lambda decay, io: decay * io.input_tensors["A"],
                                  v_mod=lambda v, io: v * io.input_tensors["dt"], custom_io=io, chunk_size=chunk_size)
+
+
+def softmax_attention_decode(B, H, S, KV, D, DV, dtype=torch.float16, HKV=None):
+    """examples/mha_decode.py:14-123: no mask, declared query length padded to a multiple of 128."""
+    scale = 1 / D ** 0.5
+    HKV = HKV or H
+    meta = (meta_tensor(B, H, ((S + 127) // 128) * 128, D, dtype=dtype), meta_tensor(B, HKV, KV, D, dtype=dtype),
+            meta_tensor(B, HKV, KV, DV, dtype=dtype))
+    return AttentionEngine(meta, CustomIO({}), score_mod=lambda score, io, b, h, q_idx, kv_idx: score * scale, mask_mod=None,
+                           online_func=OnlineSoftmax())

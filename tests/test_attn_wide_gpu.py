@@ -121,6 +121,69 @@ def test_engine_relu_64():
     oracle.assert_close(o.float().cpu(), oracle.relu_attention(q, k, v), rtol=1e-1, atol=1e-1, mismatch_ratio=1e-3)
 
 
+@pytest.mark.parametrize("D,DV,H,Hkv", [(128, 128, 8, 2), (128, 128, 6, 1), (64, 64, 4, 2), (128, 256, 4, 1)])
+@pytest.mark.parametrize("family", ["softmax", "sigmoid", "relu"])
+def test_grouped_query_prefill(D, DV, H, Hkv, family):
+    """k, v with fewer heads than q (attn_gqa_tl.py:21-24): both the 128/128 kernel and the others."""
+    hb = _hb()
+    B, S = 2, 300
+    g = torch.Generator().manual_seed(D + H)
+    q = torch.randn(B, S, H, D, generator=g).bfloat16()
+    k = (0.5 * torch.randn(B, S, Hkv, D, generator=g)).bfloat16()
+    v = (0.5 * torch.randn(B, S, Hkv, DV, generator=g)).bfloat16()
+    scale = 1 / math.sqrt(D)
+    print(f"gqa {family} D{D} DV{DV} H{H} Hkv{Hkv}", flush=True)
+    if family == "softmax":
+        ref = oracle.softmax_attention(q, k, v, causal=True)
+        o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale)
+    elif family == "sigmoid":
+        ref = oracle.sigmoid_attention(q, k, v, -3.0, causal=True, softmax_scale=scale)
+        o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_SIGMOID, causal=True, scale=scale, bias=-3.0)
+    else:
+        ref = oracle.relu_attention(q, k, v)
+        o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_RELU, causal=False, scale=scale)
+    torch.cuda.synchronize()
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=5e-2 if family == "relu" else 0.0)
+    o_rep = hb.attn_fwd(q.cuda(), k.repeat_interleave(H // Hkv, dim=2).cuda(), v.repeat_interleave(H // Hkv, dim=2).cuda(),
+                        family={"softmax": hb.MA_ATTN_SOFTMAX, "sigmoid": hb.MA_ATTN_SIGMOID, "relu": hb.MA_ATTN_RELU}[family],
+                        causal=family != "relu", scale=scale, bias=-3.0 if family == "sigmoid" else 0.0)
+    torch.cuda.synchronize()
+    assert torch.equal(o, o_rep)     # the same arithmetic on the same values
+
+
+def test_engine_grouped_query_softmax():
+    """AttentionEngine with fewer kv heads (dispatch of attn_engine.py:327-343)."""
+    B, H, Hkv, S, D = 1, 8, 2, 256, 128
+    from attn_engine import AttentionEngine
+    from core import CustomIO, meta_tensor
+    meta = (meta_tensor(B, H, S, D, dtype=torch.float16), meta_tensor(B, Hkv, S, D, dtype=torch.float16), meta_tensor(B, Hkv, S, D, dtype=torch.float16))
+    scale = 1 / math.sqrt(D)
+    mod = AttentionEngine(meta, CustomIO(), lambda score, io, b, h, q_idx, kv_idx: score * scale, specs.causal_mask, specs.OnlineSoftmax())
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(B, S, H, D, generator=g).half()
+    k = torch.randn(B, S, Hkv, D, generator=g).half()
+    v = torch.randn(B, S, Hkv, D, generator=g).half()
+    o = mod(q.cuda(), k.cuda(), v.cuda())
+    torch.cuda.synchronize()
+    oracle.assert_close(o.float().cpu(), oracle.softmax_attention(q, k, v, causal=True), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("B,H,HKV,S,KV,D,DV", [(8, 16, 16, 1, 4096, 128, 128), (2, 32, 4, 1, 1000, 128, 128), (1, 4, 4, 3, 300, 64, 64)])
+def test_engine_dense_decode(B, H, HKV, S, KV, D, DV):
+    """Decode operators (first case: testing/test.py:56, reference function :131-148): a short query against a long cache,
+    no mask, multi-head and grouped-query."""
+    mod = specs.softmax_attention_decode(B, H, S, KV, D, DV, HKV=HKV)
+    g = torch.Generator().manual_seed(KV)
+    q = torch.randn(B, S, H, D, generator=g).half()
+    k = torch.randn(B, KV, HKV, D, generator=g).half()
+    v = torch.randn(B, KV, HKV, DV, generator=g).half()
+    o = mod(q.cuda(), k.cuda(), v.cuda())
+    torch.cuda.synchronize()
+    assert o.shape == (B, S, H, DV)
+    ref = oracle.softmax_attention(q, k, v, causal=False)
+    oracle.assert_close(o.float().cpu(), ref, rtol=1e-2, atol=1e-2)      # the reference test's own tolerance (:156)
+
+
 def test_unsupported_head_size_is_an_error():
     hb = _hb()
     q = torch.zeros(1, 64, 1, 96, device="cuda", dtype=torch.bfloat16)

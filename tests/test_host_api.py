@@ -125,9 +125,12 @@ def test_engine_construction_and_dispatch():
     with pytest.raises(NotImplementedError):           # softmax score with identity row function: not in the library
         AttentionEngine(specs._meta(1, 2, 64, 128, 128, torch.bfloat16), CustomIO({}), score_mod=lambda s, c, b, h, q, k: s * 0.1,
                         mask_mod=None, online_func=specs.OnlineIdentity())
-    with pytest.raises(NotImplementedError):           # grouped-query prefill
-        AttentionEngine(specs._meta(1, 8, 64, 128, 128, torch.bfloat16, HKV=2), CustomIO({}), score_mod=None, mask_mod=None,
-                        online_func=specs.OnlineSoftmax())
+    e = AttentionEngine(specs._meta(1, 8, 64, 128, 128, torch.bfloat16, HKV=2), CustomIO({}),                # grouped-query prefill
+                        score_mod=lambda s, c, b, h, q, k: s * 0.1, mask_mod=None, online_func=specs.OnlineSoftmax())
+    assert (e.family, e.meta["Hq"], e.meta["Hkv"]) == ("softmax", 8, 2)
+    with pytest.raises(NotImplementedError):           # 8 query heads cannot share 3 kv heads
+        AttentionEngine(specs._meta(1, 8, 64, 128, 128, torch.bfloat16, HKV=3), CustomIO({}), score_mod=lambda s, c, b, h, q, k: s * 0.1,
+                        mask_mod=None, online_func=specs.OnlineSoftmax())
 
 
 def test_linear_engine_plans():

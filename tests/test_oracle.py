@@ -211,3 +211,20 @@ def test_input_generators_are_seeded():
     Cm, Bm, x, dt, A = inputs.mamba2_inputs(1, 4, 16, 8, 8)
     assert Cm.shape == (1, 1, 16, 8) and x.shape == (1, 4, 16, 8) and dt.dtype == torch.float32
     assert (A < 0).all() and (A >= -16).all() and (dt > 0).all()
+
+
+def test_grouped_query_equals_repeated_kv_heads():
+    """Hkv < H: query head h reads kv head h // (H // Hkv), i.e. the multi-head result on k, v with every
+    kv head repeated H // Hkv times."""
+    g = torch.Generator().manual_seed(4)
+    B, S, H, Hkv, D = 2, 40, 6, 2, 16
+    q = torch.randn(B, S, H, D, generator=g, dtype=torch.float64)
+    k = torch.randn(B, S, Hkv, D, generator=g, dtype=torch.float64)
+    v = torch.randn(B, S, Hkv, D, generator=g, dtype=torch.float64)
+    kr, vr = k.repeat_interleave(H // Hkv, dim=2), v.repeat_interleave(H // Hkv, dim=2)
+    kw = dict(compute_dtype=torch.float64)
+    torch.testing.assert_close(oracle.softmax_attention(q, k, v, causal=True, **kw), oracle.softmax_attention(q, kr, vr, causal=True, **kw))
+    torch.testing.assert_close(oracle.sigmoid_attention(q, k, v, 0.3, causal=True, **kw), oracle.sigmoid_attention(q, kr, vr, 0.3, causal=True, **kw))
+    torch.testing.assert_close(oracle.relu_attention(q, k, v, **kw), oracle.relu_attention(q, kr, vr, **kw))
+    sd = torch.nn.functional.scaled_dot_product_attention(q.transpose(1, 2), kr.transpose(1, 2), vr.transpose(1, 2), is_causal=True)
+    torch.testing.assert_close(oracle.softmax_attention(q, k, v, causal=True, **kw), sd.transpose(1, 2))
