@@ -77,6 +77,31 @@ typedef struct ma_attn_params {
   int32_t heads_kv;
 } ma_attn_params;
 
+/* Parallel attention backward for the SOFTMAX, SIGMOID and RELU families.  Replaces the backward of
+ * _attention (tl_template/attn/attn_tl.py:669-692): delta pre-pass, dK/dV kernel with fp32 dQ atomics,
+ * dQ post-pass.  Tensors and strides as in ma_attn_params; o and lse are the forward pass's output and
+ * fp32 [B,H,Sq] row scale (SOFTMAX only; may be NULL otherwise), dout is the gradient of o; dq [B,Sq,H,Dqk],
+ * dk [B,Skv,Hkv,Dqk], dv [B,Skv,Hkv,Dv] are written (not accumulated into), in `dtype`.  The workspace
+ * (ma_attn_bwd_workspace_bytes: fp32 [B,H,Sq]) carries delta = sum_d dout*o between the two kernels. */
+typedef struct ma_attn_bwd_params {
+  int32_t family; /* ma_attn_family: SOFTMAX, SIGMOID or RELU */
+  int32_t dtype;
+  int32_t mask;   /* ma_mask_kind */
+  int32_t batch, heads, heads_kv /* 0 = heads */, seqlen_q, seqlen_kv, dim_qk, dim_v;
+  const void* q;    int64_t q_stride_b, q_stride_s, q_stride_h;
+  const void* k;    int64_t k_stride_b, k_stride_s, k_stride_h;
+  const void* v;    int64_t v_stride_b, v_stride_s, v_stride_h;
+  const void* o;    int64_t o_stride_b, o_stride_s, o_stride_h;
+  const void* dout; int64_t do_stride_b, do_stride_s, do_stride_h;
+  void* dq;         int64_t dq_stride_b, dq_stride_s, dq_stride_h;
+  void* dk;         int64_t dk_stride_b, dk_stride_s, dk_stride_h;
+  void* dv;         int64_t dv_stride_b, dv_stride_s, dv_stride_h;
+  const float* lse;
+  float scale, bias;
+  const float* bias_ptr;
+  void* workspace; size_t workspace_bytes;
+} ma_attn_bwd_params;
+
 /* Chunked linear / stateful attention forward.  Replaces the three launches
  * of LinearAttention.forward (tl_template/linear/linear_tl.py:1240-1269):
  * chunk-local cumsum (:36-60), chunk_fwd_h (:146-221), chunk_o (:322-399).
@@ -124,6 +149,10 @@ const char* ma_last_error(void);
 
 /* attn_tl.py:92-190 (`main`) behind _attention.forward (:654-667) */
 int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream);
+
+/* attn_tl.py:669-692 (`_attention.backward`: mod_prep, mod_bwd, mod_post) */
+size_t ma_attn_bwd_workspace_bytes(const ma_attn_bwd_params* p);
+int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream);
 
 /* linear_tl.py:1240-1269 */
 size_t ma_linear_workspace_bytes(const ma_linear_params* p);

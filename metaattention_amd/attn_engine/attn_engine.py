@@ -71,8 +71,8 @@ _FAMILY = {
 
 
 class _ForwardOnly(torch.autograd.Function):
-    """Gives outputs a grad_fn whose backward fails loudly: the library holds
-    forward kernels only."""
+    """Gives outputs a grad_fn whose backward fails loudly, for the operators whose
+    backward kernels are not in the library."""
 
     @staticmethod
     def forward(ctx, run, *tensors):
@@ -80,7 +80,30 @@ class _ForwardOnly(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, *grads):
-        raise NotImplementedError("this operator is forward-only: backward kernels are not part of the gfx950 kernel library")
+        raise NotImplementedError("this operator is forward-only: its backward kernel is not part of the gfx950 kernel library")
+
+
+class _Attention(torch.autograd.Function):
+    """Forward + backward of the softmax / sigmoid / relu operators, as _attention of
+    tl_template/attn/attn_tl.py:654-692: saves q, k, v, o and the final row scale, returns
+    (dq, dk, dv) and None for every custom input."""
+
+    @staticmethod
+    def forward(ctx, engine, run, fam_code, bias_t, q, k, v):
+        out = run(q, k, v)
+        lse = engine.final_rowscales
+        ctx.engine, ctx.fam_code, ctx.bias_t = engine, fam_code, bias_t
+        ctx.save_for_backward(q, k, v, out, *([lse] if lse is not None else []))
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        from hip_backend import attn_bwd
+        q, k, v, out, *rest = ctx.saved_tensors
+        form = ctx.engine.score_form
+        dq, dk, dv = attn_bwd(q, k, v, out, dout, rest[0] if rest else None, family=ctx.fam_code,
+                              causal=ctx.engine.mask_kind == "causal", scale=form.scale, bias=form.bias, bias_tensor=ctx.bias_t)
+        return None, None, None, None, dq, dk, dv
 
 
 class AttentionEngine:
@@ -169,7 +192,10 @@ class AttentionEngine:
             return out
 
         if any(t.requires_grad for t in (q, k, v)):
-            return _ForwardOnly.apply(run, q, k, v)
+            if self.family == "retention":
+                return _ForwardOnly.apply(run, q, k, v)
+            bias_t = given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None
+            return _Attention.apply(self, run, fam_code, bias_t, q, k, v)
         return run(q, k, v)
 
     # ------------------------------------------------------------------ MLA decode

@@ -2,6 +2,7 @@
 // error strings, kernel selection.  No allocation, no synchronisation.
 #include "../../include/metaattention_hip.h"
 #include "attn_fwd.h"
+#include "attn_bwd.h"
 #include "linear_fwd.h"
 #include "mla_decode.h"
 
@@ -68,6 +69,62 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
   if (rc == -2)
     return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: no kernel for family %d, Dqk=%d, Dv=%d", p->family, p->dim_qk, p->dim_v);
   if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_attn_fwd: launch failed: %s", hipGetErrorString(hipGetLastError()));
+  return MA_OK;
+}
+
+size_t ma_attn_bwd_workspace_bytes(const ma_attn_bwd_params* p) {
+  if (!p || p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->family != MA_ATTN_SOFTMAX) return 0;
+  return (size_t)p->batch * p->heads * p->seqlen_q * sizeof(float);
+}
+
+int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
+  if (!p) return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: params is NULL");
+  if (!p->q || !p->k || !p->v || !p->dout || !p->dq || !p->dk || !p->dv)
+    return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: q/k/v/dout/dq/dk/dv must be non-NULL");
+  if (p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->seqlen_kv <= 0 || p->dim_qk <= 0 || p->dim_v <= 0)
+    return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: sizes must be positive");
+  if (p->dtype != MA_BF16 && p->dtype != MA_FP16) return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: dtype %d", p->dtype);
+  if (p->family != MA_ATTN_SOFTMAX && p->family != MA_ATTN_SIGMOID && p->family != MA_ATTN_RELU)
+    return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: family %d has no backward kernel", p->family);
+  if (!(p->scale > 0.f)) return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: scale must be > 0 (got %g)", (double)p->scale);
+  if (p->mask == MA_MASK_CAUSAL && p->seqlen_q != p->seqlen_kv)
+    return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: causal mask needs seqlen_q == seqlen_kv (%d vs %d)", p->seqlen_q, p->seqlen_kv);
+  const int hkv = p->heads_kv > 0 ? p->heads_kv : p->heads;
+  if (p->heads_kv < 0 || p->heads % hkv != 0)
+    return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: heads (%d) must be a multiple of heads_kv (%d)", p->heads, p->heads_kv);
+  if (p->family == MA_ATTN_SOFTMAX) {
+    if (!p->o || !p->lse) return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: SOFTMAX needs o and lse of the forward pass");
+    if (!p->workspace || p->workspace_bytes < ma_attn_bwd_workspace_bytes(p) || (uintptr_t)p->workspace % 4 != 0)
+      return fail(MA_ERR_WORKSPACE, "ma_attn_bwd: workspace of %zu bytes needed", ma_attn_bwd_workspace_bytes(p));
+  }
+  const int64_t strides[] = {p->q_stride_b, p->q_stride_s, p->q_stride_h, p->k_stride_b, p->k_stride_s, p->k_stride_h,
+                             p->v_stride_b, p->v_stride_s, p->v_stride_h, p->o_stride_b, p->o_stride_s, p->o_stride_h,
+                             p->do_stride_b, p->do_stride_s, p->do_stride_h, p->dq_stride_b, p->dq_stride_s, p->dq_stride_h,
+                             p->dk_stride_b, p->dk_stride_s, p->dk_stride_h, p->dv_stride_b, p->dv_stride_s, p->dv_stride_h};
+  for (int64_t s : strides)
+    if (s % 8 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: strides must be multiples of 8 elements (16-byte rows)");
+  const uintptr_t ptrs[] = {(uintptr_t)p->q, (uintptr_t)p->k, (uintptr_t)p->v, (uintptr_t)p->o, (uintptr_t)p->dout,
+                            (uintptr_t)p->dq, (uintptr_t)p->dk, (uintptr_t)p->dv};
+  for (uintptr_t x : ptrs)
+    if (x % 16 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: tensors must be 16-byte aligned");
+
+  ma::AttnBwdArgs a{};
+  a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.dout = p->dout; a.dq = p->dq; a.dk = p->dk; a.dv = p->dv;
+  a.lse = p->lse; a.delta = (float*)p->workspace; a.bias_ptr = p->bias_ptr;
+  a.qsb = p->q_stride_b; a.qss = p->q_stride_s; a.qsh = p->q_stride_h;
+  a.ksb = p->k_stride_b; a.kss = p->k_stride_s; a.ksh = p->k_stride_h;
+  a.vsb = p->v_stride_b; a.vss = p->v_stride_s; a.vsh = p->v_stride_h;
+  a.osb = p->o_stride_b; a.oss = p->o_stride_s; a.osh = p->o_stride_h;
+  a.dosb = p->do_stride_b; a.doss = p->do_stride_s; a.dosh = p->do_stride_h;
+  a.dqsb = p->dq_stride_b; a.dqss = p->dq_stride_s; a.dqsh = p->dq_stride_h;
+  a.dksb = p->dk_stride_b; a.dkss = p->dk_stride_s; a.dksh = p->dk_stride_h;
+  a.dvsb = p->dv_stride_b; a.dvss = p->dv_stride_s; a.dvsh = p->dv_stride_h;
+  a.B = p->batch; a.H = p->heads; a.Hkv = hkv; a.Sq = p->seqlen_q; a.Skv = p->seqlen_kv;
+  a.kv_group = p->heads / hkv;
+  a.scale = p->scale; a.bias = p->bias;
+  const int rc = ma::attn_bwd_dispatch(a, p->family, p->mask == MA_MASK_CAUSAL, p->dtype == MA_BF16, p->dim_qk, p->dim_v, (hipStream_t)stream);
+  if (rc == -2) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: no kernel for family %d, Dqk=%d, Dv=%d", p->family, p->dim_qk, p->dim_v);
+  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_attn_bwd: launch failed: %s", hipGetErrorString(hipGetLastError()));
   return MA_OK;
 }
 

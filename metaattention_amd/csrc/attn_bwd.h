@@ -1,0 +1,22 @@
+// Kernel-side argument block of the parallel attention backward kernels.
+#pragma once
+#include "common.h"
+
+namespace ma {
+
+struct AttnBwdArgs {
+  const void* q; const void* k; const void* v; const void* o; const void* dout;
+  void* dq; void* dk; void* dv;
+  const float* lse;    // [B,H,Sq] natural-log row scale of the forward pass (softmax)
+  float* delta;        // [B,H,Sq] workspace: sum_d dout * o per row (softmax)
+  const float* bias_ptr;
+  int64_t qsb, qss, qsh, ksb, kss, ksh, vsb, vss, vsh, osb, oss, osh, dosb, doss, dosh;
+  int64_t dqsb, dqss, dqsh, dksb, dkss, dksh, dvsb, dvss, dvsh;
+  int B, H, Hkv, Sq, Skv, num_blocks;
+  int kv_group;   // query heads per kv head
+  float scale, bias;
+};
+
+int attn_bwd_dispatch(const AttnBwdArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);
+
+}  // namespace ma

@@ -1,0 +1,420 @@
+// Parallel attention backward (dq, dk, dv) for gfx950: softmax, sigmoid and relu row functions.
+//
+// Replaces the backward of _attention (attention_engine/core/template/tl_template/attn/attn_tl.py:
+// 669-692): the delta pre-pass (:212-237), the dK/dV kernel with fp32 dQ atomics (:301-420) and the
+// dQ post-pass (:239-262).  With p = rowfn(x), x = s * scale + bias, s = q.k^T:
+//   softmax   p = exp(x - lse),       ds = p * (dp - delta) * scale,   delta_i = sum_d do_id * o_id
+//   sigmoid   p = 1 / (1 + exp(-x)),  ds = dp * p * (1 - p) * scale
+//   relu      p = max(x, 0),          ds = dp * [x > 0] * scale
+//   dp = do.v^T,   dv = p^T do,   dk = ds^T q,   dq = ds k
+// (p and ds are rounded to the tensor dtype before the second products, as there: :357-362).
+//
+// No atomics: two kernels, each owning its outputs.
+//   attn_bwd_dq_kernel   a wave owns 32 query rows and walks the kv sequence; everything transposed as in
+//                        the forward kernels (S^T = K Q^T, dP^T = V dO^T: lane = query row, so lse and
+//                        delta are per-lane scalars; dS^T is directly the B operand of dQ^T += K^T dS^T).
+//                        It also computes delta and leaves it in the workspace for the second kernel.
+//   attn_bwd_dkv_kernel  a wave owns 32 keys of one kv head (K and V fragments in registers as B
+//                        operands) and walks the query rows of every query head of its group; here
+//                        S = Q K^T and dP = dO V^T are NOT transposed (lane = key), so P and dS are
+//                        directly the B operands of dV^T += dO^T P and dK^T += Q^T dS; lse and delta of
+//                        the 16 rows a lane holds come from global memory.
+// The scores are recomputed in both (7 tile products instead of 5), which is what avoiding the fp32
+// atomics and the post-pass costs.  Tiles of 32 rows arrive by direct-to-LDS DMA, double buffered,
+// one barrier per tile, XOR-swizzled like the forward tiles; the column-side operands (K^T, dO^T,
+// Q^T) come from the same tiles through the transposing LDS read.
+#include "attn_bwd.h"
+
+namespace ma {
+
+namespace {
+enum { BF_SOFTMAX = 0, BF_SIGMOID = 1, BF_RELU = 2 };   // = MA_ATTN_* of the C interface
+
+// ds (and p) of one score element.  x2 = (s * scale + bias) * log2(e) for softmax / sigmoid.
+template <int FAMILY>
+__device__ __forceinline__ void row_fn_bwd(float s, float dp, bool masked, float c_scale, float c_bias, float scale, float bias,
+                                           float lse2, float delta, float& p, float& ds) {
+  if constexpr (FAMILY == BF_SOFTMAX) {
+    p = masked ? 0.f : fast_exp2(s * c_scale + c_bias - lse2);
+    ds = p * (dp - delta) * scale;
+  } else if constexpr (FAMILY == BF_SIGMOID) {
+    p = masked ? 0.f : fast_rcp(1.f + fast_exp2(-(s * c_scale + c_bias)));
+    ds = dp * p * (1.f - p) * scale;
+  } else {
+    const float x = s * scale + bias;
+    p = masked ? 0.f : fmaxf(x, 0.f);
+    ds = (!masked && x > 0.f) ? dp * scale : 0.f;
+  }
+}
+
+// DMA of a [32 x ROWB bytes] tile whose rows are `row_stride` bytes apart in memory: each instruction
+// moves 1 KB; lane i fetches the 16-byte chunk that belongs at physical position i of that KB.  Rows
+// beyond `limit` are clamped to the last one (whatever is computed from them is masked).
+template <int ROWB, int NWAVES>
+__device__ __forceinline__ void dma_tile(const char* src, int64_t row_stride, int row0, int limit, uint32_t lds_base, int wave, int lane) {
+  constexpr int CPR = ROWB / 16, NI = 32 * ROWB / 1024;
+  for (int ii = wave; ii < NI; ii += NWAVES) {
+    const int row = ii * (1024 / ROWB) + lane / CPR, c = lane % CPR;
+    const int grow = min(row0 + row, limit - 1);
+    dma16(src + grow * row_stride + ((c ^ swz_tile<CPR>(row)) << 4), lds_base + ii * 1024);
+  }
+}
+
+// [32 x 32] += A B^T over DIM columns, A = the 32 rows of an LDS tile (row reads), B = fragments in registers
+template <typename T, int DIM>
+__device__ __forceinline__ f32x16 mm_rows(uint32_t tile, int r, int g, const typename Elem<T>::x8 (&bf)[DIM / 16]) {
+  using E = Elem<T>;
+  using x8 = typename E::x8;
+  constexpr int ROWB = DIM * 2, CPR = DIM / 8, KS = DIM / 16, AH = 2, RING = 3;
+  const uint32_t row_off = tile + r * ROWB;
+  const int c0 = g ^ swz_tile<CPR>(r);
+  f32x16 acc;
+#pragma unroll
+  for (int j = 0; j < 16; j++) acc[j] = 0.f;
+  x8 af[RING];
+#pragma unroll
+  for (int ks = 0; ks < AH && ks < KS; ks++) af[ks] = lds_read<x8>(row_off + (uint32_t)((c0 ^ (2 * ks)) << 4));
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) {
+    if (ks + AH < KS) af[(ks + AH) % RING] = lds_read<x8>(row_off + (uint32_t)((c0 ^ (2 * (ks + AH))) << 4));
+    __builtin_amdgcn_sched_barrier(0);
+    acc = E::mfma32(af[ks % RING], bf[ks], acc);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  return acc;
+}
+
+// acc[DIM/32 blocks of 32 columns] += (tile columns)^T . pf, where pf holds a [32 x 32] factor in
+// accumulator order rounded to T (k slot i of slice s for lane half g is tile row 16s + 8(i/4) + 4g + i%4,
+// which is the row order the transposing reads below fetch)
+template <typename T, int DIM>
+__device__ __forceinline__ void mm_cols(uint32_t tile, int lane, const typename Elem<T>::x8 (&pf)[2], f32x16 (&acc)[DIM / 32]) {
+  using E = Elem<T>;
+  using x8 = typename E::x8;
+  using x4 = typename E::x4;
+  constexpr int ROWB = DIM * 2, CPR = DIM / 8, NB = DIM / 32, PF = NB >= 2 ? 4 : 2;
+  const int g = lane >> 5, jr = (lane & 15) >> 2;
+  const int lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
+  const uint32_t row_off = tile + (4 * g + jr) * ROWB + (lane & 1) * 8;
+  const int c0 = lc ^ swz_tile<CPR>(4 * g + jr);
+  x4 lo[PF], hi[PF];
+  auto request = [&](int idx) {   // idx = 2 block + slice
+    const int db = idx >> 1, sl = idx & 1;
+    const uint32_t rb = row_off + 16 * sl * ROWB;
+    lo[idx % PF] = lds_read_tr4<T>(rb + (uint32_t)((c0 ^ (4 * db)) << 4));
+    hi[idx % PF] = lds_read_tr4<T>(rb + 8 * ROWB + (uint32_t)((c0 ^ (4 * db) ^ 2) << 4));
+  };
+#pragma unroll
+  for (int i = 0; i < PF - 1; i++) request(i);
+#pragma unroll
+  for (int idx = 0; idx < 2 * NB; idx++) {
+    if (idx + PF - 1 < 2 * NB) request(idx + PF - 1);
+    __builtin_amdgcn_sched_barrier(0);
+    x8 af = __builtin_shufflevector(lo[idx % PF], hi[idx % PF], 0, 1, 2, 3, 4, 5, 6, 7);
+    acc[idx >> 1] = E::mfma32(af, pf[idx & 1], acc[idx >> 1]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// a wave's [DIM x 32] accumulator (lane = output row, elements = columns) to global rows of DIM
+// elements, through a wave-private LDS block in two halves, 16-byte coalesced stores
+template <typename T, int DIM>
+__device__ __forceinline__ void store_rows(const f32x16 (&acc)[DIM / 32], float mult, uint32_t stage, T* gbase, int64_t row_stride,
+                                           int row0, int row_limit, int lane) {
+  using x4 = typename Elem<T>::x4;
+  constexpr int NB = DIM / 32, HALF = DIM / 2, OROW = HALF * 2 + 16;
+  const int r = lane & 31, g = lane >> 5;
+#pragma unroll
+  for (int hp = 0; hp < 2; hp++) {
+#pragma unroll
+    for (int dbl = 0; dbl < NB / 2; dbl++)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (T)(acc[hp * (NB / 2) + dbl][4 * q4 + i] * mult);
+        lds_write<x4>(stage + r * OROW + (32 * dbl + 8 * q4 + 4 * g) * 2, w);
+      }
+#pragma unroll
+    for (int it = 0; it < 32 * (HALF / 8) / 64; it++) {
+      const int ci = lane + 64 * it, row = ci / (HALF / 8), c = ci % (HALF / 8);
+      const u32x4 w = lds_read<u32x4>(stage + row * OROW + c * 16);
+      if (row0 + row < row_limit) *(u32x4*)(gbase + (int64_t)(row0 + row) * row_stride + hp * HALF + c * 8) = w;
+    }
+  }
+}
+}  // namespace
+
+// ------------------------------------------------------------------------------------------------
+// dq (and delta)
+// ------------------------------------------------------------------------------------------------
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
+__global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_kernel(const AttnBwdArgs a) {
+  using E = Elem<T>;
+  using x8 = typename E::x8;
+  constexpr int BM = 128, BN = 32;
+  constexpr int KS = DQK / 16, VS = DV / 16, QB = DQK / 32;
+  constexpr int KROW = DQK * 2, VROW = DV * 2;
+  constexpr int KTILE = BN * KROW, VTILE = BN * VROW, STAGE = KTILE + VTILE;
+
+  extern __shared__ __align__(16) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, g = lane >> 5;
+
+  const int nmb = a.num_blocks, BH = a.B * a.H;
+  int bh, mb;
+  if ((BH & 7) == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    bh = (slot / nmb) * 8 + xcd;
+    mb = slot % nmb;
+  } else {
+    bh = blockIdx.x / nmb;
+    mb = blockIdx.x % nmb;
+  }
+  if (CAUSAL) mb = nmb - 1 - mb;
+  const int b = bh / a.H, h = bh % a.H, hk = h / a.kv_group;
+  const int m_wave = mb * BM + wave * 32, m_lane = m_wave + r;
+  const int m_ld = min(m_lane, a.Sq - 1);
+
+  // B operands of this wave's 32 rows: Q (for S^T = K Q^T) and dO (for dP^T = V dO^T)
+  x8 qf[KS], dof[VS];
+  float delta = 0.f, lse2 = 0.f;
+  {
+    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)m_ld * a.qss + (int64_t)h * a.qsh + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 16 * ks);
+    const T* dop = (const T*)a.dout + (int64_t)b * a.dosb + (int64_t)m_ld * a.doss + (int64_t)h * a.dosh + 8 * g;
+#pragma unroll
+    for (int sl = 0; sl < VS; sl++) dof[sl] = *(const x8*)(dop + 16 * sl);
+    if constexpr (FAMILY == BF_SOFTMAX) {
+      const T* op = (const T*)a.o + (int64_t)b * a.osb + (int64_t)m_ld * a.oss + (int64_t)h * a.osh + 8 * g;
+      float part = 0.f;
+#pragma unroll
+      for (int sl = 0; sl < VS; sl++) {
+        const x8 of = *(const x8*)(op + 16 * sl);
+#pragma unroll
+        for (int i = 0; i < 8; i++) part += (float)dof[sl][i] * (float)of[i];
+      }
+      delta = part + xhalf(part);
+      const int64_t ri = ((int64_t)b * a.H + h) * a.Sq + m_ld;
+      lse2 = a.lse[ri] * kLog2e;
+      if (g == 0 && m_lane < a.Sq) a.delta[ri] = delta;
+    }
+  }
+  const char* kb = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)hk * a.ksh);
+  const char* vb = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)hk * a.vsh);
+  const int64_t k_row_bytes = a.kss * 2, v_row_bytes = a.vss * 2;
+
+  int n_tiles = (a.Skv + BN - 1) / BN;
+  if (CAUSAL) n_tiles = min(n_tiles, (mb * BM + BM + BN - 1) / BN);
+
+  auto issue_tile = [&](int n0, int buf) {
+    dma_tile<KROW, 4>(kb, k_row_bytes, n0, a.Skv, lds0 + buf * STAGE, wave, lane);
+    dma_tile<VROW, 4>(vb, v_row_bytes, n0, a.Skv, lds0 + buf * STAGE + KTILE, wave, lane);
+  };
+
+  f32x16 dq[QB];
+#pragma unroll
+  for (int i = 0; i < QB; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) dq[i][j] = 0.f;
+  const float bias = a.bias + (a.bias_ptr ? *a.bias_ptr : 0.f);
+  const float c_scale = a.scale * kLog2e, c_bias = bias * kLog2e;
+
+  if (n_tiles > 0) issue_tile(0, 0);
+  for (int jt = 0; jt < n_tiles; jt++) {
+    const int buf = jt & 1, n0 = jt * BN;
+    wait_dma();
+    __syncthreads();
+    if (jt + 1 < n_tiles) issue_tile(n0 + BN, buf ^ 1);
+    const uint32_t kbase = lds0 + buf * STAGE, vbase = kbase + KTILE;
+
+    const f32x16 s = mm_rows<T, DQK>(kbase, r, g, qf);     // S^T: lane = row m_lane, element jj = key n0 + 8(jj/4) + 4g + jj%4
+    const f32x16 dp = mm_rows<T, DV>(vbase, r, g, dof);   // dP^T, same layout
+    x8 dsf[2];
+#pragma unroll
+    for (int jj = 0; jj < 16; jj++) {
+      const int n = n0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
+      const bool masked = (CAUSAL && n > m_lane) || n >= a.Skv;
+      float p, ds;
+      row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, lse2, delta, p, ds);
+      dsf[jj >> 3][jj & 7] = (T)ds;
+    }
+    mm_cols<T, DQK>(kbase, lane, dsf, dq);                 // dQ^T += K^T dS^T
+  }
+  __syncthreads();   // every wave is done with the tiles: they become output staging
+
+  constexpr int OROW = DQK + 16;
+  T* dqb = (T*)a.dq + (int64_t)b * a.dqsb + (int64_t)h * a.dqsh;
+  store_rows<T, DQK>(dq, 1.f, lds0 + wave * 32 * OROW, dqb, a.dqss, m_wave, a.Sq, lane);
+}
+
+// ------------------------------------------------------------------------------------------------
+// dk, dv
+// ------------------------------------------------------------------------------------------------
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
+// (the two [D x 32] accumulators plus the K and V fragments take 192 registers at 128/128: one wave per SIMD there)
+__global__ __launch_bounds__(256, (DQK + DV >= 256 ? 1 : 2)) void attn_bwd_dkv_kernel(const AttnBwdArgs a) {
+  using E = Elem<T>;
+  using x8 = typename E::x8;
+  constexpr int BNW = 128, BMT = 32;   // keys per workgroup, query rows per tile
+  constexpr int KS = DQK / 16, VS = DV / 16, QB = DQK / 32, VB = DV / 32;
+  constexpr int QROW = DQK * 2, DOROW = DV * 2;
+  constexpr int QTILE = BMT * QROW, DOTILE = BMT * DOROW, STAGE = QTILE + DOTILE;
+
+  extern __shared__ __align__(16) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, g = lane >> 5;
+
+  const int nnb = a.num_blocks, BHK = a.B * a.Hkv;
+  int bhk, nb;
+  if ((BHK & 7) == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    bhk = (slot / nnb) * 8 + xcd;
+    nb = slot % nnb;
+  } else {
+    bhk = blockIdx.x / nnb;
+    nb = blockIdx.x % nnb;
+  }
+  const int b = bhk / a.Hkv, hk = bhk % a.Hkv;
+  const int n_wave = nb * BNW + wave * 32, n_lane = n_wave + r;
+  const int n_ld = min(n_lane, a.Skv - 1);
+
+  // B operands of this wave's 32 keys: K (for S = Q K^T) and V (for dP = dO V^T)
+  x8 kf[KS], vf[VS];
+  {
+    const T* kp = (const T*)a.k + (int64_t)b * a.ksb + (int64_t)n_ld * a.kss + (int64_t)hk * a.ksh + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) kf[ks] = *(const x8*)(kp + 16 * ks);
+    const T* vp = (const T*)a.v + (int64_t)b * a.vsb + (int64_t)n_ld * a.vss + (int64_t)hk * a.vsh + 8 * g;
+#pragma unroll
+    for (int sl = 0; sl < VS; sl++) vf[sl] = *(const x8*)(vp + 16 * sl);
+  }
+  f32x16 dk[QB], dv[VB];
+#pragma unroll
+  for (int i = 0; i < QB; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) dk[i][j] = 0.f;
+#pragma unroll
+  for (int i = 0; i < VB; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) dv[i][j] = 0.f;
+  const float bias = a.bias + (a.bias_ptr ? *a.bias_ptr : 0.f);
+  const float c_scale = a.scale * kLog2e, c_bias = bias * kLog2e;
+
+  // query tiles that can see this workgroup's keys, for every query head of the kv head's group
+  const int t_first = CAUSAL ? (nb * BNW) / BMT : 0;
+  const int t_count = (a.Sq + BMT - 1) / BMT - t_first;
+  const int n_steps = t_count > 0 ? t_count * a.kv_group : 0;
+  const int64_t q_row_bytes = a.qss * 2, do_row_bytes = a.doss * 2;
+  auto issue_step = [&](int step, int buf) {
+    const int h = hk * a.kv_group + step / t_count, m0 = (t_first + step % t_count) * BMT;
+    const char* qb = (const char*)((const T*)a.q + (int64_t)b * a.qsb + (int64_t)h * a.qsh);
+    const char* dob = (const char*)((const T*)a.dout + (int64_t)b * a.dosb + (int64_t)h * a.dosh);
+    dma_tile<QROW, 4>(qb, q_row_bytes, m0, a.Sq, lds0 + buf * STAGE, wave, lane);
+    dma_tile<DOROW, 4>(dob, do_row_bytes, m0, a.Sq, lds0 + buf * STAGE + QTILE, wave, lane);
+  };
+
+  if (n_steps > 0) issue_step(0, 0);
+  for (int step = 0; step < n_steps; step++) {
+    const int buf = step & 1;
+    const int h = hk * a.kv_group + step / t_count, m0 = (t_first + step % t_count) * BMT;
+    wait_dma();
+    __syncthreads();
+    if (step + 1 < n_steps) issue_step(step + 1, buf ^ 1);
+    // (a wave whose keys all lie behind this tile's rows has nothing to add; it still takes part in the barriers)
+    if (CAUSAL && m0 + BMT - 1 < n_wave) continue;
+    const uint32_t qbase = lds0 + buf * STAGE, dobase = qbase + QTILE;
+
+    // lse and delta of the rows this lane holds: m0 + 8q4 + 4g + {0..3}
+    float lse2[16], dl[16];
+    if constexpr (FAMILY == BF_SOFTMAX) {
+      const int64_t rbase = ((int64_t)b * a.H + h) * a.Sq;
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int m = min(m0 + 8 * q4 + 4 * g + i, a.Sq - 1);
+          lse2[4 * q4 + i] = a.lse[rbase + m] * kLog2e;
+          dl[4 * q4 + i] = a.delta[rbase + m];
+        }
+    }
+    const f32x16 s = mm_rows<T, DQK>(qbase, r, g, kf);     // S: lane = key n_lane, element jj = row m0 + 8(jj/4) + 4g + jj%4
+    const f32x16 dp = mm_rows<T, DV>(dobase, r, g, vf);   // dP, same layout
+    x8 pf[2], dsf[2];
+#pragma unroll
+    for (int jj = 0; jj < 16; jj++) {
+      const int m = m0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
+      const bool masked = (CAUSAL && n_lane > m) || m >= a.Sq || n_lane >= a.Skv;
+      float p, ds;
+      row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX ? lse2[jj] : 0.f,
+                         FAMILY == BF_SOFTMAX ? dl[jj] : 0.f, p, ds);
+      if (masked) ds = 0.f;
+      pf[jj >> 3][jj & 7] = (T)p;
+      dsf[jj >> 3][jj & 7] = (T)ds;
+    }
+    mm_cols<T, DV>(dobase, lane, pf, dv);     // dV^T += dO^T P
+    mm_cols<T, DQK>(qbase, lane, dsf, dk);    // dK^T += Q^T dS
+  }
+  __syncthreads();   // every wave is done with the tiles: they become output staging
+
+  constexpr int DMAX = DQK > DV ? DQK : DV, OROW = DMAX + 16;
+  const uint32_t stage = lds0 + wave * 32 * OROW;
+  T* dkb = (T*)a.dk + (int64_t)b * a.dksb + (int64_t)hk * a.dksh;
+  T* dvb = (T*)a.dv + (int64_t)b * a.dvsb + (int64_t)hk * a.dvsh;
+  store_rows<T, DQK>(dk, 1.f, stage, dkb, a.dkss, n_wave, a.Skv, lane);
+  store_rows<T, DV>(dv, 1.f, stage, dvb, a.dvss, n_wave, a.Skv, lane);
+}
+
+// ------------------------------------------------------------------------------------------------
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
+static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
+  constexpr int DMAX = DQK > DV ? DQK : DV;
+  constexpr size_t tiles = 2 * (size_t)32 * (DQK + DV) * 2;
+  constexpr size_t ostage = 4 * 32 * (size_t)(DMAX + 16);
+  constexpr size_t lds = tiles > ostage ? tiles : ostage;
+  auto k1 = attn_bwd_dq_kernel<T, DQK, DV, FAMILY, CAUSAL>;
+  auto k2 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
+    if (hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
+    attr_set = true;
+  }
+  AttnBwdArgs args = a;
+  args.num_blocks = (a.Sq + 127) / 128;
+  hipLaunchKernelGGL(k1, dim3((unsigned)(args.num_blocks * a.B * a.H)), dim3(256), lds, stream, args);
+  args.num_blocks = (a.Skv + 127) / 128;
+  hipLaunchKernelGGL(k2, dim3((unsigned)(args.num_blocks * a.B * a.Hkv)), dim3(256), lds, stream, args);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+template <typename T, int DQK, int DV>
+static int bwd_family(const AttnBwdArgs& a, int family, bool causal, hipStream_t stream) {
+  switch (family) {
+    case BF_SOFTMAX:
+      return causal ? launch_bwd<T, DQK, DV, BF_SOFTMAX, true>(a, stream) : launch_bwd<T, DQK, DV, BF_SOFTMAX, false>(a, stream);
+    case BF_SIGMOID:
+      return causal ? launch_bwd<T, DQK, DV, BF_SIGMOID, true>(a, stream) : launch_bwd<T, DQK, DV, BF_SIGMOID, false>(a, stream);
+    case BF_RELU:
+      return causal ? launch_bwd<T, DQK, DV, BF_RELU, true>(a, stream) : launch_bwd<T, DQK, DV, BF_RELU, false>(a, stream);
+  }
+  return -2;
+}
+
+template <typename T>
+static int bwd_dims(const AttnBwdArgs& a, int family, bool causal, int dqk, int dv, hipStream_t stream) {
+  if (dqk == 128 && dv == 128) return bwd_family<T, 128, 128>(a, family, causal, stream);
+  if (dqk == 64 && dv == 64) return bwd_family<T, 64, 64>(a, family, causal, stream);
+  if (dqk == 128 && dv == 256) return bwd_family<T, 128, 256>(a, family, causal, stream);
+  return -2;
+}
+
+// returns 0 ok, -1 launch failure, -2 unsupported
+int attn_bwd_dispatch(const AttnBwdArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream) {
+  return is_bf16 ? bwd_dims<__bf16>(a, family, causal, dqk, dv, stream) : bwd_dims<_Float16>(a, family, causal, dqk, dv, stream);
+}
+
+}  // namespace ma

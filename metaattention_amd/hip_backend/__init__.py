@@ -22,7 +22,7 @@ MA_ATTN_SOFTMAX, MA_ATTN_SIGMOID, MA_ATTN_RELU, MA_ATTN_RETENTION = 0, 1, 2, 3
 MA_MASK_NONE, MA_MASK_CAUSAL = 0, 1
 
 EXPORTED_SYMBOLS = (
-    "ma_version", "ma_last_error", "ma_attn_fwd",
+    "ma_version", "ma_last_error", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes", "ma_attn_bwd",
     "ma_linear_workspace_bytes", "ma_linear_fwd",
     "ma_mla_choose_split", "ma_mla_workspace_bytes", "ma_mla_decode",
 )
@@ -47,6 +47,24 @@ class AttnParams(Structure):
         ("scale", c_float), ("bias", c_float), ("bias_ptr", c_void_p),
         ("score_mask", c_void_p), ("sm_stride_b", c_int64), ("sm_stride_h", c_int64), ("sm_stride_q", c_int64),
         ("heads_kv", c_int32),
+    ]
+
+
+def _tensor_fields(name):
+    return [(name, c_void_p), (f"{name}_stride_b", c_int64), (f"{name}_stride_s", c_int64), (f"{name}_stride_h", c_int64)]
+
+
+class AttnBwdParams(Structure):
+    _fields_ = [
+        ("family", c_int32), ("dtype", c_int32), ("mask", c_int32),
+        ("batch", c_int32), ("heads", c_int32), ("heads_kv", c_int32), ("seqlen_q", c_int32), ("seqlen_kv", c_int32),
+        ("dim_qk", c_int32), ("dim_v", c_int32),
+        *_tensor_fields("q"), *_tensor_fields("k"), *_tensor_fields("v"), *_tensor_fields("o"),
+        ("dout", c_void_p), ("do_stride_b", c_int64), ("do_stride_s", c_int64), ("do_stride_h", c_int64),
+        *_tensor_fields("dq"), *_tensor_fields("dk"), *_tensor_fields("dv"),
+        ("lse", c_void_p),
+        ("scale", c_float), ("bias", c_float), ("bias_ptr", c_void_p),
+        ("workspace", c_void_p), ("workspace_bytes", c_size_t),
     ]
 
 
@@ -94,6 +112,10 @@ def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
     lib.ma_last_error.restype = c_char_p
     lib.ma_attn_fwd.argtypes = [POINTER(AttnParams), c_void_p]
     lib.ma_attn_fwd.restype = c_int
+    lib.ma_attn_bwd.argtypes = [POINTER(AttnBwdParams), c_void_p]
+    lib.ma_attn_bwd.restype = c_int
+    lib.ma_attn_bwd_workspace_bytes.argtypes = [POINTER(AttnBwdParams)]
+    lib.ma_attn_bwd_workspace_bytes.restype = c_size_t
     lib.ma_linear_workspace_bytes.argtypes = [POINTER(LinearParams)]
     lib.ma_linear_workspace_bytes.restype = c_size_t
     lib.ma_linear_fwd.argtypes = [POINTER(LinearParams), c_void_p]
@@ -167,6 +189,44 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
         p.sm_stride_h, p.sm_stride_q = score_mask.stride(1), score_mask.stride(2)
     _check(load_library().ma_attn_fwd(ctypes.byref(p), _stream()))
     return out
+
+
+def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None):
+    """Gradients (dq, dk, dv) of the parallel attention forward on BSHD tensors.  ``o`` and ``lse``
+    (fp32 [B,H,Sq]) are the forward pass's output and row scale (softmax only; None otherwise),
+    ``dout`` the gradient of ``o``."""
+    _require_gpu(q, k, v, o, dout, lse, bias_tensor)
+    B, Sq, H, Dqk = q.shape
+    Skv, Hkv, Dv = k.shape[1], k.shape[2], v.shape[-1]
+    assert k.shape == (B, Skv, Hkv, Dqk) and v.shape == (B, Skv, Hkv, Dv) and dout.shape == (B, Sq, H, Dv) and H % Hkv == 0
+    dout = dout if dout.stride(-1) == 1 else dout.contiguous()
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    p = AttnBwdParams()
+    p.family, p.dtype, p.mask = family, _dtype_code(q.dtype), MA_MASK_CAUSAL if causal else MA_MASK_NONE
+    p.batch, p.heads, p.heads_kv, p.seqlen_q, p.seqlen_kv, p.dim_qk, p.dim_v = B, H, Hkv, Sq, Skv, Dqk, Dv
+    for name, prefix, t in (("q", "q", q), ("k", "k", k), ("v", "v", v), ("o", "o", o), ("dout", "do", dout), ("dq", "dq", dq),
+                            ("dk", "dk", dk), ("dv", "dv", dv)):
+        if t is None:
+            continue
+        assert t.stride(-1) == 1 and t.dtype == q.dtype, "last dimension must be contiguous, one dtype"
+        setattr(p, name, t.data_ptr())
+        setattr(p, f"{prefix}_stride_b", t.stride(0))
+        setattr(p, f"{prefix}_stride_s", t.stride(1))
+        setattr(p, f"{prefix}_stride_h", t.stride(2))
+    if lse is not None:
+        assert lse.dtype == torch.float32 and lse.shape == (B, H, Sq) and lse.is_contiguous()
+        p.lse = lse.data_ptr()
+    p.scale, p.bias = float(scale), float(bias)
+    if bias_tensor is not None:
+        assert bias_tensor.dtype == torch.float32 and bias_tensor.numel() == 1
+        p.bias_ptr = bias_tensor.data_ptr()
+    lib = load_library()
+    need = lib.ma_attn_bwd_workspace_bytes(ctypes.byref(p))
+    if need:
+        ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+        p.workspace, p.workspace_bytes = ws.data_ptr(), need
+    _check(lib.ma_attn_bwd(ctypes.byref(p), _stream()))
+    return dq, dk, dv
 
 
 def mla_decode(q, q_pe, kv, k_pe, *, scale: float, num_split: int = 0, out=None, lse=None, workspace=None):

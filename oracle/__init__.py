@@ -27,6 +27,10 @@ ssd_chunk_scan         3-way agreement: chunked reference == naive sequential
                        state-space recurrence; chunk-size independence
 simple_gla             token-by-token recurrence (fp64)
 mla_decode             SDPA with K=concat(kv,k_pe), V=kv; split-KV invariance
+attention_grads        central differences of the pinned forward functions in
+                       fp64 along random directions; SDPA's own autograd
+(all of the above)     tests/golden/*.npz: the operators' definitions evaluated
+                       element by element in fp64 numpy by independent code
 =====================  =====================================================
 
 No function here is "parity unpinned".
@@ -38,6 +42,7 @@ from .attention_ref import (  # noqa: F401
     retention_parallel,
     mla_decode,
     retention_decay_mask,
+    attention_grads,
 )
 from .linear_ref import (  # noqa: F401
     retnet_quadratic,

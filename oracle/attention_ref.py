@@ -141,3 +141,13 @@ def mla_decode(q, q_pe, kv, k_pe, compute_dtype=torch.float32, return_lse: bool 
             lse[b, hs] = torch.logsumexp(s, dim=-1)
             out[b, 0, hs] = torch.softmax(s, dim=-1) @ kv[b, :, g].to(compute_dtype)
     return (out, lse) if return_lse else out
+
+
+def attention_grads(forward, q, k, v, dout, **kwargs):
+    """(dq, dk, dv) of ``sum(forward(q, k, v, **kwargs) * dout)`` by PyTorch autograd over the fp64
+    restated forward, the way the reference's tests obtain reference gradients
+    (testing/test.py:119-125: ``ref_o.backward(do)``)."""
+    qd, kd, vd = (t.detach().to(torch.float64).requires_grad_(True) for t in (q, k, v))
+    out = forward(qd, kd, vd, compute_dtype=torch.float64, **kwargs)
+    out.backward(dout.to(torch.float64))
+    return qd.grad, kd.grad, vd.grad

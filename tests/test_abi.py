@@ -40,7 +40,8 @@ def test_struct_layout_matches_c():
     import subprocess
     import tempfile
     from metaattention_amd import hip_backend as hb
-    checks = [("ma_attn_params", hb.AttnParams), ("ma_linear_params", hb.LinearParams), ("ma_mla_params", hb.MlaParams)]
+    checks = [("ma_attn_params", hb.AttnParams), ("ma_attn_bwd_params", hb.AttnBwdParams), ("ma_linear_params", hb.LinearParams),
+              ("ma_mla_params", hb.MlaParams)]
     src = ['#include <stdio.h>', '#include <stddef.h>', '#include "metaattention_hip.h"', 'int main(void){']
     for cname, cls in checks:
         src.append(f'printf("%zu\\n", sizeof({cname}));')

@@ -1,0 +1,141 @@
+"""Parity of the parallel attention backward (dq, dk, dv through the C ABI and through autograd on
+the AttentionEngine operators) with the gradient oracle (autograd over the fp64 restated forward, as
+the reference's tests obtain their reference gradients: testing/test.py:119-125).  Tolerance atol 2e-2 /
+rtol 1e-2 with a small allowance for the bf16/fp16 rounding of p and ds (the reference's own checks
+use rtol = atol = 1e-1, :123-125, which is asserted with no allowance)."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from oracle import inputs
+import specs
+
+pytestmark = pytest.mark.gpu
+ATOL, RTOL = 2e-2, 1e-2
+
+
+def _hb():
+    from metaattention_amd import hip_backend as hb
+    hb.load_library()
+    return hb
+
+
+def _check(got, ref, what):
+    for name, a, b in zip(("dq", "dk", "dv"), got, ref):
+        a, b = a.float().cpu(), b.float()
+        oracle.assert_close(a, b, rtol=1e-1, atol=1e-1, msg=f"{what}:{name} (reference acceptance)")
+        oracle.assert_close(a, b, rtol=RTOL, atol=ATOL, mismatch_ratio=1e-3, msg=f"{what}:{name}")
+
+
+def _run(hb, family, q, k, v, dout, causal, scale, bias=0.0):
+    fam = {"softmax": hb.MA_ATTN_SOFTMAX, "sigmoid": hb.MA_ATTN_SIGMOID, "relu": hb.MA_ATTN_RELU}[family]
+    qc, kc, vc, dc = q.cuda(), k.cuda(), v.cuda(), dout.cuda()
+    B, S, H, _ = q.shape
+    lse = torch.empty(B, H, S, device="cuda") if family == "softmax" else None
+    o = hb.attn_fwd(qc, kc, vc, family=fam, causal=causal, scale=scale, bias=bias, row_scale=lse)
+    got = hb.attn_bwd(qc, kc, vc, o, dc, lse, family=fam, causal=causal, scale=scale, bias=bias)
+    torch.cuda.synchronize()
+    if family == "softmax":
+        ref = oracle.attention_grads(oracle.softmax_attention, q, k, v, dout, causal=causal, softmax_scale=scale)
+    elif family == "sigmoid":
+        ref = oracle.attention_grads(oracle.sigmoid_attention, q, k, v, dout, bias=bias, causal=causal, softmax_scale=scale)
+    else:
+        ref = oracle.attention_grads(oracle.relu_attention, q, k, v, dout, softmax_scale=scale)
+    return got, ref
+
+
+@pytest.mark.parametrize("D,DV", [(128, 128), (64, 64), (128, 256)])
+@pytest.mark.parametrize("B,H,Hkv,S,causal", [(1, 2, 2, 256, True), (2, 3, 3, 200, True), (1, 2, 2, 333, False), (1, 4, 2, 129, True), (1, 1, 1, 1, True)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_softmax_backward(D, DV, B, H, Hkv, S, causal, dtype):
+    hb = _hb()
+    g = torch.Generator().manual_seed(S + D)
+    q = torch.randn(B, S, H, D, generator=g).to(dtype)
+    k = torch.randn(B, S, Hkv, D, generator=g).to(dtype)
+    v = torch.randn(B, S, Hkv, DV, generator=g).to(dtype)
+    dout = torch.randn(B, S, H, DV, generator=g).to(dtype)
+    print(f"softmax bwd D{D} DV{DV} B{B} H{H} Hkv{Hkv} S{S} causal={causal} {dtype}", flush=True)
+    got, ref = _run(hb, "softmax", q, k, v, dout, causal, 1 / math.sqrt(D))
+    _check(got, ref, "softmax")
+
+
+@pytest.mark.parametrize("family", ["sigmoid", "relu"])
+@pytest.mark.parametrize("D,DV,S,causal", [(128, 128, 256, True), (64, 64, 200, False), (128, 128, 130, True)])
+def test_sigmoid_relu_backward(family, D, DV, S, causal):
+    hb = _hb()
+    if family == "relu":
+        causal = False
+    B, H = 1, 2
+    g = torch.Generator().manual_seed(S)
+    q = torch.randn(B, S, H, D, generator=g).half()
+    k = (0.5 * torch.randn(B, S, H, D, generator=g)).half()
+    v = (0.5 * torch.randn(B, S, H, DV, generator=g)).half()
+    dout = (0.1 * torch.randn(B, S, H, DV, generator=g)).half()      # scale of testing/test.py:571
+    print(f"{family} bwd D{D} DV{DV} S{S} causal={causal}", flush=True)
+    got, ref = _run(hb, family, q, k, v, dout, causal, 1 / math.sqrt(D), bias=-1.0 if family == "sigmoid" else 0.0)
+    _check(got, ref, family)
+
+
+def test_backward_mask_is_exact():
+    """Gradients of rows / keys must not depend on anything behind the causal diagonal: poisoning q, dout
+    of later rows leaves dk, dv contributions of earlier rows... checked as: truncating the sequence gives
+    the same dq for the kept rows, bit for bit."""
+    hb = _hb()
+    B, H, S, D = 1, 2, 256, 128
+    g = torch.Generator().manual_seed(1)
+    q, k, v, dout = (torch.randn(B, S, H, D, generator=g).bfloat16().cuda() for _ in range(4))
+    lse = torch.empty(B, H, S, device="cuda")
+    o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=0.1, row_scale=lse)
+    dq, dk, dv = hb.attn_bwd(q, k, v, o, dout, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=0.1)
+    cut = 128
+    q2, k2, v2, do2 = (t[:, :cut].contiguous() for t in (q, k, v, dout))
+    lse2 = torch.empty(B, H, cut, device="cuda")
+    o2 = hb.attn_fwd(q2, k2, v2, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=0.1, row_scale=lse2)
+    dq2, _, _ = hb.attn_bwd(q2, k2, v2, o2, do2, lse2, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=0.1)
+    torch.cuda.synchronize()
+    assert torch.equal(dq[:, :cut], dq2)
+
+
+def test_engine_backward_like_the_reference_test():
+    """testing/test.py:107-125 at a reduced size: o.backward(do) on the operator built from the spec."""
+    B, H, S, D = 1, 4, 512, 128
+    mod = specs.softmax_attention(B, H, S, D, D, dtype=torch.float16)
+    g = torch.Generator().manual_seed(2)
+    q, k, v, dout = (torch.randn(B, S, H, D, generator=g).half() for _ in range(4))
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = mod(qc, kc, vc)
+    o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    ref = oracle.attention_grads(oracle.softmax_attention, q, k, v, dout, causal=True)
+    _check((qc.grad, kc.grad, vc.grad), ref, "engine softmax")
+
+
+def test_engine_sigmoid_backward_with_bias_tensor():
+    """examples/sigmoid_attn.py operator: the bias is a custom input; its gradient slot is None (attn_tl.py:690-691)."""
+    B, H, S, D = 1, 2, 256, 128
+    mod = specs.sigmoid_attention(B, H, S, D, D, dtype=torch.float16)
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(B, S, H, D, generator=g).half()
+    k = (0.5 * torch.randn(B, S, H, D, generator=g)).half()
+    v = torch.randn(B, S, H, D, generator=g).half()
+    dout = (0.1 * torch.randn(B, S, H, D, generator=g)).half()
+    bias = torch.tensor([-2.0])
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = mod(qc, kc, vc, bias.cuda())
+    o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    ref = oracle.attention_grads(oracle.sigmoid_attention, q, k, v, dout, bias=-2.0, causal=True, softmax_scale=1.0)
+    _check((qc.grad, kc.grad, vc.grad), ref, "engine sigmoid")
+
+
+def test_retention_backward_still_raises():
+    B, H, S = 1, 2, 128
+    mod = specs.retention_parallel(B, H, S, 256, 512)
+    q, k, v, _ = inputs.retnet_inputs(B, H, S, 256, 512, seed=1, layout="bshd")
+    mask = oracle.retention_decay_mask(H, S).bfloat16().cuda()
+    qc = q.cuda().requires_grad_(True)
+    o = mod(qc, k.cuda(), v.cuda(), mask)
+    with pytest.raises(NotImplementedError):
+        o.sum().backward()

@@ -228,3 +228,33 @@ def test_grouped_query_equals_repeated_kv_heads():
     torch.testing.assert_close(oracle.relu_attention(q, k, v, **kw), oracle.relu_attention(q, kr, vr, **kw))
     sd = torch.nn.functional.scaled_dot_product_attention(q.transpose(1, 2), kr.transpose(1, 2), vr.transpose(1, 2), is_causal=True)
     torch.testing.assert_close(oracle.softmax_attention(q, k, v, causal=True, **kw), sd.transpose(1, 2))
+
+
+def test_attention_grads_vs_finite_differences_and_sdpa():
+    """The gradient oracle is autograd over the pinned fp64 forward; checked against central
+    differences along random directions and, for softmax, against SDPA's own backward."""
+    g = torch.Generator().manual_seed(9)
+    B, S, H, Hkv, D, DV = 1, 12, 4, 2, 8, 6
+    q = torch.randn(B, S, H, D, generator=g, dtype=torch.float64)
+    k = torch.randn(B, S, Hkv, D, generator=g, dtype=torch.float64)
+    v = torch.randn(B, S, Hkv, DV, generator=g, dtype=torch.float64)
+    dout = torch.randn(B, S, H, DV, generator=g, dtype=torch.float64)
+    cases = [(oracle.softmax_attention, dict(causal=True)), (oracle.sigmoid_attention, dict(bias=-0.7, causal=True, softmax_scale=0.3)),
+             (oracle.relu_attention, dict())]
+    for fwd, kw in cases:
+        dq, dk, dv = oracle.attention_grads(fwd, q, k, v, dout, **kw)
+        f = lambda q_, k_, v_: float((fwd(q_, k_, v_, compute_dtype=torch.float64, **kw) * dout).sum())
+        for t, grad, idx in ((q, dq, 0), (k, dk, 1), (v, dv, 2)):
+            direction = torch.randn(t.shape, generator=g, dtype=torch.float64)
+            eps = 1e-6
+            args_p, args_m = [q, k, v], [q, k, v]
+            args_p[idx], args_m[idx] = t + eps * direction, t - eps * direction
+            fd = (f(*args_p) - f(*args_m)) / (2 * eps)
+            assert abs(fd - float((grad * direction).sum())) < 1e-5 * max(1.0, abs(fd)), (fwd.__name__, idx)
+    qs, ks, vs = (t.clone().requires_grad_(True) for t in (q, k, v))
+    o = torch.nn.functional.scaled_dot_product_attention(qs.transpose(1, 2), ks.repeat_interleave(2, dim=2).transpose(1, 2),
+                                                         vs.repeat_interleave(2, dim=2).transpose(1, 2), is_causal=True)
+    o.transpose(1, 2).backward(dout)
+    dq, dk, dv = oracle.attention_grads(oracle.softmax_attention, q, k, v, dout, causal=True)
+    for a, b in ((dq, qs.grad), (dk, ks.grad), (dv, vs.grad)):
+        torch.testing.assert_close(a, b, rtol=1e-9, atol=1e-9)
