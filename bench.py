@@ -11,6 +11,7 @@ sample of the same workload) and, under "other_workloads", the remaining
 benchmark configurations, each with its own roofline fraction:
 
   c2_sigmoid_causal   same shape, sigmoid(q.k*scale - log S) row function
+  c2_softmax_causal_bwd  backward of the headline workload (dq, dk, dv)
   c3_retnet_chunked   RetNet retention, chunked operator, B8 H16 S2048 Dqk256 Dv512
   c3_retnet_parallel  same shape, normalised parallel operator with a [1,H,S,S] decay mask
   c4_mamba2_ssd       Mamba2 SSD, B8 H64 S2048 P64 N128, one B/C group
@@ -89,6 +90,22 @@ def bench_softmax(steps, warmup, family="softmax"):
     ms = time_gpu(fn, steps, warmup)
     flops = 0.5 * 4.0 * B * H * S * S * D
     return dict(ms=ms, flops=flops, tflops=flops / ms / 1e9, shape=dict(B=B, H=H, S=S, D=D, DV=D, causal=True))
+
+
+def bench_softmax_bwd(steps, warmup):
+    """Backward of the headline workload (dq, dk, dv given o, lse, do).  FLOPs by the usual convention:
+    5 tile products against the forward's 2, causal at one half."""
+    import torch
+    from metaattention_amd import hip_backend as hb
+    B, H, S, D = 8, 32, 4096, 128
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q, k, v, do = (torch.randn(B, S, H, D, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(4))
+    lse = torch.empty(B, H, S, device="cuda", dtype=torch.float32)
+    scale = 1.0 / math.sqrt(D)
+    o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale, row_scale=lse)
+    ms = time_gpu(lambda: hb.attn_bwd(q, k, v, o, do, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale), max(steps // 3, 3), 2)
+    flops = 2.5 * 0.5 * 4.0 * B * H * S * S * D
+    return _mfma_entry(ms, flops, "backward, 2.5 x the forward's algorithmic FLOPs (5 tile products; the two kernels execute 7)")
 
 
 def bench_retnet_chunked(steps, warmup):
@@ -223,6 +240,7 @@ def main():
     others = {}
     want = [w for w in args.only.split(",") if w]
     table = [("c2_sigmoid_causal", "sigmoid", lambda: (lambda r: _mfma_entry(r["ms"], r["flops"]))(bench_softmax(args.steps, args.warmup, "sigmoid"))),
+             ("c2_softmax_causal_bwd", "bwd", lambda: bench_softmax_bwd(args.steps, args.warmup)),
              ("c3_retnet_chunked", "retnet", lambda: bench_retnet_chunked(args.steps, args.warmup)),
              ("c3_retnet_parallel", "retention", lambda: bench_retnet_parallel(args.steps, args.warmup)),
              ("c4_mamba2_ssd", "mamba", lambda: bench_mamba2(args.steps, args.warmup)),
