@@ -254,7 +254,8 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
 // dk, dv
 // ------------------------------------------------------------------------------------------------
 template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
-// (the two [D x 32] accumulators plus the K and V fragments take 192 registers at 128/128: one wave per SIMD there)
+// (the two [D x 32] accumulators plus the K and V fragments take 192 registers at 128/128: one wave per SIMD there;
+// forcing two makes the compiler spill the fragments and is slower)
 __global__ __launch_bounds__(256, (DQK + DV >= 256 ? 1 : 2)) void attn_bwd_dkv_kernel(const AttnBwdArgs a) {
   using E = Elem<T>;
   using x8 = typename E::x8;
@@ -332,14 +333,27 @@ __global__ __launch_bounds__(256, (DQK + DV >= 256 ? 1 : 2)) void attn_bwd_dkv_k
     float lse2[16], dl[16];
     if constexpr (FAMILY == BF_SOFTMAX) {
       const int64_t rbase = ((int64_t)b * a.H + h) * a.Sq;
+      if ((a.Sq & 3) == 0 && m0 + BMT <= a.Sq) {   // whole tile, 16-byte aligned groups of four rows
 #pragma unroll
-      for (int q4 = 0; q4 < 4; q4++)
+        for (int q4 = 0; q4 < 4; q4++) {
+          const f32x4 tl = *(const f32x4*)(a.lse + rbase + m0 + 8 * q4 + 4 * g);
+          const f32x4 td = *(const f32x4*)(a.delta + rbase + m0 + 8 * q4 + 4 * g);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const int m = min(m0 + 8 * q4 + 4 * g + i, a.Sq - 1);
-          lse2[4 * q4 + i] = a.lse[rbase + m] * kLog2e;
-          dl[4 * q4 + i] = a.delta[rbase + m];
+          for (int i = 0; i < 4; i++) {
+            lse2[4 * q4 + i] = tl[i] * kLog2e;
+            dl[4 * q4 + i] = td[i];
+          }
         }
+      } else {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int m = min(m0 + 8 * q4 + 4 * g + i, a.Sq - 1);
+            lse2[4 * q4 + i] = a.lse[rbase + m] * kLog2e;
+            dl[4 * q4 + i] = a.delta[rbase + m];
+          }
+      }
     }
     const f32x16 s = mm_rows<T, DQK>(qbase, r, g, kf);     // S: lane = key n_lane, element jj = row m0 + 8(jj/4) + 4g + jj%4
     const f32x16 dp = mm_rows<T, DV>(dobase, r, g, vf);   // dP, same layout
