@@ -118,6 +118,7 @@ typedef struct ma_linear_params {
   const float* v_scale;
   float q_scale;
   int32_t segments; /* 0 = let the library choose; 1 = single pass; n = cut the sequence into at most n segments */
+  int32_t out_fp32; /* non-zero: o is fp32 [B,H,T,Dv] (the backward pass builds the decay gradient from such outputs) */
   void* workspace; size_t workspace_bytes; /* see ma_linear_workspace_bytes; may be NULL (then single pass) */
 } ma_linear_params;
 

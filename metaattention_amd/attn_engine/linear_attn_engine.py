@@ -17,6 +17,30 @@ from core.eager import evaluate, custom_tensor_view
 from core.transform.core import CustomIO
 
 
+class _LinearAttention(torch.autograd.Function):
+    """Forward + backward of the chunked operator on (q, k, v, log decay, value scale), as LinearAttention
+    of tl_template/linear/linear_tl.py:1240-1340; the mods around it (decay_mod, the tensors behind v_mod)
+    are ordinary PyTorch operations, so autograd carries the gradients on to decay, A, dt."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, g, v_scale, q_scale, chunk):
+        from hip_backend import linear_fwd
+        ctx.q_scale = q_scale
+        ctx.has_vs = v_scale is not None
+        ctx.save_for_backward(q, k, v, g, *([v_scale] if v_scale is not None else []))
+        return linear_fwd(q, k, v, g, q_scale=q_scale, v_scale=v_scale, chunk=chunk)
+
+    @staticmethod
+    def backward(ctx, dout):
+        from hip_backend import linear_bwd
+        q, k, v, g, *rest = ctx.saved_tensors
+        vs = rest[0] if ctx.has_vs else None
+        dq, dk, dv, dg, dvs = linear_bwd(q, k, v, g, dout, q_scale=ctx.q_scale, v_scale=vs)
+        if dvs is not None:
+            dvs = dvs.to(vs.dtype)
+        return dq, dk, dv, dg.to(g.dtype), dvs, None, None
+
+
 class LinearAttentionEngine:
     def __init__(self, qkv_meta, q_mod=None, k_mod=None, v_mod=None, decay_mod=None, custom_io=None,
                  tune=False, tune_filename="tune_result", tune_bwd=False, chunk_size=None):
@@ -60,13 +84,9 @@ class LinearAttentionEngine:
         g = self._log_decay(decay.to(torch.float32), given)
         v_scale = given[self.plan.v_scale_tensor] if self.plan.v_scale_tensor else None
 
-        def run(q, k, v):
-            return linear_fwd(q, k, v, g, q_scale=self.plan.q_scale, v_scale=v_scale, chunk=self.chunk_size)
-
-        if any(t.requires_grad for t in (q, k, v)):
-            from .attn_engine import _ForwardOnly
-            return _ForwardOnly.apply(run, q, k, v)
-        return run(q, k, v)
+        if any(t is not None and t.requires_grad for t in (q, k, v, g, v_scale)):
+            return _LinearAttention.apply(q, k, v, g, v_scale, self.plan.q_scale, self.chunk_size)
+        return linear_fwd(q, k, v, g, q_scale=self.plan.q_scale, v_scale=v_scale, chunk=self.chunk_size)
 
     def __call__(self, *args, **kargs):
         return self.attention(*args, **kargs)

@@ -145,6 +145,7 @@ static ma::LinArgs linear_args(const ma_linear_params* p) {
   ma::LinArgs a{};
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.log_decay = p->log_decay; a.v_scale = p->v_scale;
   a.q_scale = p->q_scale;
+  a.out_f32 = p->out_fp32 != 0;
   a.B = p->batch; a.H = p->heads; a.Hq = p->heads_q; a.Hk = p->heads_k; a.T = p->seqlen; a.Dv = p->dim_v;
   return a;
 }

@@ -389,7 +389,32 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
     // ---- write this wave's [32 tokens x 32 columns] block: stage (wave private), then 16-byte row pieces.
     //      With ALIAS_OST the staging block is the wave's own 4 chunks per row of the V tile just consumed
     //      (only this wave reads them, and the next DMA into this buffer is issued behind the next barrier).
-    if constexpr (MODE != 1) {
+    if (MODE != 1 && a.out_f32) {
+      // fp32 outputs (used by the backward pass, whose decay gradient is a difference of sums over these
+      // values): the same staging block, 16 columns at a time
+      const int sw_r = swz_tile<CPRV>(r);
+      float* ob32 = (float*)a.o + (int64_t)bh * Tn * a.Dv + dvb * (32 * NWH) + 32 * (wave % NWH);
+#pragma unroll
+      for (int half = 0; half < 2; half++) {
+#pragma unroll
+        for (int q2 = 0; q2 < 2; q2++) {
+          const int q4 = 2 * half + q2;
+          f32x4 w;
+#pragma unroll
+          for (int i = 0; i < 4; i++)
+            w[i] = (DK < 256 && HG == 1 ? o_inter[4 * q4 + i] + o_inter2[4 * q4 + i] : o_inter[4 * q4 + i]) * eg + o_intra[4 * q4 + i];
+          if (ALIAS_OST) lds_write<f32x4>(vbase + r * RBV + (uint32_t)(((4 * wave + 2 * q2 + g) ^ sw_r) << 4), w);
+          else lds_write<f32x4>(lds_ost + r * OROW + (8 * q2 + 4 * g) * 4, w);
+        }
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+          const int ci = ln + 64 * it, row = ci >> 2, cc = ci & 3;
+          const u32x4 w = ALIAS_OST ? lds_read<u32x4>(vbase + row * RBV + (uint32_t)(((4 * wave + cc) ^ swz_tile<CPRV>(row)) << 4))
+                                    : lds_read<u32x4>(lds_ost + row * OROW + cc * 16);
+          if (t0 + row < Tn) *(u32x4*)(ob32 + (int64_t)(t0 + row) * a.Dv + 16 * half + cc * 4) = w;
+        }
+      }
+    } else if constexpr (MODE != 1) {
       const int sw_r = swz_tile<CPRV>(r);
 #pragma unroll
       for (int q4 = 0; q4 < 4; q4++) {

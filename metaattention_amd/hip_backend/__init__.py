@@ -75,7 +75,7 @@ class LinearParams(Structure):
         ("seqlen", c_int32), ("dim_k", c_int32), ("dim_v", c_int32), ("chunk", c_int32),
         ("q", c_void_p), ("k", c_void_p), ("v", c_void_p), ("o", c_void_p),
         ("log_decay", c_void_p), ("v_scale", c_void_p),
-        ("q_scale", c_float), ("segments", c_int32),
+        ("q_scale", c_float), ("segments", c_int32), ("out_fp32", c_int32),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
     ]
 
@@ -270,7 +270,7 @@ def mla_workspace_bytes(B, Hq, Skv, D=512, Dpe=64, num_split=0) -> int:
 
 
 def linear_fwd(q, k, v, log_decay, *, q_scale: float = 1.0, v_scale=None, chunk=None, out=None, segments: int = 0,
-               workspace=None):
+               workspace=None, out_fp32: bool = False):
     """Chunked linear attention forward on BHSD tensors: q [B,Hq,T,Dk], k [B,Hk,T,Dk],
     v [B,H,T,Dv] (bf16, contiguous), log_decay fp32 [B,H,T], optional per-token value
     scale [B,H,T].  ``chunk`` is accepted for API compatibility; the result does not
@@ -289,8 +289,10 @@ def linear_fwd(q, k, v, log_decay, *, q_scale: float = 1.0, v_scale=None, chunk=
         assert v_scale.shape == (B, H, T)
         v_scale = v_scale.to(torch.float32).contiguous()
     if out is None:
-        out = torch.empty(B, H, T, Dv, dtype=v.dtype, device=v.device)
+        out = torch.empty(B, H, T, Dv, dtype=torch.float32 if out_fp32 else v.dtype, device=v.device)
+    assert out.dtype == (torch.float32 if out_fp32 else v.dtype) and out.is_contiguous()
     p = LinearParams()
+    p.out_fp32 = int(out_fp32)
     p.dtype = _dtype_code(v.dtype)
     p.batch, p.heads, p.heads_q, p.heads_k, p.seqlen, p.dim_k, p.dim_v = B, H, Hq, Hk, T, Dk, Dv
     p.chunk = int(chunk or 0)
@@ -308,6 +310,66 @@ def linear_fwd(q, k, v, log_decay, *, q_scale: float = 1.0, v_scale=None, chunk=
         p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
     _check(lib.ma_linear_fwd(ctypes.byref(p), _stream()))
     return out
+
+
+def _linear_any_width(q, k, v, log_decay, q_scale, v_scale=None):
+    """linear_fwd with fp32 outputs for any key width: the kernels contract over 128 or 256 key columns;
+    narrower keys are zero-padded, wider ones are cut into slices of 256 whose results add (the operator
+    is linear in q.k)."""
+    D = q.shape[-1]
+    if D in (128, 256):
+        return linear_fwd(q, k, v, log_decay, q_scale=q_scale, v_scale=v_scale, out_fp32=True)
+    if D < 256:
+        W = 128 if D < 128 else 256
+        pad = lambda t: torch.nn.functional.pad(t, (0, W - D))
+        return linear_fwd(pad(q), pad(k), v, log_decay, q_scale=q_scale, v_scale=v_scale, out_fp32=True)
+    acc = None
+    for c0 in range(0, D, 256):
+        part = _linear_any_width(q[..., c0:c0 + 256].contiguous(), k[..., c0:c0 + 256].contiguous(), v, log_decay, q_scale, v_scale)
+        acc = part if acc is None else acc + part
+    return acc
+
+
+def linear_bwd(q, k, v, log_decay, dout, *, q_scale: float = 1.0, v_scale=None):
+    """Gradients of linear_fwd with respect to q, k, v, log_decay and v_scale (None when no v_scale).
+
+    With A_ts = q_scale (q_t.k_s) exp(G_t - G_s) [s <= t] and u = v * v_scale, o = A u and
+        dq_t = q_scale sum_{s<=t} exp(G_t-G_s) (do_t.u_s) k_s
+        du_s = sum_{t>=s} A_ts do_t,      dk_s = q_scale sum_{t>=s} exp(G_t-G_s) (do_t.u_s) q_t
+    are the SAME operator on permuted (and, for the two sums over later tokens, time-reversed) inputs:
+        dq = LA(do, v, k; v_scale),   du = flip LA(flip k, flip q, flip do),   dk = v_scale * flip LA(flip v, flip do, flip q)
+    with the reversed log decay shifted by one token.  So the backward pass is three launches of the
+    parity-tested forward kernel plus element-wise glue; heads that share a q / k head have their
+    gradients summed, as LinearAttention.backward does (linear_tl.py:1300-1303).  The decay gradient
+    follows from dG_t = q_t.dq_t - k_t.dk_t and G = cumsum(log_decay) (a reversed cumulative sum,
+    compute_final_dg of the reference)."""
+    _require_gpu(q, k, v, log_decay, dout, v_scale)
+    B, H, T, Dv = v.shape
+    Hq, Hk, Dk = q.shape[1], k.shape[1], q.shape[-1]
+    g = log_decay.to(torch.float32).contiguous()
+    vs = v_scale.to(torch.float32).contiguous() if v_scale is not None else None
+    dout = dout.to(v.dtype).contiguous()
+    flip = lambda t: torch.flip(t, dims=(2,)).contiguous()
+    expand = lambda t, h: t if t.shape[1] == H else t.repeat_interleave(H // h, dim=1)
+    qe, ke = expand(q, Hq), expand(k, Hk)
+    g_rev = torch.zeros_like(g)
+    if T > 1:
+        g_rev[:, :, 1:] = torch.flip(g, dims=(2,))[:, :, :-1]          # g_rev[t'] = g[T - t'], t' >= 1
+    dq_h = _linear_any_width(dout, v, ke, g, q_scale, vs)                                     # [B,H,T,Dk]
+    du = flip(_linear_any_width(flip(k), flip(q), flip(dout), g_rev, q_scale))                # [B,H,T,Dv]
+    dk_h = flip(_linear_any_width(flip(v), flip(dout), flip(qe), g_rev, q_scale))             # [B,H,T,Dk], before the v_scale factor
+    # (dq_h, du, dk_h are fp32 from here on)
+    if vs is not None:
+        dk_h = dk_h * vs.unsqueeze(-1)
+        dv = (du * vs.unsqueeze(-1)).to(v.dtype)
+        dvs = (v.float() * du).sum(-1)
+    else:
+        dv, dvs = du.to(v.dtype), None
+    dG = (qe.float() * dq_h).sum(-1) - (ke.float() * dk_h).sum(-1)                            # [B,H,T]
+    dld = torch.flip(torch.cumsum(torch.flip(dG, dims=(2,)), dim=2), dims=(2,))
+    dq = (dq_h if Hq == H else dq_h.view(B, Hq, H // Hq, T, Dk).sum(2)).to(q.dtype)
+    dk = (dk_h if Hk == H else dk_h.view(B, Hk, H // Hk, T, Dk).sum(2)).to(k.dtype)
+    return dq, dk, dv, dld, dvs
 
 
 def linear_workspace_bytes(B, H, Hq, Hk, T, Dk, Dv, segments: int = 0) -> int:

@@ -27,8 +27,8 @@ ssd_chunk_scan         3-way agreement: chunked reference == naive sequential
                        state-space recurrence; chunk-size independence
 simple_gla             token-by-token recurrence (fp64)
 mla_decode             SDPA with K=concat(kv,k_pe), V=kv; split-KV invariance
-attention_grads        central differences of the pinned forward functions in
-                       fp64 along random directions; SDPA's own autograd
+attention_grads,       central differences of the pinned forward functions in
+linear_attention_grads fp64 along random directions; SDPA's own autograd
 (all of the above)     tests/golden/*.npz: the operators' definitions evaluated
                        element by element in fp64 numpy by independent code
 =====================  =====================================================
@@ -52,6 +52,7 @@ from .linear_ref import (  # noqa: F401
     ssd_sequential,
     simple_gla_chunked,
     simple_gla_recurrence,
+    linear_attention_grads,
 )
 from .compare import assert_close, mismatch_report  # noqa: F401
 from . import inputs  # noqa: F401

@@ -186,3 +186,17 @@ def simple_gla_recurrence(q, k, v, g, scale: Optional[float] = None, compute_dty
                     torch.outer(k[b, h, t].to(compute_dtype), v[b, h, t].to(compute_dtype))
                 out[b, h, t] = (q[b, h, t].to(compute_dtype) * scale) @ S
     return out
+
+
+def linear_attention_grads(q, k, v, log_decay, dout, q_scale: float = 1.0, v_scale: Optional[torch.Tensor] = None, chunk: int = 16):
+    """Gradients of sum(linear_attention_chunked(...) * dout) with respect to q, k, v, log_decay and
+    v_scale (None without one), by PyTorch autograd over the fp64 chunked form - the way the
+    reference's tests obtain reference gradients (testing/test.py:360-361, 483-484: ``o_ref.backward(do)``)."""
+    T = q.shape[2]
+    while T % chunk:
+        chunk //= 2
+    leaves = [t.detach().to(torch.float64).requires_grad_(True) for t in (q, k, v, log_decay)]
+    vs = v_scale.detach().to(torch.float64).requires_grad_(True) if v_scale is not None else None
+    out = linear_attention_chunked(*leaves, chunk=max(chunk, 1), q_scale=q_scale, v_scale=vs, compute_dtype=torch.float64)
+    out.backward(dout.to(torch.float64))
+    return tuple(t.grad for t in leaves) + ((vs.grad,) if vs is not None else (None,))

@@ -1,0 +1,113 @@
+"""Gradients of the chunked linear / stateful operators (q, k, v, log decay, value scale) against the
+gradient oracle (autograd over the fp64 chunked form, as the reference's tests obtain theirs).
+q, k, v gradients at atol 2e-2 / rtol 1e-2 with a small allowance for the bf16 rounding of the
+intermediate gradients (the reference's own checks: rtol = atol = 1e-1, testing/test.py:364-385,
+488-505, which is also asserted); the decay and value-scale gradients, which the reference's tests
+leave unchecked (:386-397, :506-511), are sums of bf16-rounded products over the head dimension and
+are held to 5 % of their largest magnitude (at least 1e-2)."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from oracle import inputs
+import specs
+
+pytestmark = pytest.mark.gpu
+ATOL, RTOL = 2e-2, 1e-2
+
+
+def _hb():
+    from metaattention_amd import hip_backend as hb
+    hb.load_library()
+    return hb
+
+
+def _check(got, ref, what):
+    names = ("dq", "dk", "dv", "dlog_decay", "dv_scale")
+    for name, a, b in zip(names, got, ref):
+        if b is None:
+            assert a is None
+            continue
+        a, b = a.float().cpu(), b.float()
+        if name in ("dq", "dk", "dv"):
+            oracle.assert_close(a, b, rtol=1e-1, atol=1e-1, mismatch_ratio=1e-2, msg=f"{what}:{name} (reference acceptance)")
+            oracle.assert_close(a, b, rtol=RTOL, atol=ATOL, mismatch_ratio=5e-3, msg=f"{what}:{name}")
+        else:
+            tol = max(0.05 * float(b.abs().max()), 1e-2)
+            assert float((a - b).abs().max()) <= tol, f"{what}:{name}: {float((a - b).abs().max())} > {tol}"
+
+
+@pytest.mark.parametrize("B,Hq,H,T,Dk,Dv,use_vs", [
+    (1, 2, 2, 256, 256, 256, False),    # gated retention (testing/test.py:58 head sizes)
+    (1, 2, 2, 200, 256, 512, False),    # RetNet head sizes: the dq / dk launches contract over 512 = 2 x 256
+    (2, 1, 4, 256, 128, 64, True),      # Mamba2: one q/k head for all heads, value scale, 64-wide contraction padded
+    (1, 2, 4, 100, 128, 128, True),
+    (1, 1, 1, 1, 128, 64, False),
+])
+def test_linear_backward(B, Hq, H, T, Dk, Dv, use_vs):
+    hb = _hb()
+    g = torch.Generator().manual_seed(T + Dv)
+    q = torch.randn(B, Hq, T, Dk, generator=g).bfloat16()
+    k = (0.1 * torch.randn(B, Hq, T, Dk, generator=g)).bfloat16()
+    v = torch.randn(B, H, T, Dv, generator=g).bfloat16()
+    ld = torch.nn.functional.logsigmoid(torch.randn(B, H, T, generator=g) + 3.0)
+    vs = (torch.rand(B, H, T, generator=g) + 0.5) if use_vs else None
+    dout = (0.5 * torch.randn(B, H, T, Dv, generator=g)).bfloat16()
+    q_scale = Dk ** -0.5
+    print(f"linear bwd B{B} H{H}/{Hq} T{T} Dk{Dk} Dv{Dv} v_scale={use_vs}", flush=True)
+    got = hb.linear_bwd(q.cuda(), k.cuda(), v.cuda(), ld.cuda(), dout.cuda(), q_scale=q_scale, v_scale=vs.cuda() if use_vs else None)
+    torch.cuda.synchronize()
+    ref = oracle.linear_attention_grads(q, k, v, ld, dout, q_scale=q_scale, v_scale=vs)
+    _check(got, ref, "linear")
+
+
+def test_engine_mamba2_backward():
+    """mod(C, B, x, dt, A, dt_bf16) as testing/test.py:198-204 followed by o.backward(do): gradients reach
+    C, B, x and, through the eager mods, dt and A."""
+    B, H, T, P, N = 1, 8, 256, 64, 128
+    mod = specs.mamba2(B, 1, T, N, P, HK=1, HV=H)
+    Cm, Bm, x, dt, A = inputs.mamba2_inputs(B, H, T, P, N, seed=7)
+    dout = (0.5 * torch.randn(B, H, T, P, generator=torch.Generator().manual_seed(1))).bfloat16()
+    Cc, Bc, xc = (t.cuda().requires_grad_(True) for t in (Cm, Bm, x))
+    dtc, Ac = dt.cuda().requires_grad_(True), A.cuda().requires_grad_(True)
+    o = mod(Cc, Bc, xc, dtc, Ac, dtc.bfloat16())
+    o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    # oracle: the same composition in fp64 (log decay = dt * A, value scale = the bf16 copy of dt)
+    dt64, A64 = dt.double().requires_grad_(True), A.double().requires_grad_(True)
+    q64, k64, v64 = (t.double().requires_grad_(True) for t in (Cm, Bm, x))
+    out = oracle.linear_attention_chunked(q64, k64, v64, dt64 * A64.view(1, H, 1), chunk=64, v_scale=dt64.bfloat16().double(),
+                                          compute_dtype=torch.float64)
+    out.backward(dout.double())
+    _check((Cc.grad, Bc.grad, xc.grad), (q64.grad, k64.grad, v64.grad), "mamba2")
+    tol = max(0.05 * float(dt64.grad.abs().max()), 1e-2)
+    err = float((dtc.grad.double().cpu() - dt64.grad).abs().max())
+    assert err <= tol, f"ddt: {err} > {tol}"
+    # dA_h = sum_t dlog_decay_t dt_t = sum_j dG_j C_j with C_j = sum_{t<=j} dt_t (up to ~40 here): a residual of T large terms
+    # of both signs.  Every dG_j carries the relative 2^-8 of the bf16 intermediates inside the kernels (scores, state), so
+    # the bound that can be asserted is 1 % of sum_j |dG_j| C_j; per-token accuracy is what the ddt check above pins.
+    dld_ref = oracle.linear_attention_grads(Cm, Bm, x, dt * A.view(1, H, 1), dout, v_scale=dt.bfloat16().float())[3]
+    dG_ref = dld_ref - torch.cat([dld_ref[:, :, 1:], torch.zeros(B, H, 1, dtype=dld_ref.dtype)], dim=2)
+    tol_a = 1e-2 * (dG_ref.abs() * torch.cumsum(dt.double(), dim=2)).sum(dim=(0, 2))
+    err_a = (Ac.grad.double().cpu().view(-1) - A64.grad.view(-1)).abs()
+    assert bool((err_a <= tol_a).all()), f"dA: {err_a} > {tol_a}"
+
+
+def test_engine_retnet_backward():
+    """testing/test.py:749-800: q, k, v gradients of the RetNet operator."""
+    B, H, T, Dk, Dv = 1, 4, 256, 256, 512
+    mod = specs.retnet_recurrent(B, H, T, Dk, Dv)
+    gen = torch.Generator().manual_seed(5)
+    q = torch.randn(B, H, T, Dk, generator=gen).bfloat16()
+    k = (0.1 * torch.randn(B, H, T, Dk, generator=gen)).bfloat16()
+    v = torch.randn(B, H, T, Dv, generator=gen).bfloat16()
+    dout = (0.5 * torch.randn(B, H, T, Dv, generator=gen)).bfloat16()
+    decay = (1 - torch.exp2(-5 - torch.arange(H, dtype=torch.float32)))[None, :, None].expand(B, H, T).contiguous()
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = mod(qc, kc, vc, decay.cuda())
+    o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    ref = oracle.linear_attention_grads(q, k, v, torch.log(decay), dout, q_scale=Dk ** -0.5)
+    _check((qc.grad, kc.grad, vc.grad), ref[:3], "retnet")

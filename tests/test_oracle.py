@@ -258,3 +258,25 @@ def test_attention_grads_vs_finite_differences_and_sdpa():
     dq, dk, dv = oracle.attention_grads(oracle.softmax_attention, q, k, v, dout, causal=True)
     for a, b in ((dq, qs.grad), (dk, ks.grad), (dv, vs.grad)):
         torch.testing.assert_close(a, b, rtol=1e-9, atol=1e-9)
+
+
+def test_linear_attention_grads_vs_finite_differences():
+    g = torch.Generator().manual_seed(11)
+    B, Hq, H, T, Dk, Dv = 1, 1, 2, 24, 6, 5
+    q = torch.randn(B, Hq, T, Dk, generator=g, dtype=torch.float64)
+    k = torch.randn(B, Hq, T, Dk, generator=g, dtype=torch.float64)
+    v = torch.randn(B, H, T, Dv, generator=g, dtype=torch.float64)
+    ld = -torch.rand(B, H, T, generator=g, dtype=torch.float64)
+    vs = torch.rand(B, H, T, generator=g, dtype=torch.float64) + 0.5
+    dout = torch.randn(B, H, T, Dv, generator=g, dtype=torch.float64)
+    grads = oracle.linear_attention_grads(q, k, v, ld, dout, q_scale=0.4, v_scale=vs, chunk=8)
+    args = [q, k, v, ld, vs]
+    f = lambda a: float((oracle.linear_attention_chunked(a[0], a[1], a[2], a[3], chunk=8, q_scale=0.4, v_scale=a[4],
+                                                         compute_dtype=torch.float64) * dout).sum())
+    for idx, grad in enumerate(grads):
+        direction = torch.randn(args[idx].shape, generator=g, dtype=torch.float64)
+        eps = 1e-6
+        ap, am = list(args), list(args)
+        ap[idx], am[idx] = args[idx] + eps * direction, args[idx] - eps * direction
+        fd = (f(ap) - f(am)) / (2 * eps)
+        assert abs(fd - float((grad * direction).sum())) < 1e-5 * max(1.0, abs(fd)), idx
