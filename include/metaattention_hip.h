@@ -75,6 +75,14 @@ typedef struct ma_attn_params {
   /* grouped-query attention (attn_gqa_tl.py:21-24, :80, :95): k and v have heads_kv heads and query
    * head h reads kv head h / (heads / heads_kv); 0 means heads_kv = heads */
   int32_t heads_kv;
+  /* decode-style kv selection (blockattn_decode_varlen_tl.py:16, :57-75); both optional:
+   * kv_seqlens int32 [B]: keys at or beyond kv_seqlens[b] do not exist for batch entry b;
+   * kv_block_mask uint8/bool [B, heads_kv, ceil(Skv / kv_block_size)]: blocks of kv_block_size keys
+   * (a multiple of 32) whose entry is 0 are skipped for that (batch, kv head).  A row left with no
+   * key at all gets zeros (lse = -inf). */
+  int32_t kv_block_size;
+  const int32_t* kv_seqlens;
+  const uint8_t* kv_block_mask; int64_t kbm_stride_b, kbm_stride_h;
 } ma_attn_params;
 
 /* Parallel attention backward for the SOFTMAX, SIGMOID and RELU families.  Replaces the backward of

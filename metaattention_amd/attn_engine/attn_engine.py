@@ -114,13 +114,18 @@ class AttentionEngine:
                  extern_block_mask=False, use_varlen=False, kv_shared=False):
         # `backend`, `tune*`, `infer_mask*` select code generators / tuners in the
         # reference; here there is one pre-built backend and fixed tile tables, so
-        # they are accepted and ignored.
+        # they are accepted and ignored, except infer_mask_block_N: the block size of an
+        # external kv block mask (examples/sparse_gqa_decode.py:100-107).
         self.device = device if device is not None else MI355X()
         self.use_varlen = use_varlen
         self.block_mask = None
         self.tl_code = ""     # no source is generated
-        if use_varlen or extern_block_mask:
-            raise NotImplementedError("varlen / external block masks are not in the kernel library")
+        self.extern_block_mask = extern_block_mask
+        self.kv_block_size = int(infer_mask_block_N)
+        if (use_varlen or extern_block_mask) and (self.kv_block_size < 32 or self.kv_block_size % 32 != 0):
+            raise NotImplementedError("kv block masks need a block size that is a multiple of 32 (infer_mask_block_N)")
+        if (use_varlen or extern_block_mask) and (kv_shared or qkv_meta[0].shape[2] == qkv_meta[2].shape[2]):
+            raise NotImplementedError("varlen / external block masks are only in the decode operators of the kernel library")
         dtype = qkv_meta[0].dtype
         if dtype not in (torch.float16, torch.bfloat16):
             raise KeyError(dtype)      # the reference's dtype map has only these two (attn_engine.py:234-237)
@@ -170,7 +175,7 @@ class AttentionEngine:
         self.final_rowscales = None
         self.attention = self._call_prefill
 
-    def _call_prefill(self, q, k, v, *custom):
+    def _call_prefill(self, q, k, v, *custom, block_mask=None, cache_seqlens=None):
         from hip_backend import attn_fwd, MA_ATTN_SOFTMAX, MA_ATTN_SIGMOID, MA_ATTN_RELU, MA_ATTN_RETENTION
         fam_code = {"softmax": MA_ATTN_SOFTMAX, "sigmoid": MA_ATTN_SIGMOID, "relu": MA_ATTN_RELU,
                     "retention": MA_ATTN_RETENTION}[self.family]
@@ -179,17 +184,44 @@ class AttentionEngine:
         given = dict(zip(self.names, custom))
         form = self.score_form
 
+        sparse = block_mask is not None or cache_seqlens is not None
+        if sparse and (self.mask_kind == "causal" or self.family == "retention"):
+            raise NotImplementedError("block_mask / cache_seqlens are for the unmasked decode operators")
+        if block_mask is not None and block_mask.dim() != 3:
+            raise NotImplementedError("only kv block masks [batch, heads_kv, blocks] (decode) are in the kernel library; "
+                                      "block-sparse prefill masks [batch, heads, q blocks, kv blocks] are not")
+
         def run(q, k, v):
-            B, Sq, H, _ = q.shape
-            rs = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if self.family in ("softmax", "retention") else None
-            bias_t = given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None
+            B, Sq, H, D = q.shape
+            Hkv, Dv = k.shape[2], v.shape[-1]
+            grp = H // Hkv
+            kw = dict(family=fam_code, causal=self.mask_kind == "causal", scale=form.scale, bias=form.bias,
+                      bias_tensor=given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None)
+            if sparse:
+                kw.update(kv_seqlens=cache_seqlens.to(torch.int32) if cache_seqlens is not None else None, kv_block_mask=block_mask,
+                          kv_block_size=self.kv_block_size if block_mask is not None else 0)
+            has_rs = self.family in ("softmax", "retention")
+            if Sq == 1 and grp > 1 and self.mask_kind != "causal" and self.family != "retention":
+                # one query token, grouped-query: the query heads of a kv head become the rows of that head
+                # (the decode kernels of the reference pack them the same way, attn_gqa_decode_tl.py:81-84)
+                out = torch.empty(B, 1, H, Dv, dtype=q.dtype, device=q.device)
+                rs = torch.empty(B, Hkv, grp, dtype=torch.float32, device=q.device) if has_rs else None
+                attn_fwd(q.contiguous().view(B, Hkv, grp, D).transpose(1, 2), k, v, out=out.view(B, Hkv, grp, Dv).transpose(1, 2),
+                         row_scale=rs, **kw)
+                self.final_rowscales = rs.view(B, H, 1) if has_rs else None
+                return out
+            rs = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if has_rs else None
             mask_t = given[form.mask_tensor] if form.mask_tensor else None
             if mask_t is not None and mask_t.dtype != q.dtype:
                 mask_t = mask_t.to(q.dtype)
-            out = attn_fwd(q, k, v, family=fam_code, causal=self.mask_kind == "causal", scale=form.scale, bias=form.bias,
-                           bias_tensor=bias_t, score_mask=mask_t, row_scale=rs)
+            out = attn_fwd(q, k, v, score_mask=mask_t, row_scale=rs, **kw)
             self.final_rowscales = rs     # kept for a backward pass, not returned (attn_tl.py:661-667)
             return out
+
+        if sparse:
+            # the varlen block-sparse decode operator squeezes the query token and has no backward
+            # (blockattn_decode_varlen_tl.py:17, :250)
+            return run(q, k, v).squeeze(1)
 
         if any(t.requires_grad for t in (q, k, v)):
             if self.family == "retention":
@@ -216,6 +248,9 @@ class AttentionEngine:
         return mla_decode(q, q_pe, kv, k_pe, scale=self.mla_scale)
 
     def __call__(self, *args, **kargs):
-        if kargs.get("block_mask") is not None:
-            raise NotImplementedError("block masks are not in the kernel library")
-        return self.attention(*args)
+        block_mask, cache_seqlens = kargs.get("block_mask"), kargs.get("cache_seqlens")
+        if block_mask is None and cache_seqlens is None:
+            return self.attention(*args)
+        if self.attention != self._call_prefill:
+            raise NotImplementedError("block_mask / cache_seqlens are not taken by this operator")
+        return self._call_prefill(*args, block_mask=block_mask, cache_seqlens=cache_seqlens)

@@ -40,6 +40,10 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
     return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: causal mask needs seqlen_q == seqlen_kv (%d vs %d)", p->seqlen_q, p->seqlen_kv);
   if (p->heads_kv < 0 || (p->heads_kv > 0 && p->heads % p->heads_kv != 0))
     return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: heads (%d) must be a multiple of heads_kv (%d)", p->heads, p->heads_kv);
+  if (p->kv_block_mask && (p->kv_block_size < 32 || p->kv_block_size % 32 != 0))
+    return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: kv_block_size must be a positive multiple of 32 (got %d)", p->kv_block_size);
+  if ((p->kv_block_mask || p->kv_seqlens) && p->mask == MA_MASK_CAUSAL)
+    return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: kv_seqlens / kv_block_mask are for the unmasked (decode) operators");
   if (p->family == MA_ATTN_RETENTION) {
     if (!p->score_mask) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: RETENTION needs score_mask");
     if ((uintptr_t)p->score_mask % 8 != 0 || p->sm_stride_b % 4 != 0 || p->sm_stride_h % 4 != 0 || p->sm_stride_q % 4 != 0)
@@ -63,6 +67,9 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
   a.msb = p->sm_stride_b; a.msh = p->sm_stride_h; a.msq = p->sm_stride_q;
   a.B = p->batch; a.H = p->heads; a.Sq = p->seqlen_q; a.Skv = p->seqlen_kv;
   a.kv_group = p->heads_kv > 0 ? p->heads / p->heads_kv : 1;
+  a.kv_lens = p->kv_seqlens;
+  a.kv_block_mask = p->kv_block_mask; a.kbm_sb = p->kbm_stride_b; a.kbm_sh = p->kbm_stride_h;
+  a.kv_block = p->kv_block_size;
   a.scale = p->scale; a.bias = p->bias;
   const int rc = ma::attn_fwd_dispatch(a, p->family, p->mask == MA_MASK_CAUSAL, p->dtype == MA_BF16, p->dim_qk, p->dim_v,
                                        (hipStream_t)stream);

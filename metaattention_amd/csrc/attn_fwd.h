@@ -12,6 +12,12 @@ struct AttnArgs {
   int64_t qsb, qss, qsh, ksb, kss, ksh, vsb, vss, vsh, osb, oss, osh, msb, msh, msq;
   int B, H, Sq, Skv, num_m_blocks;
   int kv_group;   // query heads per kv head (1 unless grouped-query)
+  // decode-style kv selection (attn_wide_fwd_kernel only): per-batch cache length and a per-(batch, kv head)
+  // mask over blocks of kv_block keys (a multiple of 32)
+  const int32_t* kv_lens;
+  const uint8_t* kv_block_mask;
+  int64_t kbm_sb, kbm_sh;
+  int kv_block;
   float scale, bias;
 };
 

@@ -77,8 +77,18 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
   const T* mrow = nullptr;
   if constexpr (FAMILY == WF_RETENTION) mrow = (const T*)a.smask + (int64_t)b * a.msb + (int64_t)h * a.msh + (int64_t)m_ld * a.msq;
 
-  int n_tiles = (a.Skv + BN - 1) / BN;
+  // keys beyond this batch entry's cache length do not exist (blockattn_decode_varlen_tl.py:66-75)
+  const int skv = a.kv_lens ? min(a.Skv, max(a.kv_lens[b], 0)) : a.Skv;
+  int n_tiles = (skv + BN - 1) / BN;
   if (CAUSAL) n_tiles = min(n_tiles, (mb * BM + BM + BN - 1) / BN);
+  // tiles whose block of keys is switched off for this (batch, kv head) are skipped (:57-64)
+  const uint8_t* bm_row = a.kv_block_mask ? a.kv_block_mask + (int64_t)b * a.kbm_sb + (int64_t)(h / a.kv_group) * a.kbm_sh : nullptr;
+  const int tiles_per_block = a.kv_block / BN;
+  auto next_tile = [&](int jt) {
+    if (bm_row)
+      while (jt < n_tiles && !bm_row[jt / tiles_per_block]) jt++;
+    return jt;
+  };
 
   // DMA of one tile: each instruction moves 1 KB (1024 / row bytes tile rows); lane i fetches the
   // 16-byte chunk that belongs at physical position i of that KB.  Rows beyond the sequence are clamped
@@ -88,12 +98,12 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
     for (int ii = wave; ii < NIK + NIV; ii += 4) {
       if (ii < NIK) {
         const int row = ii * (1024 / KROW) + lane / CPRK, c = lane % CPRK;
-        const int nrow = min(n0 + row, a.Skv - 1);
+        const int nrow = min(n0 + row, skv - 1);
         dma16(kb + nrow * k_row_bytes + ((c ^ swz_tile<CPRK>(row)) << 4), base + ii * 1024);
       } else {
         const int i2 = ii - NIK;
         const int row = i2 * (1024 / VROW) + lane / CPRV, c = lane % CPRV;
-        const int nrow = min(n0 + row, a.Skv - 1);
+        const int nrow = min(n0 + row, skv - 1);
         dma16(vb + nrow * v_row_bytes + ((c ^ swz_tile<CPRV>(row)) << 4), base + KTILE + i2 * 1024);
       }
     }
@@ -103,11 +113,11 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
 #pragma unroll
     for (int q4 = 0; q4 < 4; q4++) {
       const int n = n0 + 8 * q4 + 4 * g;
-      if (n + 3 < a.Skv) {
+      if (n + 3 < skv) {
         mk[q4] = *(const x4*)(mrow + n);
       } else {
 #pragma unroll
-        for (int i = 0; i < 4; i++) mk[q4][i] = n + i < a.Skv ? mrow[n + i] : (T)0.f;
+        for (int i = 0; i < 4; i++) mk[q4][i] = n + i < skv ? mrow[n + i] : (T)0.f;
       }
     }
   };
@@ -130,23 +140,25 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
   const float c_scale = a.scale * kLog2e, c_bias = bias * kLog2e;
 
   x4 mk_next[4];
-  if (n_tiles > 0) {
-    issue_tile(0, 0);
-    if constexpr (FAMILY == WF_RETENTION) load_mask(0, mk_next);
+  int jt = next_tile(0);
+  if (jt < n_tiles) {
+    issue_tile(jt * BN, 0);
+    if constexpr (FAMILY == WF_RETENTION) load_mask(jt * BN, mk_next);
   }
 
-  for (int jt = 0; jt < n_tiles; jt++) {
-    const int buf = jt & 1, n0 = jt * BN;
+  for (int it = 0; jt < n_tiles; it++) {
+    const int buf = it & 1, n0 = jt * BN;
     wait_dma();
     __syncthreads();
+    jt = next_tile(jt + 1);   // from here on: the tile after this one
     x4 mk[4];
     if constexpr (FAMILY == WF_RETENTION) {
 #pragma unroll
       for (int q4 = 0; q4 < 4; q4++) mk[q4] = mk_next[q4];
     }
-    if (jt + 1 < n_tiles) {
-      if constexpr (FAMILY == WF_RETENTION) load_mask(n0 + BN, mk_next);
-      issue_tile(n0 + BN, buf ^ 1);
+    if (jt < n_tiles) {
+      if constexpr (FAMILY == WF_RETENTION) load_mask(jt * BN, mk_next);
+      issue_tile(jt * BN, buf ^ 1);
     }
     const uint32_t kbase = lds0 + buf * STAGE, vbase = kbase + KTILE;
 
@@ -178,12 +190,12 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
       }
     } else {
       // element-wise mask only on tiles that reach past the diagonal or the end of the sequence
-      const bool edge = (CAUSAL && n0 + BN - 1 > m_wave) || n0 + BN > a.Skv;
+      const bool edge = (CAUSAL && n0 + BN - 1 > m_wave) || n0 + BN > skv;
       if (edge) {
 #pragma unroll
         for (int jj = 0; jj < 16; jj++) {
           const int n = n0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
-          if ((CAUSAL && n > m_lane) || n >= a.Skv) s[jj] = -INFINITY;
+          if ((CAUSAL && n > m_lane) || n >= skv) s[jj] = -INFINITY;
         }
       }
       if constexpr (FAMILY == WF_SOFTMAX) {
@@ -249,8 +261,8 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
     if (rs_ptr) *rs_ptr = r_tot;
   } else if constexpr (FAMILY == WF_SOFTMAX) {
     const float tot = r_part + xhalf(r_part);
-    inv = 1.f / tot;
-    if (rs_ptr) *rs_ptr = (row_max + fast_log2(tot)) * kLn2;
+    inv = tot > 0.f ? 1.f / tot : 0.f;   // (a row that was left no key at all gives zeros and lse = -inf)
+    if (rs_ptr) *rs_ptr = tot > 0.f ? (row_max + fast_log2(tot)) * kLn2 : -INFINITY;
   }
 
   // ---- O: two halves of DV/2 columns through a wave-private LDS block, coalesced 16-byte stores
@@ -318,6 +330,7 @@ static int wide_dims(const AttnArgs& a, int family, bool causal, int dqk, int dv
       return causal ? launch_wide<T, 128, 128, WF_RETENTION, true>(a, stream) : launch_wide<T, 128, 128, WF_RETENTION, false>(a, stream);
     return -2;
   }
+  if (dqk == 128 && dv == 128) return wide_family<T, 128, 128>(a, family, causal, stream);   // (only with kv selection: see attn_fwd_dispatch)
   if (dqk == 64 && dv == 64) return wide_family<T, 64, 64>(a, family, causal, stream);
   if (dqk == 128 && dv == 256) return wide_family<T, 128, 256>(a, family, causal, stream);
   if (dqk == 256 && dv == 256) return wide_family<T, 256, 256>(a, family, causal, stream);

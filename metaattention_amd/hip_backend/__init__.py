@@ -47,6 +47,8 @@ class AttnParams(Structure):
         ("scale", c_float), ("bias", c_float), ("bias_ptr", c_void_p),
         ("score_mask", c_void_p), ("sm_stride_b", c_int64), ("sm_stride_h", c_int64), ("sm_stride_q", c_int64),
         ("heads_kv", c_int32),
+        ("kv_block_size", c_int32), ("kv_seqlens", c_void_p),
+        ("kv_block_mask", c_void_p), ("kbm_stride_b", c_int64), ("kbm_stride_h", c_int64),
     ]
 
 
@@ -154,10 +156,10 @@ def _require_gpu(*tensors):
 
 
 def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None,
-             score_mask=None, out=None, row_scale=None):
+             score_mask=None, out=None, row_scale=None, kv_seqlens=None, kv_block_mask=None, kv_block_size: int = 0):
     """Parallel attention forward on BSHD tensors.  Returns ``out`` ([B,Sq,H,Dv]).  k and v may
     have fewer heads than q (grouped-query: query head h reads kv head h // (H // Hkv))."""
-    _require_gpu(q, k, v, bias_tensor, score_mask, out, row_scale)
+    _require_gpu(q, k, v, bias_tensor, score_mask, out, row_scale, kv_seqlens, kv_block_mask)
     B, Sq, H, Dqk = q.shape
     Skv, Hkv, Dv = k.shape[1], k.shape[2], v.shape[-1]
     assert k.shape == (B, Skv, Hkv, Dqk) and v.shape == (B, Skv, Hkv, Dv) and H % Hkv == 0, "q/k/v shapes disagree"
@@ -187,6 +189,14 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
         p.score_mask = score_mask.data_ptr()
         p.sm_stride_b = score_mask.stride(0) if score_mask.shape[0] > 1 else 0
         p.sm_stride_h, p.sm_stride_q = score_mask.stride(1), score_mask.stride(2)
+    if kv_seqlens is not None:
+        assert kv_seqlens.dtype == torch.int32 and kv_seqlens.shape == (B,) and kv_seqlens.is_contiguous()
+        p.kv_seqlens = kv_seqlens.data_ptr()
+    if kv_block_mask is not None:
+        nblk = (Skv + kv_block_size - 1) // kv_block_size
+        assert kv_block_mask.dtype in (torch.bool, torch.uint8) and kv_block_mask.shape == (B, Hkv, nblk) and kv_block_mask.stride(-1) == 1
+        p.kv_block_mask, p.kv_block_size = kv_block_mask.data_ptr(), int(kv_block_size)
+        p.kbm_stride_b, p.kbm_stride_h = kv_block_mask.stride(0), kv_block_mask.stride(1)
     _check(load_library().ma_attn_fwd(ctypes.byref(p), _stream()))
     return out
 

@@ -27,6 +27,7 @@ ssd_chunk_scan         3-way agreement: chunked reference == naive sequential
                        state-space recurrence; chunk-size independence
 simple_gla             token-by-token recurrence (fp64)
 mla_decode             SDPA with K=concat(kv,k_pe), V=kv; split-KV invariance
+sparse_decode_attention  dense attention over the gathered kept keys only
 attention_grads,       central differences of the pinned forward functions in
 linear_attention_grads fp64 along random directions; SDPA's own autograd
 (all of the above)     tests/golden/*.npz: the operators' definitions evaluated
@@ -43,6 +44,7 @@ from .attention_ref import (  # noqa: F401
     mla_decode,
     retention_decay_mask,
     attention_grads,
+    sparse_decode_attention,
 )
 from .linear_ref import (  # noqa: F401
     retnet_quadratic,

@@ -151,3 +151,26 @@ def attention_grads(forward, q, k, v, dout, **kwargs):
     out = forward(qd, kd, vd, compute_dtype=torch.float64, **kwargs)
     out.backward(dout.to(torch.float64))
     return qd.grad, kd.grad, vd.grad
+
+
+def sparse_decode_attention(q, k, v, block_mask=None, cache_seqlens=None, block_size: int = 32, compute_dtype=torch.float32):
+    """Decode attention over a selected part of the cache, testing/test.py:654-693 (``ref_program_torch``):
+    q [B,1,H,D], k [B,S,G,D], v [B,S,G,Dv]; keys in blocks of ``block_size`` whose ``block_mask[b, g, block]``
+    is false, and keys at or beyond ``cache_seqlens[b]``, are set to -inf before softmax(scores / sqrt(D)).
+    Query head h reads kv head h // (H // G).  Returns [B,H,Dv] (the query token squeezed, as there)."""
+    B, _, H, D = q.shape
+    S, G, Dv = k.shape[1], k.shape[2], v.shape[-1]
+    out = torch.empty(B, H, Dv, dtype=compute_dtype)
+    pos = torch.arange(S)
+    for b in range(B):
+        for h in range(H):
+            g = h // (H // G)
+            s = (k[b, :, g].to(compute_dtype) @ q[b, 0, h].to(compute_dtype)) / math.sqrt(D)
+            keep = torch.ones(S, dtype=torch.bool)
+            if block_mask is not None:
+                keep &= block_mask[b, g].to(torch.bool).cpu()[pos // block_size]
+            if cache_seqlens is not None:
+                keep &= pos < int(cache_seqlens[b])
+            s = s.masked_fill(~keep, float("-inf"))
+            out[b, h] = torch.softmax(s, dim=-1) @ v[b, :, g].to(compute_dtype)
+    return out

@@ -172,3 +172,11 @@ def softmax_attention_decode(B, H, S, KV, D, DV, dtype=torch.float16, HKV=None):
             meta_tensor(B, HKV, KV, DV, dtype=dtype))
     return AttentionEngine(meta, CustomIO({}), score_mod=lambda score, io, b, h, q_idx, kv_idx: score * scale, mask_mod=None,
                            online_func=OnlineSoftmax())
+
+
+def sparse_gqa_decode(B, H, G, S, D, DV, dtype=torch.float16, block=32):
+    """examples/sparse_gqa_decode.py:13-107: one query token, G kv heads, external kv block mask and per-batch cache lengths."""
+    scale = 1 / D ** 0.5
+    meta = (meta_tensor(B, H, 1, D, dtype=dtype), meta_tensor(B, G, S, D, dtype=dtype), meta_tensor(B, G, S, DV, dtype=dtype))
+    return AttentionEngine(meta, CustomIO({}), score_mod=lambda score, io, b, h, q_idx, kv_idx: score * scale, mask_mod=None,
+                           online_func=OnlineSoftmax(), extern_block_mask=True, use_varlen=True, infer_mask_block_N=block)

@@ -184,6 +184,45 @@ def test_engine_dense_decode(B, H, HKV, S, KV, D, DV):
     oracle.assert_close(o.float().cpu(), ref, rtol=1e-2, atol=1e-2)      # the reference test's own tolerance (:156)
 
 
+@pytest.mark.parametrize("B,H,G,S,D,DV,block", [(8, 32, 8, 2048, 128, 128, 32), (2, 8, 2, 500, 128, 128, 64), (3, 6, 6, 300, 64, 64, 32)])
+def test_engine_sparse_gqa_decode(B, H, G, S, D, DV, block):
+    """First case: testing/test.py:60 (block mask generated as there, :697-726, half of the blocks kept); the others add
+    ragged cache lengths, a wider block and plain multi-head."""
+    mod = specs.sparse_gqa_decode(B, H, G, S, D, DV, block=block)
+    g = torch.Generator().manual_seed(S)
+    q = torch.randn(B, 1, H, D, generator=g).half()
+    k = torch.randn(B, S, G, D, generator=g).half()
+    v = torch.randn(B, S, G, DV, generator=g).half()
+    lens = torch.full((B,), S, dtype=torch.int32) if S == 2048 else torch.randint(1, S + 1, (B,), generator=g, dtype=torch.int32)
+    nblk = (S + block - 1) // block
+    bm = torch.zeros(B, G, nblk, dtype=torch.bool)
+    for b in range(B):
+        valid = (int(lens[b]) + block - 1) // block
+        keep = max(1, math.ceil(int(lens[b]) * 0.5 / block))
+        for gi in range(G):
+            bm[b, gi, torch.randperm(valid, generator=g)[:keep]] = True
+    o = mod(q.cuda(), k.cuda(), v.cuda(), block_mask=bm.cuda(), cache_seqlens=lens.cuda())
+    torch.cuda.synchronize()
+    assert o.shape == (B, H, DV)
+    ref = oracle.sparse_decode_attention(q, k, v, bm, lens, block_size=block)
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    # cache lengths alone (every block kept) through the same operator
+    o2 = mod(q.cuda(), k.cuda(), v.cuda(), cache_seqlens=lens.cuda())
+    torch.cuda.synchronize()
+    oracle.assert_close(o2.float().cpu(), oracle.sparse_decode_attention(q, k, v, None, lens), rtol=RTOL, atol=ATOL)
+
+
+def test_row_without_any_key_gives_zeros():
+    hb = _hb()
+    B, S, H, D = 1, 64, 1, 128
+    q, k, v = (t.cuda() for t in inputs.softmax_inputs(B, H, S, D, D, seed=1))
+    bm = torch.zeros(B, H, 2, dtype=torch.bool, device="cuda")
+    lse = torch.empty(B, H, 1, device="cuda")
+    o = hb.attn_fwd(q[:, :1].contiguous(), k, v, family=hb.MA_ATTN_SOFTMAX, causal=False, scale=0.1, kv_block_mask=bm, kv_block_size=32, row_scale=lse)
+    torch.cuda.synchronize()
+    assert float(o.float().abs().max()) == 0.0 and bool(torch.isinf(lse).all())
+
+
 def test_unsupported_head_size_is_an_error():
     hb = _hb()
     q = torch.zeros(1, 64, 1, 96, device="cuda", dtype=torch.bfloat16)

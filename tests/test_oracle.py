@@ -280,3 +280,21 @@ def test_linear_attention_grads_vs_finite_differences():
         ap[idx], am[idx] = args[idx] + eps * direction, args[idx] - eps * direction
         fd = (f(ap) - f(am)) / (2 * eps)
         assert abs(fd - float((grad * direction).sum())) < 1e-5 * max(1.0, abs(fd)), idx
+
+
+def test_sparse_decode_equals_dense_attention_over_kept_keys():
+    g = torch.Generator().manual_seed(13)
+    B, H, G, S, D, bs = 2, 4, 2, 96, 16, 32
+    q = torch.randn(B, 1, H, D, generator=g, dtype=torch.float64)
+    k = torch.randn(B, S, G, D, generator=g, dtype=torch.float64)
+    v = torch.randn(B, S, G, D, generator=g, dtype=torch.float64)
+    bm = torch.tensor([[[1, 0, 1], [0, 1, 1]], [[1, 1, 0], [1, 0, 0]]], dtype=torch.bool)
+    lens = torch.tensor([96, 70], dtype=torch.int32)
+    got = oracle.sparse_decode_attention(q, k, v, bm, lens, block_size=bs, compute_dtype=torch.float64)
+    for b in range(B):
+        for h in range(H):
+            gi = h // (H // G)
+            idx = [n for n in range(S) if bm[b, gi, n // bs] and n < int(lens[b])]
+            ref = oracle.softmax_attention(q[b:b + 1, :, h:h + 1], k[b:b + 1, idx, gi:gi + 1], v[b:b + 1, idx, gi:gi + 1], causal=False,
+                                           compute_dtype=torch.float64)
+            torch.testing.assert_close(got[b, h], ref[0, 0, 0])
