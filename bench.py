@@ -16,6 +16,7 @@ benchmark configurations, each with its own roofline fraction:
   c3_retnet_parallel  same shape, normalised parallel operator with a [1,H,S,S] decay mask
   c4_mamba2_ssd       Mamba2 SSD, B8 H64 S2048 P64 N128, one B/C group
   c5_mla_decode       absorbed MLA decode, B64 Hq128 KV4096 d512+64 (HBM bound)
+  gqa_decode          grouped-query softmax decode, B64 H32 Hkv8 KV4096 D128 (HBM bound)
 """
 from __future__ import annotations
 
@@ -106,6 +107,30 @@ def bench_softmax_bwd(steps, warmup):
     ms = time_gpu(lambda: hb.attn_bwd(q, k, v, o, do, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale), max(steps // 3, 3), 2)
     flops = 2.5 * 0.5 * 4.0 * B * H * S * S * D
     return _mfma_entry(ms, flops, "backward, 2.5 x the forward's algorithmic FLOPs (5 tile products; the two kernels execute 7)")
+
+
+def bench_decode(steps, warmup, B=64, H=32, Hkv=8, Skv=4096, D=128):
+    """Grouped-query decode, one query token per sequence (HBM bound): the query heads of a kv head are handed to the
+    kernel as the rows of that head, the cache is cut into kv splits."""
+    import torch
+    from metaattention_amd import hip_backend as hb
+    g = torch.Generator(device="cuda").manual_seed(0)
+    grp = H // Hkv
+    q = torch.randn(B, 1, H, D, device="cuda", dtype=torch.bfloat16, generator=g)
+    k = torch.randn(B, Skv, Hkv, D, device="cuda", dtype=torch.bfloat16, generator=g)
+    v = torch.randn(B, Skv, Hkv, D, device="cuda", dtype=torch.bfloat16, generator=g)
+    o = torch.empty_like(q)
+    qv, ov = q.view(B, Hkv, grp, D).transpose(1, 2), o.view(B, Hkv, grp, D).transpose(1, 2)
+    ws = torch.empty(1 << 26, dtype=torch.uint8, device="cuda")
+    junk = torch.empty(512 * 2 ** 20, dtype=torch.uint8, device="cuda")
+    fn = lambda: hb.attn_fwd(qv, k, v, family=hb.MA_ATTN_SOFTMAX, causal=False, scale=1 / math.sqrt(D), out=ov, workspace=ws)
+    ms = time_gpu(fn, steps, warmup, flush=lambda: junk.fill_(1))
+    ms_warm = time_gpu(fn, steps, warmup)
+    nbytes = 2.0 * (k.numel() + v.numel() + q.numel() + o.numel())
+    gbs = nbytes / ms / 1e6
+    return dict(ms=round(ms, 4), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / PEAK_HBM_GBS, 4), algorithmic_bytes=nbytes,
+                ms_without_cache_flush=round(ms_warm, 4), shape=dict(B=B, H=H, Hkv=Hkv, Sq=1, Skv=Skv, D=D),
+                note="split-KV kernel + combine kernel per call; caches overwritten before every timed call")
 
 
 def bench_retnet_chunked(steps, warmup):
@@ -244,7 +269,8 @@ def main():
              ("c3_retnet_chunked", "retnet", lambda: bench_retnet_chunked(args.steps, args.warmup)),
              ("c3_retnet_parallel", "retention", lambda: bench_retnet_parallel(args.steps, args.warmup)),
              ("c4_mamba2_ssd", "mamba", lambda: bench_mamba2(args.steps, args.warmup)),
-             ("c5_mla_decode", "mla", lambda: bench_mla(args.steps, args.warmup))]
+             ("c5_mla_decode", "mla", lambda: bench_mla(args.steps, args.warmup)),
+             ("gqa_decode", "decode", lambda: bench_decode(args.steps, args.warmup))]
     for name, key, fn in table:
         if want and (want == ["none"] or not any(key.startswith(w) or w in name for w in want)):
             continue

@@ -83,6 +83,9 @@ typedef struct ma_attn_params {
   int32_t kv_block_size;
   const int32_t* kv_seqlens;
   const uint8_t* kv_block_mask; int64_t kbm_stride_b, kbm_stride_h;
+  /* optional; with ma_attn_workspace_bytes(&params) bytes, decode shapes (at most 32 query rows, SOFTMAX, no
+   * structural mask) run as split-KV + combine (attn_decode_tl.py:63-206); without it they run unsplit */
+  void* workspace; size_t workspace_bytes;
 } ma_attn_params;
 
 /* Parallel attention backward for the SOFTMAX, SIGMOID and RELU families.  Replaces the backward of
@@ -156,7 +159,8 @@ typedef void* ma_stream_t; /* a hipStream_t */
 int ma_version(void);
 const char* ma_last_error(void);
 
-/* attn_tl.py:92-190 (`main`) behind _attention.forward (:654-667) */
+/* attn_tl.py:92-190 (`main`) behind _attention.forward (:654-667); attn_decode_tl.py:63-206 for decode shapes */
+size_t ma_attn_workspace_bytes(const ma_attn_params* p);
 int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream);
 
 /* attn_tl.py:669-692 (`_attention.backward`: mod_prep, mod_bwd, mod_post) */

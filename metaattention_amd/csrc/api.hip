@@ -25,6 +25,19 @@ extern "C" {
 int ma_version(void) { return MA_VERSION; }
 const char* ma_last_error(void) { return g_err; }
 
+static int attn_splits(const ma_attn_params* p) {
+  return ma::attn_decode_splits(p->family, p->mask == MA_MASK_CAUSAL, p->batch, p->heads, p->seqlen_q, p->seqlen_kv, p->dim_qk, p->dim_v);
+}
+
+// partial outputs [B, splits, H, Sq, Dv] in the tensor dtype, then their fp32 row scales [B, splits, H, Sq]
+size_t ma_attn_workspace_bytes(const ma_attn_params* p) {
+  if (!p || p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->seqlen_kv <= 0 || p->dim_v <= 0) return 0;
+  const int n = attn_splits(p);
+  if (n <= 1) return 0;
+  const size_t rows = (size_t)p->batch * n * p->heads * p->seqlen_q;
+  return rows * p->dim_v * 2 + rows * sizeof(float);
+}
+
 int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
   if (!p) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: params is NULL");
   if (!p->q || !p->k || !p->v || !p->o) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: q/k/v/o must be non-NULL");
@@ -70,6 +83,16 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
   a.kv_lens = p->kv_seqlens;
   a.kv_block_mask = p->kv_block_mask; a.kbm_sb = p->kbm_stride_b; a.kbm_sh = p->kbm_stride_h;
   a.kv_block = p->kv_block_size;
+  a.n_split = 1;
+  if (p->workspace && ((uintptr_t)p->workspace % 16) == 0) {
+    const int n = attn_splits(p);
+    if (n > 1 && p->workspace_bytes >= ma_attn_workspace_bytes(p)) {
+      const size_t rows = (size_t)p->batch * n * p->heads * p->seqlen_q;
+      a.n_split = n;
+      a.o_part = p->workspace;
+      a.lse_part = (float*)((char*)p->workspace + rows * p->dim_v * 2);
+    }
+  }
   a.scale = p->scale; a.bias = p->bias;
   const int rc = ma::attn_fwd_dispatch(a, p->family, p->mask == MA_MASK_CAUSAL, p->dtype == MA_BF16, p->dim_qk, p->dim_v,
                                        (hipStream_t)stream);

@@ -18,10 +18,18 @@ struct AttnArgs {
   const uint8_t* kv_block_mask;
   int64_t kbm_sb, kbm_sh;
   int kv_block;
+  // split-kv decode (attn_wide_fwd_kernel with one wave per workgroup): n_split kv ranges per (batch, head,
+  // row block), normalised partial outputs [B, n_split, H, Sq, Dv] in the tensor dtype and their fp32
+  // natural-log row scale [B, n_split, H, Sq], merged by attn_split_combine_kernel
+  int n_split;
+  void* o_part;
+  float* lse_part;
   float scale, bias;
 };
 
 int attn_wide_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);
+// number of kv splits the decode path would use for these sizes (1: not a decode shape / nothing to gain)
+int attn_decode_splits(int family, bool causal, int B, int H, int Sq, int Skv, int dqk, int dv);
 int attn_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);
 
 }  // namespace ma

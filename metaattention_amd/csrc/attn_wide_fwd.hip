@@ -14,6 +14,11 @@
 // The head sizes of the reference's own test list are covered (testing/test.py:54-63: 128/256 softmax,
 // 64/64 relu, 256/512 retention) next to 256/256 and, without softmax, 256/512.
 //
+// Decode shapes (a few query rows against a long cache, softmax, no mask) run with one wave per
+// workgroup and the kv sequence cut into splits, each writing a normalised partial output and its
+// log-sum-exp to a workspace; attn_split_combine_kernel merges them (the split-KV scheme of
+// tl_template/attn/attn_decode_tl.py:63-206 with the `combine` of examples/mha_decode.py:72-80).
+//
 // Structure.  One workgroup of 4 waves owns 128 query rows (32 per wave, Q fragments in registers)
 // and walks the kv sequence in tiles of 32 rows; K and V tiles arrive by direct-to-LDS DMA, double
 // buffered, one barrier per tile.  Scores are computed transposed (S^T = K Q^T) as in attn_fwd.hip, so
@@ -32,12 +37,12 @@ namespace {
 enum { WF_SOFTMAX = 0, WF_SIGMOID = 1, WF_RELU = 2, WF_RETENTION = 3 };   // = MA_ATTN_* of the C interface
 }
 
-template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
-__global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_kernel(const AttnArgs a) {
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL, int NW>
+__global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_kernel(const AttnArgs a) {
   using E = Elem<T>;
   using x8 = typename E::x8;
   using x4 = typename E::x4;
-  constexpr int BM = 128, BN = 32;
+  constexpr int BM = 32 * NW, BN = 32;
   constexpr int KS = DQK / 16, DB = DV / 32;
   constexpr int KROW = DQK * 2, VROW = DV * 2;
   constexpr int CPRK = DQK / 8, CPRV = DV / 8;
@@ -51,14 +56,22 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
   const int r = lane & 31, g = lane >> 5;
 
   const int nmb = a.num_m_blocks, BH = a.B * a.H;
-  int bh, mb;
-  if ((BH & 7) == 0) {
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    bh = (slot / nmb) * 8 + xcd;
+  int bh, mb, split;
+  {
+    int slot;
+    if ((BH & 7) == 0) {
+      const int xcd = blockIdx.x & 7;
+      slot = blockIdx.x >> 3;
+      split = slot % a.n_split;
+      slot /= a.n_split;
+      bh = (slot / nmb) * 8 + xcd;
+    } else {
+      slot = blockIdx.x;
+      split = slot % a.n_split;
+      slot /= a.n_split;
+      bh = slot / nmb;
+    }
     mb = slot % nmb;
-  } else {
-    bh = blockIdx.x / nmb;
-    mb = blockIdx.x % nmb;
   }
   if (CAUSAL) mb = nmb - 1 - mb;
   const int b = bh / a.H, h = bh % a.H;
@@ -84,6 +97,10 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
   // tiles whose block of keys is switched off for this (batch, kv head) are skipped (:57-64)
   const uint8_t* bm_row = a.kv_block_mask ? a.kv_block_mask + (int64_t)b * a.kbm_sb + (int64_t)(h / a.kv_group) * a.kbm_sh : nullptr;
   const int tiles_per_block = a.kv_block / BN;
+  // this workgroup's share of the tiles
+  const int tiles_per_split = (n_tiles + a.n_split - 1) / a.n_split;
+  const int t_begin = split * tiles_per_split;
+  n_tiles = min(n_tiles, t_begin + tiles_per_split);
   auto next_tile = [&](int jt) {
     if (bm_row)
       while (jt < n_tiles && !bm_row[jt / tiles_per_block]) jt++;
@@ -95,7 +112,7 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
   // to its last row (their scores are masked, or multiplied by a zero of M).
   auto issue_tile = [&](int n0, int buf) {
     const uint32_t base = lds0 + buf * STAGE;
-    for (int ii = wave; ii < NIK + NIV; ii += 4) {
+    for (int ii = wave; ii < NIK + NIV; ii += NW) {
       if (ii < NIK) {
         const int row = ii * (1024 / KROW) + lane / CPRK, c = lane % CPRK;
         const int nrow = min(n0 + row, skv - 1);
@@ -140,7 +157,7 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
   const float c_scale = a.scale * kLog2e, c_bias = bias * kLog2e;
 
   x4 mk_next[4];
-  int jt = next_tile(0);
+  int jt = next_tile(t_begin);
   if (jt < n_tiles) {
     issue_tile(jt * BN, 0);
     if constexpr (FAMILY == WF_RETENTION) load_mask(jt * BN, mk_next);
@@ -254,7 +271,8 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
   __syncthreads();   // every wave is done with the K/V buffers: they become output staging
 
   float inv = 1.f;
-  float* const rs_ptr = a.row_scale && g == 0 && m_lane < a.Sq ? a.row_scale + ((int64_t)b * a.H + h) * a.Sq + m_lane : nullptr;
+  float* rs_ptr = a.row_scale && g == 0 && m_lane < a.Sq ? a.row_scale + ((int64_t)b * a.H + h) * a.Sq + m_lane : nullptr;
+  if (a.n_split > 1) rs_ptr = g == 0 && m_lane < a.Sq ? a.lse_part + (((int64_t)b * a.n_split + split) * a.H + h) * a.Sq + m_lane : nullptr;
   if constexpr (FAMILY == WF_RETENTION) {
     const float r_tot = fmaxf(r_part + xhalf(r_part), 1.f);
     inv = 1.f / r_tot;
@@ -269,6 +287,11 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
   constexpr int HALF = DV / 2, OROW = HALF * 2 + 16;
   const uint32_t ob = lds0 + wave * 32 * OROW;
   T* obase = (T*)a.o + (int64_t)b * a.osb + (int64_t)h * a.osh;
+  int64_t o_row_stride = a.oss;
+  if (a.n_split > 1) {
+    obase = (T*)a.o_part + ((((int64_t)b * a.n_split + split) * a.H + h) * a.Sq) * DV;
+    o_row_stride = DV;
+  }
 #pragma unroll
   for (int hf = 0; hf < 2; hf++) {
 #pragma unroll
@@ -284,34 +307,88 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_
     for (int it = 0; it < 32 * (HALF / 8) / 64; it++) {
       const int ci = lane + 64 * it, row = ci / (HALF / 8), c = ci % (HALF / 8);
       const u32x4 w = lds_read<u32x4>(ob + row * OROW + c * 16);
-      if (m_wave + row < a.Sq) *(u32x4*)(obase + (int64_t)(m_wave + row) * a.oss + hf * HALF + c * 8) = w;
+      if (m_wave + row < a.Sq) *(u32x4*)(obase + (int64_t)(m_wave + row) * o_row_stride + hf * HALF + c * 8) = w;
     }
   }
 }
 
-template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
+// Merge of the kv splits: o = sum_s exp(lse_s - lse) o_s with lse = log sum_s exp(lse_s) (examples/mha_decode.py:72-80).
+// One wave per (batch, head, row); lanes cover the value columns.
+template <typename T, int DV>
+__global__ __launch_bounds__(256) void attn_split_combine_kernel(const AttnArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);   // (b * H + h) * Sq + m
+  const int64_t rows = (int64_t)a.B * a.H * a.Sq;
+  if (row >= rows) return;
+  const int m = (int)(row % a.Sq), h = (int)((row / a.Sq) % a.H), b = (int)(row / ((int64_t)a.Sq * a.H));
+  const int64_t part_row = ((int64_t)b * a.n_split * a.H + h) * a.Sq + m, split_stride = (int64_t)a.H * a.Sq;
+  float mx = -INFINITY;
+  for (int s = 0; s < a.n_split; s++) mx = fmaxf(mx, a.lse_part[part_row + s * split_stride]);
+  float tot = 0.f;
+  for (int s = 0; s < a.n_split; s++) {
+    const float l = a.lse_part[part_row + s * split_stride];
+    tot += l == -INFINITY ? 0.f : __expf(l - mx);
+  }
+  constexpr int PER = DV / 64;   // value columns per lane
+  float acc[PER];
+#pragma unroll
+  for (int i = 0; i < PER; i++) acc[i] = 0.f;
+  for (int s = 0; s < a.n_split; s++) {
+    const float l = a.lse_part[part_row + s * split_stride];
+    if (l == -INFINITY) continue;
+    const float w = __expf(l - mx) / tot;
+    const T* src = (const T*)a.o_part + (part_row + s * split_stride) * DV + lane * PER;
+#pragma unroll
+    for (int i = 0; i < PER; i++) acc[i] += w * (float)src[i];
+  }
+  T* dst = (T*)a.o + (int64_t)b * a.osb + (int64_t)m * a.oss + (int64_t)h * a.osh + lane * PER;
+#pragma unroll
+  for (int i = 0; i < PER; i++) dst[i] = (T)acc[i];
+  if (a.row_scale && lane == 0) a.row_scale[row] = tot > 0.f ? mx + __logf(tot) : -INFINITY;
+}
+
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL, int NW = 4>
 static int launch_wide(const AttnArgs& a, hipStream_t stream) {
   constexpr size_t tiles = 2 * (size_t)32 * (DQK + DV) * 2;
-  constexpr size_t ostage = 4 * 32 * (size_t)(DV + 16);
+  constexpr size_t ostage = NW * 32 * (size_t)(DV + 16);
   constexpr size_t lds = tiles > ostage ? tiles : ostage;
-  auto kern = attn_wide_fwd_kernel<T, DQK, DV, FAMILY, CAUSAL>;
+  auto kern = attn_wide_fwd_kernel<T, DQK, DV, FAMILY, CAUSAL, NW>;
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
     attr_set = true;
   }
   AttnArgs args = a;
-  args.num_m_blocks = (a.Sq + 127) / 128;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(args.num_m_blocks * a.B * a.H)), dim3(256), lds, stream, args);
+  if (args.n_split < 1) args.n_split = 1;
+  args.num_m_blocks = (a.Sq + 32 * NW - 1) / (32 * NW);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(args.num_m_blocks * a.B * a.H * args.n_split)), dim3(64 * NW), lds, stream, args);
+  if (args.n_split > 1) {
+    const int64_t rows = (int64_t)a.B * a.H * a.Sq;
+    hipLaunchKernelGGL((attn_split_combine_kernel<T, DV>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, args);
+  }
   return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// Decode shapes: at most 32 query rows per (batch, head), softmax, no structural mask.  Splits are chosen
+// so that about four workgroups per CU are in flight, each with at least 8 tiles of 32 keys.
+int attn_decode_splits(int family, bool causal, int B, int H, int Sq, int Skv, int dqk, int dv) {
+  if (family != WF_SOFTMAX || causal || Sq > 32) return 1;
+  if (!((dqk == 128 && dv == 128) || (dqk == 64 && dv == 64) || (dqk == 128 && dv == 256) || (dqk == 256 && dv == 256))) return 1;
+  const int tiles = (Skv + 31) / 32;
+  int n = 1024 / (B * H);
+  if (n > tiles / 8) n = tiles / 8;
+  if (n > 64) n = 64;
+  return n < 1 ? 1 : n;
 }
 
 template <typename T, int DQK, int DV>
 static int wide_family(const AttnArgs& a, int family, bool causal, hipStream_t stream) {
   switch (family) {
     case WF_SOFTMAX:
-      if constexpr (DV <= 256)
+      if constexpr (DV <= 256) {
+        if (!causal && a.Sq <= 32 && a.o_part) return launch_wide<T, DQK, DV, WF_SOFTMAX, false, 1>(a, stream);   // decode
         return causal ? launch_wide<T, DQK, DV, WF_SOFTMAX, true>(a, stream) : launch_wide<T, DQK, DV, WF_SOFTMAX, false>(a, stream);
+      }
       return -2;
     case WF_SIGMOID:
       return causal ? launch_wide<T, DQK, DV, WF_SIGMOID, true>(a, stream) : launch_wide<T, DQK, DV, WF_SIGMOID, false>(a, stream);

@@ -22,7 +22,7 @@ MA_ATTN_SOFTMAX, MA_ATTN_SIGMOID, MA_ATTN_RELU, MA_ATTN_RETENTION = 0, 1, 2, 3
 MA_MASK_NONE, MA_MASK_CAUSAL = 0, 1
 
 EXPORTED_SYMBOLS = (
-    "ma_version", "ma_last_error", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes", "ma_attn_bwd",
+    "ma_version", "ma_last_error", "ma_attn_workspace_bytes", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes", "ma_attn_bwd",
     "ma_linear_workspace_bytes", "ma_linear_fwd",
     "ma_mla_choose_split", "ma_mla_workspace_bytes", "ma_mla_decode",
 )
@@ -49,6 +49,7 @@ class AttnParams(Structure):
         ("heads_kv", c_int32),
         ("kv_block_size", c_int32), ("kv_seqlens", c_void_p),
         ("kv_block_mask", c_void_p), ("kbm_stride_b", c_int64), ("kbm_stride_h", c_int64),
+        ("workspace", c_void_p), ("workspace_bytes", c_size_t),
     ]
 
 
@@ -114,6 +115,8 @@ def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
     lib.ma_last_error.restype = c_char_p
     lib.ma_attn_fwd.argtypes = [POINTER(AttnParams), c_void_p]
     lib.ma_attn_fwd.restype = c_int
+    lib.ma_attn_workspace_bytes.argtypes = [POINTER(AttnParams)]
+    lib.ma_attn_workspace_bytes.restype = c_size_t
     lib.ma_attn_bwd.argtypes = [POINTER(AttnBwdParams), c_void_p]
     lib.ma_attn_bwd.restype = c_int
     lib.ma_attn_bwd_workspace_bytes.argtypes = [POINTER(AttnBwdParams)]
@@ -156,7 +159,8 @@ def _require_gpu(*tensors):
 
 
 def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None,
-             score_mask=None, out=None, row_scale=None, kv_seqlens=None, kv_block_mask=None, kv_block_size: int = 0):
+             score_mask=None, out=None, row_scale=None, kv_seqlens=None, kv_block_mask=None, kv_block_size: int = 0,
+             workspace=None, split_kv: bool = True):
     """Parallel attention forward on BSHD tensors.  Returns ``out`` ([B,Sq,H,Dv]).  k and v may
     have fewer heads than q (grouped-query: query head h reads kv head h // (H // Hkv))."""
     _require_gpu(q, k, v, bias_tensor, score_mask, out, row_scale, kv_seqlens, kv_block_mask)
@@ -197,7 +201,15 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
         assert kv_block_mask.dtype in (torch.bool, torch.uint8) and kv_block_mask.shape == (B, Hkv, nblk) and kv_block_mask.stride(-1) == 1
         p.kv_block_mask, p.kv_block_size = kv_block_mask.data_ptr(), int(kv_block_size)
         p.kbm_stride_b, p.kbm_stride_h = kv_block_mask.stride(0), kv_block_mask.stride(1)
-    _check(load_library().ma_attn_fwd(ctypes.byref(p), _stream()))
+    lib = load_library()
+    if split_kv:
+        need = lib.ma_attn_workspace_bytes(ctypes.byref(p))
+        if need:
+            if workspace is None:
+                workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+            assert workspace.numel() * workspace.element_size() >= need
+            p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    _check(lib.ma_attn_fwd(ctypes.byref(p), _stream()))
     return out
 
 

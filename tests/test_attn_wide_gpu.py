@@ -223,6 +223,44 @@ def test_row_without_any_key_gives_zeros():
     assert float(o.float().abs().max()) == 0.0 and bool(torch.isinf(lse).all())
 
 
+@pytest.mark.parametrize("D,DV", [(128, 128), (64, 64), (128, 256), (256, 256)])
+@pytest.mark.parametrize("B,H,Hkv,Sq,Skv", [(8, 16, 16, 1, 4096), (2, 8, 2, 1, 1000), (1, 4, 4, 17, 700), (1, 2, 1, 32, 2048)])
+def test_split_kv_decode_matches_unsplit(D, DV, B, H, Hkv, Sq, Skv):
+    """Decode shapes through the split-KV path (workspace given: the default of the wrapper) and unsplit: both against
+    the oracle, lse included, and against each other."""
+    hb = _hb()
+    g = torch.Generator().manual_seed(Skv + D)
+    q = torch.randn(B, Sq, H, D, generator=g).half()
+    k = torch.randn(B, Skv, Hkv, D, generator=g).half()
+    v = torch.randn(B, Skv, Hkv, DV, generator=g).half()
+    ref, lse_ref = oracle.softmax_attention(q, k, v, causal=False, return_lse=True)
+    outs = []
+    for split in (True, False):
+        lse = torch.full((B, H, Sq), float("nan"), device="cuda")
+        o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_SOFTMAX, causal=False, scale=1 / math.sqrt(D), row_scale=lse,
+                        split_kv=split)
+        torch.cuda.synchronize()
+        oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+        torch.testing.assert_close(lse.cpu(), lse_ref, rtol=1e-3, atol=1e-3)
+        outs.append(o)
+    torch.testing.assert_close(outs[0].float(), outs[1].float(), rtol=1e-2, atol=2e-3)
+
+
+def test_decode_workspace_sizes():
+    hb = _hb()
+    import ctypes
+    p = hb.AttnParams()
+    p.family, p.dtype, p.mask = hb.MA_ATTN_SOFTMAX, hb.MA_FP16, hb.MA_MASK_NONE
+    p.batch, p.heads, p.seqlen_q, p.seqlen_kv, p.dim_qk, p.dim_v = 8, 16, 1, 4096, 128, 128
+    lib = hb.load_library()
+    need = lib.ma_attn_workspace_bytes(ctypes.byref(p))
+    assert need == 8 * 8 * 16 * 1 * (128 * 2 + 4)          # 1024 / (8 * 16) = 8 splits
+    p.mask = hb.MA_MASK_CAUSAL
+    assert lib.ma_attn_workspace_bytes(ctypes.byref(p)) == 0
+    p.mask, p.seqlen_q = hb.MA_MASK_NONE, 4096
+    assert lib.ma_attn_workspace_bytes(ctypes.byref(p)) == 0
+
+
 def test_unsupported_head_size_is_an_error():
     hb = _hb()
     q = torch.zeros(1, 64, 1, 96, device="cuda", dtype=torch.bfloat16)
