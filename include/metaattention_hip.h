@@ -152,6 +152,13 @@ typedef struct ma_mla_params {
   float* lse;       /* optional fp32 [B,Hq] natural-log lse; may be NULL */
   float scale;
   void* workspace; size_t workspace_bytes; /* see ma_mla_workspace_bytes */
+  /* optional.  kv_seqlens int32 [B]: cache length of every batch entry (seqlen_kv is then the largest).
+   * block_table int32 [B, block_table_stride]: paged cache as flash_mla_with_kvcache takes it
+   * (cute_template_kvshared/flash_mla_interface.py:75-115): kv / k_pe address a pool of pages of page_size
+   * rows (a multiple of 32; kv_stride_b / kpe_stride_b are ignored) and block_table[b][i] is the page
+   * holding rows i * page_size .. of batch entry b. */
+  const int32_t* kv_seqlens;
+  const int32_t* block_table; int64_t block_table_stride; int32_t page_size;
 } ma_mla_params;
 
 typedef void* ma_stream_t; /* a hipStream_t */

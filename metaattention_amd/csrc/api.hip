@@ -256,6 +256,15 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
   a.B = p->batch; a.Hq = p->heads_q; a.Skv = p->seqlen_kv; a.scale = p->scale;
   a.num_split = ns;
   a.split_len = ((tiles + ns - 1) / ns) * 64;
+  a.kv_lens = p->kv_seqlens;
+  if (p->block_table) {
+    if (p->page_size < 32 || p->page_size % 32 != 0)
+      return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: page_size must be a positive multiple of 32 (got %d)", p->page_size);
+    if ((int64_t)p->block_table_stride * p->page_size < p->seqlen_kv)
+      return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: block table rows of %lld pages do not cover seqlen_kv=%d", (long long)p->block_table_stride, p->seqlen_kv);
+    a.block_table = p->block_table; a.bt_stride = p->block_table_stride; a.page_size = p->page_size;
+    a.kvsb = 0; a.kpsb = 0;
+  }
   if (ns > 1) {
     const size_t need = ma_mla_workspace_bytes(p);
     if (!p->workspace || p->workspace_bytes < need)

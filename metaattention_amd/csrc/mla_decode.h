@@ -12,6 +12,13 @@ struct MlaArgs {
   int64_t qsb, qsh, qpsb, qpsh, kvsb, kvss, kpsb, kpss, osb, osh;
   int B, Hq, Skv, num_split, split_len, head_blocks;
   float scale;
+  // paged cache (flash_mla_with_kvcache of cute_template_kvshared/flash_mla_interface.py:75-115): kv / k_pe then
+  // address a pool of pages of page_size rows, block_table[b * bt_stride + i] is the page holding rows
+  // i * page_size .. of batch entry b; kv_lens[b] (optional, also without pages) is that entry's cache length
+  const int32_t* block_table;
+  int64_t bt_stride;
+  int page_size;
+  const int32_t* kv_lens;
 };
 
 int mla_decode_dispatch(const MlaArgs& a, bool is_bf16, int dim, int dim_pe, hipStream_t stream);

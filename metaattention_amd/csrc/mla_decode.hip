@@ -73,7 +73,8 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
   const int head_ld = min(head, a.Hq - 1);
 
   const int n_begin = split * a.split_len;
-  const int n_end = min(n_begin + a.split_len, a.Skv);
+  const int skv = a.kv_lens ? min(a.Skv, max(a.kv_lens[b], 0)) : a.Skv;   // this batch entry's cache length
+  const int n_end = min(n_begin + a.split_len, skv);
   const int n_tiles = n_end > n_begin ? (n_end - n_begin + BN - 1) / BN : 0;
 
   // ---- Q fragments of this wave's half of the contraction: B operand (lane: head r, k = 8g .. 8g+7 of a slice)
@@ -100,16 +101,19 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
   auto issue_tile = [&](int jt) {
     const uint32_t sb = lds0 + (jt % NSTAGE) * STAGE;
     const int n0 = n_begin + jt * BN;
+    // where the sub-tile's first row lives: with pages, in the page the block table names (a sub-tile never
+    // straddles pages: page sizes and split lengths are multiples of 32)
+    int64_t row0 = n0;
+    if (a.block_table) row0 = (int64_t)a.block_table[b * a.bt_stride + n0 / a.page_size] * a.page_size + n0 % a.page_size;
+    const int last = skv - 1 - n0;   // rows of the sub-tile beyond the cache are clamped to its last row
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int row = wave * 4 + i;
-      const int nrow = min(n0 + row, a.Skv - 1);
-      dma16_so(kvb + nrow * kv_row_bytes, lane_off, sb + row * KV_ROW);
+      dma16_so(kvb + (row0 + min(row, last)) * kv_row_bytes, lane_off, sb + row * KV_ROW);
     }
     if (wave < 4) {
       const int row = wave * 8 + (lane >> 3);
-      const int nrow = min(n0 + row, a.Skv - 1);
-      dma16(peb + nrow * pe_row_bytes + (((lane & 7) ^ swz_pe(row)) << 4), sb + KV_TILE + wave * 8 * PE_ROW);
+      dma16(peb + (row0 + min(row, last)) * pe_row_bytes + (((lane & 7) ^ swz_pe(row)) << 4), sb + KV_TILE + wave * 8 * PE_ROW);
     }
   };
 

@@ -96,6 +96,8 @@ class MlaParams(Structure):
         ("lse", c_void_p),
         ("scale", c_float),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+        ("kv_seqlens", c_void_p),
+        ("block_table", c_void_p), ("block_table_stride", c_int64), ("page_size", c_int32),
     ]
 
 
@@ -251,7 +253,7 @@ def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, 
     return dq, dk, dv
 
 
-def mla_decode(q, q_pe, kv, k_pe, *, scale: float, num_split: int = 0, out=None, lse=None, workspace=None):
+def mla_decode(q, q_pe, kv, k_pe, *, scale: float, num_split: int = 0, out=None, lse=None, workspace=None, kv_seqlens=None):
     """Absorbed MLA decode.  q [B,1,Hq,D], q_pe [B,1,Hq,Dpe], kv [B,Skv,1,D],
     k_pe [B,Skv,1,Dpe] (the reference operator's layouts) -> [B,1,Hq,D]."""
     _require_gpu(q, q_pe, kv, k_pe, out, lse, workspace)
@@ -274,6 +276,9 @@ def mla_decode(q, q_pe, kv, k_pe, *, scale: float, num_split: int = 0, out=None,
         assert lse.dtype == torch.float32 and lse.shape == (B, Hq) and lse.is_contiguous()
         p.lse = lse.data_ptr()
     p.scale = float(scale)
+    if kv_seqlens is not None:
+        assert kv_seqlens.dtype == torch.int32 and kv_seqlens.shape == (B,) and kv_seqlens.is_contiguous() and kv_seqlens.is_cuda
+        p.kv_seqlens = kv_seqlens.data_ptr()
     lib = load_library()
     need = lib.ma_mla_workspace_bytes(ctypes.byref(p))
     if need:
@@ -283,6 +288,55 @@ def mla_decode(q, q_pe, kv, k_pe, *, scale: float, num_split: int = 0, out=None,
         p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
     _check(lib.ma_mla_decode(ctypes.byref(p), _stream()))
     return out
+
+
+def get_mla_metadata(cache_seqlens, num_heads_per_head_k: int, num_heads_k: int):
+    """Counterpart of get_mla_metadata (cute_template_kvshared/flash_mla_interface.py:57-72).  The reference plans
+    per-SM work lists there; this library plans its kv splits inside ma_mla_decode from the sizes alone, so the
+    "metadata" is only the plan's summary: an int32 [1, 2] tensor (heads per kv head, kv heads) and an int32
+    [batch + 1] tensor of cumulative split counts (one unit per batch entry; the split count proper is chosen at
+    launch).  Both are accepted and ignored by flash_mla_with_kvcache."""
+    B = cache_seqlens.shape[0]
+    meta = torch.tensor([[num_heads_per_head_k, num_heads_k]], dtype=torch.int32, device=cache_seqlens.device)
+    return meta, torch.arange(B + 1, dtype=torch.int32, device=cache_seqlens.device)
+
+
+def flash_mla_with_kvcache(q, k_cache, block_table, cache_seqlens, head_dim_v: int, tile_scheduler_metadata=None, num_splits=None,
+                           softmax_scale=None, causal: bool = False):
+    """Paged absorbed-MLA decode with the signature of flash_mla_with_kvcache
+    (cute_template_kvshared/flash_mla_interface.py:75-115): q [B,1,Hq,576], k_cache [pages, page_size, 1, 576]
+    (latent 512 + rope 64 in one row), block_table int32 [B, pages per sequence], cache_seqlens int32 [B]
+    -> (out [B,1,Hq,512], softmax_lse fp32 [B,Hq,1], natural log).  One query token, so `causal` changes nothing."""
+    _require_gpu(q, k_cache, block_table, cache_seqlens)
+    B, Sq, Hq, Dfull = q.shape
+    assert Sq == 1 and k_cache.shape[2] == 1 and k_cache.shape[3] == Dfull and head_dim_v < Dfull, "one query token, one latent kv head"
+    page = k_cache.shape[1]
+    assert block_table.dtype == torch.int32 and block_table.shape[0] == B and block_table.stride(1) == 1
+    assert q.stride(-1) == 1 and k_cache.is_contiguous()
+    D, Dpe = head_dim_v, Dfull - head_dim_v
+    scale = Dfull ** -0.5 if softmax_scale is None else softmax_scale
+    out = torch.empty(B, 1, Hq, D, dtype=q.dtype, device=q.device)
+    lse = torch.empty(B, Hq, dtype=torch.float32, device=q.device)
+    seqlens = cache_seqlens.to(torch.int32).contiguous()
+    p = MlaParams()
+    p.dtype = _dtype_code(q.dtype)
+    p.batch, p.heads_q, p.seqlen_kv, p.dim, p.dim_pe, p.num_split = B, Hq, block_table.shape[1] * page, D, Dpe, 0
+    esz = q.element_size()
+    p.q, p.q_stride_b, p.q_stride_h = q.data_ptr(), q.stride(0), q.stride(2)
+    p.q_pe, p.qpe_stride_b, p.qpe_stride_h = q.data_ptr() + D * esz, q.stride(0), q.stride(2)
+    p.kv, p.kv_stride_b, p.kv_stride_s = k_cache.data_ptr(), 0, Dfull
+    p.k_pe, p.kpe_stride_b, p.kpe_stride_s = k_cache.data_ptr() + D * esz, 0, Dfull
+    p.o, p.o_stride_b, p.o_stride_h = out.data_ptr(), out.stride(0), out.stride(2)
+    p.lse, p.scale = lse.data_ptr(), float(scale)
+    p.kv_seqlens = seqlens.data_ptr()
+    p.block_table, p.block_table_stride, p.page_size = block_table.data_ptr(), block_table.stride(0), page
+    lib = load_library()
+    need = lib.ma_mla_workspace_bytes(ctypes.byref(p))
+    if need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        p.workspace, p.workspace_bytes = workspace.data_ptr(), need
+    _check(lib.ma_mla_decode(ctypes.byref(p), _stream()))
+    return out, lse.view(B, Hq, 1)
 
 
 def mla_workspace_bytes(B, Hq, Skv, D=512, Dpe=64, num_split=0) -> int:

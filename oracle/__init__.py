@@ -28,6 +28,8 @@ ssd_chunk_scan         3-way agreement: chunked reference == naive sequential
 simple_gla             token-by-token recurrence (fp64)
 mla_decode             SDPA with K=concat(kv,k_pe), V=kv; split-KV invariance
 sparse_decode_attention  dense attention over the gathered kept keys only
+paged_mla_decode       mla_decode on the contiguous cache (identity table); invariance
+                       to a permutation of the page pool
 attention_grads,       central differences of the pinned forward functions in
 linear_attention_grads fp64 along random directions; SDPA's own autograd
 (all of the above)     tests/golden/*.npz: the operators' definitions evaluated
@@ -45,6 +47,7 @@ from .attention_ref import (  # noqa: F401
     retention_decay_mask,
     attention_grads,
     sparse_decode_attention,
+    paged_mla_decode,
 )
 from .linear_ref import (  # noqa: F401
     retnet_quadratic,

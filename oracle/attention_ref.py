@@ -174,3 +174,22 @@ def sparse_decode_attention(q, k, v, block_mask=None, cache_seqlens=None, block_
             s = s.masked_fill(~keep, float("-inf"))
             out[b, h] = torch.softmax(s, dim=-1) @ v[b, :, g].to(compute_dtype)
     return out
+
+
+def paged_mla_decode(q, k_cache, block_table, cache_seqlens, head_dim_v: int = 512, compute_dtype=torch.float32):
+    """flash_mla_with_kvcache semantics (cute_template_kvshared/flash_mla_interface.py:75-115) for one query
+    token: q [B,1,Hq,d+dpe]; k_cache [pages, page_size, 1, d+dpe]; sequence b is the rows of pages
+    block_table[b, 0], block_table[b, 1], ... truncated to cache_seqlens[b]; per sequence the absorbed MLA
+    decode of ``mla_decode`` (scores over all d+dpe columns, values = the first d).  Returns (out [B,1,Hq,d],
+    lse [B,Hq,1] natural log)."""
+    B, _, Hq, Dfull = q.shape
+    d = head_dim_v
+    out = torch.empty(B, 1, Hq, d, dtype=compute_dtype)
+    lse = torch.empty(B, Hq, 1, dtype=compute_dtype)
+    for b in range(B):
+        L = int(cache_seqlens[b])
+        rows = k_cache[block_table[b].long()].reshape(-1, 1, Dfull)[:L]              # [L,1,Dfull]
+        o, l = mla_decode(q[b:b + 1, :, :, :d], q[b:b + 1, :, :, d:], rows[None, :, :, :d], rows[None, :, :, d:],
+                          compute_dtype=compute_dtype, return_lse=True)
+        out[b], lse[b, :, 0] = o[0], l[0]
+    return out, lse

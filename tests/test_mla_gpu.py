@@ -78,3 +78,37 @@ def test_mla_rejects_bad_arguments():
     kv5 = torch.zeros(1, 64, 1, 512, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(hb.MetaAttentionError):
         hb.mla_decode(q5, qp, kv5, kp, scale=SCALE, num_split=5)     # more splits than kv tiles
+
+
+@pytest.mark.parametrize("B,Hq,page,pages_per_seq,dtype", [(4, 128, 64, 8, torch.bfloat16), (3, 16, 64, 5, torch.float16), (2, 40, 32, 9, torch.bfloat16)])
+def test_paged_mla_with_kvcache(B, Hq, page, pages_per_seq, dtype):
+    """flash_mla_with_kvcache-style call: fused 576-wide rows, shuffled page pool, ragged cache lengths."""
+    hb = _hb()
+    g = torch.Generator().manual_seed(B * 100 + Hq)
+    npg = B * pages_per_seq + 3
+    q = torch.randn(B, 1, Hq, 576, generator=g).to(dtype)
+    cache = torch.randn(npg, page, 1, 576, generator=g).to(dtype)
+    table = torch.randperm(npg, generator=g)[:B * pages_per_seq].to(torch.int32).view(B, pages_per_seq)
+    lens = torch.randint(1, page * pages_per_seq + 1, (B,), generator=g, dtype=torch.int32)
+    lens[0] = page * pages_per_seq
+    meta, splits = hb.get_mla_metadata(lens.cuda(), Hq, 1)
+    print(f"paged mla B{B} Hq{Hq} page{page} x{pages_per_seq} lens {lens.tolist()} {dtype}", flush=True)
+    out, lse = hb.flash_mla_with_kvcache(q.cuda(), cache.cuda(), table.cuda(), lens.cuda(), 512, meta, splits)
+    torch.cuda.synchronize()
+    assert out.shape == (B, 1, Hq, 512) and lse.shape == (B, Hq, 1)
+    ref, lse_ref = oracle.paged_mla_decode(q, cache, table, lens)
+    oracle.assert_close(out.float().cpu(), ref, rtol=1e-2, atol=2e-2)
+    torch.testing.assert_close(lse.cpu(), lse_ref, rtol=1e-4, atol=1e-4)
+
+
+def test_mla_cache_lengths_without_pages():
+    hb = _hb()
+    B, Hq, Skv = 3, 128, 1024
+    q, q_pe, kv, k_pe = inputs.mla_inputs(B, Hq, Skv, 512, 64, seed=4)
+    lens = torch.tensor([1024, 700, 33], dtype=torch.int32)
+    o = hb.mla_decode(q.cuda(), q_pe.cuda(), kv.cuda(), k_pe.cuda(), scale=SCALE, kv_seqlens=lens.cuda())
+    torch.cuda.synchronize()
+    for b in range(B):
+        L = int(lens[b])
+        ref = oracle.mla_decode(q[b:b + 1], q_pe[b:b + 1], kv[b:b + 1, :L], k_pe[b:b + 1, :L])
+        oracle.assert_close(o[b:b + 1].float().cpu(), ref, rtol=1e-2, atol=2e-2)

@@ -298,3 +298,25 @@ def test_sparse_decode_equals_dense_attention_over_kept_keys():
             ref = oracle.softmax_attention(q[b:b + 1, :, h:h + 1], k[b:b + 1, idx, gi:gi + 1], v[b:b + 1, idx, gi:gi + 1], causal=False,
                                            compute_dtype=torch.float64)
             torch.testing.assert_close(got[b, h], ref[0, 0, 0])
+
+
+def test_paged_mla_identity_table_and_page_permutation():
+    g = torch.Generator().manual_seed(17)
+    B, Hq, page, npg = 2, 3, 4, 5
+    q = torch.randn(B, 1, Hq, 24, generator=g, dtype=torch.float64)
+    cache = torch.randn(B * npg, page, 1, 24, generator=g, dtype=torch.float64)
+    table = torch.arange(B * npg, dtype=torch.int32).view(B, npg)
+    lens = torch.tensor([20, 13], dtype=torch.int32)
+    out, lse = oracle.paged_mla_decode(q, cache, table, lens, head_dim_v=16, compute_dtype=torch.float64)
+    for b in range(B):
+        rows = cache[b * npg:(b + 1) * npg].reshape(1, -1, 1, 24)[:, :int(lens[b])]
+        o, l = oracle.mla_decode(q[b:b + 1, :, :, :16], q[b:b + 1, :, :, 16:], rows[..., :16], rows[..., 16:], compute_dtype=torch.float64,
+                                 return_lse=True)
+        torch.testing.assert_close(out[b:b + 1], o)
+        torch.testing.assert_close(lse[b, :, 0], l[0])
+    perm = torch.randperm(B * npg, generator=g)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(B * npg)
+    out2, lse2 = oracle.paged_mla_decode(q, cache[perm], inv[table.long()].to(torch.int32), lens, head_dim_v=16, compute_dtype=torch.float64)
+    torch.testing.assert_close(out2, out)
+    torch.testing.assert_close(lse2, lse)
