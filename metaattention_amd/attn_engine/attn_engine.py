@@ -137,7 +137,7 @@ class AttentionEngine:
 
         # dispatch by shape, as attn_engine.py:227-343
         if kv_shared:
-            self._init_mla()
+            self._init_mla(backend)
         elif Hq % Hkv != 0:
             raise NotImplementedError("heads of q must be a multiple of the heads of k and v")
         else:
@@ -231,7 +231,7 @@ class AttentionEngine:
         return run(q, k, v)
 
     # ------------------------------------------------------------------ MLA decode
-    def _init_mla(self):
+    def _init_mla(self, backend="tl"):
         m = self.meta
         if m["Hkv"] != 1:
             raise AssertionError("MLA decode needs a single latent kv head")   # mla_decode_tl.py:58
@@ -242,6 +242,22 @@ class AttentionEngine:
         # (core/lower/lower_decode_mla.py:25-38): fixed softmax, scale (d + d_pe)^-0.5
         self.mla_scale = 1.0 / math.sqrt(m["Dqk"])
         self.attention = self._call_mla
+        if backend in ("cute", "cute_v2"):
+            # the paged interface of the reference's second MLA backend (attn_engine.py:196-224): mod(q [B,1,Hq,576],
+            # k_cache [B * Skv / 64, 64, 1, 576]) -> (out, lse), every sequence full, pages in order
+            self.attention = self._call_mla_paged
+
+    def _call_mla_paged(self, q, k_cache):
+        from hip_backend import flash_mla_with_kvcache
+        m = self.meta
+        page = k_cache.shape[1]
+        pad = ((m["Skv"] + 255) // 256) * 256                     # as attn_engine.py:211-216
+        table = torch.arange(m["B"] * pad // page, dtype=torch.int32, device=q.device).view(m["B"], pad // page)
+        if pad != m["Skv"]:                                        # the pool holds Skv / page pages per sequence, in order
+            table = (torch.arange(m["B"], dtype=torch.int32, device=q.device).view(-1, 1) * (m["Skv"] // page)
+                     + torch.arange(pad // page, dtype=torch.int32, device=q.device).view(1, -1)).clamp_(max=k_cache.shape[0] - 1)
+        lens = torch.full((m["B"],), m["Skv"], dtype=torch.int32, device=q.device)
+        return flash_mla_with_kvcache(q, k_cache, table, lens, m["Dv"], softmax_scale=self.mla_scale)
 
     def _call_mla(self, q, q_pe, kv, k_pe):
         from hip_backend import mla_decode

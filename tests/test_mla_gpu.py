@@ -112,3 +112,25 @@ def test_mla_cache_lengths_without_pages():
         L = int(lens[b])
         ref = oracle.mla_decode(q[b:b + 1], q_pe[b:b + 1], kv[b:b + 1, :L], k_pe[b:b + 1, :L])
         oracle.assert_close(o[b:b + 1].float().cpu(), ref, rtol=1e-2, atol=2e-2)
+
+
+def test_engine_paged_mla_backend():
+    """examples/mla_decode_v2.py through the engine: mod(q [B,1,Hq,576], KV [B*Skv/64, 64, 1, 576]) -> (out, lse)
+    (testing/benchmark_h100.py:1079-1087)."""
+    from attn_engine import AttentionEngine
+    from core import CustomIO, meta_tensor
+    import specs
+    B, Hq, Skv = 2, 128, 512
+    meta = (meta_tensor(B, Hq, 1, 576, dtype=torch.bfloat16), meta_tensor(B, 1, Skv, 576, dtype=torch.bfloat16),
+            meta_tensor(B, 1, Skv, 512, dtype=torch.bfloat16))
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=lambda s, io, b, h, q, k: s * (576 ** -0.5), mask_mod=None,
+                          online_func=specs.OnlineSoftmax(), kv_shared=True, backend="cute")
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(B, 1, Hq, 576, generator=g).bfloat16()
+    cache = torch.randn(B * Skv // 64, 64, 1, 576, generator=g).bfloat16()
+    out, lse = mod(q.cuda(), cache.cuda())
+    torch.cuda.synchronize()
+    rows = cache.view(B, Skv, 1, 576)
+    ref, lse_ref = oracle.mla_decode(q[..., :512], q[..., 512:], rows[..., :512], rows[..., 512:], return_lse=True)
+    oracle.assert_close(out.float().cpu(), ref, rtol=1e-2, atol=2e-2)
+    torch.testing.assert_close(lse.cpu()[:, :, 0], lse_ref, rtol=1e-4, atol=1e-4)
