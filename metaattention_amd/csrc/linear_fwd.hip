@@ -136,19 +136,50 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
   auto issue_chunk = [&](int t0, int buf) {
     const uint32_t base = lds0 + buf * STAGE;
     constexpr int NQK = MODE == 1 ? NIQ : 2 * NIQ;      // (the state-only pass needs no Q)
-#pragma unroll (DK <= 128 && HG == 1 ? 16 : 1)   // (unrolled burst only where the state leaves registers for it)
+    constexpr int RQ = 1024 / RBQ, RV = 1024 / RBV;     // tile rows per instruction
+    if (t0 + L <= Tn && v_head_bytes < ((int64_t)1 << 31)) {
+      // Whole chunk: no row clamping, so an instruction's source is a wave-uniform base (SGPRs) plus a
+      // 32-bit lane offset.  The swizzle is a bit permutation of the row index, so it splits into the
+      // lane's part (row within the instruction) and the instruction's part (its first row): per
+      // instruction that is one XOR, against ~25 vector instructions of 64-bit address arithmetic.
+      int ln2 = lane;
+      asm volatile("" : "+v"(ln2));   // rebuilt per chunk: kept live across the chunk these would cost registers
+      const int lrq = ln2 / CPRQ, lrv = ln2 / CPRV;
+      const uint32_t offq = lrq * RBQ, lcq0 = (ln2 % CPRQ) ^ swz_tile<CPRQ>(lrq);
+      const uint32_t offv = lrv * (uint32_t)v_row_bytes, lcv0 = (ln2 % CPRV) ^ swz_tile<CPRV>(lrv);
+#pragma unroll (DK <= 128 ? 16 : 1)   // (with a 256-wide key the state leaves no registers for an unrolled burst)
+      for (int it = 0; it < (NQK + NIV + NW - 1) / NW; it++) {
+        const int ii = wave + NW * it;
+        if ((NQK + NIV) % NW != 0 && ii >= NQK + NIV) break;
+        if (ii < NQK) {
+          const int which = MODE == 1 ? 1 : ii >= NIQ, i2 = (MODE != 1 && which) ? ii - NIQ : ii;
+          const char* sb = (which ? kb : qb) + (int64_t)(t0 + i2 * RQ) * RBQ;
+          dma16_so(sb, offq + ((lcq0 ^ (uint32_t)swz_tile<CPRQ>(i2 * RQ)) << 4), base + which * QT + i2 * 1024);
+        } else {
+          const int i2 = ii - NQK;
+          const char* sb = vb + (int64_t)(t0 + i2 * RV) * v_row_bytes;
+          const uint32_t lc = lcv0 ^ (uint32_t)swz_tile<CPRV>(i2 * RV);   // logical chunk: head lc / (4 NWH), then its columns
+          uint32_t off = offv + ((lc % (4 * NWH)) << 4);
+          if (HG > 1) off += (lc / (4 * NWH)) * (uint32_t)v_head_bytes;
+          dma16_so(sb, off, base + 2 * QT + i2 * 1024);
+        }
+      }
+      return;
+    }
+    // last, partial chunk: rows beyond the sequence are clamped to its last row
+#pragma unroll 1
     for (int it = 0; it < (NQK + NIV + NW - 1) / NW; it++) {
       const int ii = wave + NW * it;
       if ((NQK + NIV) % NW != 0 && ii >= NQK + NIV) break;
       if (ii < NQK) {
         const int which = MODE == 1 ? 1 : ii >= NIQ, i2 = (MODE != 1 && which) ? ii - NIQ : ii;
-        const int row = i2 * (1024 / RBQ) + lane / CPRQ, c = lane % CPRQ;
+        const int row = i2 * RQ + lane / CPRQ, c = lane % CPRQ;
         const int trow = min(t0 + row, Tn - 1);
         const char* src = (which ? kb : qb) + (int64_t)trow * RBQ + ((c ^ swz_tile<CPRQ>(row)) << 4);
         dma16(src, base + which * QT + i2 * 1024);
       } else {
         const int i2 = ii - NQK;
-        const int row = i2 * (1024 / RBV) + lane / CPRV, c = lane % CPRV;
+        const int row = i2 * RV + lane / CPRV, c = lane % CPRV;
         const int trow = min(t0 + row, Tn - 1);
         const int lc = c ^ swz_tile<CPRV>(row);          // logical 16-byte chunk: head lc / (4 NWH), then its columns
         const char* src = vb + (int64_t)trow * v_row_bytes + ((lc % (4 * NWH)) << 4);
