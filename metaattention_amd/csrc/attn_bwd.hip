@@ -253,10 +253,13 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
 // ------------------------------------------------------------------------------------------------
 // dk, dv
 // ------------------------------------------------------------------------------------------------
-template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
-// (the two [D x 32] accumulators plus the K and V fragments take 192 registers at 128/128: one wave per SIMD there;
-// forcing two makes the compiler spill the fragments and is slower)
-__global__ __launch_bounds__(256, (DQK + DV >= 256 ? 1 : 2)) void attn_bwd_dkv_kernel(const AttnBwdArgs a) {
+// WHAT: 3 = dk and dv in one launch, 1 = dv only, 2 = dk only.  Both [D x 32] accumulators plus the K and V
+// fragments take 192 registers at 128/128, which leaves one wave per SIMD (forcing two makes the compiler
+// spill the fragments and is slower); computing dv and dk in two launches (the scores are then computed once
+// more) lets each run two waves per SIMD.
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL, int WHAT>
+__global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK + DV >= 512 ? 1 : 2))) void attn_bwd_dkv_kernel(const AttnBwdArgs a) {
+  constexpr bool DO_DV = (WHAT & 1) != 0, DO_DK = (WHAT & 2) != 0;
   using E = Elem<T>;
   using x8 = typename E::x8;
   constexpr int BNW = 128, BMT = 32;   // keys per workgroup, query rows per tile
@@ -356,7 +359,11 @@ __global__ __launch_bounds__(256, (DQK + DV >= 256 ? 1 : 2)) void attn_bwd_dkv_k
       }
     }
     const f32x16 s = mm_rows<T, DQK>(qbase, r, g, kf);     // S: lane = key n_lane, element jj = row m0 + 8(jj/4) + 4g + jj%4
-    const f32x16 dp = mm_rows<T, DV>(dobase, r, g, vf);   // dP, same layout
+    f32x16 dp;
+    if constexpr (DO_DK) dp = mm_rows<T, DV>(dobase, r, g, vf);   // dP, same layout
+    else
+#pragma unroll
+      for (int j = 0; j < 16; j++) dp[j] = 0.f;
     x8 pf[2], dsf[2];
 #pragma unroll
     for (int jj = 0; jj < 16; jj++) {
@@ -369,8 +376,8 @@ __global__ __launch_bounds__(256, (DQK + DV >= 256 ? 1 : 2)) void attn_bwd_dkv_k
       pf[jj >> 3][jj & 7] = (T)p;
       dsf[jj >> 3][jj & 7] = (T)ds;
     }
-    mm_cols<T, DV>(dobase, lane, pf, dv);     // dV^T += dO^T P
-    mm_cols<T, DQK>(qbase, lane, dsf, dk);    // dK^T += Q^T dS
+    if constexpr (DO_DV) mm_cols<T, DV>(dobase, lane, pf, dv);     // dV^T += dO^T P
+    if constexpr (DO_DK) mm_cols<T, DQK>(qbase, lane, dsf, dk);    // dK^T += Q^T dS
   }
   __syncthreads();   // every wave is done with the tiles: they become output staging
 
@@ -378,8 +385,8 @@ __global__ __launch_bounds__(256, (DQK + DV >= 256 ? 1 : 2)) void attn_bwd_dkv_k
   const uint32_t stage = lds0 + wave * 32 * OROW;
   T* dkb = (T*)a.dk + (int64_t)b * a.dksb + (int64_t)hk * a.dksh;
   T* dvb = (T*)a.dv + (int64_t)b * a.dvsb + (int64_t)hk * a.dvsh;
-  store_rows<T, DQK>(dk, 1.f, stage, dkb, a.dkss, n_wave, a.Skv, lane);
-  store_rows<T, DV>(dv, 1.f, stage, dvb, a.dvss, n_wave, a.Skv, lane);
+  if constexpr (DO_DK) store_rows<T, DQK>(dk, 1.f, stage, dkb, a.dkss, n_wave, a.Skv, lane);
+  if constexpr (DO_DV) store_rows<T, DV>(dv, 1.f, stage, dvb, a.dvss, n_wave, a.Skv, lane);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -390,11 +397,15 @@ static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   constexpr size_t ostage = 4 * 32 * (size_t)(DMAX + 16);
   constexpr size_t lds = tiles > ostage ? tiles : ostage;
   auto k1 = attn_bwd_dq_kernel<T, DQK, DV, FAMILY, CAUSAL>;
-  auto k2 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL>;
+  // one dk/dv launch where both accumulators fit beside a second wave, else one launch each
+  constexpr bool SPLIT = DQK + DV >= 256 && DQK + DV < 512;
+  auto k2 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL, SPLIT ? 1 : 3>;
+  auto k3 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL, 2>;
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
     if (hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
+    if (SPLIT && hipFuncSetAttribute((const void*)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
     attr_set = true;
   }
   AttnBwdArgs args = a;
@@ -402,6 +413,7 @@ static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL(k1, dim3((unsigned)(args.num_blocks * a.B * a.H)), dim3(256), lds, stream, args);
   args.num_blocks = (a.Skv + 127) / 128;
   hipLaunchKernelGGL(k2, dim3((unsigned)(args.num_blocks * a.B * a.Hkv)), dim3(256), lds, stream, args);
+  if (SPLIT) hipLaunchKernelGGL(k3, dim3((unsigned)(args.num_blocks * a.B * a.Hkv)), dim3(256), lds, stream, args);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
