@@ -83,6 +83,13 @@ typedef struct ma_attn_params {
   int32_t kv_block_size;
   const int32_t* kv_seqlens;
   const uint8_t* kv_block_mask; int64_t kbm_stride_b, kbm_stride_h;
+  /* arbitrary masks (blockattn_tl.py:123-234, where the mask_mod's code is generated into the kernel): elem_mask
+   * uint8/bool [1 or B, 1 or H, Sq, Skv] (strides in bytes = elements; stride 0 broadcasts; rows 4-byte aligned),
+   * 0 = the score is masked (probability exactly 0).  With it, kv_block_mask may be the prefill form
+   * [.., heads, ceil(Sq/128), ceil(Skv/kv_block_size)]: set kbm_stride_q (blocks of 128 query rows) and
+   * kbm_per_query_head = 1.  Not with MA_MASK_CAUSAL (the element mask says it all) nor RETENTION. */
+  const uint8_t* elem_mask; int64_t em_stride_b, em_stride_h, em_stride_q;
+  int64_t kbm_stride_q; int32_t kbm_per_query_head;
   /* optional; with ma_attn_workspace_bytes(&params) bytes, decode shapes (at most 32 query rows, SOFTMAX, no
    * structural mask) run as split-KV + combine (attn_decode_tl.py:63-206); without it they run unsplit */
   void* workspace; size_t workspace_bytes;

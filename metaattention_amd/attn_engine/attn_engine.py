@@ -145,8 +145,6 @@ class AttentionEngine:
             # Dense decode (seq_len_q != seq_len_kv, attn_engine.py:262-303; the examples pad the declared seq_len_q to
             # a multiple of 128 and pass the real query, examples/mha_decode.py:104-108) runs through the same kernels
             # with no structural mask; the reference's split-KV launch and its block-sparse variants have no counterpart.
-            if Sq != Skv and mask_mod is not None:
-                raise NotImplementedError("masked decode (seq_len_q != seq_len_kv with a mask_mod) is not in the kernel library")
             self._init_prefill(score_mod, mask_mod, online_func, mask_value)
 
     # ------------------------------------------------------------------ prefill
@@ -166,6 +164,17 @@ class AttentionEngine:
         if mask_value not in ("-inf", "0"):
             raise NotImplementedError(f"mask_value {mask_value!r}")
         self.mask_kind = classify_mask(mask_mod, m["B"], m["Hq"], m["Sq"], m["Skv"])
+        self.mask_mod, self._mask_tensors = mask_mod, None
+        if self.mask_kind.startswith("other"):
+            # any other mask_mod: evaluated densely once (the reference does the same to infer its block mask,
+            # lower.py:723-740) into an element-wise keep mask plus a block mask for tile skipping
+            if fam == "retention":
+                raise NotImplementedError("the retention kernel takes the causal structural mask or none")
+            if m["Sq"] != m["Skv"] and m["Sq"] % 128 != 0:
+                pass     # (a declared query length padded for decode: the mask is built for the tensors actually passed)
+            dense_bytes = (m["B"] * m["Hq"] if self.mask_kind == "other_bh" else 1) * m["Sq"] * m["Skv"]
+            if dense_bytes > 2 ** 31:
+                raise NotImplementedError("a mask_mod that depends on batch or head at this size needs more than 2 GiB as a dense mask")
         # mask_value "0": the reference applies no element-wise mask in forward, only causal
         # tile skipping (lower.py:638, attn_tl.py:140-151); the retention kernel does the same.
         if mask_value == "0" and fam != "retention" and self.mask_kind != "none":
@@ -185,7 +194,7 @@ class AttentionEngine:
         form = self.score_form
 
         sparse = block_mask is not None or cache_seqlens is not None
-        if sparse and (self.mask_kind == "causal" or self.family == "retention"):
+        if sparse and (self.mask_kind != "none" or self.family == "retention"):
             raise NotImplementedError("block_mask / cache_seqlens are for the unmasked decode operators")
         if block_mask is not None and block_mask.dim() != 3:
             raise NotImplementedError("only kv block masks [batch, heads_kv, blocks] (decode) are in the kernel library; "
@@ -197,11 +206,14 @@ class AttentionEngine:
             grp = H // Hkv
             kw = dict(family=fam_code, causal=self.mask_kind == "causal", scale=form.scale, bias=form.bias,
                       bias_tensor=given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None)
+            if self.mask_kind.startswith("other"):
+                elem, blocks = self._dense_mask(B, H, Sq, k.shape[1], q.device)
+                kw.update(elem_mask=elem, kv_block_mask=blocks, kv_block_size=32)
             if sparse:
                 kw.update(kv_seqlens=cache_seqlens.to(torch.int32) if cache_seqlens is not None else None, kv_block_mask=block_mask,
                           kv_block_size=self.kv_block_size if block_mask is not None else 0)
             has_rs = self.family in ("softmax", "retention")
-            if Sq == 1 and grp > 1 and self.mask_kind != "causal" and self.family != "retention":
+            if Sq == 1 and grp > 1 and self.mask_kind == "none" and self.family != "retention":
                 # one query token, grouped-query: the query heads of a kv head become the rows of that head
                 # (the decode kernels of the reference pack them the same way, attn_gqa_decode_tl.py:81-84)
                 out = torch.empty(B, 1, H, Dv, dtype=q.dtype, device=q.device)
@@ -224,11 +236,29 @@ class AttentionEngine:
             return run(q, k, v).squeeze(1)
 
         if any(t.requires_grad for t in (q, k, v)):
-            if self.family == "retention":
+            if self.family == "retention" or self.mask_kind.startswith("other"):
                 return _ForwardOnly.apply(run, q, k, v)
             bias_t = given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None
             return _Attention.apply(self, run, fam_code, bias_t, q, k, v)
         return run(q, k, v)
+
+    def _dense_mask(self, B, H, Sq, Skv, device):
+        """(element-wise keep mask uint8 [1|B, 1|H, Sq, Skv] with 4-byte aligned rows, block mask uint8
+        [1|B, 1|H, ceil(Sq/128), ceil(Skv/32)]: a block is kept when any of its elements is) for the mask_mod, built
+        once per shape on the device."""
+        from core.transform.core import create_mask
+        key = (B, H, Sq, Skv, str(device))
+        if self._mask_tensors is None or self._mask_tensors[0] != key:
+            Bm, Hm = (B, H) if self.mask_kind == "other_bh" else (1, 1)
+            dense = create_mask(self.mask_mod, Bm, Hm, Sq, Skv, device)
+            skp, sqp, nkp = (Skv + 3) // 4 * 4, (Sq + 127) // 128 * 128, (Skv + 31) // 32 * 32
+            buf = torch.zeros(Bm, Hm, Sq, skp, dtype=torch.uint8, device=device)
+            buf[..., :Skv] = dense
+            pad = torch.zeros(Bm, Hm, sqp, nkp, dtype=torch.bool, device=device)
+            pad[:, :, :Sq, :Skv] = dense
+            blocks = pad.view(Bm, Hm, sqp // 128, 128, nkp // 32, 32).any(dim=5).any(dim=3).to(torch.uint8).contiguous()
+            self._mask_tensors = (key, buf[..., :Skv], blocks)
+        return self._mask_tensors[1], self._mask_tensors[2]
 
     # ------------------------------------------------------------------ MLA decode
     def _init_mla(self, backend="tl"):

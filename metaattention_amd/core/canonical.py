@@ -321,9 +321,12 @@ def _allclose(a, b) -> bool:
 # mask_mod
 # ---------------------------------------------------------------------------
 def classify_mask(mask_mod, B, H, Sq, Skv, block_M=128, block_N=128) -> str:
-    """"none" | "causal".  Evaluates ``mask_mod`` densely on index grids on
-    the CPU (as the reference does at block granularity, lower.py:723-740) and
-    compares with the exact causal pattern; every (batch, head) must agree."""
+    """"none" | "causal" | "other" | "other_bh".  Evaluates ``mask_mod`` densely on index grids on
+    the CPU (as the reference does at block granularity, lower.py:723-740) and compares with the
+    exact causal pattern on a sample of (batch, head) pairs.  "other": some other pattern, the same
+    for every sampled (batch, head); "other_bh": it depends on batch or head.  Both run through an
+    element-wise keep mask built by the caller (the reference generates the mask_mod's code into
+    its block-sparse kernel instead, blockattn_tl.py:176-190)."""
     from .transform.core import create_mask
     if mask_mod is None:
         return "none"
@@ -331,12 +334,17 @@ def classify_mask(mask_mod, B, H, Sq, Skv, block_M=128, block_N=128) -> str:
     kj = torch.arange(Skv).view(1, Skv)
     causal = qi >= kj
     kinds = set()
+    first, same = None, True
     for b in sorted({0, B - 1}):
         for h in sorted({0, H // 2, H - 1}):
             m = mask_mod(torch.tensor(b), torch.tensor(h), qi, kj)
             m = m if torch.is_tensor(m) else torch.full((Sq, Skv), bool(m))
             m = m.expand(Sq, Skv)
-            if torch.equal(m, causal):
+            if first is None:
+                first = m
+            elif not torch.equal(m, first):
+                same = False
+            if Sq == Skv and torch.equal(m, causal):
                 kinds.add("causal")
             elif bool(m.all()):
                 kinds.add("none")
@@ -346,9 +354,7 @@ def classify_mask(mask_mod, B, H, Sq, Skv, block_M=128, block_N=128) -> str:
         return "causal"
     if kinds == {"none"}:
         return "none"
-    raise NotImplementedError(
-        "mask_mod is neither the causal mask (q_idx >= kv_idx) nor all-true; block-sparse and shifted masks are not "
-        "in the kernel library")
+    return "other" if same else "other_bh"
 
 
 # ---------------------------------------------------------------------------

@@ -57,6 +57,12 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
     return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: kv_block_size must be a positive multiple of 32 (got %d)", p->kv_block_size);
   if ((p->kv_block_mask || p->kv_seqlens) && p->mask == MA_MASK_CAUSAL)
     return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: kv_seqlens / kv_block_mask are for the unmasked (decode) operators");
+  if (p->elem_mask) {
+    if (p->mask == MA_MASK_CAUSAL || p->family == MA_ATTN_RETENTION)
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: elem_mask goes with MA_MASK_NONE and the softmax / sigmoid / relu families");
+    if ((uintptr_t)p->elem_mask % 4 != 0 || p->em_stride_q % 4 != 0 || p->em_stride_h % 4 != 0 || p->em_stride_b % 4 != 0)
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: elem_mask rows must be 4-byte aligned");
+  }
   if (p->family == MA_ATTN_RETENTION) {
     if (!p->score_mask) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: RETENTION needs score_mask");
     if ((uintptr_t)p->score_mask % 8 != 0 || p->sm_stride_b % 4 != 0 || p->sm_stride_h % 4 != 0 || p->sm_stride_q % 4 != 0)
@@ -83,6 +89,8 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
   a.kv_lens = p->kv_seqlens;
   a.kv_block_mask = p->kv_block_mask; a.kbm_sb = p->kbm_stride_b; a.kbm_sh = p->kbm_stride_h;
   a.kv_block = p->kv_block_size;
+  a.kbm_sq = p->kbm_stride_q; a.kbm_by_query_head = p->kbm_per_query_head;
+  a.elem_mask = p->elem_mask; a.em_sb = p->em_stride_b; a.em_sh = p->em_stride_h; a.em_sq = p->em_stride_q;
   a.n_split = 1;
   if (p->workspace && ((uintptr_t)p->workspace % 16) == 0) {
     const int n = attn_splits(p);

@@ -16,8 +16,12 @@ struct AttnArgs {
   // mask over blocks of kv_block keys (a multiple of 32)
   const int32_t* kv_lens;
   const uint8_t* kv_block_mask;
-  int64_t kbm_sb, kbm_sh;
+  int64_t kbm_sb, kbm_sh, kbm_sq;   // (kbm_sq: stride between blocks of 128 query rows; 0 for the decode form)
   int kv_block;
+  int kbm_by_query_head;            // the mask's head axis counts query heads (prefill form) instead of kv heads
+  // element-wise keep mask (attn_wide_fwd_kernel only): uint8 [B|1, H|1, Sq, Skv], 0 = the score is masked
+  const uint8_t* elem_mask;
+  int64_t em_sb, em_sh, em_sq;
   // split-kv decode (attn_wide_fwd_kernel with one wave per workgroup): n_split kv ranges per (batch, head,
   // row block), normalised partial outputs [B, n_split, H, Sq, Dv] in the tensor dtype and their fp32
   // natural-log row scale [B, n_split, H, Sq], merged by attn_split_combine_kernel

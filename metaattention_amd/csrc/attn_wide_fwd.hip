@@ -95,7 +95,26 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
   int n_tiles = (skv + BN - 1) / BN;
   if (CAUSAL) n_tiles = min(n_tiles, (mb * BM + BM + BN - 1) / BN);
   // tiles whose block of keys is switched off for this (batch, kv head) are skipped (:57-64)
-  const uint8_t* bm_row = a.kv_block_mask ? a.kv_block_mask + (int64_t)b * a.kbm_sb + (int64_t)(h / a.kv_group) * a.kbm_sh : nullptr;
+  const uint8_t* bm_row = a.kv_block_mask ? a.kv_block_mask + (int64_t)b * a.kbm_sb +
+                                                (int64_t)(a.kbm_by_query_head ? h : h / a.kv_group) * a.kbm_sh + (int64_t)mb * a.kbm_sq
+                                          : nullptr;
+  // element-wise keep mask of this lane's row (any mask_mod, evaluated densely by the host: blockattn_tl.py:176-190
+  // generates its code into the kernel instead); the four bytes of a lane's four consecutive keys come as one word
+  const uint8_t* em_row = a.elem_mask ? a.elem_mask + (int64_t)b * a.em_sb + (int64_t)h * a.em_sh + (int64_t)m_ld * a.em_sq : nullptr;
+  auto load_keep = [&](int n0, uint32_t (&kp)[4]) {
+#pragma unroll
+    for (int q4 = 0; q4 < 4; q4++) {
+      const int n = n0 + 8 * q4 + 4 * g;
+      if (n + 3 < skv) {
+        kp[q4] = *(const uint32_t*)(em_row + n);
+      } else {
+        kp[q4] = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+          if (n + i < skv) kp[q4] |= (uint32_t)em_row[n + i] << (8 * i);
+      }
+    }
+  };
   const int tiles_per_block = a.kv_block / BN;
   // this workgroup's share of the tiles
   const int tiles_per_split = (n_tiles + a.n_split - 1) / a.n_split;
@@ -157,10 +176,12 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
   const float c_scale = a.scale * kLog2e, c_bias = bias * kLog2e;
 
   x4 mk_next[4];
+  uint32_t keep_next[4] = {0, 0, 0, 0};
   int jt = next_tile(t_begin);
   if (jt < n_tiles) {
     issue_tile(jt * BN, 0);
     if constexpr (FAMILY == WF_RETENTION) load_mask(jt * BN, mk_next);
+    else if (em_row) load_keep(jt * BN, keep_next);
   }
 
   for (int it = 0; jt < n_tiles; it++) {
@@ -173,8 +194,12 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
 #pragma unroll
       for (int q4 = 0; q4 < 4; q4++) mk[q4] = mk_next[q4];
     }
+    uint32_t keep[4];
+#pragma unroll
+    for (int q4 = 0; q4 < 4; q4++) keep[q4] = keep_next[q4];
     if (jt < n_tiles) {
       if constexpr (FAMILY == WF_RETENTION) load_mask(jt * BN, mk_next);
+      else if (em_row) load_keep(jt * BN, keep_next);
       issue_tile(jt * BN, buf ^ 1);
     }
     const uint32_t kbase = lds0 + buf * STAGE, vbase = kbase + KTILE;
@@ -214,6 +239,11 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
           const int n = n0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
           if ((CAUSAL && n > m_lane) || n >= skv) s[jj] = -INFINITY;
         }
+      }
+      if (em_row) {
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++)
+          if (((keep[jj >> 2] >> (8 * (jj & 3))) & 0xff) == 0) s[jj] = -INFINITY;
       }
       if constexpr (FAMILY == WF_SOFTMAX) {
         float mx = s[0];

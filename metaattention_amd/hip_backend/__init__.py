@@ -49,6 +49,8 @@ class AttnParams(Structure):
         ("heads_kv", c_int32),
         ("kv_block_size", c_int32), ("kv_seqlens", c_void_p),
         ("kv_block_mask", c_void_p), ("kbm_stride_b", c_int64), ("kbm_stride_h", c_int64),
+        ("elem_mask", c_void_p), ("em_stride_b", c_int64), ("em_stride_h", c_int64), ("em_stride_q", c_int64),
+        ("kbm_stride_q", c_int64), ("kbm_per_query_head", c_int32),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
     ]
 
@@ -162,7 +164,7 @@ def _require_gpu(*tensors):
 
 def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None,
              score_mask=None, out=None, row_scale=None, kv_seqlens=None, kv_block_mask=None, kv_block_size: int = 0,
-             workspace=None, split_kv: bool = True):
+             workspace=None, split_kv: bool = True, elem_mask=None):
     """Parallel attention forward on BSHD tensors.  Returns ``out`` ([B,Sq,H,Dv]).  k and v may
     have fewer heads than q (grouped-query: query head h reads kv head h // (H // Hkv))."""
     _require_gpu(q, k, v, bias_tensor, score_mask, out, row_scale, kv_seqlens, kv_block_mask)
@@ -200,9 +202,23 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
         p.kv_seqlens = kv_seqlens.data_ptr()
     if kv_block_mask is not None:
         nblk = (Skv + kv_block_size - 1) // kv_block_size
-        assert kv_block_mask.dtype in (torch.bool, torch.uint8) and kv_block_mask.shape == (B, Hkv, nblk) and kv_block_mask.stride(-1) == 1
+        assert kv_block_mask.dtype in (torch.bool, torch.uint8) and kv_block_mask.stride(-1) == 1 and kv_block_mask.is_cuda
         p.kv_block_mask, p.kv_block_size = kv_block_mask.data_ptr(), int(kv_block_size)
-        p.kbm_stride_b, p.kbm_stride_h = kv_block_mask.stride(0), kv_block_mask.stride(1)
+        if kv_block_mask.dim() == 3:          # decode form: per (batch, kv head)
+            assert kv_block_mask.shape == (B, Hkv, nblk)
+            p.kbm_stride_b, p.kbm_stride_h = kv_block_mask.stride(0), kv_block_mask.stride(1)
+        else:                                 # prefill form: per (batch | 1, query head | 1, block of 128 query rows)
+            assert kv_block_mask.shape[2:] == ((Sq + 127) // 128, nblk) and kv_block_mask.shape[0] in (1, B) and kv_block_mask.shape[1] in (1, H)
+            p.kbm_stride_b = kv_block_mask.stride(0) if kv_block_mask.shape[0] > 1 else 0
+            p.kbm_stride_h = kv_block_mask.stride(1) if kv_block_mask.shape[1] > 1 else 0
+            p.kbm_stride_q, p.kbm_per_query_head = kv_block_mask.stride(2), 1
+    if elem_mask is not None:
+        assert elem_mask.dtype in (torch.bool, torch.uint8) and elem_mask.dim() == 4 and elem_mask.shape[2:] == (Sq, Skv)
+        assert elem_mask.shape[0] in (1, B) and elem_mask.shape[1] in (1, H) and elem_mask.stride(-1) == 1 and elem_mask.is_cuda
+        p.elem_mask = elem_mask.data_ptr()
+        p.em_stride_b = elem_mask.stride(0) if elem_mask.shape[0] > 1 else 0
+        p.em_stride_h = elem_mask.stride(1) if elem_mask.shape[1] > 1 else 0
+        p.em_stride_q = elem_mask.stride(2)
     lib = load_library()
     if split_kv:
         need = lib.ma_attn_workspace_bytes(ctypes.byref(p))

@@ -102,7 +102,7 @@ def softmax_attention(B, H, S, D, DV, dtype=torch.bfloat16, causal=True, online=
                            tune=tune, tune_file=f"tuned_config/{dev.name}/attn_tl.json", infer_mask=True)
 
 
-def sigmoid_attention(B, H, S, D, DV, dtype=torch.bfloat16, scale=1.0, form="tanh", const_bias=None, causal=True):
+def sigmoid_attention(B, H, S, D, DV, dtype=torch.bfloat16, scale=1.0, form="tanh", const_bias=None, causal=True, mask_mod=None):
     def score_mod(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
         x = score * scale if scale != 1.0 else score
         x = x + (const_bias if const_bias is not None else custom_fwd_inputs.input_tensors["softmax_bias"])
@@ -112,7 +112,7 @@ def sigmoid_attention(B, H, S, D, DV, dtype=torch.bfloat16, scale=1.0, form="tan
 
     io = CustomIO({} if const_bias is not None else {"softmax_bias": (1,)})
     return AttentionEngine(_meta(B, H, S, D, DV, dtype), io, score_mod=score_mod,
-                           mask_mod=causal_mask if causal else None, online_func=OnlineIdentity())
+                           mask_mod=mask_mod if mask_mod is not None else (causal_mask if causal else None), online_func=OnlineIdentity())
 
 
 def relu_attention(B, H, S, D, DV, dtype=torch.bfloat16):

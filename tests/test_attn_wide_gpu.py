@@ -261,6 +261,55 @@ def test_decode_workspace_sizes():
     assert lib.ma_attn_workspace_bytes(ctypes.byref(p)) == 0
 
 
+MASKS = {
+    "sliding_window": lambda b, h, q, k: (q >= k) & (q - k < 100),
+    "shifted_causal": lambda b, h, q, k: q - 128 >= k,                    # attention_engine/tests/test_blockmask.py:19-26
+    "prefix_lm": lambda b, h, q, k: (q >= k) | (k < 64),
+    "per_head_window": lambda b, h, q, k: (q >= k) & (q - k < 32 * (h + 1)),
+    "document": lambda b, h, q, k: (q >= k) & ((q // 150) == (k // 150)),
+}
+
+
+@pytest.mark.parametrize("name", sorted(MASKS))
+@pytest.mark.parametrize("D,S,family", [(128, 512, "softmax"), (64, 300, "softmax"), (128, 300, "sigmoid")])
+def test_engine_arbitrary_mask_mod(name, D, S, family):
+    """Any mask_mod (the reference generates its code into the block-sparse kernel, blockattn_tl.py:123-234): here through
+    a dense keep mask + block mask.  Oracle: scores masked with -inf before the row function, rows without any key give 0."""
+    from attn_engine import AttentionEngine
+    from core import CustomIO, meta_tensor
+    B, H = 2, 3
+    mask_mod = MASKS[name]
+    meta = tuple(meta_tensor(B, H, S, D, dtype=torch.bfloat16) for _ in range(3))
+    scale = 1 / math.sqrt(D)
+    if family == "softmax":
+        mod = AttentionEngine(meta, CustomIO(), lambda s_, io, b, h, q, k: s_ * scale, mask_mod, specs.OnlineSoftmax())
+    else:
+        mod = specs.sigmoid_attention(B, H, S, D, D, scale=scale, const_bias=-math.log(S), form="exp", mask_mod=mask_mod)
+    assert mod.mask_kind in ("other", "other_bh")
+    g = torch.Generator().manual_seed(S)
+    q = torch.randn(B, S, H, D, generator=g).bfloat16()
+    k = torch.randn(B, S, H, D, generator=g).bfloat16()
+    v = torch.randn(B, S, H, D, generator=g).bfloat16()
+    o = mod(q.cuda(), k.cuda(), v.cuda())
+    o2 = mod(q.cuda(), k.cuda(), v.cuda())          # second call re-uses the cached mask tensors
+    torch.cuda.synchronize()
+    assert torch.equal(o, o2)
+    bi, hi = torch.arange(B).view(B, 1, 1, 1), torch.arange(H).view(1, H, 1, 1)
+    keep = mask_mod(bi, hi, torch.arange(S).view(1, 1, S, 1), torch.arange(S).view(1, 1, 1, S)).expand(B, H, S, S)
+    ref = torch.empty(B, S, H, D)
+    for b in range(B):
+        for h in range(H):
+            s_ = (q[b, :, h].float() @ k[b, :, h].float().T) * scale
+            if family == "softmax":
+                s_ = s_.masked_fill(~keep[b, h], float("-inf"))
+                p = torch.softmax(s_, dim=-1)
+                p = torch.where(keep[b, h].any(dim=-1, keepdim=True), p, torch.zeros_like(p))
+            else:
+                p = torch.sigmoid(s_ - math.log(S)) * keep[b, h]
+            ref[b, :, h] = p @ v[b, :, h].float()
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
 def test_unsupported_head_size_is_an_error():
     hb = _hb()
     q = torch.zeros(1, 64, 1, 96, device="cuda", dtype=torch.bfloat16)

@@ -56,10 +56,10 @@ def test_classify_mask():
     assert classify_mask(None, 1, 2, 64, 64) == "none"
     assert classify_mask(lambda b, h, q, k: q >= k, 2, 4, 300, 300) == "causal"
     assert classify_mask(lambda b, h, q, k: (q >= k) | (q < k), 2, 4, 64, 64) == "none"
-    with pytest.raises(NotImplementedError):
-        classify_mask(lambda b, h, q, k: q - 4 >= k, 1, 1, 64, 64)
-    with pytest.raises(NotImplementedError):
-        classify_mask(lambda b, h, q, k: (q >= k) & (h > 0), 1, 2, 64, 64)
+    assert classify_mask(lambda b, h, q, k: q - 4 >= k, 1, 1, 64, 64) == "other"              # shifted: element-wise keep mask
+    assert classify_mask(lambda b, h, q, k: (q >= k) & (q - k < 16), 2, 4, 64, 64) == "other"  # sliding window
+    assert classify_mask(lambda b, h, q, k: (q >= k) & (h > 0), 1, 2, 64, 64) == "other_bh"    # depends on the head
+    assert classify_mask(lambda b, h, q, k: q >= k, 1, 1, 64, 128) == "other"                  # "causal" needs equal lengths
 
 
 def test_canonical_score_forms():
