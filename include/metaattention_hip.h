@@ -1,5 +1,5 @@
 /*
- * C ABI of the MI355X (gfx950) attention forward kernel library.
+ * C ABI of the MI355X (gfx950) attention kernel library (forward operators and their backward).
  *
  * This is the boundary the Python host side binds with ctypes.  Each entry
  * point replaces one compiled operator that the reference builds at run time
