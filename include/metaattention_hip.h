@@ -85,9 +85,11 @@ typedef struct ma_attn_params {
   const uint8_t* kv_block_mask; int64_t kbm_stride_b, kbm_stride_h;
   /* arbitrary masks (blockattn_tl.py:123-234, where the mask_mod's code is generated into the kernel): elem_mask
    * uint8/bool [1 or B, 1 or H, Sq, Skv] (strides in bytes = elements; stride 0 broadcasts; rows 4-byte aligned),
-   * 0 = the score is masked (probability exactly 0).  With it, kv_block_mask may be the prefill form
-   * [.., heads, ceil(Sq/128), ceil(Skv/kv_block_size)]: set kbm_stride_q (blocks of 128 query rows) and
-   * kbm_per_query_head = 1.  Not with MA_MASK_CAUSAL (the element mask says it all) nor RETENTION. */
+   * 0 = the score is masked (probability exactly 0).  Not with MA_MASK_CAUSAL (the element mask says it all) nor
+   * RETENTION.  With or without it, kv_block_mask may be the prefill form
+   * [1 or B, 1 or heads, ceil(Sq/128), ceil(Skv/kv_block_size)] of the block-sparse prefill operator: set
+   * kbm_stride_q (blocks of 128 query rows; strides 0 broadcast) and kbm_per_query_head = 1.  This form also goes
+   * with MA_MASK_CAUSAL. */
   const uint8_t* elem_mask; int64_t em_stride_b, em_stride_h, em_stride_q;
   int64_t kbm_stride_q; int32_t kbm_per_query_head;
   /* optional; with ma_attn_workspace_bytes(&params) bytes, decode shapes (at most 32 query rows, SOFTMAX, no

@@ -124,8 +124,10 @@ class AttentionEngine:
         self.kv_block_size = int(infer_mask_block_N)
         if (use_varlen or extern_block_mask) and (self.kv_block_size < 32 or self.kv_block_size % 32 != 0):
             raise NotImplementedError("kv block masks need a block size that is a multiple of 32 (infer_mask_block_N)")
-        if (use_varlen or extern_block_mask) and (kv_shared or qkv_meta[0].shape[2] == qkv_meta[2].shape[2]):
-            raise NotImplementedError("varlen / external block masks are only in the decode operators of the kernel library")
+        if (use_varlen or extern_block_mask) and kv_shared:
+            raise NotImplementedError("varlen / external block masks are not in the MLA decode operator")
+        if use_varlen and qkv_meta[0].shape[2] == qkv_meta[2].shape[2]:
+            raise NotImplementedError("cache lengths (use_varlen) are only in the decode operators of the kernel library")
         dtype = qkv_meta[0].dtype
         if dtype not in (torch.float16, torch.bfloat16):
             raise KeyError(dtype)      # the reference's dtype map has only these two (attn_engine.py:234-237)
@@ -193,12 +195,18 @@ class AttentionEngine:
         given = dict(zip(self.names, custom))
         form = self.score_form
 
+        # block_mask [batch, heads, q blocks, kv blocks]: the block-sparse prefill operator (blockattn_tl.py:123-234);
+        # [batch, heads_kv, kv blocks] (+ cache_seqlens): the varlen block-sparse decode operator
+        prefill_blocks = block_mask if block_mask is not None and block_mask.dim() == 4 else None
+        if prefill_blocks is not None:
+            block_mask = None
+            if self.family == "retention" or cache_seqlens is not None:
+                raise NotImplementedError("block-sparse prefill masks go with the softmax / sigmoid / relu kernels, without cache_seqlens")
         sparse = block_mask is not None or cache_seqlens is not None
         if sparse and (self.mask_kind != "none" or self.family == "retention"):
             raise NotImplementedError("block_mask / cache_seqlens are for the unmasked decode operators")
         if block_mask is not None and block_mask.dim() != 3:
-            raise NotImplementedError("only kv block masks [batch, heads_kv, blocks] (decode) are in the kernel library; "
-                                      "block-sparse prefill masks [batch, heads, q blocks, kv blocks] are not")
+            raise NotImplementedError("block masks are [batch, heads_kv, kv blocks] (decode) or [batch, heads, q blocks, kv blocks] (prefill)")
 
         def run(q, k, v):
             B, Sq, H, D = q.shape
@@ -209,6 +217,11 @@ class AttentionEngine:
             if self.mask_kind.startswith("other"):
                 elem, blocks = self._dense_mask(B, H, Sq, k.shape[1], q.device)
                 kw.update(elem_mask=elem, kv_block_mask=blocks, kv_block_size=32)
+            if prefill_blocks is not None:
+                ext = self._expand_block_mask(prefill_blocks, B, H, Sq, k.shape[1])
+                if "kv_block_mask" in kw:
+                    ext = ext & kw["kv_block_mask"]        # (the mask_mod's own block mask: broadcast over batch / heads)
+                kw.update(kv_block_mask=ext.contiguous(), kv_block_size=32)
             if sparse:
                 kw.update(kv_seqlens=cache_seqlens.to(torch.int32) if cache_seqlens is not None else None, kv_block_mask=block_mask,
                           kv_block_size=self.kv_block_size if block_mask is not None else 0)
@@ -236,11 +249,24 @@ class AttentionEngine:
             return run(q, k, v).squeeze(1)
 
         if any(t.requires_grad for t in (q, k, v)):
-            if self.family == "retention" or self.mask_kind.startswith("other"):
+            if self.family == "retention" or self.mask_kind.startswith("other") or prefill_blocks is not None:
                 return _ForwardOnly.apply(run, q, k, v)
             bias_t = given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None
             return _Attention.apply(self, run, fam_code, bias_t, q, k, v)
         return run(q, k, v)
+
+    @staticmethod
+    def _expand_block_mask(block_mask, B, H, Sq, Skv):
+        """A caller's block mask [1|B, 1|H, nq, nk] (non-zero = keep; a block covers Sq/nq query rows and Skv/nk keys,
+        blockattn_tl.py:109-112, :170) at the kernel's granularity: uint8 [.., Sq/128, Skv/32]."""
+        if block_mask.shape[0] not in (1, B) or block_mask.shape[1] not in (1, H):
+            raise ValueError(f"block_mask {tuple(block_mask.shape)} does not fit batch {B}, heads {H}")
+        nq, nk = block_mask.shape[2:]
+        if nq < 1 or nk < 1 or Sq % nq or Skv % nk or (Sq // nq) % 128 or (Skv // nk) % 32:
+            raise NotImplementedError(f"block_mask of {nq} x {nk} blocks over {Sq} x {Skv}: blocks must be a whole multiple of "
+                                      "128 query rows by 32 keys")
+        keep = (block_mask != 0).to(torch.uint8)
+        return keep.repeat_interleave(Sq // nq // 128, dim=2).repeat_interleave(Skv // nk // 32, dim=3)
 
     def _dense_mask(self, B, H, Sq, Skv, device):
         """(element-wise keep mask uint8 [1|B, 1|H, Sq, Skv] with 4-byte aligned rows, block mask uint8

@@ -55,8 +55,9 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
     return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: heads (%d) must be a multiple of heads_kv (%d)", p->heads, p->heads_kv);
   if (p->kv_block_mask && (p->kv_block_size < 32 || p->kv_block_size % 32 != 0))
     return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: kv_block_size must be a positive multiple of 32 (got %d)", p->kv_block_size);
-  if ((p->kv_block_mask || p->kv_seqlens) && p->mask == MA_MASK_CAUSAL)
-    return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: kv_seqlens / kv_block_mask are for the unmasked (decode) operators");
+  // (a block mask with a row per 128 queries goes with either mask: the block-sparse prefill operator)
+  if ((p->kv_seqlens || (p->kv_block_mask && !p->kbm_per_query_head)) && p->mask == MA_MASK_CAUSAL)
+    return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: kv_seqlens / a kv_block_mask per kv head are for the unmasked (decode) operators");
   if (p->elem_mask) {
     if (p->mask == MA_MASK_CAUSAL || p->family == MA_ATTN_RETENTION)
       return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: elem_mask goes with MA_MASK_NONE and the softmax / sigmoid / relu families");

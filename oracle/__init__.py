@@ -30,6 +30,10 @@ mla_decode             SDPA with K=concat(kv,k_pe), V=kv; split-KV invariance
 sparse_decode_attention  dense attention over the gathered kept keys only
 paged_mla_decode       mla_decode on the contiguous cache (identity table); invariance
                        to a permutation of the page pool
+masked_attention       SDPA with a boolean attn_mask (fp64); tril keep mask ==
+                       softmax_attention(causal); a block mask == attention over
+                       the gathered kept keys of each query block; rows without
+                       keys are 0; sigmoid / relu by element-wise brute force
 attention_grads,       central differences of the pinned forward functions in
 linear_attention_grads fp64 along random directions; SDPA's own autograd
 (all of the above)     tests/golden/*.npz: the operators' definitions evaluated
@@ -48,6 +52,7 @@ from .attention_ref import (  # noqa: F401
     attention_grads,
     sparse_decode_attention,
     paged_mla_decode,
+    masked_attention,
 )
 from .linear_ref import (  # noqa: F401
     retnet_quadratic,

@@ -176,6 +176,42 @@ def sparse_decode_attention(q, k, v, block_mask=None, cache_seqlens=None, block_
     return out
 
 
+def masked_attention(q, k, v, keep=None, block_mask=None, family: str = "softmax", softmax_scale: Optional[float] = None,
+                     bias: float = 0.0, compute_dtype=torch.float32):
+    """Attention under an arbitrary element-wise mask and / or a block mask: the block-sparse prefill operator,
+    tl_template/attn/blockattn_tl.py:123-234.  ``keep`` bool [1|B, 1|H, Sq, Skv] is the mask_mod evaluated densely
+    (scores of dropped elements are -inf before the score function, :176-190); ``block_mask`` [1|B, 1|H, nq, nk]
+    (non-zero = visit, :170) switches whole blocks of Sq/nq rows x Skv/nk keys off (:109-112).  family "softmax":
+    softmax(scores * scale); "sigmoid": sigmoid(scores * scale + bias); "relu": max(scores * scale, 0); a dropped
+    element contributes exactly 0 in each.  A row left without any key is all zeros (the epilogue is skipped when no
+    block was visited, :225-227; a visited block whose elements are all dropped gives 0/0 there, defined as 0 here)."""
+    B, Sq, H, D = q.shape
+    Skv, Dv = k.shape[1], v.shape[-1]
+    scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+    out = torch.empty(B, Sq, H, Dv, dtype=compute_dtype)
+    for b in range(B):
+        for h in range(H):
+            m = torch.ones(Sq, Skv, dtype=torch.bool)
+            if keep is not None:
+                m &= keep[b if keep.shape[0] > 1 else 0, h if keep.shape[1] > 1 else 0].to(torch.bool).cpu()
+            if block_mask is not None:
+                bm = block_mask[b if block_mask.shape[0] > 1 else 0, h if block_mask.shape[1] > 1 else 0].cpu() != 0
+                nq, nk = bm.shape
+                m &= bm.repeat_interleave(Sq // nq, dim=0).repeat_interleave(Skv // nk, dim=1)
+            s = (q[b, :, h].to(compute_dtype) @ k[b, :, h // (H // k.shape[2])].to(compute_dtype).T) * scale
+            if family == "softmax":
+                p = torch.softmax(s.masked_fill(~m, float("-inf")), dim=-1)
+                p = torch.where(m.any(dim=-1, keepdim=True), p, torch.zeros_like(p))
+            elif family == "sigmoid":
+                p = torch.sigmoid(s + bias) * m
+            elif family == "relu":
+                p = torch.relu(s) * m
+            else:
+                raise ValueError(family)
+            out[b, :, h] = p @ v[b, :, h // (H // v.shape[2])].to(compute_dtype)
+    return out
+
+
 def paged_mla_decode(q, k_cache, block_table, cache_seqlens, head_dim_v: int = 512, compute_dtype=torch.float32):
     """flash_mla_with_kvcache semantics (cute_template_kvshared/flash_mla_interface.py:75-115) for one query
     token: q [B,1,Hq,d+dpe]; k_cache [pages, page_size, 1, d+dpe]; sequence b is the rows of pages

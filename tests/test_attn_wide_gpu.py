@@ -296,18 +296,69 @@ def test_engine_arbitrary_mask_mod(name, D, S, family):
     assert torch.equal(o, o2)
     bi, hi = torch.arange(B).view(B, 1, 1, 1), torch.arange(H).view(1, H, 1, 1)
     keep = mask_mod(bi, hi, torch.arange(S).view(1, 1, S, 1), torch.arange(S).view(1, 1, 1, S)).expand(B, H, S, S)
-    ref = torch.empty(B, S, H, D)
-    for b in range(B):
-        for h in range(H):
-            s_ = (q[b, :, h].float() @ k[b, :, h].float().T) * scale
-            if family == "softmax":
-                s_ = s_.masked_fill(~keep[b, h], float("-inf"))
-                p = torch.softmax(s_, dim=-1)
-                p = torch.where(keep[b, h].any(dim=-1, keepdim=True), p, torch.zeros_like(p))
-            else:
-                p = torch.sigmoid(s_ - math.log(S)) * keep[b, h]
-            ref[b, :, h] = p @ v[b, :, h].float()
+    ref = oracle.masked_attention(q, k, v, keep=keep, family=family, softmax_scale=scale, bias=-math.log(S))
     oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
+def _sparse_prefill_engine(family, causal, mask_mod, B, H, S, D, dtype=torch.bfloat16):
+    from attn_engine import AttentionEngine
+    from core import CustomIO, meta_tensor
+    meta = tuple(meta_tensor(B, H, S, D, dtype=dtype) for _ in range(3))
+    scale = 1 / math.sqrt(D)
+    mm = mask_mod if mask_mod is not None else (specs.causal_mask if causal else None)
+    if family == "softmax":
+        return AttentionEngine(meta, CustomIO(), lambda s_, io, b, h, q, k: s_ * scale, mm, specs.OnlineSoftmax(), extern_block_mask=True)
+    if family == "relu":
+        return AttentionEngine(meta, CustomIO(), lambda s_, io, b, h, q, k: (s_ * scale).max(0), mm, specs.OnlineIdentity(),
+                               extern_block_mask=True)
+    return AttentionEngine(meta, CustomIO(), lambda s_, io, b, h, q, k: 1 / (1 + (-(s_ * scale + (-math.log(S)))).exp()), mm,
+                           specs.OnlineIdentity(), extern_block_mask=True)
+
+
+@pytest.mark.parametrize("family,mask,D,S,bq,bk", [
+    ("softmax", "none", 128, 512, 128, 128),
+    ("softmax", "causal", 128, 512, 128, 128),       # the reference's default block size (attn_engine.py:113)
+    ("softmax", "causal", 64, 768, 256, 64),
+    ("softmax", "sliding_window", 128, 512, 128, 32),
+    ("sigmoid", "causal", 128, 512, 128, 64),
+    ("relu", "none", 64, 256, 128, 32),
+])
+def test_engine_block_sparse_prefill(family, mask, D, S, bq, bk):
+    """extern_block_mask=True at prefill shapes: mod(q, k, v, block_mask=[B, H, S/bq, S/bk]) visits only the kept blocks
+    (blockattn_tl.py:123-234), on top of the mask_mod's element-wise mask; query blocks with no kept block give zeros."""
+    B, H = 2, 3
+    mask_mod = MASKS.get(mask)
+    mod = _sparse_prefill_engine(family, mask == "causal", mask_mod, B, H, S, D)
+    g = torch.Generator().manual_seed(S + bq + bk)
+    q, k, v = (torch.randn(B, S, H, D, generator=g).bfloat16() for _ in range(3))
+    bm = (torch.rand(B, H, S // bq, S // bk, generator=g) < 0.5).to(torch.int8)
+    bm[0, 0, 1] = 0                                   # a whole block of query rows without keys
+    bm[1, 2, 0] = 1
+    o = mod(q.cuda(), k.cuda(), v.cuda(), block_mask=bm.cuda())
+    torch.cuda.synchronize()
+    keep = None
+    if mask != "none":
+        fn = mask_mod if mask_mod is not None else specs.causal_mask
+        keep = fn(torch.arange(B).view(B, 1, 1, 1), torch.arange(H).view(1, H, 1, 1), torch.arange(S).view(1, 1, S, 1),
+                  torch.arange(S).view(1, 1, 1, S)).expand(B, H, S, S)
+    ref = oracle.masked_attention(q, k, v, keep=keep, block_mask=bm, family=family, softmax_scale=1 / math.sqrt(D), bias=-math.log(S))
+    # (un-normalised relu sums: the rounding of the probabilities to bf16 alone is ~2.5e-2 rms at these sizes)
+    ratio = 5e-2 if family == "relu" else 0.0
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=ratio)
+    assert torch.count_nonzero(o[0, bq:2 * bq, 0]) == 0
+    # a broadcast mask [1, 1, nq, nk], and the all-ones mask == the dense operator
+    o1 = mod(q.cuda(), k.cuda(), v.cuda(), block_mask=bm[:1, :1].cuda())
+    ref1 = oracle.masked_attention(q, k, v, keep=keep, block_mask=bm[:1, :1], family=family, softmax_scale=1 / math.sqrt(D), bias=-math.log(S))
+    oracle.assert_close(o1.float().cpu(), ref1, rtol=RTOL, atol=ATOL, mismatch_ratio=ratio)
+
+
+def test_block_sparse_prefill_rejects_odd_blocks():
+    mod = _sparse_prefill_engine("softmax", True, None, 1, 2, 512, 128)
+    q = torch.zeros(1, 512, 2, 128, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError):
+        mod(q, q, q, block_mask=torch.ones(1, 2, 8, 4, dtype=torch.int8, device="cuda"))      # 64-row query blocks
+    with pytest.raises(ValueError):
+        mod(q, q, q, block_mask=torch.ones(3, 2, 4, 4, dtype=torch.int8, device="cuda"))
 
 
 def test_unsupported_head_size_is_an_error():

@@ -320,3 +320,42 @@ def test_paged_mla_identity_table_and_page_permutation():
     out2, lse2 = oracle.paged_mla_decode(q, cache[perm], inv[table.long()].to(torch.int32), lens, head_dim_v=16, compute_dtype=torch.float64)
     torch.testing.assert_close(out2, out)
     torch.testing.assert_close(lse2, lse)
+
+
+def test_masked_attention_against_sdpa_and_special_cases():
+    g = torch.Generator().manual_seed(19)
+    B, H, S, D = 2, 3, 24, 8
+    q, k, v = (torch.randn(B, S, H, D, generator=g, dtype=torch.float64) for _ in range(3))
+    keep = torch.rand(B, H, S, S, generator=g) < 0.4
+    keep[0, 1, 5] = False                                   # a row without any key
+    got = oracle.masked_attention(q, k, v, keep=keep, compute_dtype=torch.float64)
+    sd = torch.nn.functional.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), attn_mask=keep)
+    sd = torch.nan_to_num(sd, nan=0.0).transpose(1, 2)      # SDPA gives NaN for the empty row
+    assert keep.any(-1).all(-1).tolist() != [[True] * H] * B
+    torch.testing.assert_close(got, sd)
+    assert torch.equal(got[0, 5, 1], torch.zeros(D, dtype=torch.float64))
+    # the lower-triangular keep mask is the causal operator; a broadcast mask is the same for every (batch, head)
+    tril = torch.tril(torch.ones(S, S, dtype=torch.bool)).view(1, 1, S, S)
+    torch.testing.assert_close(oracle.masked_attention(q, k, v, keep=tril, compute_dtype=torch.float64),
+                               oracle.softmax_attention(q, k, v, causal=True, compute_dtype=torch.float64))
+    # a block mask: every query block attends to the gathered keys of its kept blocks only
+    bm = torch.tensor([[1, 0, 1], [0, 0, 0], [0, 1, 1], [1, 1, 1]], dtype=torch.int8).view(1, 1, 4, 3).expand(B, H, 4, 3)
+    got = oracle.masked_attention(q, k, v, block_mask=bm, compute_dtype=torch.float64)
+    for qb in range(4):
+        rows = slice(qb * 6, qb * 6 + 6)
+        idx = [n for n in range(S) if bm[0, 0, qb, n // 8]]
+        if not idx:
+            assert torch.count_nonzero(got[:, rows]) == 0
+            continue
+        ref = oracle.softmax_attention(q[:, rows], k[:, idx], v[:, idx], causal=False, compute_dtype=torch.float64)
+        torch.testing.assert_close(got[:, rows], ref)
+    # sigmoid / relu: element by element
+    for family, fn in (("sigmoid", lambda x: 1 / (1 + math.exp(-(x - 0.3)))), ("relu", lambda x: max(x, 0.0))):
+        got = oracle.masked_attention(q[:1, :6, :1], k[:1, :6, :1], v[:1, :6, :1], keep=keep[:1, :1, :6, :6], family=family,
+                                      softmax_scale=0.5, bias=-0.3, compute_dtype=torch.float64)
+        for i in range(6):
+            acc = torch.zeros(D, dtype=torch.float64)
+            for j in range(6):
+                if keep[0, 0, i, j]:
+                    acc += fn(0.5 * float(q[0, i, 0] @ k[0, j, 0])) * v[0, j, 0]
+            torch.testing.assert_close(got[0, i, 0], acc)
