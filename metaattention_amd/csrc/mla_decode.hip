@@ -65,7 +65,8 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
   const uint32_t lds_x = lds0 + NSTAGE * STAGE;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int hg = wave & 3, hf = wave >> 2;   // head group, half
+  const int hg = wave >> 1, hf = wave & 1;   // head group, half: partners are on different SIMDs (wave % 4)
+  const bool late = wave >= 4;               // head groups 2 and 3 run half a sub-tile behind (see the main loop)
   const int r = lane & 31, g = lane >> 5;
   const int hblk = blockIdx.x % a.head_blocks, bs = blockIdx.x / a.head_blocks;
   const int b = bs / a.num_split, split = bs % a.num_split;
@@ -129,7 +130,7 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
   const uint32_t v_lo_off = (4 * g + jr) * KV_ROW + (lc << 4) + (lane & 1) * 8 + hf * (DBH * 64);
   const uint32_t v_hi_off = (4 * g + jr + 8) * KV_ROW + ((lc ^ 1) << 4) + (lane & 1) * 8 + hf * (DBH * 64);
   // exchange of the half score tiles: 4 x 16 bytes per lane, lane-major
-  const uint32_t x_mine = lds_x + wave * XCHG + lane * 16, x_other = lds_x + (wave ^ 4) * XCHG + lane * 16;
+  const uint32_t x_mine = lds_x + wave * XCHG + lane * 16, x_other = lds_x + (wave ^ 1) * XCHG + lane * 16;
 
   f32x16 o[DBH];
 #pragma unroll
@@ -143,48 +144,39 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
   if (n_tiles > 0) issue_tile(0);
   if (n_tiles > 1) issue_tile(1);
 
-  for (int jt = 0; jt < n_tiles; jt++) {
-    // Sub-tile jt has landed for every wave (a wave's loads complete in order: only those of sub-tile jt+1
-    // may still be in flight), every wave is done with sub-tile jt-1, whose stage takes sub-tile jt+2, and
-    // every wave has read its partner's half scores of sub-tile jt-1.
-    if (jt + 1 < n_tiles) {
-      if (wave < 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 5); else __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
-    } else {
-      wait_dma();
-    }
-    __syncthreads();
-    if (jt + 2 < n_tiles) issue_tile(jt + 2);
-    const int n0 = n_begin + jt * BN;
-    const uint32_t base = lds0 + (jt % NSTAGE) * STAGE;
+  f32x16 sc;   // this wave's half scores, then the full scores, of the sub-tile it is working on
 
-    // ---- half scores: S^T_half = KV_half Q_half^T over this wave's 18 k-slices
-    f32x16 sc;
-    {
-      constexpr int AH = 2, RING = AH + 1;
-      x8 kf[RING];
-      uint32_t kb = base + k_off, pb = base + pe_off;
-      asm volatile("" : "+v"(kb), "+v"(pb));   // one address register + immediates for the reads below
-      // the last four slices of the second half are the rope columns (their own, XOR-swizzled tile)
-      uint32_t tail[NSL - NLAT1];
+  // ---- phase A of sub-tile jt: half scores S^T_half = KV_half Q_half^T over this wave's 18 k-slices, handed to the partner
+  auto half_scores = [&](int jt) {
+    const uint32_t base = lds0 + (jt % NSTAGE) * STAGE;
+    constexpr int AH = 2, RING = AH + 1;
+    x8 kf[RING];
+    uint32_t kb = base + k_off, pb = base + pe_off;
+    asm volatile("" : "+v"(kb), "+v"(pb));   // one address register + immediates for the reads below
+    // the last four slices of the second half are the rope columns (their own, XOR-swizzled tile)
+    uint32_t tail[NSL - NLAT1];
 #pragma unroll
-      for (int j = 0; j < NSL - NLAT1; j++) tail[j] = hf ? pb + (uint32_t)((pe_c0 ^ (2 * j)) << 4) : kb + 32 * (NLAT1 + j);
-      auto request = [&](int sl) {
-        kf[sl % RING] = lds_read<x8>(sl < NLAT1 ? kb + 32 * sl : tail[sl < NLAT1 ? 0 : sl - NLAT1]);
-      };
+    for (int j = 0; j < NSL - NLAT1; j++) tail[j] = hf ? pb + (uint32_t)((pe_c0 ^ (2 * j)) << 4) : kb + 32 * (NLAT1 + j);
+    auto request = [&](int sl) {
+      kf[sl % RING] = lds_read<x8>(sl < NLAT1 ? kb + 32 * sl : tail[sl < NLAT1 ? 0 : sl - NLAT1]);
+    };
 #pragma unroll
-      for (int sl = 0; sl < AH; sl++) request(sl);
+    for (int sl = 0; sl < AH; sl++) request(sl);
 #pragma unroll
-      for (int sl = 0; sl < NSL; sl++) {
-        if (sl + AH < NSL) request(sl + AH);
-        __builtin_amdgcn_sched_barrier(0);   // keep the requests ahead of the MFMAs that hide their latency
-        sc = E::mfma32(kf[sl % RING], qf[sl], sl == 0 ? zero16 : sc);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+    for (int sl = 0; sl < NSL; sl++) {
+      if (sl + AH < NSL) request(sl + AH);
+      __builtin_amdgcn_sched_barrier(0);   // keep the requests ahead of the MFMAs that hide their latency
+      sc = E::mfma32(kf[sl % RING], qf[sl], sl == 0 ? zero16 : sc);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    // ---- exchange and add the halves
 #pragma unroll
     for (int j4 = 0; j4 < 4; j4++) lds_write<f32x4>(x_mine + j4 * 1024, f32x4{sc[4 * j4], sc[4 * j4 + 1], sc[4 * j4 + 2], sc[4 * j4 + 3]});
-    __syncthreads();
+  };
+
+  // ---- phase B of sub-tile jt (a barrier after the partner's phase A): add the halves, softmax, O^T_half += KV_half^T P^T
+  auto softmax_pv = [&](int jt) {
+    const int n0 = n_begin + jt * BN;
+    const uint32_t base = lds0 + (jt % NSTAGE) * STAGE;
 #pragma unroll
     for (int j4 = 0; j4 < 4; j4++) {
       const f32x4 t = lds_read<f32x4>(x_other + j4 * 1024);
@@ -205,7 +197,7 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
 #pragma unroll
     for (int i = 0; i < PF - 1; i++) v_request(i);
 
-    // ---- mask, online softmax in the log2 domain: lane holds head r, kv rows 8(j/4) + 4g + j%4
+    // mask, online softmax in the log2 domain: lane holds head r, kv rows 8(j/4) + 4g + j%4
     if (n0 + BN > n_end) {
 #pragma unroll
       for (int j = 0; j < 16; j++)
@@ -246,7 +238,6 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
     }
     row_sum += part;
 
-    // ---- O^T_half += KV_half^T P^T
 #pragma unroll
     for (int i = 0; i < NPV; i++) {
       if (i + PF - 1 < NPV) v_request(i + PF - 1);
@@ -255,7 +246,38 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
       o[i % DBH] = E::mfma32(vf, p[i / DBH], o[i % DBH]);
       __builtin_amdgcn_sched_barrier(0);
     }
+  };
+
+  // Two barriers per sub-tile: [barrier, phase A, barrier, phase B].  Head groups 2 and 3 (waves 4..7) pass one
+  // barrier more before their first sub-tile and groups 0 and 1 one more after their last, so the late groups
+  // run half a sub-tile behind: while an early wave is in phase A the late wave on its SIMD is in phase B of
+  // the sub-tile before, and the other way round.  One wave's softmax (vector ALU) then always runs beside the
+  // other wave's MFMAs instead of both doing the same thing at the same time.  With the global barrier count
+  // k = 1, 2, ..: early waves run A(j) after k = 2j+1 and B(j) after 2j+2, late waves A(j) after 2j+2 and B(j)
+  // after 2j+3.  Sub-tile j is read from k = 2j+1 on, so every wave has waited for its own loads of it before
+  // that barrier; its stage is free after k = 2j+4, which is where sub-tile j+3 is requested.
+  auto wait_tile = [&](int t) {   // this wave's loads of sub-tile t have landed (they complete in order: only those of t+1 may be in flight)
+    if (t + 1 < n_tiles) {
+      if (wave < 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 5); else __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+    } else {
+      wait_dma();
+    }
+  };
+  if (late) {
+    wait_tile(0);
+    __syncthreads();
   }
+  for (int jt = 0; jt < n_tiles; jt++) {
+    if (!late) wait_tile(jt);
+    __syncthreads();
+    if (late && jt + 2 < n_tiles) issue_tile(jt + 2);
+    half_scores(jt);
+    if (late && jt + 1 < n_tiles) wait_tile(jt + 1);
+    __syncthreads();
+    if (!late && jt + 2 < n_tiles) issue_tile(jt + 2);
+    softmax_pv(jt);
+  }
+  if (!late) __syncthreads();
 
   // ---- epilogue: lane holds head r, output columns 256 hf + 32db + 8(j/4) + 4g + j%4
   float t_lo, t_hi;
