@@ -79,6 +79,14 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
   constexpr int SCAL_BYTES = 3 * L * 4;            // per-wave g / pv*q_scale / w
   constexpr int NIQ = QT / 1024, NIV = VT / 1024;  // DMA instructions per tile
   static_assert(CPRQ >= 16, "DK < 128 needs its own Q/K swizzle");
+  // Every wave of the workgroup needs the same 32 x 32 tile A^T = K Q^T.  With four or more waves it is computed
+  // once: in 16 x 16 quadrants (v_mfma_f32_16x16x32; the quadrant of keys 16..31 x queries 0..15 lies above the
+  // diagonal and is left out), each over 1 / KP of the key dims, one (quadrant, part) per wave, exchanged
+  // through LDS.  16 MFMAs of 32x32x16 and 2 x DK / 16 KB of operand reads per wave become at most 4 half-size
+  // MFMAs plus a 1 KB write and 4 KP KB of reads, for one more barrier per chunk.
+  constexpr bool SHARE_A = NW >= 4 && MODE != 1;
+  constexpr int KP = NW >= 8 ? 2 : 1;               // parts of the key dims per quadrant
+  constexpr int A_ITEMS = 3 * KP;
 
   extern __shared__ __align__(16) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
@@ -86,6 +94,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
   const int r0 = lane & 31;
   const uint32_t lds_scal = lds0 + 2 * STAGE + wave * SCAL_BYTES;
   const uint32_t lds_ost = lds0 + 2 * STAGE + NW * SCAL_BYTES + wave * (L * OROW);   // (unused with ALIAS_OST)
+  const uint32_t lds_apart = lds0 + 2 * STAGE + NW * SCAL_BYTES + (ALIAS_OST ? 0 : NW * (L * OROW));   // A^T quadrants, 1 KB each
 
   // workgroup -> (head group, value slice, segment); the workgroups of one head group share
   // id % 8 (one XCD, shared L2)
@@ -238,6 +247,28 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
     const uint32_t base = lds0 + buf * STAGE;
     const uint32_t qbase = base, kbase = base + QT, vbase = base + 2 * QT;
 
+    // ---- this wave's share of A^T = K Q^T: quadrant slot 0 = keys 0..15 x queries 0..15, 1 = keys 0..15 x queries
+    //      16..31, 2 = keys 16..31 x queries 16..31; A / B operand: lane holds row (column) lane % 16, k = 8 (lane / 16) .. +7
+    //      of a 32-wide slice; C: lane holds column lane % 16, rows 4 (lane / 16) + {0..3}
+    if constexpr (SHARE_A) {
+      if (wave < A_ITEMS) {
+        const int slot = wave / KP, kp = wave % KP;
+        int la = lane;
+        asm volatile("" : "+v"(la));
+        const int rr = la & 15, kg = la >> 4;
+        const uint32_t krow = kbase + (16 * (slot >> 1) + rr) * RBQ, qrow = qbase + (16 * (slot > 0) + rr) * RBQ;
+        const int c0 = kg ^ swz16(rr);
+        constexpr int NS16 = DK / 32 / KP;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s2 = 0; s2 < NS16; s2++) {
+          const uint32_t off = (uint32_t)((c0 ^ (4 * (kp * NS16 + s2))) << 4);
+          acc = E::mfma16(lds_read<x8>(krow + off), lds_read<x8>(qrow + off), acc);
+        }
+        lds_write<f32x4>(lds_apart + wave * 1024 + la * 16, acc);
+      }
+    }
+
     // ---- per-lane LDS read offsets.  They are loop invariant; left outside the loop, they (and every
     //      swizzled address derived from them, dozens) stay in registers across chunks, which the state
     //      accumulator leaves no room for.  The lane id is laundered so that they are rebuilt per chunk.
@@ -273,24 +304,42 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
     gi += dpp_f32<0x118>(gi);
     gi += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, gi), 0x142, 0xa, 0xf, false));   // row_bcast:15
     const float g_last = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, gi), 31));
+    const float gi2 = gi * kLog2e, g_last2 = g_last * kLog2e;    // (exponents in the log2 domain from here on)
     const float pvq = valid ? vs * a.q_scale : 0.f;               // factor of column j in P
-    const float wl = valid ? vs * fast_exp2((g_last - gi) * kLog2e) : 0.f;   // factor of row l in the state update
-    const float eg = fast_exp2(gi * kLog2e) * a.q_scale;          // factor of token i in the inter-chunk term
-    const float decay_all = fast_exp2(g_last * kLog2e);
+    const float wl = valid ? vs * fast_exp2(g_last2 - gi2) : 0.f;   // factor of row l in the state update
+    const float eg = fast_exp2(gi2) * a.q_scale;                  // factor of token i in the inter-chunk term
+    const float decay_all = fast_exp2(g_last2);
     if (MODE == 1) seg_log += g_last;
     if (g == 0) {
-      lds_write<float>(lds_scal + ti * 4, gi);
+      lds_write<float>(lds_scal + ti * 4, gi2);
       lds_write<float>(lds_scal + (L + ti) * 4, pvq);
       lds_write<float>(lds_scal + (2 * L + ti) * 4, wl);
     }
     // ---- A^T = K Q^T (lane: token i = r, rows j = 8(jj/4) + 4g + jj%4)
     // two accumulation chains, so that consecutive MFMAs do not wait for each other, where registers
     // allow (with three waves per SIMD the other waves fill those gaps)
-    constexpr bool TWO_CHAINS = HG == 1;
+    constexpr bool TWO_CHAINS = HG == 1 && !SHARE_A;
     f32x16 sacc, sacc2;
 #pragma unroll
     for (int j = 0; j < 16; j++) { sacc[j] = 0.f; sacc2[j] = 0.f; }
-    if constexpr (MODE != 1) {
+    if constexpr (SHARE_A) {
+      // gather the quadrants: this lane's rows 8 q4 + 4g + {0..3} of column r sit in lane (r % 16) + 16 (2 (q4 % 2) + g)
+      // of quadrant slot (q4 / 2) + (r / 16); for the quadrant that was left out this reads its neighbour, and the
+      // causal select below discards it
+      __syncthreads();
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const uint32_t src = lds_apart + (uint32_t)(((q4 >> 1) + (r >> 4)) * KP) * 1024 + (uint32_t)((r & 15) + 16 * (2 * (q4 & 1) + g)) * 16;
+        f32x4 t = lds_read<f32x4>(src);
+        if constexpr (KP == 2) {
+          const f32x4 t2 = lds_read<f32x4>(src + 1024);
+#pragma unroll
+          for (int i = 0; i < 4; i++) t[i] += t2[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) sacc[4 * q4 + i] = t[i];
+      }
+    } else if constexpr (MODE != 1) {
       constexpr int NS = DK / 16, AH = 2, RING = 3;
       x8 kf[RING], qf[RING];
       auto request = [&](int ks) {
@@ -329,7 +378,8 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
 #pragma unroll
     for (int jj = 0; jj < 16; jj++) {
       const int j = 8 * (jj >> 2) + 4 * g + (jj & 3);
-      const float e = fast_exp2(fminf(gi - gj[jj], 0.f) * kLog2e);
+      // (above the diagonal the exponent is positive and the product may be inf or NaN: the select drops it)
+      const float e = fast_exp2(gi2 - gj[jj]);
       float p = (TWO_CHAINS ? sacc[jj] + sacc2[jj] : sacc[jj]) * e * pj[jj];
       asm volatile("" : "+v"(p));   // computed for every lane, then selected: no branch per element
       pf[jj >> 3][jj & 7] = (T)(j <= ti ? p : 0.f);
@@ -482,7 +532,7 @@ template <int DK, int NWH, int HG>
 struct Config {
   static constexpr int NW = NWH * HG;
   static constexpr size_t stage = (size_t)L * (4 * DK + 2 * 32 * NW);
-  static constexpr size_t lds = 2 * stage + NW * (3 * L * 4) + (HG > 1 ? 0 : NW * (L * 80));
+  static constexpr size_t lds = 2 * stage + NW * (3 * L * 4) + (HG > 1 ? 0 : NW * (L * 80)) + (NW >= 4 ? 3 * (NW >= 8 ? 2 : 1) * 1024 : 0);
   static constexpr int64_t ws_wave_floats = (int64_t)(DK / 32) * 16 * 64;
 
   static bool prepare(int& resident, int& cus) {
