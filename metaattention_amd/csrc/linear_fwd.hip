@@ -256,15 +256,15 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
         int la = lane;
         asm volatile("" : "+v"(la));
         const int rr = la & 15, kg = la >> 4;
-        const uint32_t krow = kbase + (16 * (slot >> 1) + rr) * RBQ, qrow = qbase + (16 * (slot > 0) + rr) * RBQ;
-        const int c0 = kg ^ swz16(rr);
+        // (tile bases and row offsets are multiples of the row size, so the swizzled chunk index occupies its own
+        // address bits: one XOR with a constant per read moves to another slice)
         constexpr int NS16 = DK / 32 / KP;
+        const uint32_t c0 = (uint32_t)((kg ^ swz16(rr)) << 4) ^ (uint32_t)(kp * NS16 * 64);
+        const uint32_t ka = kbase + (16 * (slot >> 1) + rr) * RBQ + c0, qa = qbase + (16 * (slot > 0) + rr) * RBQ + c0;
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s2 = 0; s2 < NS16; s2++) {
-          const uint32_t off = (uint32_t)((c0 ^ (4 * (kp * NS16 + s2))) << 4);
-          acc = E::mfma16(lds_read<x8>(krow + off), lds_read<x8>(qrow + off), acc);
-        }
+        for (int s2 = 0; s2 < NS16; s2++)
+          acc = E::mfma16(lds_read<x8>(ka ^ (uint32_t)(s2 * 64)), lds_read<x8>(qa ^ (uint32_t)(s2 * 64)), acc);
         lds_write<f32x4>(lds_apart + wave * 1024 + la * 16, acc);
       }
     }
@@ -342,10 +342,10 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
     } else if constexpr (MODE != 1) {
       constexpr int NS = DK / 16, AH = 2, RING = 3;
       x8 kf[RING], qf[RING];
+      const uint32_t kq_a = kbase + qk_row + (uint32_t)(qk_c0 << 4), qq_a = qbase + qk_row + (uint32_t)(qk_c0 << 4);
       auto request = [&](int ks) {
-        const uint32_t off = qk_row + (uint32_t)((qk_c0 ^ (2 * ks)) << 4);
-        kf[ks % RING] = lds_read<x8>(kbase + off);
-        qf[ks % RING] = lds_read<x8>(qbase + off);
+        kf[ks % RING] = lds_read<x8>(kq_a ^ (uint32_t)(ks * 32));
+        qf[ks % RING] = lds_read<x8>(qq_a ^ (uint32_t)(ks * 32));
       };
 #pragma unroll
       for (int ks = 0; ks < AH; ks++) request(ks);
@@ -389,12 +389,15 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
     // ---- V^T fragments (rows = this wave's 32 value columns; k-slot i of slice s is token
     //      16s + 8(i/4) + 4g + i%4, the order P^T comes in)
     x8 vf[2];
+    {
+      const uint32_t va = vbase + vt_row + (uint32_t)(vt_c0 << 4);
 #pragma unroll
-    for (int s = 0; s < 2; s++) {
-      const int cx = s ? V_X16 : 0;
-      x4 lo = lds_read_tr4<T>(vbase + vt_row + 16 * s * RBV + (uint32_t)((vt_c0 ^ cx) << 4));
-      x4 hi = lds_read_tr4<T>(vbase + vt_row + (16 * s + 8) * RBV + (uint32_t)((vt_c0 ^ cx ^ V_X8) << 4));
-      vf[s] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      for (int s = 0; s < 2; s++) {
+        const int cx = s ? V_X16 : 0;
+        x4 lo = lds_read_tr4<T>((va ^ (uint32_t)(cx << 4)) + 16 * s * RBV);
+        x4 hi = lds_read_tr4<T>((va ^ (uint32_t)((cx ^ V_X8) << 4)) + (16 * s + 8) * RBV);
+        vf[s] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
     }
 
     // ---- O^T = (h^T Q^T) * eg + V^T P^T
@@ -423,17 +426,18 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
       // per 32-row state block b: inter-chunk product with the OLD state, then the state update
       constexpr int RING = 2;
       x4 qlo[RING][2], qhi[RING][2], klo[RING][2], khi[RING][2];
+      const uint32_t qpa = qbase + qp_row + (uint32_t)(qp_swz << 4), kta = kbase + kt_row + (uint32_t)(kt_c0 << 4);
       auto request = [&](int bb) {
 #pragma unroll
         for (int s = 0; s < 2; s++) {
           const int lcq = 4 * bb + 2 * s;
           if constexpr (MODE != 1) {
-            qlo[bb % RING][s] = lds_read<x4>(qbase + qp_row + (uint32_t)((lcq ^ qp_swz) << 4));
-            qhi[bb % RING][s] = lds_read<x4>(qbase + qp_row + (uint32_t)(((lcq + 1) ^ qp_swz) << 4));
+            qlo[bb % RING][s] = lds_read<x4>(qpa ^ (uint32_t)(lcq << 4));
+            qhi[bb % RING][s] = lds_read<x4>(qpa ^ (uint32_t)((lcq + 1) << 4));
           }
           const int cx = s ? Q_X16 : 0;
-          klo[bb % RING][s] = lds_read_tr4<T>(kbase + kt_row + 16 * s * RBQ + (uint32_t)((kt_c0 ^ (4 * bb) ^ cx) << 4));
-          khi[bb % RING][s] = lds_read_tr4<T>(kbase + kt_row + (16 * s + 8) * RBQ + (uint32_t)((kt_c0 ^ (4 * bb) ^ cx ^ Q_X8) << 4));
+          klo[bb % RING][s] = lds_read_tr4<T>((kta ^ (uint32_t)(((4 * bb) ^ cx) << 4)) + 16 * s * RBQ);
+          khi[bb % RING][s] = lds_read_tr4<T>((kta ^ (uint32_t)(((4 * bb) ^ cx ^ Q_X8) << 4)) + (16 * s + 8) * RBQ);
         }
       };
       // operands are requested one block ahead, except where three waves per SIMD hide the LDS latency
@@ -503,14 +507,15 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
 #pragma unroll
         for (int i = 0; i < 4; i++)
           w[i] = (T)((DK < 256 && HG == 1 ? o_inter[4 * q4 + i] + o_inter2[4 * q4 + i] : o_inter[4 * q4 + i]) * eg + o_intra[4 * q4 + i]);
-        if (ALIAS_OST) lds_write<x4>(vbase + r * RBV + (uint32_t)(((4 * wave + q4) ^ sw_r) << 4) + g * 8, w);
+        if (ALIAS_OST) lds_write<x4>((vbase + r * RBV + (uint32_t)(((4 * wave) ^ sw_r) << 4) + g * 8) ^ (uint32_t)(q4 << 4), w);
         else lds_write<x4>(lds_ost + r * OROW + (8 * q4 + 4 * g) * 2, w);
       }
+      // (rows 16 apart share their swizzle)
+      const uint32_t ra = vbase + (ln >> 2) * RBV + (uint32_t)(((4 * wave + (ln & 3)) ^ swz_tile<CPRV>(ln >> 2)) << 4);
 #pragma unroll
       for (int it = 0; it < 2; it++) {
         const int ci = ln + 64 * it, row = ci >> 2, cc = ci & 3;
-        const u32x4 w = ALIAS_OST ? lds_read<u32x4>(vbase + row * RBV + (uint32_t)(((4 * wave + cc) ^ swz_tile<CPRV>(row)) << 4))
-                                  : lds_read<u32x4>(lds_ost + row * OROW + cc * 16);
+        const u32x4 w = ALIAS_OST ? lds_read<u32x4>(ra + 16 * it * RBV) : lds_read<u32x4>(lds_ost + row * OROW + cc * 16);
         if (t0 + row < Tn) *(u32x4*)(ob + (int64_t)(t0 + row) * a.Dv + cc * 8) = w;
       }
     }
