@@ -319,6 +319,8 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
     // two accumulation chains, so that consecutive MFMAs do not wait for each other, where registers
     // allow (with three waves per SIMD the other waves fill those gaps)
     constexpr bool TWO_CHAINS = HG == 1 && !SHARE_A;
+    // (a chain's first MFMA takes the constant zero as its accumulator input: no registers to clear)
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     f32x16 sacc, sacc2;
 #pragma unroll
     for (int j = 0; j < 16; j++) { sacc[j] = 0.f; sacc2[j] = 0.f; }
@@ -353,18 +355,20 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
       for (int ks = 0; ks < NS; ks++) {
         if (ks + AH < NS) request(ks + AH);
         __builtin_amdgcn_sched_barrier(0);
-        if (TWO_CHAINS && (ks & 1)) sacc2 = E::mfma32(kf[ks % RING], qf[ks % RING], sacc2);
-        else sacc = E::mfma32(kf[ks % RING], qf[ks % RING], sacc);
+        if (TWO_CHAINS && (ks & 1)) sacc2 = E::mfma32(kf[ks % RING], qf[ks % RING], ks == 1 ? zero16 : sacc2);
+        else sacc = E::mfma32(kf[ks % RING], qf[ks % RING], ks == 0 ? zero16 : sacc);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
     // rows held by this lane in a 32 x 32 accumulator block: 8q4 + 4g + {0..3}
     float gj[16], pj[16];
+    uint32_t scal_g = lds_scal + 16 * g;   // one lane register; every read below is this plus an immediate
+    asm volatile("" : "+v"(scal_g));
     if constexpr (MODE != 1) {
 #pragma unroll
     for (int q4 = 0; q4 < 4; q4++) {
-      const f32x4 tg = lds_read<f32x4>(lds_scal + (8 * q4 + 4 * g) * 4);
-      const f32x4 tp = lds_read<f32x4>(lds_scal + (L + 8 * q4 + 4 * g) * 4);
+      const f32x4 tg = lds_read<f32x4>(scal_g + 32 * q4);
+      const f32x4 tp = lds_read<f32x4>(scal_g + (L + 8 * q4) * 4);
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         gj[4 * q4 + i] = tg[i];
@@ -405,7 +409,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
 #pragma unroll
     for (int j = 0; j < 16; j++) { o_inter[j] = 0.f; o_inter2[j] = 0.f; o_intra[j] = 0.f; }
     if constexpr (MODE != 1) {
-      o_intra = E::mfma32(vf[0], pf[0], o_intra);
+      o_intra = E::mfma32(vf[0], pf[0], zero16);
       o_intra = E::mfma32(vf[1], pf[1], o_intra);
     }
     // value-scaled V^T for the state update (k-slot i of slice s is token 16s + 8(i/4) + 4g + i%4 -> wj[8s + i])
@@ -415,7 +419,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
       float w8[8];
 #pragma unroll
       for (int h2 = 0; h2 < 2; h2++) {
-        const f32x4 tw = lds_read<f32x4>(lds_scal + (2 * L + 16 * s + 8 * h2 + 4 * g) * 4);
+        const f32x4 tw = lds_read<f32x4>(scal_g + (2 * L + 16 * s + 8 * h2) * 4);
 #pragma unroll
         for (int i = 0; i < 4; i++) w8[4 * h2 + i] = tw[i];
       }
@@ -449,19 +453,26 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
         if (!AHEAD) request(bb);
         else if (bb + 1 < KB) request(bb + 1);
         __builtin_amdgcn_sched_barrier(0);
+        // the old state as bf16 operands first, then the decay in place (left to itself the compiler decays into a
+        // second register block while the old values are still waiting to be converted, and copies it back)
+        x8 hf[2];
         if constexpr (MODE != 1) {
 #pragma unroll
-          for (int s = 0; s < 2; s++) {
-            x8 hf;
+          for (int s = 0; s < 2; s++)
 #pragma unroll
-            for (int i = 0; i < 8; i++) hf[i] = (T)hst[bb][8 * s + i];
-            x8 qf = __builtin_shufflevector(qlo[bb % RING][s], qhi[bb % RING][s], 0, 1, 2, 3, 4, 5, 6, 7);
-            if (DK < 256 && HG == 1 && s) o_inter2 = E::mfma32(hf, qf, o_inter2);   // (a second chain where registers allow)
-            else o_inter = E::mfma32(hf, qf, o_inter);
-          }
+            for (int i = 0; i < 8; i++) hf[s][i] = (T)hst[bb][8 * s + i];
+          __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int j = 0; j < 16; j++) hst[bb][j] *= decay_all;
+        if constexpr (MODE != 1) {
+#pragma unroll
+          for (int s = 0; s < 2; s++) {
+            x8 qf = __builtin_shufflevector(qlo[bb % RING][s], qhi[bb % RING][s], 0, 1, 2, 3, 4, 5, 6, 7);
+            if (DK < 256 && HG == 1 && s) o_inter2 = E::mfma32(hf[s], qf, bb == 0 ? zero16 : o_inter2);   // (a second chain where registers allow)
+            else o_inter = E::mfma32(hf[s], qf, (bb == 0 && (s == 0 || (DK < 256 && HG == 1))) ? zero16 : o_inter);
+          }
+        }
 #pragma unroll
         for (int s = 0; s < 2; s++) {
           x8 kf = __builtin_shufflevector(klo[bb % RING][s], khi[bb % RING][s], 0, 1, 2, 3, 4, 5, 6, 7);
