@@ -142,20 +142,25 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
 
   // ---- DMA of one chunk: each instruction moves 1 KB (1024/row_bytes tile rows); lane i fetches
   //      the 16-byte chunk that belongs at physical position i of that KB.
+  //      (Spreading a chunk's instructions over the chunk's phases instead of issuing them together behind the
+  //      barrier was measured: no gain at the RetNet shape, 5 % slower at the Mamba2 shape.)
   auto issue_chunk = [&](int t0, int buf) {
     const uint32_t base = lds0 + buf * STAGE;
     constexpr int NQK = MODE == 1 ? NIQ : 2 * NIQ;      // (the state-only pass needs no Q)
     constexpr int RQ = 1024 / RBQ, RV = 1024 / RBV;     // tile rows per instruction
+    static_assert(HG == 1 || RV % 4 == 0, "the V swizzle of an instruction's first row must stay inside a head's columns");
     if (t0 + L <= Tn && v_head_bytes < ((int64_t)1 << 31)) {
       // Whole chunk: no row clamping, so an instruction's source is a wave-uniform base (SGPRs) plus a
       // 32-bit lane offset.  The swizzle is a bit permutation of the row index, so it splits into the
-      // lane's part (row within the instruction) and the instruction's part (its first row): per
-      // instruction that is one XOR, against ~25 vector instructions of 64-bit address arithmetic.
+      // lane's part (row within the instruction) and the instruction's part (its first row), and since row
+      // offsets are multiples of the row size the instruction's part is one XOR on the finished lane offset.
       int ln2 = lane;
       asm volatile("" : "+v"(ln2));   // rebuilt per chunk: kept live across the chunk these would cost registers
       const int lrq = ln2 / CPRQ, lrv = ln2 / CPRV;
-      const uint32_t offq = lrq * RBQ, lcq0 = (ln2 % CPRQ) ^ swz_tile<CPRQ>(lrq);
-      const uint32_t offv = lrv * (uint32_t)v_row_bytes, lcv0 = (ln2 % CPRV) ^ swz_tile<CPRV>(lrv);
+      const uint32_t aq = lrq * RBQ + (uint32_t)(((ln2 % CPRQ) ^ swz_tile<CPRQ>(lrq)) << 4);
+      const uint32_t lc0 = (ln2 % CPRV) ^ swz_tile<CPRV>(lrv);       // logical chunk: head lc / (4 NWH), then its columns
+      uint32_t av = lrv * (uint32_t)v_row_bytes + ((lc0 % (4 * NWH)) << 4);
+      if (HG > 1) av += (lc0 / (4 * NWH)) * (uint32_t)v_head_bytes;
 #pragma unroll (DK <= 128 ? 16 : 1)   // (with a 256-wide key the state leaves no registers for an unrolled burst)
       for (int it = 0; it < (NQK + NIV + NW - 1) / NW; it++) {
         const int ii = wave + NW * it;
@@ -163,14 +168,11 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
         if (ii < NQK) {
           const int which = MODE == 1 ? 1 : ii >= NIQ, i2 = (MODE != 1 && which) ? ii - NIQ : ii;
           const char* sb = (which ? kb : qb) + (int64_t)(t0 + i2 * RQ) * RBQ;
-          dma16_so(sb, offq + ((lcq0 ^ (uint32_t)swz_tile<CPRQ>(i2 * RQ)) << 4), base + which * QT + i2 * 1024);
+          dma16_so(sb, aq ^ (uint32_t)(swz_tile<CPRQ>(i2 * RQ) << 4), base + which * QT + i2 * 1024);
         } else {
           const int i2 = ii - NQK;
           const char* sb = vb + (int64_t)(t0 + i2 * RV) * v_row_bytes;
-          const uint32_t lc = lcv0 ^ (uint32_t)swz_tile<CPRV>(i2 * RV);   // logical chunk: head lc / (4 NWH), then its columns
-          uint32_t off = offv + ((lc % (4 * NWH)) << 4);
-          if (HG > 1) off += (lc / (4 * NWH)) * (uint32_t)v_head_bytes;
-          dma16_so(sb, off, base + 2 * QT + i2 * 1024);
+          dma16_so(sb, av ^ (uint32_t)(swz_tile<CPRV>(i2 * RV) << 4), base + 2 * QT + i2 * 1024);
         }
       }
       return;
@@ -234,7 +236,8 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
     wait_dma();
     __syncthreads();
     const float ld = ld_next, vs = vs_next;
-    if (c + 1 < c_end) {
+    const bool has_next = c + 1 < c_end;
+    if (has_next) {
       const int tn = t0 + L + ti;
       ld_next = 0.f;
       vs_next = 1.f;
@@ -242,8 +245,8 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
         ld_next = ldp[tn];
         if (vsp) vs_next = vsp[tn];
       }
-      issue_chunk(t0 + L, buf ^ 1);
     }
+    if (has_next) issue_chunk(t0 + L, buf ^ 1);
     const uint32_t base = lds0 + buf * STAGE;
     const uint32_t qbase = base, kbase = base + QT, vbase = base + 2 * QT;
 
