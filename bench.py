@@ -35,7 +35,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a
 # 1 GiB copy (profiles/attn_fwd_kernel_c2_softmax_sigmoid.md): 1414 MB read + 273 MB written
-ATTN_FWD_HBM_BYTES = 1.687e9
+ATTN_FWD_HBM_BYTES = 1.709e9
 
 
 def time_gpu(fn, steps, warmup, flush=None):
@@ -106,7 +106,7 @@ def bench_softmax_bwd(steps, warmup):
     o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale, row_scale=lse)
     ms = time_gpu(lambda: hb.attn_bwd(q, k, v, o, do, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale), max(steps // 3, 3), 2)
     flops = 2.5 * 0.5 * 4.0 * B * H * S * S * D
-    return _mfma_entry(ms, flops, "backward, 2.5 x the forward's algorithmic FLOPs (5 tile products; the two kernels execute 7)")
+    return _mfma_entry(ms, flops, "backward, 2.5 x the forward's algorithmic FLOPs (5 tile products; the three kernels dq, dv, dk execute 8: each recomputes the scores)")
 
 
 def bench_decode(steps, warmup, B=64, H=32, Hkv=8, Skv=4096, D=128):
