@@ -66,19 +66,19 @@ __device__ __forceinline__ f32x16 mm_rows(uint32_t tile, int r, int g, const typ
   using E = Elem<T>;
   using x8 = typename E::x8;
   constexpr int ROWB = DIM * 2, CPR = DIM / 8, KS = DIM / 16, AH = 2, RING = 3;
-  const uint32_t row_off = tile + r * ROWB;
-  const int c0 = g ^ swz_tile<CPR>(r);
+  // (tile bases and row offsets are multiples of the row size, so the swizzled chunk index has its own address
+  // bits: another k-slice is one XOR with a constant away)
+  const uint32_t a0 = tile + r * ROWB + (uint32_t)((g ^ swz_tile<CPR>(r)) << 4);
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   f32x16 acc;
-#pragma unroll
-  for (int j = 0; j < 16; j++) acc[j] = 0.f;
   x8 af[RING];
 #pragma unroll
-  for (int ks = 0; ks < AH && ks < KS; ks++) af[ks] = lds_read<x8>(row_off + (uint32_t)((c0 ^ (2 * ks)) << 4));
+  for (int ks = 0; ks < AH && ks < KS; ks++) af[ks] = lds_read<x8>(a0 ^ (uint32_t)(ks * 32));
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) {
-    if (ks + AH < KS) af[(ks + AH) % RING] = lds_read<x8>(row_off + (uint32_t)((c0 ^ (2 * (ks + AH))) << 4));
+    if (ks + AH < KS) af[(ks + AH) % RING] = lds_read<x8>(a0 ^ (uint32_t)((ks + AH) * 32));
     __builtin_amdgcn_sched_barrier(0);
-    acc = E::mfma32(af[ks % RING], bf[ks], acc);
+    acc = E::mfma32(af[ks % RING], bf[ks], ks == 0 ? zero16 : acc);
     __builtin_amdgcn_sched_barrier(0);
   }
   return acc;
@@ -95,14 +95,12 @@ __device__ __forceinline__ void mm_cols(uint32_t tile, int lane, const typename 
   constexpr int ROWB = DIM * 2, CPR = DIM / 8, NB = DIM / 32, PF = NB >= 2 ? 4 : 2;
   const int g = lane >> 5, jr = (lane & 15) >> 2;
   const int lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
-  const uint32_t row_off = tile + (4 * g + jr) * ROWB + (lane & 1) * 8;
-  const int c0 = lc ^ swz_tile<CPR>(4 * g + jr);
+  const uint32_t b0 = tile + (4 * g + jr) * ROWB + (lane & 1) * 8 + (uint32_t)((lc ^ swz_tile<CPR>(4 * g + jr)) << 4);
   x4 lo[PF], hi[PF];
   auto request = [&](int idx) {   // idx = 2 block + slice
     const int db = idx >> 1, sl = idx & 1;
-    const uint32_t rb = row_off + 16 * sl * ROWB;
-    lo[idx % PF] = lds_read_tr4<T>(rb + (uint32_t)((c0 ^ (4 * db)) << 4));
-    hi[idx % PF] = lds_read_tr4<T>(rb + 8 * ROWB + (uint32_t)((c0 ^ (4 * db) ^ 2) << 4));
+    lo[idx % PF] = lds_read_tr4<T>((b0 ^ (uint32_t)((4 * db) << 4)) + 16 * sl * ROWB);
+    hi[idx % PF] = lds_read_tr4<T>((b0 ^ (uint32_t)(((4 * db) ^ 2) << 4)) + (16 * sl + 8) * ROWB);
   };
 #pragma unroll
   for (int i = 0; i < PF - 1; i++) request(i);
@@ -233,13 +231,23 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
     const f32x16 s = mm_rows<T, DQK>(kbase, r, g, qf);     // S^T: lane = row m_lane, element jj = key n0 + 8(jj/4) + 4g + jj%4
     const f32x16 dp = mm_rows<T, DV>(vbase, r, g, dof);   // dP^T, same layout
     x8 dsf[2];
+    // only tiles that touch the diagonal or the end of the keys pay for the mask (the test is wave-uniform)
+    if ((CAUSAL && n0 + BN - 1 > m_wave) || n0 + BN > a.Skv) {
 #pragma unroll
-    for (int jj = 0; jj < 16; jj++) {
-      const int n = n0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
-      const bool masked = (CAUSAL && n > m_lane) || n >= a.Skv;
-      float p, ds;
-      row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, lse2, delta, p, ds);
-      dsf[jj >> 3][jj & 7] = (T)ds;
+      for (int jj = 0; jj < 16; jj++) {
+        const int n = n0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
+        const bool masked = (CAUSAL && n > m_lane) || n >= a.Skv;
+        float p, ds;
+        row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, lse2, delta, p, ds);
+        dsf[jj >> 3][jj & 7] = (T)ds;
+      }
+    } else {
+#pragma unroll
+      for (int jj = 0; jj < 16; jj++) {
+        float p, ds;
+        row_fn_bwd<FAMILY>(s[jj], dp[jj], false, c_scale, c_bias, a.scale, bias, lse2, delta, p, ds);
+        dsf[jj >> 3][jj & 7] = (T)ds;
+      }
     }
     mm_cols<T, DQK>(kbase, lane, dsf, dq);                 // dQ^T += K^T dS^T
   }
@@ -365,16 +373,28 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
 #pragma unroll
       for (int j = 0; j < 16; j++) dp[j] = 0.f;
     x8 pf[2], dsf[2];
+    // only tiles that touch the diagonal or an end of the sequences pay for the mask (the test is wave-uniform)
+    if ((CAUSAL && n_wave + 31 > m0) || m0 + BMT > a.Sq || n_wave + 32 > a.Skv) {
 #pragma unroll
-    for (int jj = 0; jj < 16; jj++) {
-      const int m = m0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
-      const bool masked = (CAUSAL && n_lane > m) || m >= a.Sq || n_lane >= a.Skv;
-      float p, ds;
-      row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX ? lse2[jj] : 0.f,
-                         FAMILY == BF_SOFTMAX ? dl[jj] : 0.f, p, ds);
-      if (masked) ds = 0.f;
-      pf[jj >> 3][jj & 7] = (T)p;
-      dsf[jj >> 3][jj & 7] = (T)ds;
+      for (int jj = 0; jj < 16; jj++) {
+        const int m = m0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
+        const bool masked = (CAUSAL && n_lane > m) || m >= a.Sq || n_lane >= a.Skv;
+        float p, ds;
+        row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX ? lse2[jj] : 0.f,
+                           FAMILY == BF_SOFTMAX ? dl[jj] : 0.f, p, ds);
+        if (masked) ds = 0.f;
+        pf[jj >> 3][jj & 7] = (T)p;
+        dsf[jj >> 3][jj & 7] = (T)ds;
+      }
+    } else {
+#pragma unroll
+      for (int jj = 0; jj < 16; jj++) {
+        float p, ds;
+        row_fn_bwd<FAMILY>(s[jj], dp[jj], false, c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX ? lse2[jj] : 0.f,
+                           FAMILY == BF_SOFTMAX ? dl[jj] : 0.f, p, ds);
+        pf[jj >> 3][jj & 7] = (T)p;
+        dsf[jj >> 3][jj & 7] = (T)ds;
+      }
     }
     if constexpr (DO_DV) mm_cols<T, DV>(dobase, lane, pf, dv);     // dV^T += dO^T P
     if constexpr (DO_DK) mm_cols<T, DQK>(qbase, lane, dsf, dk);    // dK^T += Q^T dS
