@@ -30,20 +30,21 @@ namespace ma {
 namespace {
 enum { BF_SOFTMAX = 0, BF_SIGMOID = 1, BF_RELU = 2 };   // = MA_ATTN_* of the C interface
 
-// ds (and p) of one score element.  x2 = (s * scale + bias) * log2(e) for softmax / sigmoid.
+// ds / scale (and p) of one score element: the common factor `scale` of dq and dk is applied once, when the
+// accumulators are stored.  x2 = (s * scale + bias) * log2(e) for softmax / sigmoid.
 template <int FAMILY>
 __device__ __forceinline__ void row_fn_bwd(float s, float dp, bool masked, float c_scale, float c_bias, float scale, float bias,
                                            float lse2, float delta, float& p, float& ds) {
   if constexpr (FAMILY == BF_SOFTMAX) {
-    p = masked ? 0.f : fast_exp2(s * c_scale + c_bias - lse2);
-    ds = p * (dp - delta) * scale;
+    p = masked ? 0.f : fast_exp2(s * c_scale + lse2);   // (lse2 = c_bias - lse * log2(e), folded by the caller)
+    ds = p * (dp - delta);
   } else if constexpr (FAMILY == BF_SIGMOID) {
     p = masked ? 0.f : fast_rcp(1.f + fast_exp2(-(s * c_scale + c_bias)));
-    ds = dp * p * (1.f - p) * scale;
+    ds = dp * p * (1.f - p);
   } else {
     const float x = s * scale + bias;
     p = masked ? 0.f : fmaxf(x, 0.f);
-    ds = (!masked && x > 0.f) ? dp * scale : 0.f;
+    ds = (!masked && x > 0.f) ? dp : 0.f;
   }
 }
 
@@ -219,6 +220,7 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
     for (int j = 0; j < 16; j++) dq[i][j] = 0.f;
   const float bias = a.bias + (a.bias_ptr ? *a.bias_ptr : 0.f);
   const float c_scale = a.scale * kLog2e, c_bias = bias * kLog2e;
+  lse2 = c_bias - lse2;   // what the row function adds to s * c_scale
 
   if (n_tiles > 0) issue_tile(0, 0);
   for (int jt = 0; jt < n_tiles; jt++) {
@@ -255,7 +257,7 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
 
   constexpr int OROW = DQK + 16;
   T* dqb = (T*)a.dq + (int64_t)b * a.dqsb + (int64_t)h * a.dqsh;
-  store_rows<T, DQK>(dq, 1.f, lds0 + wave * 32 * OROW, dqb, a.dqss, m_wave, a.Sq, lane);
+  store_rows<T, DQK>(dq, a.scale, lds0 + wave * 32 * OROW, dqb, a.dqss, m_wave, a.Sq, lane);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -351,7 +353,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
           const f32x4 td = *(const f32x4*)(a.delta + rbase + m0 + 8 * q4 + 4 * g);
 #pragma unroll
           for (int i = 0; i < 4; i++) {
-            lse2[4 * q4 + i] = tl[i] * kLog2e;
+            lse2[4 * q4 + i] = c_bias - tl[i] * kLog2e;   // what the row function adds to s * c_scale
             dl[4 * q4 + i] = td[i];
           }
         }
@@ -361,7 +363,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
 #pragma unroll
           for (int i = 0; i < 4; i++) {
             const int m = min(m0 + 8 * q4 + 4 * g + i, a.Sq - 1);
-            lse2[4 * q4 + i] = a.lse[rbase + m] * kLog2e;
+            lse2[4 * q4 + i] = c_bias - a.lse[rbase + m] * kLog2e;
             dl[4 * q4 + i] = a.delta[rbase + m];
           }
       }
@@ -405,7 +407,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
   const uint32_t stage = lds0 + wave * 32 * OROW;
   T* dkb = (T*)a.dk + (int64_t)b * a.dksb + (int64_t)hk * a.dksh;
   T* dvb = (T*)a.dv + (int64_t)b * a.dvsb + (int64_t)hk * a.dvsh;
-  if constexpr (DO_DK) store_rows<T, DQK>(dk, 1.f, stage, dkb, a.dkss, n_wave, a.Skv, lane);
+  if constexpr (DO_DK) store_rows<T, DQK>(dk, a.scale, stage, dkb, a.dkss, n_wave, a.Skv, lane);
   if constexpr (DO_DV) store_rows<T, DV>(dv, 1.f, stage, dvb, a.dvss, n_wave, a.Skv, lane);
 }
 
