@@ -120,6 +120,13 @@ typedef struct ma_attn_bwd_params {
   float scale, bias;
   const float* bias_ptr;
   void* workspace; size_t workspace_bytes;
+  /* arbitrary masks, as elem_mask of ma_attn_params (with MA_MASK_NONE only): the same uint8/bool keep mask in both
+   * orientations, strides in bytes, stride 0 broadcasts, rows 4-byte aligned.  elem_mask [1 or B, 1 or H, Sq, Skv]
+   * serves the dq kernel, elem_mask_t [1 or B, 1 or H, Skv, Sq] (its transpose) the dk / dv kernels, where a lane
+   * walks down a key's column; give both or neither.  (The reference generates the mask_mod's code into its backward
+   * kernels as well, attn_tl.py:212-525.) */
+  const uint8_t* elem_mask;   int64_t em_stride_b, em_stride_h, em_stride_q;
+  const uint8_t* elem_mask_t; int64_t emt_stride_b, emt_stride_h, emt_stride_k;
 } ma_attn_bwd_params;
 
 /* Chunked linear / stateful attention forward.  Replaces the three launches

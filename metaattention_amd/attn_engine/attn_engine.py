@@ -101,8 +101,13 @@ class _Attention(torch.autograd.Function):
         from hip_backend import attn_bwd
         q, k, v, out, *rest = ctx.saved_tensors
         form = ctx.engine.score_form
+        eng = ctx.engine
+        masks = {}
+        if eng.mask_kind.startswith("other"):
+            masks = dict(zip(("elem_mask", "elem_mask_t"), eng._dense_mask(q.shape[0], q.shape[2], q.shape[1], k.shape[1], q.device,
+                                                                           transposed=True)))
         dq, dk, dv = attn_bwd(q, k, v, out, dout, rest[0] if rest else None, family=ctx.fam_code,
-                              causal=ctx.engine.mask_kind == "causal", scale=form.scale, bias=form.bias, bias_tensor=ctx.bias_t)
+                              causal=eng.mask_kind == "causal", scale=form.scale, bias=form.bias, bias_tensor=ctx.bias_t, **masks)
         return None, None, None, None, dq, dk, dv
 
 
@@ -249,7 +254,7 @@ class AttentionEngine:
             return run(q, k, v).squeeze(1)
 
         if any(t.requires_grad for t in (q, k, v)):
-            if self.family == "retention" or self.mask_kind.startswith("other") or prefill_blocks is not None:
+            if self.family == "retention" or prefill_blocks is not None:
                 return _ForwardOnly.apply(run, q, k, v)
             bias_t = given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None
             return _Attention.apply(self, run, fam_code, bias_t, q, k, v)
@@ -268,10 +273,11 @@ class AttentionEngine:
         keep = (block_mask != 0).to(torch.uint8)
         return keep.repeat_interleave(Sq // nq // 128, dim=2).repeat_interleave(Skv // nk // 32, dim=3)
 
-    def _dense_mask(self, B, H, Sq, Skv, device):
+    def _dense_mask(self, B, H, Sq, Skv, device, transposed=False):
         """(element-wise keep mask uint8 [1|B, 1|H, Sq, Skv] with 4-byte aligned rows, block mask uint8
         [1|B, 1|H, ceil(Sq/128), ceil(Skv/32)]: a block is kept when any of its elements is) for the mask_mod, built
-        once per shape on the device."""
+        once per shape on the device.  transposed=True: (the keep mask, its transpose [.., Skv, Sq] with 4-byte aligned
+        rows) for the backward kernels; the transpose is built on first use."""
         from core.transform.core import create_mask
         key = (B, H, Sq, Skv, str(device))
         if self._mask_tensors is None or self._mask_tensors[0] != key:
@@ -283,7 +289,14 @@ class AttentionEngine:
             pad = torch.zeros(Bm, Hm, sqp, nkp, dtype=torch.bool, device=device)
             pad[:, :, :Sq, :Skv] = dense
             blocks = pad.view(Bm, Hm, sqp // 128, 128, nkp // 32, 32).any(dim=5).any(dim=3).to(torch.uint8).contiguous()
-            self._mask_tensors = (key, buf[..., :Skv], blocks)
+            self._mask_tensors = [key, buf[..., :Skv], blocks, None]
+        if transposed:
+            if self._mask_tensors[3] is None:
+                elem = self._mask_tensors[1]
+                buf_t = torch.zeros(elem.shape[0], elem.shape[1], Skv, (Sq + 3) // 4 * 4, dtype=torch.uint8, device=device)
+                buf_t[..., :Sq] = elem.transpose(2, 3)
+                self._mask_tensors[3] = buf_t[..., :Sq]
+            return self._mask_tensors[1], self._mask_tensors[3]
         return self._mask_tensors[1], self._mask_tensors[2]
 
     # ------------------------------------------------------------------ MLA decode

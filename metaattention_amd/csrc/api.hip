@@ -146,6 +146,14 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
                             (uintptr_t)p->dq, (uintptr_t)p->dk, (uintptr_t)p->dv};
   for (uintptr_t x : ptrs)
     if (x % 16 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: tensors must be 16-byte aligned");
+  if (p->elem_mask || p->elem_mask_t) {
+    if (!p->elem_mask || !p->elem_mask_t) return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: elem_mask and elem_mask_t go together");
+    if (p->mask == MA_MASK_CAUSAL) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: elem_mask goes with MA_MASK_NONE");
+    const int64_t ms[] = {(int64_t)(uintptr_t)p->elem_mask, p->em_stride_b, p->em_stride_h, p->em_stride_q,
+                          (int64_t)(uintptr_t)p->elem_mask_t, p->emt_stride_b, p->emt_stride_h, p->emt_stride_k};
+    for (int64_t x : ms)
+      if (x % 4 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: elem_mask rows must be 4-byte aligned");
+  }
 
   ma::AttnBwdArgs a{};
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.dout = p->dout; a.dq = p->dq; a.dk = p->dk; a.dv = p->dv;
@@ -161,6 +169,8 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
   a.B = p->batch; a.H = p->heads; a.Hkv = hkv; a.Sq = p->seqlen_q; a.Skv = p->seqlen_kv;
   a.kv_group = p->heads / hkv;
   a.scale = p->scale; a.bias = p->bias;
+  a.elem_mask = p->elem_mask; a.em_sb = p->em_stride_b; a.em_sh = p->em_stride_h; a.em_sq = p->em_stride_q;
+  a.elem_mask_t = p->elem_mask_t; a.emt_sb = p->emt_stride_b; a.emt_sh = p->emt_stride_h; a.emt_sk = p->emt_stride_k;
   const int rc = ma::attn_bwd_dispatch(a, p->family, p->mask == MA_MASK_CAUSAL, p->dtype == MA_BF16, p->dim_qk, p->dim_v, (hipStream_t)stream);
   if (rc == -2) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: no kernel for family %d, Dqk=%d, Dv=%d", p->family, p->dim_qk, p->dim_v);
   if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_attn_bwd: launch failed: %s", hipGetErrorString(hipGetLastError()));

@@ -15,6 +15,11 @@ struct AttnBwdArgs {
   int B, H, Hkv, Sq, Skv, num_blocks;
   int kv_group;   // query heads per kv head
   float scale, bias;
+  // optional element-wise keep mask (0 = masked) in both orientations, strides in bytes, 0 broadcasts:
+  // elem_mask [.., .., Sq, Skv] for the dq kernel (a lane walks a query row), elem_mask_t [.., .., Skv, Sq]
+  // for the dk / dv kernel (a lane walks a key's column); rows are 4-byte aligned
+  const uint8_t* elem_mask; int64_t em_sb, em_sh, em_sq;
+  const uint8_t* elem_mask_t; int64_t emt_sb, emt_sh, emt_sk;
 };
 
 int attn_bwd_dispatch(const AttnBwdArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);

@@ -7,7 +7,11 @@
 //   sigmoid   p = 1 / (1 + exp(-x)),  ds = dp * p * (1 - p) * scale
 //   relu      p = max(x, 0),          ds = dp * [x > 0] * scale
 //   dp = do.v^T,   dv = p^T do,   dk = ds^T q,   dq = ds k
-// (p and ds are rounded to the tensor dtype before the second products, as there: :357-362).
+// (p and ds are rounded to the tensor dtype before the second products, as there: :357-362; the factor
+// `scale` common to dq and dk is applied once, when their accumulators are stored).
+// Masks: none, causal, or an element-wise keep mask given in both orientations (the dq kernel walks a
+// query row of it, the dk / dv kernel a key's column of its transpose); only tiles that a mask can
+// touch evaluate it.
 //
 // No atomics: two kernels, each owning its outputs.
 //   attn_bwd_dq_kernel   a wave owns 32 query rows and walks the kv sequence; everything transposed as in
@@ -222,6 +226,9 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
   const float c_scale = a.scale * kLog2e, c_bias = bias * kLog2e;
   lse2 = c_bias - lse2;   // what the row function adds to s * c_scale
 
+  // element-wise keep mask of this lane's query row
+  const uint8_t* em_row = a.elem_mask ? a.elem_mask + (int64_t)b * a.em_sb + (int64_t)h * a.em_sh + (int64_t)m_ld * a.em_sq : nullptr;
+
   if (n_tiles > 0) issue_tile(0, 0);
   for (int jt = 0; jt < n_tiles; jt++) {
     const int buf = jt & 1, n0 = jt * BN;
@@ -233,12 +240,28 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
     const f32x16 s = mm_rows<T, DQK>(kbase, r, g, qf);     // S^T: lane = row m_lane, element jj = key n0 + 8(jj/4) + 4g + jj%4
     const f32x16 dp = mm_rows<T, DV>(vbase, r, g, dof);   // dP^T, same layout
     x8 dsf[2];
-    // only tiles that touch the diagonal or the end of the keys pay for the mask (the test is wave-uniform)
-    if ((CAUSAL && n0 + BN - 1 > m_wave) || n0 + BN > a.Skv) {
+    // only tiles that touch the diagonal or the end of the keys pay for the mask (the test is wave-uniform);
+    // with an element-wise mask every tile does
+    if ((CAUSAL && n0 + BN - 1 > m_wave) || n0 + BN > a.Skv || em_row) {
+      uint32_t keep[4] = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};   // the bytes of this lane's four keys per group
+      if (em_row) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+          const int n = n0 + 8 * q4 + 4 * g;
+          if (n + 3 < a.Skv) {
+            keep[q4] = *(const uint32_t*)(em_row + n);
+          } else {
+            keep[q4] = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+              if (n + i < a.Skv) keep[q4] |= (uint32_t)em_row[n + i] << (8 * i);
+          }
+        }
+      }
 #pragma unroll
       for (int jj = 0; jj < 16; jj++) {
         const int n = n0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
-        const bool masked = (CAUSAL && n > m_lane) || n >= a.Skv;
+        const bool masked = (CAUSAL && n > m_lane) || n >= a.Skv || ((keep[jj >> 2] >> (8 * (jj & 3))) & 0xffu) == 0;
         float p, ds;
         row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, lse2, delta, p, ds);
         dsf[jj >> 3][jj & 7] = (T)ds;
@@ -375,12 +398,30 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
 #pragma unroll
       for (int j = 0; j < 16; j++) dp[j] = 0.f;
     x8 pf[2], dsf[2];
-    // only tiles that touch the diagonal or an end of the sequences pay for the mask (the test is wave-uniform)
-    if ((CAUSAL && n_wave + 31 > m0) || m0 + BMT > a.Sq || n_wave + 32 > a.Skv) {
+    // only tiles that touch the diagonal or an end of the sequences pay for the mask (the test is wave-uniform);
+    // with an element-wise mask every tile does
+    if ((CAUSAL && n_wave + 31 > m0) || m0 + BMT > a.Sq || n_wave + 32 > a.Skv || a.elem_mask_t) {
+      uint32_t keep[4] = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};   // the bytes of this lane's four rows per group
+      if (a.elem_mask_t) {
+        // the transposed mask: this key's row, indexed by query position
+        const uint8_t* emt_row = a.elem_mask_t + (int64_t)b * a.emt_sb + (int64_t)h * a.emt_sh + (int64_t)n_ld * a.emt_sk;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+          const int m = m0 + 8 * q4 + 4 * g;
+          if (m + 3 < a.Sq) {
+            keep[q4] = *(const uint32_t*)(emt_row + m);
+          } else {
+            keep[q4] = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+              if (m + i < a.Sq) keep[q4] |= (uint32_t)emt_row[m + i] << (8 * i);
+          }
+        }
+      }
 #pragma unroll
       for (int jj = 0; jj < 16; jj++) {
         const int m = m0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
-        const bool masked = (CAUSAL && n_lane > m) || m >= a.Sq || n_lane >= a.Skv;
+        const bool masked = (CAUSAL && n_lane > m) || m >= a.Sq || n_lane >= a.Skv || ((keep[jj >> 2] >> (8 * (jj & 3))) & 0xffu) == 0;
         float p, ds;
         row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX ? lse2[jj] : 0.f,
                            FAMILY == BF_SOFTMAX ? dl[jj] : 0.f, p, ds);

@@ -70,6 +70,8 @@ class AttnBwdParams(Structure):
         ("lse", c_void_p),
         ("scale", c_float), ("bias", c_float), ("bias_ptr", c_void_p),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+        ("elem_mask", c_void_p), ("em_stride_b", c_int64), ("em_stride_h", c_int64), ("em_stride_q", c_int64),
+        ("elem_mask_t", c_void_p), ("emt_stride_b", c_int64), ("emt_stride_h", c_int64), ("emt_stride_k", c_int64),
     ]
 
 
@@ -231,11 +233,13 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
     return out
 
 
-def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None):
+def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None,
+             elem_mask=None, elem_mask_t=None):
     """Gradients (dq, dk, dv) of the parallel attention forward on BSHD tensors.  ``o`` and ``lse``
     (fp32 [B,H,Sq]) are the forward pass's output and row scale (softmax only; None otherwise),
-    ``dout`` the gradient of ``o``."""
-    _require_gpu(q, k, v, o, dout, lse, bias_tensor)
+    ``dout`` the gradient of ``o``.  ``elem_mask`` (the forward pass's keep mask, [1|B, 1|H, Sq, Skv]) comes with
+    its transpose ``elem_mask_t`` [1|B, 1|H, Skv, Sq]; both with rows at 4-byte aligned addresses."""
+    _require_gpu(q, k, v, o, dout, lse, bias_tensor, elem_mask, elem_mask_t)
     B, Sq, H, Dqk = q.shape
     Skv, Hkv, Dv = k.shape[1], k.shape[2], v.shape[-1]
     assert k.shape == (B, Skv, Hkv, Dqk) and v.shape == (B, Skv, Hkv, Dv) and dout.shape == (B, Sq, H, Dv) and H % Hkv == 0
@@ -260,6 +264,15 @@ def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, 
     if bias_tensor is not None:
         assert bias_tensor.dtype == torch.float32 and bias_tensor.numel() == 1
         p.bias_ptr = bias_tensor.data_ptr()
+    if elem_mask is not None or elem_mask_t is not None:
+        assert elem_mask is not None and elem_mask_t is not None, "elem_mask and elem_mask_t go together"
+        for t, rows, cols, pre, last in ((elem_mask, Sq, Skv, "em", "q"), (elem_mask_t, Skv, Sq, "emt", "k")):
+            assert t.dtype in (torch.bool, torch.uint8) and t.dim() == 4 and t.shape[2:] == (rows, cols) and t.stride(-1) == 1
+            assert t.shape[0] in (1, B) and t.shape[1] in (1, H)
+            setattr(p, "elem_mask" if pre == "em" else "elem_mask_t", t.data_ptr())
+            setattr(p, f"{pre}_stride_b", t.stride(0) if t.shape[0] > 1 else 0)
+            setattr(p, f"{pre}_stride_h", t.stride(1) if t.shape[1] > 1 else 0)
+            setattr(p, f"{pre}_stride_{last}", t.stride(2))
     lib = load_library()
     need = lib.ma_attn_bwd_workspace_bytes(ctypes.byref(p))
     if need:

@@ -139,3 +139,78 @@ def test_retention_backward_still_raises():
     o = mod(qc, k.cuda(), v.cuda(), mask)
     with pytest.raises(NotImplementedError):
         o.sum().backward()
+
+
+MASKS = {
+    "sliding_window": lambda b, h, q, k: (q >= k) & (q - k < 100),
+    "prefix_lm": lambda b, h, q, k: (q >= k) | (k < 64),
+    "per_head_window": lambda b, h, q, k: (q >= k) & (q - k < 32 * (h + 1)),
+    "document": lambda b, h, q, k: (q >= k) & ((q // 150) == (k // 150)),
+    "shifted_causal": lambda b, h, q, k: q - 128 >= k,          # rows 0..127 have no key at all
+}
+
+
+def _keep(mask_mod, B, H, Sq, Skv):
+    return mask_mod(torch.arange(B).view(B, 1, 1, 1), torch.arange(H).view(1, H, 1, 1), torch.arange(Sq).view(1, 1, Sq, 1),
+                    torch.arange(Skv).view(1, 1, 1, Skv)).expand(B, H, Sq, Skv)
+
+
+@pytest.mark.parametrize("name", sorted(MASKS))
+@pytest.mark.parametrize("family,D,S", [("softmax", 128, 300), ("softmax", 64, 512), ("sigmoid", 128, 260)])
+def test_engine_backward_with_arbitrary_mask_mod(name, family, D, S):
+    """Gradients under any mask_mod (the reference generates the mask_mod's code into its backward kernels,
+    attn_tl.py:212-525): the element-wise keep mask in both orientations.  Oracle: autograd over
+    oracle.masked_attention in fp64."""
+    from attn_engine import AttentionEngine
+    from core import CustomIO, meta_tensor
+    B, H = 2, 3
+    mask_mod = MASKS[name]
+    scale = 1 / math.sqrt(D)
+    if family == "softmax":
+        meta = tuple(meta_tensor(B, H, S, D, dtype=torch.bfloat16) for _ in range(3))
+        mod = AttentionEngine(meta, CustomIO(), lambda s_, io, b, h, q, k: s_ * scale, mask_mod, specs.OnlineSoftmax())
+    else:
+        mod = specs.sigmoid_attention(B, H, S, D, D, scale=scale, const_bias=-math.log(S), form="exp", mask_mod=mask_mod)
+    assert mod.mask_kind in ("other", "other_bh")
+    g = torch.Generator().manual_seed(S + D)
+    q, k, v, dout = (torch.randn(B, S, H, D, generator=g).bfloat16() for _ in range(4))
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = mod(qc, kc, vc)
+    o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    keep = _keep(mask_mod, B, H, S, S)
+    ref = oracle.attention_grads(oracle.masked_attention, q, k, v, dout, keep=keep, family=family, softmax_scale=scale, bias=-math.log(S))
+    _check((qc.grad, kc.grad, vc.grad), ref, f"engine {family} {name}")
+    # what is masked gets exactly no gradient: keys no query may see
+    unseen = ~keep.any(dim=2)                                   # [B, H, Skv]
+    if unseen.any():
+        idx = unseen.permute(0, 2, 1).cuda()                    # [B, Skv, H]
+        assert torch.count_nonzero(kc.grad[idx]) == 0 and torch.count_nonzero(vc.grad[idx]) == 0
+
+
+def test_masked_backward_through_the_c_abi_matches_causal():
+    """A lower-triangular keep mask through elem_mask / elem_mask_t gives the gradients of the causal flag (bit for bit:
+    the same tiles, the same masked elements), grouped-query heads included."""
+    hb = _hb()
+    B, H, Hkv, S, D = 1, 4, 2, 257, 128
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(B, S, H, D, generator=g).bfloat16().cuda()
+    k = torch.randn(B, S, Hkv, D, generator=g).bfloat16().cuda()
+    v = torch.randn(B, S, Hkv, D, generator=g).bfloat16().cuda()
+    dout = torch.randn(B, S, H, D, generator=g).bfloat16().cuda()
+    lse = torch.empty(B, H, S, device="cuda")
+    o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=D ** -0.5, row_scale=lse)
+    ref = hb.attn_bwd(q, k, v, o, dout, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=D ** -0.5)
+    sp = (S + 3) // 4 * 4
+    buf = torch.zeros(1, 1, S, sp, dtype=torch.uint8, device="cuda")
+    buf[0, 0, :, :S] = torch.tril(torch.ones(S, S, dtype=torch.uint8, device="cuda"))
+    buf_t = torch.zeros(1, 1, S, sp, dtype=torch.uint8, device="cuda")
+    buf_t[0, 0, :, :S] = torch.triu(torch.ones(S, S, dtype=torch.uint8, device="cuda"))
+    got = hb.attn_bwd(q, k, v, o, dout, lse, family=hb.MA_ATTN_SOFTMAX, causal=False, scale=D ** -0.5,
+                      elem_mask=buf[..., :S], elem_mask_t=buf_t[..., :S])
+    torch.cuda.synchronize()
+    for a, b_ in zip(got, ref):
+        assert torch.equal(a, b_)
+    with pytest.raises(hb.MetaAttentionError):
+        hb.attn_bwd(q, k, v, o, dout, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=D ** -0.5,
+                    elem_mask=buf[..., :S], elem_mask_t=buf_t[..., :S])
