@@ -104,8 +104,8 @@ class _Attention(torch.autograd.Function):
         eng = ctx.engine
         masks = {}
         if eng.mask_kind.startswith("other"):
-            masks = dict(zip(("elem_mask", "elem_mask_t"), eng._dense_mask(q.shape[0], q.shape[2], q.shape[1], k.shape[1], q.device,
-                                                                           transposed=True)))
+            masks = dict(zip(("elem_mask", "elem_mask_t", "kv_block_mask", "q_block_mask"),
+                             eng._dense_mask(q.shape[0], q.shape[2], q.shape[1], k.shape[1], q.device, transposed=True)))
         dq, dk, dv = attn_bwd(q, k, v, out, dout, rest[0] if rest else None, family=ctx.fam_code,
                               causal=eng.mask_kind == "causal", scale=form.scale, bias=form.bias, bias_tensor=ctx.bias_t, **masks)
         return None, None, None, None, dq, dk, dv
@@ -277,7 +277,8 @@ class AttentionEngine:
         """(element-wise keep mask uint8 [1|B, 1|H, Sq, Skv] with 4-byte aligned rows, block mask uint8
         [1|B, 1|H, ceil(Sq/128), ceil(Skv/32)]: a block is kept when any of its elements is) for the mask_mod, built
         once per shape on the device.  transposed=True: (the keep mask, its transpose [.., Skv, Sq] with 4-byte aligned
-        rows) for the backward kernels; the transpose is built on first use."""
+        rows, the block mask, the block mask of the transpose [.., ceil(Skv/128), ceil(Sq/32)]) for the backward kernels;
+        the transposed pair is built on first use."""
         from core.transform.core import create_mask
         key = (B, H, Sq, Skv, str(device))
         if self._mask_tensors is None or self._mask_tensors[0] != key:
@@ -295,8 +296,12 @@ class AttentionEngine:
                 elem = self._mask_tensors[1]
                 buf_t = torch.zeros(elem.shape[0], elem.shape[1], Skv, (Sq + 3) // 4 * 4, dtype=torch.uint8, device=device)
                 buf_t[..., :Sq] = elem.transpose(2, 3)
-                self._mask_tensors[3] = buf_t[..., :Sq]
-            return self._mask_tensors[1], self._mask_tensors[3]
+                skp, sqp = (Skv + 127) // 128 * 128, (Sq + 31) // 32 * 32
+                pad = torch.zeros(elem.shape[0], elem.shape[1], skp, sqp, dtype=torch.bool, device=device)
+                pad[:, :, :Skv, :Sq] = elem.transpose(2, 3) != 0
+                blocks_t = pad.view(elem.shape[0], elem.shape[1], skp // 128, 128, sqp // 32, 32).any(dim=5).any(dim=3)
+                self._mask_tensors[3] = (buf_t[..., :Sq], blocks_t.to(torch.uint8).contiguous())
+            return self._mask_tensors[1], self._mask_tensors[3][0], self._mask_tensors[2], self._mask_tensors[3][1]
         return self._mask_tensors[1], self._mask_tensors[2]
 
     # ------------------------------------------------------------------ MLA decode

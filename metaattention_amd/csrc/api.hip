@@ -154,6 +154,10 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
     for (int64_t x : ms)
       if (x % 4 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: elem_mask rows must be 4-byte aligned");
   }
+  if ((p->kv_block_mask != nullptr) != (p->q_block_mask != nullptr))
+    return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: kv_block_mask and q_block_mask go together");
+  if (p->kv_block_mask && !p->elem_mask)
+    return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: block masks come with an element-wise mask");
 
   ma::AttnBwdArgs a{};
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.dout = p->dout; a.dq = p->dq; a.dk = p->dk; a.dv = p->dv;
@@ -171,6 +175,8 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
   a.scale = p->scale; a.bias = p->bias;
   a.elem_mask = p->elem_mask; a.em_sb = p->em_stride_b; a.em_sh = p->em_stride_h; a.em_sq = p->em_stride_q;
   a.elem_mask_t = p->elem_mask_t; a.emt_sb = p->emt_stride_b; a.emt_sh = p->emt_stride_h; a.emt_sk = p->emt_stride_k;
+  a.kv_block_mask = p->kv_block_mask; a.kbm_sb = p->kbm_stride_b; a.kbm_sh = p->kbm_stride_h; a.kbm_sq = p->kbm_stride_q;
+  a.q_block_mask = p->q_block_mask; a.qbm_sb = p->qbm_stride_b; a.qbm_sh = p->qbm_stride_h; a.qbm_sk = p->qbm_stride_k;
   const int rc = ma::attn_bwd_dispatch(a, p->family, p->mask == MA_MASK_CAUSAL, p->dtype == MA_BF16, p->dim_qk, p->dim_v, (hipStream_t)stream);
   if (rc == -2) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: no kernel for family %d, Dqk=%d, Dv=%d", p->family, p->dim_qk, p->dim_v);
   if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_attn_bwd: launch failed: %s", hipGetErrorString(hipGetLastError()));

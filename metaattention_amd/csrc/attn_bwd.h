@@ -20,6 +20,11 @@ struct AttnBwdArgs {
   // for the dk / dv kernel (a lane walks a key's column); rows are 4-byte aligned
   const uint8_t* elem_mask; int64_t em_sb, em_sh, em_sq;
   const uint8_t* elem_mask_t; int64_t emt_sb, emt_sh, emt_sk;
+  // optional tile masks (0 = nothing kept in the tile: skipped), strides in bytes, 0 broadcasts:
+  // kv_block_mask [.., .., ceil(Sq/128), ceil(Skv/32)] for the dq kernel (a workgroup's 128 rows x a 32-key tile),
+  // q_block_mask  [.., .., ceil(Skv/128), ceil(Sq/32)] for the dk / dv kernel (a workgroup's 128 keys x a 32-row tile)
+  const uint8_t* kv_block_mask; int64_t kbm_sb, kbm_sh, kbm_sq;
+  const uint8_t* q_block_mask; int64_t qbm_sb, qbm_sh, qbm_sk;
 };
 
 int attn_bwd_dispatch(const AttnBwdArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);

@@ -229,12 +229,22 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
   // element-wise keep mask of this lane's query row
   const uint8_t* em_row = a.elem_mask ? a.elem_mask + (int64_t)b * a.em_sb + (int64_t)h * a.em_sh + (int64_t)m_ld * a.em_sq : nullptr;
 
-  if (n_tiles > 0) issue_tile(0, 0);
-  for (int jt = 0; jt < n_tiles; jt++) {
-    const int buf = jt & 1, n0 = jt * BN;
+  // tiles in which the mask keeps nothing for this workgroup's rows are never fetched
+  const uint8_t* bm_row = a.kv_block_mask ? a.kv_block_mask + (int64_t)b * a.kbm_sb + (int64_t)h * a.kbm_sh + (int64_t)mb * a.kbm_sq : nullptr;
+  auto next_tile = [&](int jt) {
+    if (bm_row)
+      while (jt < n_tiles && !bm_row[jt]) jt++;
+    return jt;
+  };
+
+  int jt = next_tile(0);
+  if (jt < n_tiles) issue_tile(jt * BN, 0);
+  for (int it = 0; jt < n_tiles; it++) {
+    const int buf = it & 1, n0 = jt * BN;
     wait_dma();
     __syncthreads();
-    if (jt + 1 < n_tiles) issue_tile(n0 + BN, buf ^ 1);
+    jt = next_tile(jt + 1);
+    if (jt < n_tiles) issue_tile(jt * BN, buf ^ 1);
     const uint32_t kbase = lds0 + buf * STAGE, vbase = kbase + KTILE;
 
     const f32x16 s = mm_rows<T, DQK>(kbase, r, g, qf);     // S^T: lane = row m_lane, element jj = key n0 + 8(jj/4) + 4g + jj%4
@@ -346,6 +356,13 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
   const int t_count = (a.Sq + BMT - 1) / BMT - t_first;
   const int n_steps = t_count > 0 ? t_count * a.kv_group : 0;
   const int64_t q_row_bytes = a.qss * 2, do_row_bytes = a.doss * 2;
+  // tiles in which the mask keeps nothing for this workgroup's keys are never fetched
+  const uint8_t* qbm = a.q_block_mask ? a.q_block_mask + (int64_t)b * a.qbm_sb + (int64_t)nb * a.qbm_sk : nullptr;
+  auto next_step = [&](int step) {
+    if (qbm)
+      while (step < n_steps && !qbm[(int64_t)(hk * a.kv_group + step / t_count) * a.qbm_sh + t_first + step % t_count]) step++;
+    return step;
+  };
   auto issue_step = [&](int step, int buf) {
     const int h = hk * a.kv_group + step / t_count, m0 = (t_first + step % t_count) * BMT;
     const char* qb = (const char*)((const T*)a.q + (int64_t)b * a.qsb + (int64_t)h * a.qsh);
@@ -354,13 +371,15 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
     dma_tile<DOROW, 4>(dob, do_row_bytes, m0, a.Sq, lds0 + buf * STAGE + QTILE, wave, lane);
   };
 
-  if (n_steps > 0) issue_step(0, 0);
-  for (int step = 0; step < n_steps; step++) {
-    const int buf = step & 1;
+  int step_next = next_step(0);
+  if (step_next < n_steps) issue_step(step_next, 0);
+  for (int it = 0; step_next < n_steps; it++) {
+    const int buf = it & 1, step = step_next;
     const int h = hk * a.kv_group + step / t_count, m0 = (t_first + step % t_count) * BMT;
     wait_dma();
     __syncthreads();
-    if (step + 1 < n_steps) issue_step(step + 1, buf ^ 1);
+    step_next = next_step(step + 1);
+    if (step_next < n_steps) issue_step(step_next, buf ^ 1);
     // (a wave whose keys all lie behind this tile's rows has nothing to add; it still takes part in the barriers)
     if (CAUSAL && m0 + BMT - 1 < n_wave) continue;
     const uint32_t qbase = lds0 + buf * STAGE, dobase = qbase + QTILE;

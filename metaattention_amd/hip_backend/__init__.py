@@ -72,6 +72,8 @@ class AttnBwdParams(Structure):
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("elem_mask", c_void_p), ("em_stride_b", c_int64), ("em_stride_h", c_int64), ("em_stride_q", c_int64),
         ("elem_mask_t", c_void_p), ("emt_stride_b", c_int64), ("emt_stride_h", c_int64), ("emt_stride_k", c_int64),
+        ("kv_block_mask", c_void_p), ("kbm_stride_b", c_int64), ("kbm_stride_h", c_int64), ("kbm_stride_q", c_int64),
+        ("q_block_mask", c_void_p), ("qbm_stride_b", c_int64), ("qbm_stride_h", c_int64), ("qbm_stride_k", c_int64),
     ]
 
 
@@ -234,12 +236,14 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
 
 
 def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None,
-             elem_mask=None, elem_mask_t=None):
+             elem_mask=None, elem_mask_t=None, kv_block_mask=None, q_block_mask=None):
     """Gradients (dq, dk, dv) of the parallel attention forward on BSHD tensors.  ``o`` and ``lse``
     (fp32 [B,H,Sq]) are the forward pass's output and row scale (softmax only; None otherwise),
     ``dout`` the gradient of ``o``.  ``elem_mask`` (the forward pass's keep mask, [1|B, 1|H, Sq, Skv]) comes with
-    its transpose ``elem_mask_t`` [1|B, 1|H, Skv, Sq]; both with rows at 4-byte aligned addresses."""
-    _require_gpu(q, k, v, o, dout, lse, bias_tensor, elem_mask, elem_mask_t)
+    its transpose ``elem_mask_t`` [1|B, 1|H, Skv, Sq]; both with rows at 4-byte aligned addresses.  Optional tile masks
+    for skipping: ``kv_block_mask`` [1|B, 1|H, ceil(Sq/128), ceil(Skv/32)] and ``q_block_mask`` [1|B, 1|H, ceil(Skv/128),
+    ceil(Sq/32)] (a tile is kept when any of its elements is)."""
+    _require_gpu(q, k, v, o, dout, lse, bias_tensor, elem_mask, elem_mask_t, kv_block_mask, q_block_mask)
     B, Sq, H, Dqk = q.shape
     Skv, Hkv, Dv = k.shape[1], k.shape[2], v.shape[-1]
     assert k.shape == (B, Skv, Hkv, Dqk) and v.shape == (B, Skv, Hkv, Dv) and dout.shape == (B, Sq, H, Dv) and H % Hkv == 0
@@ -270,6 +274,16 @@ def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, 
             assert t.dtype in (torch.bool, torch.uint8) and t.dim() == 4 and t.shape[2:] == (rows, cols) and t.stride(-1) == 1
             assert t.shape[0] in (1, B) and t.shape[1] in (1, H)
             setattr(p, "elem_mask" if pre == "em" else "elem_mask_t", t.data_ptr())
+            setattr(p, f"{pre}_stride_b", t.stride(0) if t.shape[0] > 1 else 0)
+            setattr(p, f"{pre}_stride_h", t.stride(1) if t.shape[1] > 1 else 0)
+            setattr(p, f"{pre}_stride_{last}", t.stride(2))
+    if kv_block_mask is not None or q_block_mask is not None:
+        assert kv_block_mask is not None and q_block_mask is not None, "kv_block_mask and q_block_mask go together"
+        for t, shape, pre, last in ((kv_block_mask, ((Sq + 127) // 128, (Skv + 31) // 32), "kbm", "q"),
+                                    (q_block_mask, ((Skv + 127) // 128, (Sq + 31) // 32), "qbm", "k")):
+            assert t.dtype in (torch.bool, torch.uint8) and t.dim() == 4 and t.shape[2:] == shape and t.stride(-1) == 1
+            assert t.shape[0] in (1, B) and t.shape[1] in (1, H)
+            setattr(p, "kv_block_mask" if pre == "kbm" else "q_block_mask", t.data_ptr())
             setattr(p, f"{pre}_stride_b", t.stride(0) if t.shape[0] > 1 else 0)
             setattr(p, f"{pre}_stride_h", t.stride(1) if t.shape[1] > 1 else 0)
             setattr(p, f"{pre}_stride_{last}", t.stride(2))
