@@ -30,6 +30,7 @@
 //     un-normalised (O = sum_j P_j V_j, r = sum_j |P_j| in fp32) and divided by max(r, 1) once at the
 //     end; the online form of the reference rescales every tile and gives the same value up to rounding.
 #include "attn_fwd.h"
+#include <type_traits>
 
 namespace ma {
 
@@ -431,8 +432,7 @@ static int wide_family(const AttnArgs& a, int family, bool causal, hipStream_t s
 template <typename T>
 static int wide_dims(const AttnArgs& a, int family, bool causal, int dqk, int dv, hipStream_t stream) {
   if (family == WF_RETENTION) {
-    if (dqk == 256 && dv == 512)
-      return causal ? launch_wide<T, 256, 512, WF_RETENTION, true>(a, stream) : launch_wide<T, 256, 512, WF_RETENTION, false>(a, stream);
+    if (dqk == 256 && dv == 512) return retention_pair_fwd_dispatch(a, causal, std::is_same<T, __bf16>::value, stream);   // retention_fwd.hip
     if (dqk == 128 && dv == 128)
       return causal ? launch_wide<T, 128, 128, WF_RETENTION, true>(a, stream) : launch_wide<T, 128, 128, WF_RETENTION, false>(a, stream);
     return -2;
