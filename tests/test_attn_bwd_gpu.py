@@ -238,3 +238,31 @@ def test_backward_tile_skipping_changes_nothing():
         assert torch.equal(a, b_)
     with pytest.raises(hb.MetaAttentionError):
         hb.attn_bwd(q, k, v, o, dout, lse, kv_block_mask=kbm, q_block_mask=qbm, family=hb.MA_ATTN_SOFTMAX, causal=False, scale=D ** -0.5)
+
+
+def test_backward_full_size_properties():
+    """Benchmark shape (B8 H32 S4096 D128, causal): (batch, head) slices against the gradient oracle, the last key's
+    dk / dv come from the last query alone (closed form), and the gradients are linear in dout."""
+    hb = _hb()
+    B, H, S, D = 8, 32, 4096, 128
+    scale = 1 / math.sqrt(D)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q, k, v, dout = (torch.randn(B, S, H, D, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(4))
+    lse = torch.empty(B, H, S, device="cuda")
+    o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale, row_scale=lse)
+    dq, dk, dv = hb.attn_bwd(q, k, v, o, dout, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale)
+    torch.cuda.synchronize()
+    for t in (dq, dk, dv):
+        assert torch.isfinite(t.float()).all()
+    # the last key is seen by the last query only: dv[S-1] = p * dout[S-1], with p = exp(s * scale - lse)
+    s_last = (q[:, -1].float() * k[:, -1].float()).sum(-1) * scale                      # [B, H]
+    p_last = torch.exp(s_last - lse[:, :, -1])
+    torch.testing.assert_close(dv[:, -1].float(), p_last.unsqueeze(-1) * dout[:, -1].float(), rtol=2e-2, atol=2e-2)
+    for b, h in [(0, 0), (7, 31)]:
+        sl = lambda t: t[b:b + 1, :, h:h + 1].cpu()
+        ref = oracle.attention_grads(oracle.softmax_attention, sl(q), sl(k), sl(v), sl(dout), causal=True, softmax_scale=scale)
+        _check((sl(dq), sl(dk), sl(dv)), ref, f"full size slice ({b},{h})")
+    # linearity in dout (exact: a power of two commutes with every rounding on the way)
+    dq2, dk2, dv2 = hb.attn_bwd(q, k, v, o, dout * 2, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale)
+    torch.cuda.synchronize()
+    assert torch.equal(dq2, dq * 2) and torch.equal(dk2, dk * 2) and torch.equal(dv2, dv * 2)
