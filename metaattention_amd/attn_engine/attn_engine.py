@@ -127,6 +127,7 @@ class AttentionEngine:
         self.tl_code = ""     # no source is generated
         self.extern_block_mask = extern_block_mask
         self.kv_block_size = int(infer_mask_block_N)
+        self._infer_blocks = (int(infer_mask_block_M), int(infer_mask_block_N)) if infer_mask else None
         if (use_varlen or extern_block_mask) and (self.kv_block_size < 32 or self.kv_block_size % 32 != 0):
             raise NotImplementedError("kv block masks need a block size that is a multiple of 32 (infer_mask_block_N)")
         if (use_varlen or extern_block_mask) and kv_shared:
@@ -291,6 +292,14 @@ class AttentionEngine:
             pad[:, :, :Sq, :Skv] = dense
             blocks = pad.view(Bm, Hm, sqp // 128, 128, nkp // 32, 32).any(dim=5).any(dim=3).to(torch.uint8).contiguous()
             self._mask_tensors = [key, buf[..., :Skv], blocks, None]
+            if self._infer_blocks is not None:
+                # the attribute the reference keeps for operators whose mask is not the exact causal one
+                # (attn_engine.py:394-397): the mask_mod pooled to infer_mask_block_M x infer_mask_block_N blocks
+                bm_, bn_ = self._infer_blocks
+                qp, kp = (Sq + bm_ - 1) // bm_ * bm_, (Skv + bn_ - 1) // bn_ * bn_
+                padb = torch.zeros(Bm, Hm, qp, kp, dtype=torch.bool, device=device)
+                padb[:, :, :Sq, :Skv] = dense
+                self.block_mask = padb.view(Bm, Hm, qp // bm_, bm_, kp // bn_, bn_).any(dim=5).any(dim=3).to(torch.int8)
         if transposed:
             if self._mask_tensors[3] is None:
                 elem = self._mask_tensors[1]

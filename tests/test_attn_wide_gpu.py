@@ -294,6 +294,9 @@ def test_engine_arbitrary_mask_mod(name, D, S, family):
     o2 = mod(q.cuda(), k.cuda(), v.cuda())          # second call re-uses the cached mask tensors
     torch.cuda.synchronize()
     assert torch.equal(o, o2)
+    # the block mask attribute of the reference (attn_engine.py:394-397), at its default 128 x 128 blocks
+    nb = (S + 127) // 128
+    assert mod.block_mask is not None and mod.block_mask.shape[2:] == (nb, nb) and mod.block_mask.dtype == torch.int8
     bi, hi = torch.arange(B).view(B, 1, 1, 1), torch.arange(H).view(1, H, 1, 1)
     keep = mask_mod(bi, hi, torch.arange(S).view(1, 1, S, 1), torch.arange(S).view(1, 1, 1, S)).expand(B, H, S, S)
     ref = oracle.masked_attention(q, k, v, keep=keep, family=family, softmax_scale=scale, bias=-math.log(S))
