@@ -181,9 +181,25 @@ typedef struct ma_mla_params {
    * holding rows i * page_size .. of batch entry b. */
   const int32_t* kv_seqlens;
   const int32_t* block_table; int64_t block_table_stride; int32_t page_size;
+  /* optional work plan for ragged batches, as written by ma_mla_get_metadata (kv_seqlens is then required and
+   * num_split ignored): tile_scheduler_metadata int32 [num_sm_parts, 8], num_splits int32 [batch + 1], device memory.
+   * Every workgroup then takes the contiguous run of (batch entry, token range) pieces its part of the plan names
+   * instead of one of num_split equal ranges of one batch entry. */
+  const int32_t* tile_scheduler_metadata;
+  const int32_t* num_splits;
+  int32_t num_sm_parts;
 } ma_mla_params;
 
 typedef void* ma_stream_t; /* a hipStream_t */
+
+/* get_mla_metadata of the paged MLA interface (cute_template_kvshared/flash_mla_interface.py:57-72, kernels/
+ * get_mla_metadata.cu:8-75): the number of parts the work of a launch is dealt to (one workgroup of 128 heads per CU),
+ * and the plan itself, written on `stream` into device memory: tile_scheduler_metadata int32 [parts, 8] =
+ * {first batch, first token, last batch, end token, split index of the first piece, 0, 0, 0} per part and num_splits
+ * int32 [batch + 1], the number of pieces of the batch entries before each.  kv_seqlens is device memory, int32 [batch]. */
+int ma_mla_num_sm_parts(int heads_q);
+int ma_mla_get_metadata(const int32_t* kv_seqlens, int batch, int num_sm_parts, int32_t* tile_scheduler_metadata, int32_t* num_splits,
+                        ma_stream_t stream);
 
 int ma_version(void);
 const char* ma_last_error(void);

@@ -248,11 +248,34 @@ int ma_mla_choose_split(const ma_mla_params* p) {
 
 static int mla_split_of(const ma_mla_params* p) { return p->num_split > 0 ? p->num_split : ma_mla_choose_split(p); }
 
+// One workgroup serves 128 heads and owns a CU: the plan has as many parts as CUs per block of heads
+// (flash_api.cpp:39 with this library's block of heads).
+int ma_mla_num_sm_parts(int heads_q) {
+  if (heads_q <= 0) return 0;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  const int parts = cus / ((heads_q + 127) / 128);
+  return parts < 1 ? 1 : parts;
+}
+
+int ma_mla_get_metadata(const int32_t* kv_seqlens, int batch, int num_sm_parts, int32_t* tile_scheduler_metadata, int32_t* num_splits,
+                        ma_stream_t stream) {
+  if (!kv_seqlens || !tile_scheduler_metadata || !num_splits) return fail(MA_ERR_INVALID_ARG, "ma_mla_get_metadata: NULL argument");
+  if (batch <= 0 || num_sm_parts <= 0) return fail(MA_ERR_INVALID_ARG, "ma_mla_get_metadata: batch and num_sm_parts must be positive");
+  // blocks of 64 tokens and 5 blocks of fixed cost per batch entry, as kernels/config.h:6,11
+  if (ma::mla_plan_dispatch(kv_seqlens, batch, num_sm_parts, 64, 5, tile_scheduler_metadata, num_splits, (hipStream_t)stream) != 0)
+    return fail(MA_ERR_LAUNCH, "ma_mla_get_metadata: launch failed: %s", hipGetErrorString(hipGetLastError()));
+  return MA_OK;
+}
+
 size_t ma_mla_workspace_bytes(const ma_mla_params* p) {
   if (!p) return 0;
+  const size_t per_slot = (size_t)p->heads_q * ((size_t)p->dim * 2 + sizeof(float));   // 2-byte partial outputs + fp32 lse
+  if (p->tile_scheduler_metadata) return ((size_t)p->batch + (size_t)p->num_sm_parts) * per_slot;   // at most one piece more per part
   const int ns = mla_split_of(p);
   if (ns <= 1) return 0;
-  return (size_t)p->batch * ns * p->heads_q * ((size_t)p->dim * 2 + sizeof(float));   // 2-byte partial outputs + fp32 lse
+  return (size_t)p->batch * ns * per_slot;
 }
 
 int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
@@ -270,7 +293,14 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
   const uintptr_t ptrs[] = {(uintptr_t)p->q, (uintptr_t)p->q_pe, (uintptr_t)p->kv, (uintptr_t)p->k_pe, (uintptr_t)p->o};
   for (uintptr_t x : ptrs)
     if (x % 16 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: tensors must be 16-byte aligned");
-  const int ns = mla_split_of(p);
+  const bool planned = p->tile_scheduler_metadata != nullptr;
+  if (planned) {
+    if (!p->num_splits || !p->kv_seqlens || p->num_sm_parts <= 0)
+      return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: a work plan needs num_splits, kv_seqlens and num_sm_parts > 0");
+    // (a batch entry is cut into at most one piece per part, and the combine kernel merges at most 64)
+    if (p->num_sm_parts > 65535) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: num_sm_parts > 65535");
+  }
+  const int ns = planned ? 1 : mla_split_of(p);
   const int tiles = (p->seqlen_kv + 63) / 64;
   if (ns > tiles || ns > 64) return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: num_split %d exceeds min(kv tiles=%d, 64)", ns, tiles);
   ma::MlaArgs a{};
@@ -290,7 +320,15 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
     a.block_table = p->block_table; a.bt_stride = p->block_table_stride; a.page_size = p->page_size;
     a.kvsb = 0; a.kpsb = 0;
   }
-  if (ns > 1) {
+  if (planned) {
+    const size_t need = ma_mla_workspace_bytes(p);
+    if (!p->workspace || p->workspace_bytes < need)
+      return fail(MA_ERR_WORKSPACE, "ma_mla_decode: workspace of %zu bytes needed for the work plan, got %zu", need, p->workspace_bytes);
+    if ((uintptr_t)p->workspace % 16 != 0) return fail(MA_ERR_WORKSPACE, "ma_mla_decode: workspace must be 16-byte aligned");
+    a.plan_meta = p->tile_scheduler_metadata; a.plan_splits = p->num_splits; a.plan_parts = p->num_sm_parts;
+    a.o_part = p->workspace;
+    a.lse_part = (float*)((char*)p->workspace + ((size_t)p->batch + (size_t)p->num_sm_parts) * p->heads_q * p->dim * 2);
+  } else if (ns > 1) {
     const size_t need = ma_mla_workspace_bytes(p);
     if (!p->workspace || p->workspace_bytes < need)
       return fail(MA_ERR_WORKSPACE, "ma_mla_decode: workspace of %zu bytes needed for %d splits, got %zu", need, ns, p->workspace_bytes);

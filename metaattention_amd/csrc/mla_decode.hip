@@ -50,7 +50,10 @@ __device__ __forceinline__ int kv_flip(int row) { return (row >> 3) & 1; }
 __device__ __forceinline__ int swz_pe(int row) { return (row >> 1) & 7; }
 }  // namespace
 
-template <typename T>
+// PLANNED: the workgroup does not own one (batch, kv split) but the contiguous run of work that the plan gives
+// its part (plan_part of the kernel below the split kernel): a sequence of pieces (batch entry, token range, split
+// index), each handled like one (batch, split) of the unplanned launch.
+template <typename T, bool PLANNED>
 __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) {
   using E = Elem<T>;
   using x8 = typename E::x8;
@@ -69,30 +72,28 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
   const bool late = wave >= 4;               // head groups 2 and 3 run half a sub-tile behind (see the main loop)
   const int r = lane & 31, g = lane >> 5;
   const int hblk = blockIdx.x % a.head_blocks, bs = blockIdx.x / a.head_blocks;
-  const int b = bs / a.num_split, split = bs % a.num_split;
   const int head = hblk * HB + hg * 32 + r;
   const int head_ld = min(head, a.Hq - 1);
-
-  const int n_begin = split * a.split_len;
-  const int skv = a.kv_lens ? min(a.Skv, max(a.kv_lens[b], 0)) : a.Skv;   // this batch entry's cache length
-  const int n_end = min(n_begin + a.split_len, skv);
-  const int n_tiles = n_end > n_begin ? (n_end - n_begin + BN - 1) / BN : 0;
-
-  // ---- Q fragments of this wave's half of the contraction: B operand (lane: head r, k = 8g .. 8g+7 of a slice)
-  x8 qf[NSL];
-  {
-    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)head_ld * a.qsh + 8 * g + hf * (NSL * 16);
-    const T* qpe = (const T*)a.q_pe + (int64_t)b * a.qpsb + (int64_t)head_ld * a.qpsh + 8 * g;
-#pragma unroll
-    for (int sl = 0; sl < NSL; sl++) {
-      const T* src = (hf == 1 && sl >= NLAT1) ? qpe + 16 * (sl - NLAT1) : qp + 16 * sl;
-      qf[sl] = *(const x8*)src;
-    }
-  }
-
-  const char* kvb = (const char*)a.kv + (int64_t)b * a.kvsb * 2;
-  const char* peb = (const char*)a.k_pe + (int64_t)b * a.kpsb * 2;
   const int64_t kv_row_bytes = a.kvss * 2, pe_row_bytes = a.kpss * 2;
+
+  // ---- the pieces of this workgroup: one (batch, split) of the uniform launch, or the run its part of the plan names
+  //      (tile_scheduler_metadata[part] = {first batch, its first token, last batch, its end token, split index of the
+  //      first piece}; a later piece of the run starts a batch entry: token 0, split index 0)
+  int b_first, b_last, first_token = 0, last_end = 0, first_split = 0;
+  if constexpr (PLANNED) {
+    const int32_t* md = a.plan_meta + (int64_t)bs * 8;
+    b_first = md[0]; first_token = md[1]; b_last = md[2]; last_end = md[3]; first_split = md[4];
+    if (b_first >= a.B) return;   // a part the plan left without work
+  } else {
+    b_first = b_last = bs / a.num_split;
+  }
+  // per piece
+  int b = 0, split = 0, n_begin = 0, skv = 0, n_end = 0, n_tiles = 0;
+  bool direct = true;          // the piece is its batch entry's only one: it writes the final output
+  int64_t slot = 0;            // else: its slot among the partial results
+  const char* kvb = nullptr;
+  const char* peb = nullptr;
+  x8 qf[NSL];   // Q fragments of this wave's half of the contraction: B operand (lane: head r, k = 8g .. 8g+7 of a slice)
 
   // ---- DMA.  Wave w streams latent rows 4w..4w+3 of a sub-tile, one instruction per row (64 lanes x 16 B =
   //      the 1 KB row; lane i fetches the chunk that belongs at physical chunk i); waves 0..3 also fetch 8
@@ -133,16 +134,9 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
   const uint32_t x_mine = lds_x + wave * XCHG + lane * 16, x_other = lds_x + (wave ^ 1) * XCHG + lane * 16;
 
   f32x16 o[DBH];
-#pragma unroll
-  for (int i = 0; i < DBH; i++)
-#pragma unroll
-    for (int j = 0; j < 16; j++) o[i][j] = 0.f;
   const float c_scale = a.scale * kLog2e;
   float row_ref = -1e30f, row_sum = 0.f;
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-
-  if (n_tiles > 0) issue_tile(0);
-  if (n_tiles > 1) issue_tile(1);
 
   f32x16 sc;   // this wave's half scores, then the full scores, of the sub-tile it is working on
 
@@ -263,6 +257,45 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
       wait_dma();
     }
   };
+  for (b = b_first; b <= b_last; b++) {
+  // ---- this piece
+  if constexpr (PLANNED) {
+    skv = min(a.Skv, max(a.kv_lens[b], 0));
+    n_begin = b == b_first ? first_token : 0;
+    n_end = min(b == b_last ? last_end : skv, skv);
+    split = b == b_first ? first_split : 0;
+    const int first_slot = a.plan_splits[b];
+    direct = a.plan_splits[b + 1] - first_slot == 1;
+    slot = first_slot + split;
+  } else {
+    split = bs % a.num_split;
+    n_begin = split * a.split_len;
+    skv = a.kv_lens ? min(a.Skv, max(a.kv_lens[b], 0)) : a.Skv;   // this batch entry's cache length
+    n_end = min(n_begin + a.split_len, skv);
+    direct = a.num_split == 1;
+    slot = (int64_t)b * a.num_split + split;
+  }
+  n_tiles = n_end > n_begin ? (n_end - n_begin + BN - 1) / BN : 0;
+  kvb = (const char*)a.kv + (int64_t)b * a.kvsb * 2;
+  peb = (const char*)a.k_pe + (int64_t)b * a.kpsb * 2;
+  {
+    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)head_ld * a.qsh + 8 * g + hf * (NSL * 16);
+    const T* qpe = (const T*)a.q_pe + (int64_t)b * a.qpsb + (int64_t)head_ld * a.qpsh + 8 * g;
+#pragma unroll
+    for (int sl = 0; sl < NSL; sl++) {
+      const T* src = (hf == 1 && sl >= NLAT1) ? qpe + 16 * (sl - NLAT1) : qp + 16 * sl;
+      qf[sl] = *(const x8*)src;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < DBH; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) o[i][j] = 0.f;
+  row_ref = -1e30f;
+  row_sum = 0.f;
+  if (n_tiles > 0) issue_tile(0);
+  if (n_tiles > 1) issue_tile(1);
+
   if (late) {
     wait_tile(0);
     __syncthreads();
@@ -302,8 +335,8 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
         for (int i = 0; i < 4; i++) w[i] = (T)(o[db][4 * q4 + i] * inv);
         lds_write<x4>(sb + r * SROW + (((4 * db + q4) ^ (r & 31)) << 4) + 8 * g, w);
       }
-    T* obase = a.num_split == 1 ? (T*)a.o + (int64_t)b * a.osb : (T*)a.o_part + ((int64_t)b * a.num_split + split) * a.Hq * D;
-    const int64_t ostride = a.num_split == 1 ? a.osh : D;
+    T* obase = direct ? (T*)a.o + (int64_t)b * a.osb : (T*)a.o_part + slot * a.Hq * D;
+    const int64_t ostride = direct ? a.osh : D;
     const int head0 = hblk * HB + hg * 32;
 #pragma unroll
     for (int it = 0; it < 32 * (SROW / 16) / 64; it++) {
@@ -313,12 +346,14 @@ __global__ __launch_bounds__(64 * NW, 2) void mla_split_kernel(const MlaArgs a) 
     }
   }
   if (head < a.Hq && hf == 0 && g == 0) {
-    if (a.num_split == 1) {
+    if (direct) {
       if (a.lse) a.lse[(int64_t)b * a.Hq + head] = lse2 * kLn2;
     } else {
-      a.lse_part[((int64_t)b * a.num_split + split) * a.Hq + head] = lse2;
+      a.lse_part[slot * a.Hq + head] = lse2;
     }
   }
+  if (PLANNED && b < b_last) __syncthreads();   // the staged output has left the stages: the next piece may fill them
+  }   // pieces
 }
 
 // Four (batch, head) pairs per workgroup: 64 threads x 8 output columns each.
@@ -329,9 +364,42 @@ __global__ __launch_bounds__(256) void mla_combine_kernel(const MlaArgs a) {
   const int64_t bh = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (bh >= (int64_t)a.B * a.Hq) return;
   const int b = (int)(bh / a.Hq), head = (int)(bh % a.Hq);
-  const int ns = a.num_split;
-  // lane s of the wave holds the log-sum-exp of split s (at most 64 splits): one load, wave reductions
-  const float* lp = a.lse_part + (int64_t)b * ns * a.Hq + head;
+  // the partial results of this batch entry: num_split slots from b * num_split on, or what the plan says (an entry with
+  // a single piece has written its output itself)
+  int ns = a.num_split;
+  int64_t first = (int64_t)b * ns;
+  if (a.plan_splits) {
+    first = a.plan_splits[b];
+    ns = a.plan_splits[b + 1] - (int)first;
+    if (ns <= 1) return;
+  }
+  const float* lp = a.lse_part + first * a.Hq + head;
+  if (ns > 64) {
+    // (only a plan can cut a batch entry into this many pieces: one very long sequence on many parts)
+    float mx = -INFINITY;
+    for (int s2 = tid; s2 < ns; s2 += 64) mx = fmaxf(mx, lp[(int64_t)s2 * a.Hq]);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+    float sum = 0.f;
+    for (int s2 = tid; s2 < ns; s2 += 64) sum += fast_exp2(lp[(int64_t)s2 * a.Hq] - mx);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, 64);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const T* pp = (const T*)a.o_part + (first * a.Hq + head) * D + tid * 8;
+    for (int s2 = 0; s2 < ns; s2++) {
+      const float w = fast_exp2(lp[(int64_t)s2 * a.Hq] - mx) / sum;
+      const x8 v = *(const x8*)(pp + (int64_t)s2 * a.Hq * D);
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc[i] += (float)v[i] * w;
+    }
+    x8 w;
+#pragma unroll
+    for (int i = 0; i < 8; i++) w[i] = (T)acc[i];
+    *(x8*)((T*)a.o + (int64_t)b * a.osb + (int64_t)head * a.osh + tid * 8) = w;
+    if (a.lse && tid == 0) a.lse[(int64_t)b * a.Hq + head] = (mx + fast_log2(sum)) * kLn2;
+    return;
+  }
+  // lane s of the wave holds the log-sum-exp of split s (at most 64 splits here): one load, wave reductions
   const float my = tid < ns ? lp[(int64_t)tid * a.Hq] : -INFINITY;
   float mx = my;
 #pragma unroll
@@ -342,7 +410,7 @@ __global__ __launch_bounds__(256) void mla_combine_kernel(const MlaArgs a) {
   for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, 64);
   const float wgt = e / sum;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const T* pp = (const T*)a.o_part + ((int64_t)b * ns * a.Hq + head) * D + tid * 8;
+  const T* pp = (const T*)a.o_part + (first * a.Hq + head) * D + tid * 8;
   int s0 = 0;
   for (; s0 + 4 <= ns; s0 += 4) {   // four independent loads in flight
     x8 v[4];
@@ -368,17 +436,74 @@ __global__ __launch_bounds__(256) void mla_combine_kernel(const MlaArgs a) {
   if (a.lse && tid == 0) a.lse[(int64_t)b * a.Hq + head] = (mx + fast_log2(sum)) * kLn2;
 }
 
+// The work plan of get_mla_metadata.cu:8-75, one lane: cache blocks of block_n tokens plus a fixed overhead per batch
+// entry are dealt to `parts` workgroups in order, each taking about total / parts (+ overhead); a batch entry cut by a
+// part boundary gets one more split.  meta[p] = {first batch, first token, last batch, end token, split index of the
+// first piece, 0, 0, 0}; splits[b] = number of pieces of the batch entries before b.
+__global__ __launch_bounds__(64) void mla_plan_kernel(const int32_t* seqlens, int batch, int parts, int block_n, int overhead,
+                                                      int32_t* meta, int32_t* splits) {
+  if (threadIdx.x != 0) return;
+  int total = 0;
+  for (int i = 0; i < batch; i++) total += (max(seqlens[i], 0) + block_n - 1) / block_n + overhead;
+  const int payload = max((total + parts - 1) / parts + overhead, 2 * overhead);
+  int now_idx = 0, now_block = 0, now_split = 0, cum = 0;
+  splits[0] = 0;
+  for (int p = 0; p < parts; p++) {
+    int32_t* m = meta + (int64_t)p * 8;
+    m[0] = now_idx;
+    m[1] = now_block * block_n;
+    m[4] = now_split;
+    int remain = payload;
+    while (now_idx < batch) {
+      const int blocks = (max(seqlens[now_idx], 0) + block_n - 1) / block_n;
+      const int left = blocks - now_block;
+      if (remain >= left + overhead) {
+        cum += now_split + 1;
+        splits[now_idx + 1] = cum;
+        remain -= left + overhead;
+        now_idx++;
+        now_block = 0;
+        now_split = 0;
+      } else {
+        if (remain - overhead > 0) {
+          now_block += remain - overhead;
+          now_split++;
+          remain = 0;
+        }
+        break;
+      }
+    }
+    m[2] = now_block > 0 ? now_idx : now_idx - 1;
+    m[3] = now_block > 0 ? now_block * block_n : (now_idx > 0 ? max(seqlens[now_idx - 1], 0) : 0);
+    m[5] = m[6] = m[7] = 0;
+  }
+}
+
+int mla_plan_dispatch(const int32_t* seqlens, int batch, int parts, int block_n, int overhead_blocks, int32_t* meta, int32_t* splits,
+                      hipStream_t stream) {
+  hipLaunchKernelGGL(mla_plan_kernel, dim3(1), dim3(64), 0, stream, seqlens, batch, parts, block_n, overhead_blocks, meta, splits);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
 template <typename T>
 static int launch_t(const MlaArgs& a, hipStream_t stream) {
   constexpr size_t lds = NSTAGE * (size_t)STAGE + NW * (size_t)XCHG;
-  auto kern = mla_split_kernel<T>;
+  auto kern = mla_split_kernel<T, false>;
+  auto kern_planned = mla_split_kernel<T, true>;
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
+    if (hipFuncSetAttribute((const void*)kern_planned, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
     attr_set = true;
   }
   MlaArgs args = a;
   args.head_blocks = (a.Hq + HB - 1) / HB;
+  if (a.plan_meta) {
+    hipLaunchKernelGGL(kern_planned, dim3((unsigned)(a.plan_parts * args.head_blocks)), dim3(64 * NW), lds, stream, args);
+    if (hipGetLastError() != hipSuccess) return -1;
+    hipLaunchKernelGGL(mla_combine_kernel<T>, dim3((unsigned)(((int64_t)a.B * a.Hq + 3) / 4)), dim3(256), 0, stream, args);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+  }
   const unsigned grid = (unsigned)(a.B * a.num_split * args.head_blocks);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, args);
   if (hipGetLastError() != hipSuccess) return -1;

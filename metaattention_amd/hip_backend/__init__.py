@@ -24,7 +24,7 @@ MA_MASK_NONE, MA_MASK_CAUSAL = 0, 1
 EXPORTED_SYMBOLS = (
     "ma_version", "ma_last_error", "ma_attn_workspace_bytes", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes", "ma_attn_bwd",
     "ma_linear_workspace_bytes", "ma_linear_fwd",
-    "ma_mla_choose_split", "ma_mla_workspace_bytes", "ma_mla_decode",
+    "ma_mla_choose_split", "ma_mla_workspace_bytes", "ma_mla_decode", "ma_mla_num_sm_parts", "ma_mla_get_metadata",
 )
 
 
@@ -104,6 +104,7 @@ class MlaParams(Structure):
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("kv_seqlens", c_void_p),
         ("block_table", c_void_p), ("block_table_stride", c_int64), ("page_size", c_int32),
+        ("tile_scheduler_metadata", c_void_p), ("num_splits", c_void_p), ("num_sm_parts", c_int32),
     ]
 
 
@@ -138,6 +139,10 @@ def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
     lib.ma_mla_workspace_bytes.argtypes = [POINTER(MlaParams)]
     lib.ma_mla_workspace_bytes.restype = c_size_t
     lib.ma_mla_decode.argtypes = [POINTER(MlaParams), c_void_p]
+    lib.ma_mla_num_sm_parts.argtypes = [c_int]
+    lib.ma_mla_num_sm_parts.restype = c_int
+    lib.ma_mla_get_metadata.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]
+    lib.ma_mla_get_metadata.restype = c_int
     lib.ma_mla_decode.restype = c_int
     _lib = lib
     return lib
@@ -333,15 +338,22 @@ def mla_decode(q, q_pe, kv, k_pe, *, scale: float, num_split: int = 0, out=None,
     return out
 
 
-def get_mla_metadata(cache_seqlens, num_heads_per_head_k: int, num_heads_k: int):
-    """Counterpart of get_mla_metadata (cute_template_kvshared/flash_mla_interface.py:57-72).  The reference plans
-    per-SM work lists there; this library plans its kv splits inside ma_mla_decode from the sizes alone, so the
-    "metadata" is only the plan's summary: an int32 [1, 2] tensor (heads per kv head, kv heads) and an int32
-    [batch + 1] tensor of cumulative split counts (one unit per batch entry; the split count proper is chosen at
-    launch).  Both are accepted and ignored by flash_mla_with_kvcache."""
-    B = cache_seqlens.shape[0]
-    meta = torch.tensor([[num_heads_per_head_k, num_heads_k]], dtype=torch.int32, device=cache_seqlens.device)
-    return meta, torch.arange(B + 1, dtype=torch.int32, device=cache_seqlens.device)
+def get_mla_metadata(cache_seqlens, num_heads_per_head_k: int, num_heads_k: int, num_sm_parts: int = 0):
+    """get_mla_metadata of the paged MLA interface (cute_template_kvshared/flash_mla_interface.py:57-72): the work plan
+    for a ragged batch, computed on the device from cache_seqlens (int32 [B]) by the greedy scheme of
+    kernels/get_mla_metadata.cu:8-75.  Returns (tile_scheduler_metadata int32 [num_sm_parts, 8], num_splits int32 [B + 1]);
+    flash_mla_with_kvcache hands every workgroup the run of (batch entry, token range) pieces its part names.
+    num_sm_parts defaults to one part per CU and block of 128 query heads."""
+    _require_gpu(cache_seqlens)
+    assert num_heads_k == 1, "one latent kv head"
+    lib = load_library()
+    seqlens = cache_seqlens.to(torch.int32).contiguous()
+    B = seqlens.shape[0]
+    parts = int(num_sm_parts) if num_sm_parts else lib.ma_mla_num_sm_parts(int(num_heads_per_head_k))
+    meta = torch.empty(parts, 8, dtype=torch.int32, device=seqlens.device)
+    splits = torch.empty(B + 1, dtype=torch.int32, device=seqlens.device)
+    _check(lib.ma_mla_get_metadata(seqlens.data_ptr(), B, parts, meta.data_ptr(), splits.data_ptr(), _stream()))
+    return meta, splits
 
 
 def flash_mla_with_kvcache(q, k_cache, block_table, cache_seqlens, head_dim_v: int, tile_scheduler_metadata=None, num_splits=None,
@@ -373,6 +385,14 @@ def flash_mla_with_kvcache(q, k_cache, block_table, cache_seqlens, head_dim_v: i
     p.lse, p.scale = lse.data_ptr(), float(scale)
     p.kv_seqlens = seqlens.data_ptr()
     p.block_table, p.block_table_stride, p.page_size = block_table.data_ptr(), block_table.stride(0), page
+    if tile_scheduler_metadata is not None and tile_scheduler_metadata.dim() == 2 and tile_scheduler_metadata.shape[1] == 8:
+        # the plan of get_mla_metadata: every workgroup walks its part's pieces
+        assert num_splits is not None and num_splits.shape == (B + 1,), "num_splits of get_mla_metadata goes with its metadata"
+        assert tile_scheduler_metadata.dtype == torch.int32 and num_splits.dtype == torch.int32
+        assert tile_scheduler_metadata.is_contiguous() and num_splits.is_contiguous()
+        _require_gpu(tile_scheduler_metadata, num_splits)
+        p.tile_scheduler_metadata, p.num_splits = tile_scheduler_metadata.data_ptr(), num_splits.data_ptr()
+        p.num_sm_parts = tile_scheduler_metadata.shape[0]
     lib = load_library()
     need = lib.ma_mla_workspace_bytes(ctypes.byref(p))
     if need:

@@ -30,6 +30,9 @@ mla_decode             SDPA with K=concat(kv,k_pe), V=kv; split-KV invariance
 sparse_decode_attention  dense attention over the gathered kept keys only
 paged_mla_decode       mla_decode on the contiguous cache (identity table); invariance
                        to a permutation of the page pool
+mla_work_plan          hand-computed small plans; invariants on random ragged batches:
+                       the pieces tile every batch entry exactly once in order, piece
+                       counts equal num_splits, no part exceeds its payload
 masked_attention       SDPA with a boolean attn_mask (fp64); tril keep mask ==
                        softmax_attention(causal); a block mask == attention over
                        the gathered kept keys of each query block; rows without
@@ -64,5 +67,6 @@ from .linear_ref import (  # noqa: F401
     simple_gla_recurrence,
     linear_attention_grads,
 )
+from .mla_plan_ref import mla_work_plan, plan_pieces  # noqa: F401
 from .compare import assert_close, mismatch_report  # noqa: F401
 from . import inputs  # noqa: F401

@@ -134,3 +134,61 @@ def test_engine_paged_mla_backend():
     ref, lse_ref = oracle.mla_decode(q[..., :512], q[..., 512:], rows[..., :512], rows[..., 512:], return_lse=True)
     oracle.assert_close(out.float().cpu(), ref, rtol=1e-2, atol=2e-2)
     torch.testing.assert_close(lse.cpu()[:, :, 0], lse_ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_mla_plan_kernel_matches_the_oracle(seed):
+    """get_mla_metadata (cute_template_kvshared/kernels/get_mla_metadata.cu:8-75) is integer work: bit-exact."""
+    hb = _hb()
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    for _ in range(12):
+        B = int(rng.integers(1, 70))
+        lens = rng.integers(0, 9000, size=B).astype(np.int32)
+        if rng.random() < 0.3:
+            lens[:] = int(rng.integers(1, 5000))
+        parts = int(rng.choice([1, 2, 7, 64, 128, 256, 300]))
+        meta, splits = hb.get_mla_metadata(torch.from_numpy(lens).cuda(), 128, 1, num_sm_parts=parts)
+        torch.cuda.synchronize()
+        ref_meta, ref_splits = oracle.mla_work_plan(lens, parts)
+        assert meta.shape == (parts, 8) and np.array_equal(meta.cpu().numpy(), ref_meta), (B, parts, lens.tolist())
+        assert np.array_equal(splits.cpu().numpy(), ref_splits)
+    assert hb.get_mla_metadata(torch.ones(3, dtype=torch.int32, device="cuda"), 128, 1)[0].shape[0] == hb.load_library().ma_mla_num_sm_parts(128)
+
+
+@pytest.mark.parametrize("B,Hq,parts,maxlen", [(24, 128, 0, 4096), (5, 128, 7, 3000), (3, 64, 256, 700), (1, 128, 256, 32768)])
+def test_planned_paged_mla_decode(B, Hq, parts, maxlen):
+    """Ragged batches through the work plan: every workgroup walks the pieces of its part (batch entries cut at part
+    boundaries are merged by the combine kernel; the last case cuts one long sequence into more than 64 pieces).  Same
+    results as the paged oracle, and as the launch without a plan up to the rounding of the partial outputs."""
+    hb = _hb()
+    page = 64
+    g = torch.Generator().manual_seed(B + maxlen)
+    pages_per_seq = (maxlen + page - 1) // page
+    npg = B * pages_per_seq + 2
+    q = torch.randn(B, 1, Hq, 576, generator=g).bfloat16()
+    cache = torch.randn(npg, page, 1, 576, generator=g).bfloat16()
+    table = torch.randperm(npg, generator=g)[:B * pages_per_seq].to(torch.int32).view(B, pages_per_seq)
+    lens = torch.randint(1, maxlen + 1, (B,), generator=g, dtype=torch.int32)
+    lens[0] = maxlen
+    if B > 2:
+        lens[1] = 0            # an empty cache entry: zeros, lse = -inf
+        lens[2] = 1
+    meta, splits = hb.get_mla_metadata(lens.cuda(), Hq, 1, num_sm_parts=parts)
+    print(f"planned mla B{B} Hq{Hq} parts{meta.shape[0]} pieces {int(splits[-1])} lens {lens.tolist()[:8]}..", flush=True)
+    out, lse = hb.flash_mla_with_kvcache(q.cuda(), cache.cuda(), table.cuda(), lens.cuda(), 512, meta, splits)
+    out_u, lse_u = hb.flash_mla_with_kvcache(q.cuda(), cache.cuda(), table.cuda(), lens.cuda(), 512)
+    torch.cuda.synchronize()
+    if B == 1:
+        assert int(splits[-1]) > 64
+    check = list(range(B)) if B <= 6 else [0, 1, 2, 3, B - 1]
+    for b in check:
+        if int(lens[b]) == 0:
+            assert torch.count_nonzero(out[b]) == 0 and torch.isinf(lse[b]).all() and (lse[b] < 0).all()
+            continue
+        ref, lse_ref = oracle.paged_mla_decode(q[b:b + 1], cache, table[b:b + 1], lens[b:b + 1])
+        oracle.assert_close(out[b:b + 1].float().cpu(), ref, rtol=1e-2, atol=2e-2)
+        torch.testing.assert_close(lse[b:b + 1].cpu(), lse_ref, rtol=1e-4, atol=1e-4)
+    keep = lens > 0
+    torch.testing.assert_close(out[keep.cuda()].float(), out_u[keep.cuda()].float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(lse[keep.cuda()], lse_u[keep.cuda()], rtol=1e-4, atol=1e-4)

@@ -3,6 +3,8 @@ formula: library routines, closed forms, brute-force loops, or an
 algebraically different evaluation of the same operator."""
 import math
 
+import numpy as np
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -359,3 +361,37 @@ def test_masked_attention_against_sdpa_and_special_cases():
                 if keep[0, 0, i, j]:
                     acc += fn(0.5 * float(q[0, i, 0] @ k[0, j, 0])) * v[0, j, 0]
             torch.testing.assert_close(got[0, i, 0], acc)
+
+
+def test_mla_work_plan_small_cases_and_invariants():
+    # two entries of 3 and 1 blocks on two parts: total = (3+5) + (1+5) = 14, payload = max(7 + 5, 10) = 12;
+    # part 0 takes entry 0 whole (8) and has 4 left, not enough for entry 1 (6) nor for one block beside the overhead
+    meta, splits = oracle.mla_work_plan([192, 64], parts=2)
+    assert meta[:, :5].tolist() == [[0, 0, 0, 192, 0], [1, 0, 1, 64, 0]] and splits.tolist() == [0, 1, 2]
+    # one entry of 40 blocks on 4 parts: payload = max(ceil(45/4) + 5, 10) = 17 -> pieces of 12 blocks, the last of 4
+    meta, splits = oracle.mla_work_plan([40 * 64], parts=4)
+    assert meta[:, :5].tolist() == [[0, 0, 0, 768, 0], [0, 768, 0, 1536, 1], [0, 1536, 0, 2304, 2], [0, 2304, 0, 2560, 3]]
+    assert splits.tolist() == [0, 4]
+    # more parts than work: the surplus parts start at batch == B and are empty
+    meta, splits = oracle.mla_work_plan([64], parts=3)
+    assert meta[0, :5].tolist() == [0, 0, 0, 64, 0] and meta[1, 0] == 1 and meta[2, 0] == 1 and splits.tolist() == [0, 1]
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        B = int(rng.integers(1, 40))
+        lens = rng.integers(0, 5000, size=B)
+        parts = int(rng.integers(1, 300))
+        meta, splits = oracle.mla_work_plan(lens, parts)
+        pieces = oracle.plan_pieces(meta, splits, lens)
+        payload = max(-(-sum(-(-int(x) // 64) + 5 for x in lens) // parts) + 5, 10)
+        cover = {b: [] for b in range(B)}
+        load = {}
+        for p, b, begin, end, sidx in pieces:
+            assert sidx == len(cover[b])                                    # split indices count up per batch entry
+            cover[b].append((begin, end))
+            load[p] = load.get(p, 0) + -(-(end - begin) // 64) + 5
+        for b in range(B):
+            assert cover[b][0][0] == 0 and cover[b][-1][1] == lens[b]       # every token exactly once, in order
+            assert all(a[1] == c[0] for a, c in zip(cover[b], cover[b][1:]))
+            assert all(e > s_ for s_, e in cover[b]) or lens[b] == 0
+            assert splits[b + 1] - splits[b] == len(cover[b])
+        assert all(v <= payload for v in load.values())
