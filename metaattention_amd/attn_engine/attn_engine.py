@@ -89,10 +89,10 @@ class _Attention(torch.autograd.Function):
     (dq, dk, dv) and None for every custom input."""
 
     @staticmethod
-    def forward(ctx, engine, run, fam_code, bias_t, q, k, v):
+    def forward(ctx, engine, run, fam_code, bias_t, call_masks, q, k, v):
         out = run(q, k, v)
         lse = engine.final_rowscales
-        ctx.engine, ctx.fam_code, ctx.bias_t = engine, fam_code, bias_t
+        ctx.engine, ctx.fam_code, ctx.bias_t, ctx.call_masks = engine, fam_code, bias_t, call_masks
         ctx.save_for_backward(q, k, v, out, *([lse] if lse is not None else []))
         return out
 
@@ -102,13 +102,16 @@ class _Attention(torch.autograd.Function):
         q, k, v, out, *rest = ctx.saved_tensors
         form = ctx.engine.score_form
         eng = ctx.engine
-        masks = {}
-        if eng.mask_kind.startswith("other"):
+        masks, causal = {}, eng.mask_kind == "causal"
+        if ctx.call_masks is not None:
+            # a call with an external block mask: the whole mask (the caller's blocks, the mask_mod, causal) as elements
+            masks, causal = ctx.call_masks(), False
+        elif eng.mask_kind.startswith("other"):
             masks = dict(zip(("elem_mask", "elem_mask_t", "kv_block_mask", "q_block_mask"),
                              eng._dense_mask(q.shape[0], q.shape[2], q.shape[1], k.shape[1], q.device, transposed=True)))
         dq, dk, dv = attn_bwd(q, k, v, out, dout, rest[0] if rest else None, family=ctx.fam_code,
-                              causal=eng.mask_kind == "causal", scale=form.scale, bias=form.bias, bias_tensor=ctx.bias_t, **masks)
-        return None, None, None, None, dq, dk, dv
+                              causal=causal, scale=form.scale, bias=form.bias, bias_tensor=ctx.bias_t, **masks)
+        return None, None, None, None, None, dq, dk, dv
 
 
 class AttentionEngine:
@@ -255,10 +258,14 @@ class AttentionEngine:
             return run(q, k, v).squeeze(1)
 
         if any(t.requires_grad for t in (q, k, v)):
-            if self.family == "retention" or prefill_blocks is not None:
+            if self.family == "retention":
                 return _ForwardOnly.apply(run, q, k, v)
             bias_t = given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None
-            return _Attention.apply(self, run, fam_code, bias_t, q, k, v)
+            call_masks = None
+            if prefill_blocks is not None:
+                shape = (q.shape[0], q.shape[2], q.shape[1], k.shape[1], q.device)
+                call_masks = lambda: self._block_mask_backward_masks(prefill_blocks, *shape)
+            return _Attention.apply(self, run, fam_code, bias_t, call_masks, q, k, v)
         return run(q, k, v)
 
     @staticmethod
@@ -273,6 +280,28 @@ class AttentionEngine:
                                       "128 query rows by 32 keys")
         keep = (block_mask != 0).to(torch.uint8)
         return keep.repeat_interleave(Sq // nq // 128, dim=2).repeat_interleave(Skv // nk // 32, dim=3)
+
+    def _block_mask_backward_masks(self, block_mask, B, H, Sq, Skv, device):
+        """The masks the backward kernels take, for a call with an external block mask: the caller's blocks spread to
+        elements and ANDed with the operator's own mask (the mask_mod, or causal), its transpose, and both pooled to the
+        blocks the kernels skip by.  Built per backward call (the block mask is an argument of the call, not of the
+        operator); 2 x batch x heads x Sq x Skv bytes unless the mask broadcasts."""
+        nq, nk = block_mask.shape[2:]
+        elem = (block_mask != 0).repeat_interleave(Sq // nq, dim=2).repeat_interleave(Skv // nk, dim=3)
+        if self.mask_kind == "causal":
+            elem = elem & torch.ones(Sq, Skv, dtype=torch.bool, device=device).tril_()
+        elif self.mask_kind.startswith("other"):
+            elem = elem & (self._dense_mask(B, H, Sq, Skv, device)[0] != 0)
+        Bm, Hm = elem.shape[:2]
+        elem_t = elem.transpose(2, 3)
+
+        def pool(m, r, c):                        # blocks of 128 rows x 32 columns, kept when any element is
+            rp = (r + 127) // 128 * 128
+            m = torch.nn.functional.pad(m, (0, 0, 0, rp - r)) if rp != r else m
+            return m.reshape(Bm, Hm, rp // 128, 128, c // 32, 32).any(dim=5).any(dim=3).to(torch.uint8).contiguous()
+
+        return dict(elem_mask=elem.to(torch.uint8).contiguous(), elem_mask_t=elem_t.to(torch.uint8).contiguous(),
+                    kv_block_mask=pool(elem, Sq, Skv), q_block_mask=pool(elem_t, Skv, Sq))
 
     def _dense_mask(self, B, H, Sq, Skv, device, transposed=False):
         """(element-wise keep mask uint8 [1|B, 1|H, Sq, Skv] with 4-byte aligned rows, block mask uint8

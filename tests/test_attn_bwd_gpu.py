@@ -188,6 +188,43 @@ def test_engine_backward_with_arbitrary_mask_mod(name, family, D, S):
         assert torch.count_nonzero(kc.grad[idx]) == 0 and torch.count_nonzero(vc.grad[idx]) == 0
 
 
+@pytest.mark.parametrize("family,mask,D,S,bq,bk", [
+    ("softmax", "causal", 128, 512, 128, 128), ("softmax", "none", 64, 384, 128, 32), ("softmax", "sliding_window", 128, 512, 128, 64),
+    ("sigmoid", "causal", 128, 512, 256, 128), ("relu", "none", 128, 256, 128, 128)])
+def test_engine_backward_with_external_block_mask(family, mask, D, S, bq, bk):
+    """Gradients of a call that passes block_mask= at prefill shapes (the block-sparse operator of the reference has a
+    forward only, blockattn_tl.py:123-234; here the caller's blocks, spread to elements and ANDed with the operator's
+    mask, drive the same masked backward kernels).  Oracle: autograd over oracle.masked_attention in fp64."""
+    from attn_engine import AttentionEngine
+    from core import CustomIO, meta_tensor
+    B, H = 2, 3
+    scale = 1 / math.sqrt(D)
+    mask_mod = specs.causal_mask if mask == "causal" else MASKS.get(mask)
+    meta = tuple(meta_tensor(B, H, S, D, dtype=torch.bfloat16) for _ in range(3))
+    score_mod = {"softmax": lambda s_, io, b, h, q, k: s_ * scale,
+                 "sigmoid": lambda s_, io, b, h, q, k: 1 / (1 + (-(s_ * scale + (-math.log(S)))).exp()),
+                 "relu": lambda s_, io, b, h, q, k: (s_ * scale).max(0)}[family]
+    mod = AttentionEngine(meta, CustomIO(), score_mod, mask_mod, specs.OnlineSoftmax() if family == "softmax" else specs.OnlineIdentity(),
+                          extern_block_mask=True)
+    g = torch.Generator().manual_seed(S + bq + bk)
+    q, k, v, dout = (torch.randn(B, S, H, D, generator=g).bfloat16() for _ in range(4))
+    if family == "relu":                              # un-normalised sums: the input scale of the relu tests above
+        k, v, dout = (0.5 * k.float()).bfloat16(), (0.5 * v.float()).bfloat16(), (0.1 * dout.float()).bfloat16()
+    bm = (torch.rand(B, H, S // bq, S // bk, generator=g) < 0.6).to(torch.int8)
+    bm[0, 0, 1] = 0                                   # a whole block of query rows without keys
+    bm[1, 1, :, 0] = 0                                # a block of keys no query sees
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = mod(qc, kc, vc, block_mask=bm.cuda())
+    o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    keep = _keep(mask_mod, B, H, S, S) if mask_mod is not None else None
+    ref = oracle.attention_grads(oracle.masked_attention, q, k, v, dout, keep=keep, block_mask=bm, family=family, softmax_scale=scale,
+                                 bias=-math.log(S))
+    _check((qc.grad, kc.grad, vc.grad), ref, f"block mask {family} {mask}")
+    assert torch.count_nonzero(qc.grad[0, bq:2 * bq, 0]) == 0
+    assert torch.count_nonzero(kc.grad[1, :bk, 1]) == 0 and torch.count_nonzero(vc.grad[1, :bk, 1]) == 0
+
+
 def test_masked_backward_through_the_c_abi_matches_causal():
     """A lower-triangular keep mask through elem_mask / elem_mask_t gives the gradients of the causal flag (bit for bit:
     the same tiles, the same masked elements), grouped-query heads included."""
