@@ -9,9 +9,10 @@
 // Mapping onto CDNA4 (wave64, v_mfma_f32_32x32x16):
 //   * a workgroup is 8 waves (two per SIMD, one workgroup per CU); each wave owns 32 query rows
 //     (block_M = 256) and every wave walks the same 32-row KV sub-tiles, which arrive in LDS by
-//     direct-to-LDS DMA through rings of 8 K and 8 V buffers (loads run 6 sub-tiles ahead, each wave
-//     issues one K and one V instruction per sub-tile, spread between its MFMAs: the CU's vector
-//     memory path moves 64 B/clk and a wave that issues a burst of loads stalls on it);
+//     direct-to-LDS DMA through rings of 6 K and 6 V buffers (K runs 7, V 4 sub-tiles ahead; each wave
+//     issues one K and one V instruction per sub-tile, spread between its MFMAs: a wave that issues a
+//     burst of loads stalls on the CU's vector memory path, so also the first sub-tiles of the NEXT work
+//     item are fetched one per step, by the last steps of the item before it);
 //   * the score tile is computed TRANSPOSED, S^T = K Q^T (A = K rows from LDS,
 //     B = Q held in registers), so that in the accumulator layout every lane
 //     owns ONE query row: the online row statistics are per-lane scalars, the
@@ -90,6 +91,13 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   x8 qf[KS];                                   // Q fragments (B operand of S^T = K Q^T), kept in registers
   const char *kbase = nullptr, *vbase = nullptr;
   int n_sub = 0, last_sub = 0;                 // sub-tiles the workgroup walks; the last one this wave has anything to do in
+  // The K/V stream runs on into the next item: the loads that an item's last steps would spend on sub-tile positions
+  // past its end (n_sub, n_sub + 1, ..) fetch the first sub-tiles of the item that follows instead.  That item expects
+  // sub-tile j in ring slot j, so the load bound for slot j fetches its sub-tile j, whatever the position: the next
+  // item's first sub-tiles arrive in rotated order, and each slot is refilled by the usual rule (after the barrier
+  // that ends the last use of what it held).  With no item after it, these loads fetch rows of the item itself.
+  const char *kbase_n = nullptr, *vbase_n = nullptr;
+  int v_fix = ATTN_NBUF - 1;                   // the one V slot that the item before this one could not refill (see the prologue)
 
   // ---- DMA of one K or V sub-tile: 8 instructions of 1 KB (4 tile rows), one per wave; lane i fetches
   //      the 16-byte chunk that belongs at physical position i of that KB.  Wave w has tile rows
@@ -101,13 +109,17 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   const uint32_t swz_lane = (uint32_t)((((lane & 15) ^ ((lane >> 4) << 2)) ^ (wave & 3)) << 4);
   const int tile_row = 4 * wave + (lane >> 4);
   const uint32_t k_row_bytes = (uint32_t)(a.kss * 2), v_row_bytes = (uint32_t)(a.vss * 2);
+  //      Positions from n_sub on fetch the next item's sub-tile `slot` (a position more than a turn of the ring past
+  //      the end repeats an earlier one: the same bytes into the same slot).
   auto issue_k_rt = [&](int su, uint32_t slot) __attribute__((always_inline)) {
-    const uint32_t row = (uint32_t)min(su * BN + tile_row, a.Skv - 1);
-    dma16_so(kbase, row * k_row_bytes + swz_lane, lds_k + slot * KTILE + wave * 1024);
+    const bool nx = su >= n_sub;
+    const uint32_t row = (uint32_t)min((nx ? (int)slot : su) * BN + tile_row, a.Skv - 1);
+    dma16_so(nx ? kbase_n : kbase, row * k_row_bytes + swz_lane, lds_k + slot * KTILE + wave * 1024);
   };
   auto issue_v_rt = [&](int su, uint32_t slot) __attribute__((always_inline)) {
-    const uint32_t row = (uint32_t)min(su * BN + tile_row, a.Skv - 1);
-    dma16_so(vbase, row * v_row_bytes + swz_lane, lds_v + slot * VTILE + wave * 1024);
+    const bool nx = su >= n_sub;
+    const uint32_t row = (uint32_t)min((nx ? (int)slot : su) * BN + tile_row, a.Skv - 1);
+    dma16_so(nx ? vbase_n : vbase, row * v_row_bytes + swz_lane, lds_v + slot * VTILE + wave * 1024);
   };
 
   // ---- per-lane LDS read addresses: all lane-dependent parts, one register each; what is added per
@@ -288,8 +300,8 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   //      its CUs work on the q blocks of the same few pairs at the same time (their K/V stays in that
   //      XCD's L2).  Under a causal mask a q block's work grows with its position, so the unit of work
   //      is a pair of q blocks (k, nmb-1-k) of one (batch, head): every unit weighs the same.
-  //      The first loads of an item (its Q rows, K(0..5), V(0..3)) are issued before the output of the
-  //      previous item is written, so their latency hides behind that epilogue.
+  //      The first sub-tiles of an item (K(0..5), V(0..3)) are fetched by the last steps of the item before it,
+  //      and its Q rows are requested before that item's output is written.
   const int nmb = a.num_m_blocks, BH = a.B * a.H, G = (int)gridDim.x;
   const bool paired = CAUSAL && BH * nmb > G;               // (few items: one q block per unit, spread wide)
   const int upb = paired ? (nmb + 1) >> 1 : nmb;            // units per (batch, head)
@@ -297,6 +309,7 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   const int units = by_xcd ? (BH >> 3) * upb : BH * upb;   // units of this workgroup's stream
   const int first = by_xcd ? (int)blockIdx.x >> 3 : (int)blockIdx.x, stride = by_xcd ? G >> 3 : G;
   // item cursor t = 2 * unit + half; returns the next cursor that names an item (or one past the end)
+  int t_next = 0;
   auto next_item = [&](int t) -> int {
     for (;;) {
       t = (t & 1) ? t + 2 * stride - 1 : t + 1;
@@ -305,38 +318,73 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
       if (paired ? !((t & 1) && k == nmb - 1 - k) : !(t & 1)) return t;   // (the middle block of an odd count is its own partner)
     }
   };
-  // decode item t into the per-item variables and start its first loads
-  auto open_item = [&](int t) __attribute__((always_inline)) {
-    const int q = t >> 1, k = q % upb;
-    mb = paired ? ((t & 1) ? k : nmb - 1 - k) : (CAUSAL ? nmb - 1 - k : k);
-    int bh = q / upb;
+  // (batch, head) planes of item t
+  auto planes_of = [&](int t, const char*& kb, const char*& vb, int& b_, int& h_) __attribute__((always_inline)) {
+    int bh = (t >> 1) / upb;
     if (by_xcd) bh = bh * 8 + ((int)blockIdx.x & 7);
-    b = bh / a.H;
-    h = bh % a.H;
+    b_ = bh / a.H;
+    h_ = bh % a.H;
+    kb = (const char*)((const T*)a.k + (int64_t)b_ * a.ksb + (int64_t)(h_ / a.kv_group) * a.ksh);
+    vb = (const char*)((const T*)a.v + (int64_t)b_ * a.vsb + (int64_t)(h_ / a.kv_group) * a.vsh);
+  };
+  // decode item t into the per-item variables, request its Q rows, and look up the item after it
+  auto open_item = [&](int t) __attribute__((always_inline)) {
+    const int k = (t >> 1) % upb;
+    mb = paired ? ((t & 1) ? k : nmb - 1 - k) : (CAUSAL ? nmb - 1 - k : k);
+    planes_of(t, kbase, vbase, b, h);
+    // V positions n_sub .. n_sub + 4 of the item before this one (its steps n_sub - 4 .. n_sub) refilled every V slot
+    // but the one of its own last sub-tile
+    v_fix = n_sub > 0 ? (n_sub - 1) % NBUF : NBUF - 1;
     m_wave = mb * BM + row_block * 32;  // first query row of this wave
     m_lane = m_wave + r;
     n_sub = (a.Skv + BN - 1) / BN;
     if (CAUSAL) n_sub = min(n_sub, (mb * BM + BM) / BN);
     last_sub = CAUSAL ? min(n_sub - 1, m_wave / BN) : n_sub - 1;
-    kbase = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)(h / a.kv_group) * a.ksh);
-    vbase = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)(h / a.kv_group) * a.vsh);
-    // K(0..5) -> slots 0..5, V(0..3) -> slots 0..3; the first step multiplies ring slot NBUF-1 with zero
-    // probabilities: it gets V(0) as well, so that whatever is there belongs to this (batch, head)
+    // Q rows, coalesced: instruction i fetches rows 4i .. 4i+3 of the wave's 32, sixteen lanes per row (the registers
+    // of qf carry them until `q_fragments` turns them into fragments)
+    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)h * a.qsh + 8 * (lane & 15);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + (int64_t)min(m_wave + 4 * ks + (lane >> 4), a.Sq - 1) * a.qss);
+    t_next = next_item(t);
+    if (t_next < 2 * units) {
+      int b_n, h_n;
+      planes_of(t_next, kbase_n, vbase_n, b_n, h_n);
+    } else {
+      kbase_n = kbase;
+      vbase_n = vbase;
+    }
+  };
+
+  // the Q rows as loaded by open_item -> fragments (lane: row r, columns 16ks + 8g ..), through this wave's rows of the
+  // output staging area (16-byte chunks XOR-swizzled by row, as the output uses it)
+  auto q_fragments = [&]() __attribute__((always_inline)) {
+    static_assert(DQK == DV, "the staging rows hold one Q row each");
+    const uint32_t qb = lds0 + NBUF * (KTILE + VTILE) + wave * 32 * VROW;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      const int row = 4 * ks + (lane >> 4);
+      lds_write<x8>(qb + row * VROW + (((lane & 15) ^ (row & 15)) << 4), qf[ks]);
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = lds_read<x8>(qb + r * VROW + (((2 * ks + g) ^ (r & 15)) << 4));
+  };
+
+  int stores_behind = 0;   // output stores this wave issued after the current item's first loads
+  int t_cur = 2 * first;
+  // An item that nobody fetched ahead for (the first of the workgroup; the one after an item of fewer than 4 sub-tiles,
+  // whose few steps do not get round the ring): K(0..5) -> slots 0..5, V(0..3) -> slots 0..3.
+  auto fetch_first = [&]() __attribute__((always_inline)) {
     static_for<0, NBUF>([&](auto t_c) __attribute__((always_inline)) {
       constexpr int tt = decltype(t_c)::value;
       issue_k_rt(tt, tt);
       if constexpr (tt < DV_AHEAD) issue_v_rt(tt, tt);
     });
-    issue_v_rt(0, NBUF - 1);
-    const int qrow = min(m_lane, a.Sq - 1);
-    const T* qp = (const T*)a.q + (int64_t)b * a.qsb + (int64_t)qrow * a.qss + (int64_t)h * a.qsh + 8 * g;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const x8*)(qp + 16 * ks);
+    v_fix = NBUF - 1;
   };
-
-  int stores_behind = 0;   // output stores this wave issued after the current item's first loads
-  int t_cur = 2 * first;
-  if (t_cur < 2 * units) open_item(t_cur);
+  if (t_cur < 2 * units) {
+    open_item(t_cur);
+    fetch_first();
+  }
   while (t_cur < 2 * units) {
 #pragma unroll
     for (int i = 0; i < DB; i++)
@@ -353,12 +401,20 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
     //      that step u refills with K(u+7) and V(u+4).  A wave's loads complete in order and every step
     //      issues K then V; K(u+3) and V(u) are the pair of step u-4, so at the top of step u the six
     //      instructions of steps u-3 .. u-1 may still be in flight.
-    // the item's first loads (see open_item) must have landed; the previous item's output stores, issued
-    // after them, need not
+    // the item's first sub-tiles (fetched by the previous item's last steps) and Q rows must have landed; the previous
+    // item's output stores, issued after them, need not
     if (stores_behind == 32 * CPRV / 64 + 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (32 * CPRV / 64 + 1));
     else if (stores_behind == 32 * CPRV / 64) __builtin_amdgcn_s_waitcnt(0x0F70 | (32 * CPRV / 64));
     else wait_dma();
+    q_fragments();
     __syncthreads();
+    // The V slot that did not get this item's sub-tile yet (slots 4 and 5 get theirs again from steps 0 and 1).  In the
+    // first item of a workgroup it is slot NBUF-1: the first step multiplies that slot with zero probabilities, and
+    // with V(5) in it whatever is there is finite unless this (batch, head)'s own values are not.
+    {
+      const uint32_t row = (uint32_t)min(v_fix * BN + tile_row, a.Skv - 1);
+      dma16_so(vbase, row * v_row_bytes + swz_lane, lds_v + (uint32_t)v_fix * VTILE + wave * 1024);
+    }
     {   // s[0] = K(0) Q^T with its maximum folded in, s[1] = K(1) Q^T; then K(6) may replace K(0)
       x8 k0[KS];
   #pragma unroll
@@ -377,7 +433,8 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
         fold_max(std::integral_constant<int, 1>{}, mx);
       }
     }
-    __syncthreads();   // every wave is done reading K(0)
+    wait_dma();
+    __syncthreads();   // every wave is done reading K(0), and V ring slot NBUF-1 is filled
     issue_k_rt(NBUF, 0);
     static_for<0, PF - 1>([&](auto i_c) __attribute__((always_inline)) {   // first fragments of step 0: zeros, K(2)
       request(i_c, std::integral_constant<int, NBUF - 1>{}, std::integral_constant<int, 2>{});
@@ -408,20 +465,26 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
         vslot = vslot + 1 == NBUF ? 0 : vslot + 1;
       }
     }
-    wait_dma();
-    __syncthreads();   // every wave is done with the K/V rings
 
-    // ---- what the epilogue needs of this item, then the next item's first loads, then the epilogue
+    // ---- what the epilogue needs of this item, then the next item's Q rows, then the epilogue
     T* const obase = (T*)a.o + (int64_t)b * a.osb + (int64_t)h * a.osh + (int64_t)m_wave * a.oss;
     const int m_out = m_wave;
     float* const lse_ptr = a.row_scale ? a.row_scale + ((int64_t)b * a.H + h) * a.Sq + m_lane : nullptr;
     const bool row_ok = m_lane < a.Sq;
-    t_cur = next_item(t_cur);
-    if (t_cur < 2 * units) open_item(t_cur);
+    t_cur = t_next;
+    if (t_cur < 2 * units) {
+      const bool unfetched = n_sub < 4;
+      open_item(t_cur);
+      if (unfetched) {
+        wait_dma();
+        __syncthreads();   // every wave is done with the K/V rings
+        fetch_first();
+      }
+    }
 
     // normalise, stage O through LDS (wave-private rows, 16-byte chunks XOR-swizzled by row so that neither
     // the 8-byte writes nor the 16-byte reads pile onto one bank group), coalesced 16-byte stores.  The
-    // staging area lies behind the rings, which already receive the next item.
+    // staging area lies behind the rings, which already hold the next item's first sub-tiles.
     float inv = 1.f, lse = 0.f;
     if constexpr (FAMILY == FAM_SOFTMAX) {
       float s_lo, s_hi;
