@@ -14,6 +14,7 @@ benchmark configurations, each with its own roofline fraction:
   c2_softmax_causal_bwd  backward of the headline workload (dq, dk, dv)
   c3_retnet_chunked   RetNet retention, chunked operator, B8 H16 S2048 Dqk256 Dv512
   c3_retnet_parallel  same shape, normalised parallel operator with a [1,H,S,S] decay mask
+  c3_retnet_parallel_bwd  backward of that operator (dq, dk, dv; the row scale held constant, as the reference defines it)
   c4_mamba2_ssd       Mamba2 SSD, B8 H64 S2048 P64 N128, one B/C group
   c5_mla_decode       absorbed MLA decode, B64 Hq128 KV4096 d512+64 (HBM bound)
   gqa_decode          grouped-query softmax decode, B64 H32 Hkv8 KV4096 D128 (HBM bound)
@@ -150,7 +151,7 @@ def bench_retnet_chunked(steps, warmup):
     return _mfma_entry(ms, flops, "chunked form, chunk 64: 2*S*C*(Dqk+Dv) + 4*S*Dqk*Dv per (batch, head)")
 
 
-def bench_retnet_parallel(steps, warmup):
+def bench_retnet_parallel(steps, warmup, backward=False):
     import torch
     import oracle
     from metaattention_amd import hip_backend as hb
@@ -165,9 +166,16 @@ def bench_retnet_parallel(steps, warmup):
     mask = (torch.exp2(diff.clamp(min=0).unsqueeze(0) * torch.log2(gam).view(H, 1, 1)) * (diff >= 0)).unsqueeze(0).bfloat16()
     o = torch.empty_like(v)
     r = torch.empty(B, H, S, device="cuda")
+    flops = 0.5 * 2.0 * B * H * S * S * (D + DV)
+    if backward:
+        hb.attn_fwd(q, k, v, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mask, out=o, row_scale=r)
+        do = torch.randn(B, S, H, DV, device="cuda", generator=g).bfloat16()
+        mask_t = mask.transpose(2, 3).contiguous()
+        ms = time_gpu(lambda: hb.attn_bwd(q, k, v, o, do, r, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mask,
+                                          score_mask_t=mask_t), max(steps // 3, 3), 2)
+        return _mfma_entry(ms, 2.5 * flops, "backward, 2.5 x the forward's algorithmic FLOPs (three kernels dq, dv, dk)")
     ms = time_gpu(lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mask, out=o,
                                       row_scale=r), steps, warmup)
-    flops = 0.5 * 2.0 * B * H * S * S * (D + DV)
     return _mfma_entry(ms, flops, "parallel form, causal counted at one half")
 
 
@@ -268,6 +276,7 @@ def main():
              ("c2_softmax_causal_bwd", "bwd", lambda: bench_softmax_bwd(args.steps, args.warmup)),
              ("c3_retnet_chunked", "retnet", lambda: bench_retnet_chunked(args.steps, args.warmup)),
              ("c3_retnet_parallel", "retention", lambda: bench_retnet_parallel(args.steps, args.warmup)),
+             ("c3_retnet_parallel_bwd", "retention_bwd", lambda: bench_retnet_parallel(args.steps, args.warmup, backward=True)),
              ("c4_mamba2_ssd", "mamba", lambda: bench_mamba2(args.steps, args.warmup)),
              ("c5_mla_decode", "mla", lambda: bench_mla(args.steps, args.warmup)),
              ("gqa_decode", "decode", lambda: bench_decode(args.steps, args.warmup))]

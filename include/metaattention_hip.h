@@ -97,14 +97,14 @@ typedef struct ma_attn_params {
   void* workspace; size_t workspace_bytes;
 } ma_attn_params;
 
-/* Parallel attention backward for the SOFTMAX, SIGMOID and RELU families.  Replaces the backward of
+/* Parallel attention backward for the SOFTMAX, SIGMOID, RELU and RETENTION families.  Replaces the backward of
  * _attention (tl_template/attn/attn_tl.py:669-692): delta pre-pass, dK/dV kernel with fp32 dQ atomics,
  * dQ post-pass.  Tensors and strides as in ma_attn_params; o and lse are the forward pass's output and
  * fp32 [B,H,Sq] row scale (SOFTMAX only; may be NULL otherwise), dout is the gradient of o; dq [B,Sq,H,Dqk],
  * dk [B,Skv,Hkv,Dqk], dv [B,Skv,Hkv,Dv] are written (not accumulated into), in `dtype`.  The workspace
  * (ma_attn_bwd_workspace_bytes: fp32 [B,H,Sq]) carries delta = sum_d dout*o between the two kernels. */
 typedef struct ma_attn_bwd_params {
-  int32_t family; /* ma_attn_family: SOFTMAX, SIGMOID or RELU */
+  int32_t family; /* ma_attn_family: SOFTMAX, SIGMOID, RELU or RETENTION (Dqk 256, Dv 512) */
   int32_t dtype;
   int32_t mask;   /* ma_mask_kind */
   int32_t batch, heads, heads_kv /* 0 = heads */, seqlen_q, seqlen_kv, dim_qk, dim_v;
@@ -133,6 +133,13 @@ typedef struct ma_attn_bwd_params {
    * q_block_mask  [1 or B, 1 or H, ceil(Skv/128), ceil(Sq/32)] for the dk / dv kernels. */
   const uint8_t* kv_block_mask; int64_t kbm_stride_b, kbm_stride_h, kbm_stride_q;
   const uint8_t* q_block_mask;  int64_t qbm_stride_b, qbm_stride_h, qbm_stride_k;
+  /* RETENTION: p = q.k * scale * M / r with r the forward pass's row scale (passed as `lse`), which the backward
+   * treats as a constant exactly as OnlineRetention.backward does (examples/retention_parallel.py:82-86:
+   * dscores = dp / r; the score_mod's own derivative contributes the factor M).  score_mask is M as given to the
+   * forward pass ([1 or B, H, Sq, Skv] in `dtype`), score_mask_t its transpose [1 or B, H, Skv, Sq] for the dk / dv
+   * kernels; strides in elements, batch stride 0 broadcasts, rows 8-byte aligned (multiples of 4 elements). */
+  const void* score_mask;   int64_t sm_stride_b, sm_stride_h, sm_stride_q;
+  const void* score_mask_t; int64_t smt_stride_b, smt_stride_h, smt_stride_k;
 } ma_attn_bwd_params;
 
 /* Chunked linear / stateful attention forward.  Replaces the three launches

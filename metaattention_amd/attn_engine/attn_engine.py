@@ -84,15 +84,15 @@ class _ForwardOnly(torch.autograd.Function):
 
 
 class _Attention(torch.autograd.Function):
-    """Forward + backward of the softmax / sigmoid / relu operators, as _attention of
+    """Forward + backward of the softmax / sigmoid / relu / retention operators, as _attention of
     tl_template/attn/attn_tl.py:654-692: saves q, k, v, o and the final row scale, returns
     (dq, dk, dv) and None for every custom input."""
 
     @staticmethod
-    def forward(ctx, engine, run, fam_code, bias_t, call_masks, q, k, v):
+    def forward(ctx, engine, run, fam_code, bias_t, call_masks, score_mask, q, k, v):
         out = run(q, k, v)
         lse = engine.final_rowscales
-        ctx.engine, ctx.fam_code, ctx.bias_t, ctx.call_masks = engine, fam_code, bias_t, call_masks
+        ctx.engine, ctx.fam_code, ctx.bias_t, ctx.call_masks, ctx.score_mask = engine, fam_code, bias_t, call_masks, score_mask
         ctx.save_for_backward(q, k, v, out, *([lse] if lse is not None else []))
         return out
 
@@ -109,9 +109,12 @@ class _Attention(torch.autograd.Function):
         elif eng.mask_kind.startswith("other"):
             masks = dict(zip(("elem_mask", "elem_mask_t", "kv_block_mask", "q_block_mask"),
                              eng._dense_mask(q.shape[0], q.shape[2], q.shape[1], k.shape[1], q.device, transposed=True)))
+        if ctx.score_mask is not None:
+            # retention: the multiplier tensor in both orientations (the dk / dv kernels walk down its columns)
+            masks = dict(score_mask=ctx.score_mask, score_mask_t=ctx.score_mask.transpose(2, 3).contiguous())
         dq, dk, dv = attn_bwd(q, k, v, out, dout, rest[0] if rest else None, family=ctx.fam_code,
                               causal=causal, scale=form.scale, bias=form.bias, bias_tensor=ctx.bias_t, **masks)
-        return None, None, None, None, None, dq, dk, dv
+        return None, None, None, None, None, None, dq, dk, dv
 
 
 class AttentionEngine:
@@ -258,14 +261,19 @@ class AttentionEngine:
             return run(q, k, v).squeeze(1)
 
         if any(t.requires_grad for t in (q, k, v)):
+            score_mask = None
             if self.family == "retention":
-                return _ForwardOnly.apply(run, q, k, v)
+                # the backward kernels of the retention operator exist for its own head size (examples/retention_parallel.py)
+                if (q.shape[-1], v.shape[-1]) != (256, 512) or not form.mask_tensor:
+                    return _ForwardOnly.apply(run, q, k, v)
+                score_mask = given[form.mask_tensor]
+                score_mask = score_mask if score_mask.dtype == q.dtype else score_mask.to(q.dtype)
             bias_t = given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None
             call_masks = None
             if prefill_blocks is not None:
                 shape = (q.shape[0], q.shape[2], q.shape[1], k.shape[1], q.device)
                 call_masks = lambda: self._block_mask_backward_masks(prefill_blocks, *shape)
-            return _Attention.apply(self, run, fam_code, bias_t, call_masks, q, k, v)
+            return _Attention.apply(self, run, fam_code, bias_t, call_masks, score_mask, q, k, v)
         return run(q, k, v)
 
     @staticmethod

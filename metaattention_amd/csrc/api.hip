@@ -123,8 +123,17 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
   if (p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->seqlen_kv <= 0 || p->dim_qk <= 0 || p->dim_v <= 0)
     return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: sizes must be positive");
   if (p->dtype != MA_BF16 && p->dtype != MA_FP16) return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: dtype %d", p->dtype);
-  if (p->family != MA_ATTN_SOFTMAX && p->family != MA_ATTN_SIGMOID && p->family != MA_ATTN_RELU)
+  if (p->family != MA_ATTN_SOFTMAX && p->family != MA_ATTN_SIGMOID && p->family != MA_ATTN_RELU && p->family != MA_ATTN_RETENTION)
     return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: family %d has no backward kernel", p->family);
+  if (p->family == MA_ATTN_RETENTION) {
+    if (!p->lse || !p->score_mask || !p->score_mask_t)
+      return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: RETENTION needs the forward's row scale (lse), score_mask and score_mask_t");
+    if (p->elem_mask || p->kv_block_mask) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: RETENTION takes no element-wise or block masks");
+    const int64_t ms[] = {(int64_t)(uintptr_t)p->score_mask / 2, p->sm_stride_b, p->sm_stride_h, p->sm_stride_q,
+                          (int64_t)(uintptr_t)p->score_mask_t / 2, p->smt_stride_b, p->smt_stride_h, p->smt_stride_k};
+    for (int64_t x : ms)
+      if (x % 4 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: score_mask rows must be 8-byte aligned");
+  }
   if (!(p->scale > 0.f)) return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: scale must be > 0 (got %g)", (double)p->scale);
   if (p->mask == MA_MASK_CAUSAL && p->seqlen_q != p->seqlen_kv)
     return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: causal mask needs seqlen_q == seqlen_kv (%d vs %d)", p->seqlen_q, p->seqlen_kv);
@@ -177,6 +186,8 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
   a.elem_mask_t = p->elem_mask_t; a.emt_sb = p->emt_stride_b; a.emt_sh = p->emt_stride_h; a.emt_sk = p->emt_stride_k;
   a.kv_block_mask = p->kv_block_mask; a.kbm_sb = p->kbm_stride_b; a.kbm_sh = p->kbm_stride_h; a.kbm_sq = p->kbm_stride_q;
   a.q_block_mask = p->q_block_mask; a.qbm_sb = p->qbm_stride_b; a.qbm_sh = p->qbm_stride_h; a.qbm_sk = p->qbm_stride_k;
+  a.smask = p->score_mask; a.sm_sb = p->sm_stride_b; a.sm_sh = p->sm_stride_h; a.sm_sq = p->sm_stride_q;
+  a.smask_t = p->score_mask_t; a.smt_sb = p->smt_stride_b; a.smt_sh = p->smt_stride_h; a.smt_sk = p->smt_stride_k;
   const int rc = ma::attn_bwd_dispatch(a, p->family, p->mask == MA_MASK_CAUSAL, p->dtype == MA_BF16, p->dim_qk, p->dim_v, (hipStream_t)stream);
   if (rc == -2) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: no kernel for family %d, Dqk=%d, Dv=%d", p->family, p->dim_qk, p->dim_v);
   if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_attn_bwd: launch failed: %s", hipGetErrorString(hipGetLastError()));

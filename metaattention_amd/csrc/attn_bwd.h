@@ -7,7 +7,7 @@ namespace ma {
 struct AttnBwdArgs {
   const void* q; const void* k; const void* v; const void* o; const void* dout;
   void* dq; void* dk; void* dv;
-  const float* lse;    // [B,H,Sq] natural-log row scale of the forward pass (softmax)
+  const float* lse;    // [B,H,Sq] row scale of the forward pass: natural-log sum (softmax), r (retention)
   float* delta;        // [B,H,Sq] workspace: sum_d dout * o per row (softmax)
   const float* bias_ptr;
   int64_t qsb, qss, qsh, ksb, kss, ksh, vsb, vss, vsh, osb, oss, osh, dosb, doss, dosh;
@@ -25,6 +25,11 @@ struct AttnBwdArgs {
   // q_block_mask  [.., .., ceil(Skv/128), ceil(Sq/32)] for the dk / dv kernel (a workgroup's 128 keys x a 32-row tile)
   const uint8_t* kv_block_mask; int64_t kbm_sb, kbm_sh, kbm_sq;
   const uint8_t* q_block_mask; int64_t qbm_sb, qbm_sh, qbm_sk;
+  // retention family: the score multiplier of the forward pass in the tensor dtype, in both orientations (strides in
+  // elements, 0 broadcasts): smask [.., H, Sq, Skv] for the dq kernel, smask_t [.., H, Skv, Sq] for the dk / dv kernels;
+  // rows are 8-byte aligned.  `lse` then holds the forward's row scale r.
+  const void* smask; int64_t sm_sb, sm_sh, sm_sq;
+  const void* smask_t; int64_t smt_sb, smt_sh, smt_sk;
 };
 
 int attn_bwd_dispatch(const AttnBwdArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);

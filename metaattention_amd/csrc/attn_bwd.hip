@@ -32,14 +32,20 @@
 namespace ma {
 
 namespace {
-enum { BF_SOFTMAX = 0, BF_SIGMOID = 1, BF_RELU = 2 };   // = MA_ATTN_* of the C interface
+enum { BF_SOFTMAX = 0, BF_SIGMOID = 1, BF_RELU = 2, BF_RETENTION = 3 };   // = MA_ATTN_* of the C interface
 
 // ds / scale (and p) of one score element: the common factor `scale` of dq and dk is applied once, when the
 // accumulators are stored.  x2 = (s * scale + bias) * log2(e) for softmax / sigmoid.
+// Retention (examples/retention_parallel.py:76-86 of the reference): p = s * scale * m / r with m the caller's score
+// multiplier and r the row scale of the forward pass, which the backward treats as a constant (dscores = dp / r);
+// `lse2` carries m / r.
 template <int FAMILY>
 __device__ __forceinline__ void row_fn_bwd(float s, float dp, bool masked, float c_scale, float c_bias, float scale, float bias,
                                            float lse2, float delta, float& p, float& ds) {
-  if constexpr (FAMILY == BF_SOFTMAX) {
+  if constexpr (FAMILY == BF_RETENTION) {
+    p = masked ? 0.f : s * scale * lse2;
+    ds = masked ? 0.f : dp * lse2;
+  } else if constexpr (FAMILY == BF_SOFTMAX) {
     p = masked ? 0.f : fast_exp2(s * c_scale + lse2);   // (lse2 = c_bias - lse * log2(e), folded by the caller)
     ds = p * (dp - delta);
   } else if constexpr (FAMILY == BF_SIGMOID) {
@@ -205,6 +211,10 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
       if (g == 0 && m_lane < a.Sq) a.delta[ri] = delta;
     }
   }
+  float r_inv = 1.f;   // retention: 1 / the row scale of the forward pass
+  if constexpr (FAMILY == BF_RETENTION) r_inv = 1.f / a.lse[((int64_t)b * a.H + h) * a.Sq + m_ld];
+  // retention: this lane's row of the score multiplier
+  const T* sm_row = FAMILY == BF_RETENTION ? (const T*)a.smask + (int64_t)b * a.sm_sb + (int64_t)h * a.sm_sh + (int64_t)m_ld * a.sm_sq : nullptr;
   const char* kb = (const char*)((const T*)a.k + (int64_t)b * a.ksb + (int64_t)hk * a.ksh);
   const char* vb = (const char*)((const T*)a.v + (int64_t)b * a.vsb + (int64_t)hk * a.vsh);
   const int64_t k_row_bytes = a.kss * 2, v_row_bytes = a.vss * 2;
@@ -247,9 +257,28 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
     if (jt < n_tiles) issue_tile(jt * BN, buf ^ 1);
     const uint32_t kbase = lds0 + buf * STAGE, vbase = kbase + KTILE;
 
+    // retention: the multipliers of this lane's 16 scores, requested before the products that hide their latency
+    typename E::x4 mk[4];
+    if constexpr (FAMILY == BF_RETENTION) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const int n = n0 + 8 * q4 + 4 * g;
+        if (n + 3 < a.Skv) {
+          mk[q4] = *(const typename E::x4*)(sm_row + n);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; i++) mk[q4][i] = n + i < a.Skv ? sm_row[n + i] : (T)0.f;
+        }
+      }
+    }
     const f32x16 s = mm_rows<T, DQK>(kbase, r, g, qf);     // S^T: lane = row m_lane, element jj = key n0 + 8(jj/4) + 4g + jj%4
     const f32x16 dp = mm_rows<T, DV>(vbase, r, g, dof);   // dP^T, same layout
     x8 dsf[2];
+    float mr[16];   // retention: multiplier / r per element
+    if constexpr (FAMILY == BF_RETENTION) {
+#pragma unroll
+      for (int jj = 0; jj < 16; jj++) mr[jj] = (float)mk[jj >> 2][jj & 3] * r_inv;
+    }
     // only tiles that touch the diagonal or the end of the keys pay for the mask (the test is wave-uniform);
     // with an element-wise mask every tile does
     if ((CAUSAL && n0 + BN - 1 > m_wave) || n0 + BN > a.Skv || em_row) {
@@ -273,14 +302,14 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
         const int n = n0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
         const bool masked = (CAUSAL && n > m_lane) || n >= a.Skv || ((keep[jj >> 2] >> (8 * (jj & 3))) & 0xffu) == 0;
         float p, ds;
-        row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, lse2, delta, p, ds);
+        row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, FAMILY == BF_RETENTION ? mr[jj] : lse2, delta, p, ds);
         dsf[jj >> 3][jj & 7] = (T)ds;
       }
     } else {
 #pragma unroll
       for (int jj = 0; jj < 16; jj++) {
         float p, ds;
-        row_fn_bwd<FAMILY>(s[jj], dp[jj], false, c_scale, c_bias, a.scale, bias, lse2, delta, p, ds);
+        row_fn_bwd<FAMILY>(s[jj], dp[jj], false, c_scale, c_bias, a.scale, bias, FAMILY == BF_RETENTION ? mr[jj] : lse2, delta, p, ds);
         dsf[jj >> 3][jj & 7] = (T)ds;
       }
     }
@@ -380,12 +409,36 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
     __syncthreads();
     step_next = next_step(step + 1);
     if (step_next < n_steps) issue_step(step_next, buf ^ 1);
-    // (a wave whose keys all lie behind this tile's rows has nothing to add; it still takes part in the barriers)
-    if (CAUSAL && m0 + BMT - 1 < n_wave) continue;
+    // (a wave whose keys all lie behind this tile's rows has nothing to add; it still takes part in the barriers.  With
+    // the large accumulators of the 256 / 512 head size the second way round the loop costs register copies that spill,
+    // and the few such tiles are computed instead: every element of them is masked)
+    if (CAUSAL && DQK + DV < 768 && m0 + BMT - 1 < n_wave) continue;
     const uint32_t qbase = lds0 + buf * STAGE, dobase = qbase + QTILE;
 
-    // lse and delta of the rows this lane holds: m0 + 8q4 + 4g + {0..3}
+    // retention: 1 / r of the rows this lane holds and the multipliers of its 16 scores (from the transposed
+    // multiplier tensor: this key's row, indexed by query position)
     float lse2[16], dl[16];
+    if constexpr (FAMILY == BF_RETENTION) {
+      const int64_t rbase = ((int64_t)b * a.H + h) * a.Sq;
+      const T* smt_row = (const T*)a.smask_t + (int64_t)b * a.smt_sb + (int64_t)h * a.smt_sh + (int64_t)n_ld * a.smt_sk;
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const int m = m0 + 8 * q4 + 4 * g;
+        if ((a.Sq & 3) == 0 && m + 3 < a.Sq) {
+          const f32x4 tr = *(const f32x4*)(a.lse + rbase + m);
+          const typename E::x4 tm = *(const typename E::x4*)(smt_row + m);
+#pragma unroll
+          for (int i = 0; i < 4; i++) lse2[4 * q4 + i] = (float)tm[i] / tr[i];
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int mm = min(m + i, a.Sq - 1);
+            lse2[4 * q4 + i] = (float)smt_row[mm] / a.lse[rbase + mm];
+          }
+        }
+      }
+    }
+    // lse and delta of the rows this lane holds: m0 + 8q4 + 4g + {0..3}
     if constexpr (FAMILY == BF_SOFTMAX) {
       const int64_t rbase = ((int64_t)b * a.H + h) * a.Sq;
       if ((a.Sq & 3) == 0 && m0 + BMT <= a.Sq) {   // whole tile, 16-byte aligned groups of four rows
@@ -442,7 +495,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
         const int m = m0 + 8 * (jj >> 2) + 4 * g + (jj & 3);
         const bool masked = (CAUSAL && n_lane > m) || m >= a.Sq || n_lane >= a.Skv || ((keep[jj >> 2] >> (8 * (jj & 3))) & 0xffu) == 0;
         float p, ds;
-        row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX ? lse2[jj] : 0.f,
+        row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX || FAMILY == BF_RETENTION ? lse2[jj] : 0.f,
                            FAMILY == BF_SOFTMAX ? dl[jj] : 0.f, p, ds);
         if (masked) ds = 0.f;
         pf[jj >> 3][jj & 7] = (T)p;
@@ -452,7 +505,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
 #pragma unroll
       for (int jj = 0; jj < 16; jj++) {
         float p, ds;
-        row_fn_bwd<FAMILY>(s[jj], dp[jj], false, c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX ? lse2[jj] : 0.f,
+        row_fn_bwd<FAMILY>(s[jj], dp[jj], false, c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX || FAMILY == BF_RETENTION ? lse2[jj] : 0.f,
                            FAMILY == BF_SOFTMAX ? dl[jj] : 0.f, p, ds);
         pf[jj >> 3][jj & 7] = (T)p;
         dsf[jj >> 3][jj & 7] = (T)ds;
@@ -480,7 +533,7 @@ static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   constexpr size_t lds = tiles > ostage ? tiles : ostage;
   auto k1 = attn_bwd_dq_kernel<T, DQK, DV, FAMILY, CAUSAL>;
   // one dk/dv launch where both accumulators fit beside a second wave, else one launch each
-  constexpr bool SPLIT = DQK + DV >= 256 && DQK + DV < 512;
+  constexpr bool SPLIT = DQK + DV >= 256 && (DQK + DV < 512 || DQK + DV > 512);
   auto k2 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL, SPLIT ? 1 : 3>;
   auto k3 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL, 2>;
   static bool attr_set = false;
@@ -514,6 +567,10 @@ static int bwd_family(const AttnBwdArgs& a, int family, bool causal, hipStream_t
 
 template <typename T>
 static int bwd_dims(const AttnBwdArgs& a, int family, bool causal, int dqk, int dv, hipStream_t stream) {
+  if (family == BF_RETENTION) {   // the head size of the retention operator (examples/retention_parallel.py: 256 / 512)
+    if (dqk != 256 || dv != 512) return -2;
+    return causal ? launch_bwd<T, 256, 512, BF_RETENTION, true>(a, stream) : launch_bwd<T, 256, 512, BF_RETENTION, false>(a, stream);
+  }
   if (dqk == 128 && dv == 128) return bwd_family<T, 128, 128>(a, family, causal, stream);
   if (dqk == 64 && dv == 64) return bwd_family<T, 64, 64>(a, family, causal, stream);
   if (dqk == 128 && dv == 256) return bwd_family<T, 128, 256>(a, family, causal, stream);

@@ -74,6 +74,8 @@ class AttnBwdParams(Structure):
         ("elem_mask_t", c_void_p), ("emt_stride_b", c_int64), ("emt_stride_h", c_int64), ("emt_stride_k", c_int64),
         ("kv_block_mask", c_void_p), ("kbm_stride_b", c_int64), ("kbm_stride_h", c_int64), ("kbm_stride_q", c_int64),
         ("q_block_mask", c_void_p), ("qbm_stride_b", c_int64), ("qbm_stride_h", c_int64), ("qbm_stride_k", c_int64),
+        ("score_mask", c_void_p), ("sm_stride_b", c_int64), ("sm_stride_h", c_int64), ("sm_stride_q", c_int64),
+        ("score_mask_t", c_void_p), ("smt_stride_b", c_int64), ("smt_stride_h", c_int64), ("smt_stride_k", c_int64),
     ]
 
 
@@ -241,14 +243,16 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
 
 
 def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None,
-             elem_mask=None, elem_mask_t=None, kv_block_mask=None, q_block_mask=None):
+             elem_mask=None, elem_mask_t=None, kv_block_mask=None, q_block_mask=None, score_mask=None, score_mask_t=None):
     """Gradients (dq, dk, dv) of the parallel attention forward on BSHD tensors.  ``o`` and ``lse``
-    (fp32 [B,H,Sq]) are the forward pass's output and row scale (softmax only; None otherwise),
-    ``dout`` the gradient of ``o``.  ``elem_mask`` (the forward pass's keep mask, [1|B, 1|H, Sq, Skv]) comes with
+    (fp32 [B,H,Sq]) are the forward pass's output and row scale (softmax and retention; None otherwise),
+    ``dout`` the gradient of ``o``.  The retention family takes the forward's multiplier tensor ``score_mask``
+    [1|B, H, Sq, Skv] and its transpose ``score_mask_t`` [1|B, H, Skv, Sq] in the tensor dtype, and treats the
+    row scale as a constant, as the reference's OnlineRetention.backward does.  ``elem_mask`` (the forward pass's keep mask, [1|B, 1|H, Sq, Skv]) comes with
     its transpose ``elem_mask_t`` [1|B, 1|H, Skv, Sq]; both with rows at 4-byte aligned addresses.  Optional tile masks
     for skipping: ``kv_block_mask`` [1|B, 1|H, ceil(Sq/128), ceil(Skv/32)] and ``q_block_mask`` [1|B, 1|H, ceil(Skv/128),
     ceil(Sq/32)] (a tile is kept when any of its elements is)."""
-    _require_gpu(q, k, v, o, dout, lse, bias_tensor, elem_mask, elem_mask_t, kv_block_mask, q_block_mask)
+    _require_gpu(q, k, v, o, dout, lse, bias_tensor, elem_mask, elem_mask_t, kv_block_mask, q_block_mask, score_mask, score_mask_t)
     B, Sq, H, Dqk = q.shape
     Skv, Hkv, Dv = k.shape[1], k.shape[2], v.shape[-1]
     assert k.shape == (B, Skv, Hkv, Dqk) and v.shape == (B, Skv, Hkv, Dv) and dout.shape == (B, Sq, H, Dv) and H % Hkv == 0
@@ -291,6 +295,14 @@ def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, 
             setattr(p, "kv_block_mask" if pre == "kbm" else "q_block_mask", t.data_ptr())
             setattr(p, f"{pre}_stride_b", t.stride(0) if t.shape[0] > 1 else 0)
             setattr(p, f"{pre}_stride_h", t.stride(1) if t.shape[1] > 1 else 0)
+            setattr(p, f"{pre}_stride_{last}", t.stride(2))
+    if score_mask is not None or score_mask_t is not None:
+        assert score_mask is not None and score_mask_t is not None, "score_mask and score_mask_t go together"
+        for t, rows, cols, pre, last in ((score_mask, Sq, Skv, "sm", "q"), (score_mask_t, Skv, Sq, "smt", "k")):
+            assert t.dtype == q.dtype and t.dim() == 4 and t.shape[1:] == (H, rows, cols) and t.shape[0] in (1, B) and t.stride(-1) == 1
+            setattr(p, "score_mask" if pre == "sm" else "score_mask_t", t.data_ptr())
+            setattr(p, f"{pre}_stride_b", t.stride(0) if t.shape[0] > 1 else 0)
+            setattr(p, f"{pre}_stride_h", t.stride(1))
             setattr(p, f"{pre}_stride_{last}", t.stride(2))
     lib = load_library()
     need = lib.ma_attn_bwd_workspace_bytes(ctypes.byref(p))

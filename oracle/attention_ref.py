@@ -98,11 +98,13 @@ def retention_decay_mask(H: int, S: int, dtype=torch.float32) -> torch.Tensor:
     return m.unsqueeze(0).to(dtype)
 
 
-def retention_parallel(q, k, v, mask, compute_dtype=torch.float32, return_r: bool = False):
+def retention_parallel(q, k, v, mask, compute_dtype=torch.float32, return_r: bool = False, freeze_r: bool = False):
     """Normalised parallel retention, attention_engine/benchmark/bench_utils.py:1158-1163
     (same as testing/benchmark_h100.py:808-813): qkm = (q.k^T) * mask,
     r = max(sum_j |qkm|, 1), o = (qkm / r) v.  q,k [B,S,H,D], v [B,S,H,Dv],
-    mask [1 or B, H, S, S] -> [B,S,H,Dv]."""
+    mask [1 or B, H, S, S] -> [B,S,H,Dv].
+    freeze_r: autograd sees r as a constant, which is the gradient the reference's operator defines
+    (OnlineRetention.backward, examples/retention_parallel.py:82-86: dscores = dp / r, nothing flows through r)."""
     B, S, H, D = q.shape
     Dv = v.shape[-1]
     out = torch.empty(B, S, H, Dv, dtype=compute_dtype)
@@ -113,7 +115,9 @@ def retention_parallel(q, k, v, mask, compute_dtype=torch.float32, return_r: boo
             s = q[b, :, h].to(compute_dtype) @ k[b, :, h // (H // k.shape[2])].to(compute_dtype).T
             s = s * mb[h].to(compute_dtype)
             r = s.abs().sum(dim=-1, keepdim=True).clamp(min=1.0)
-            r_out[b, h] = r.squeeze(-1)
+            if freeze_r:
+                r = r.detach()
+            r_out[b, h] = r.detach().squeeze(-1)
             out[b, :, h] = (s / r) @ v[b, :, h // (H // v.shape[2])].to(compute_dtype)
     return (out, r_out) if return_r else out
 

@@ -120,6 +120,33 @@ def test_retention_parallel_bruteforce_and_clamp():
     torch.testing.assert_close(o, ref, rtol=1e-12, atol=1e-12)
 
 
+def test_retention_gradient_with_the_row_scale_held_constant():
+    """The gradient the reference's retention operator defines (OnlineRetention.backward,
+    examples/retention_parallel.py:76-86: p = scores / r, dscores = dp / r, and the score_mod's factor M):
+    dq = ((dO V^T) * M / r) K, dk = ((dO V^T) * M / r)^T Q, dv = P^T dO, written out with einsum, against autograd over
+    the oracle with freeze_r; and where the clamp holds r at 1 that is the true gradient."""
+    B, S, H, D, DV = 2, 9, 2, 4, 3
+    q, k, v, do = _rand(B, S, H, D, seed=30), _rand(B, S, H, D, seed=31), _rand(B, S, H, DV, seed=32), _rand(B, S, H, DV, seed=33)
+    mask = oracle.retention_decay_mask(H, S, F64)
+    for qs in (3.0, 0.01):
+        qq = q * qs
+        got = oracle.attention_grads(oracle.retention_parallel, qq, k, v, do, mask=mask, freeze_r=True)
+        s_ = torch.einsum("bqhd,bkhd->bhqk", qq, k) * mask
+        r = s_.abs().sum(-1, keepdim=True).clamp(min=1)
+        assert bool((r > 1).any()) == (qs == 3.0)
+        dp = torch.einsum("bqhe,bkhe->bhqk", do, v)
+        ds = dp * mask / r
+        exp = (torch.einsum("bhqk,bkhd->bqhd", ds, k), torch.einsum("bhqk,bqhd->bkhd", ds, qq), torch.einsum("bhqk,bqhe->bkhe", s_ / r, do))
+        for a, b in zip(got, exp):
+            torch.testing.assert_close(a, b, rtol=1e-11, atol=1e-11)
+        true = oracle.attention_grads(oracle.retention_parallel, qq, k, v, do, mask=mask)
+        if qs == 0.01:
+            for a, b in zip(got, true):
+                torch.testing.assert_close(a, b, rtol=1e-11, atol=1e-11)
+        else:
+            assert not torch.allclose(got[0], true[0], rtol=1e-3, atol=1e-3)    # r does depend on q and k there
+
+
 # ---------------------------------------------------------------- RetNet chunked
 def test_retnet_three_way():
     B, H, T, Dk, Dv = 1, 3, 64, 8, 6

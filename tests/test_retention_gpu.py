@@ -67,6 +67,59 @@ def test_engine_retention_parallel():
     torch.testing.assert_close(mod.final_rowscales.cpu(), r_ref, rtol=1e-3, atol=1e-3)
 
 
+def _check_grads(got, ref, what):
+    for name, a, b in zip(("dq", "dk", "dv"), got, ref):
+        oracle.assert_close(a.float().cpu(), b.float(), rtol=RTOL, atol=ATOL, mismatch_ratio=1e-3, msg=f"{what}:{name}")
+
+
+@pytest.mark.parametrize("B,H,S,causal,dtype", [(1, 2, 128, True, torch.bfloat16), (2, 3, 200, True, torch.bfloat16),
+                                                (1, 2, 132, False, torch.bfloat16), (1, 1, 4, True, torch.bfloat16),
+                                                (1, 2, 260, True, torch.float16)])
+def test_retention_backward(B, H, S, causal, dtype):
+    """dq, dk, dv of the retention operator through the C ABI: the row scale r of the forward pass is a constant of the
+    backward (examples/retention_parallel.py:82-86).  Oracle: autograd over oracle.retention_parallel(freeze_r=True)
+    in fp64."""
+    hb = _hb()
+    D, DV = 256, 512
+    q, k, v, mask = _inputs(B, H, S, D, DV, seed=S)
+    q, k, v, mask = (t.to(dtype) for t in (q, k, v, mask))
+    dout = (0.5 * torch.randn(B, S, H, DV, generator=torch.Generator().manual_seed(S))).to(dtype)
+    if not causal:
+        mask = (mask.float() + mask.float().transpose(2, 3)).to(dtype)     # a full multiplier: decay on both sides of the diagonal
+    qc, kc, vc, mc = q.cuda(), k.cuda(), v.cuda(), mask.cuda()
+    rs = torch.empty(B, H, S, device="cuda")
+    print(f"retention bwd B{B} H{H} S{S} causal={causal} {dtype}", flush=True)
+    o = hb.attn_fwd(qc, kc, vc, family=hb.MA_ATTN_RETENTION, causal=causal, scale=1.0, score_mask=mc, row_scale=rs)
+    got = hb.attn_bwd(qc, kc, vc, o, dout.cuda(), rs, family=hb.MA_ATTN_RETENTION, causal=causal, scale=1.0,
+                      score_mask=mc, score_mask_t=mc.transpose(2, 3).contiguous())
+    torch.cuda.synchronize()
+    assert (rs > 1).any()
+    ref = oracle.attention_grads(oracle.retention_parallel, q, k, v, dout, mask=mask, freeze_r=True)
+    _check_grads(got, ref, "retention")
+
+
+def test_engine_retention_backward():
+    """o.backward(do) on the operator built from the spec (testing/test.py:107-125 does this for the softmax operator)."""
+    B, H, S, D, DV = 2, 4, 256, 256, 512
+    mod = specs.retention_parallel(B, H, S, D, DV)
+    q, k, v, mask = _inputs(B, H, S, D, DV, seed=5)
+    dout = (0.5 * torch.randn(B, S, H, DV, generator=torch.Generator().manual_seed(5))).bfloat16()
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = mod(qc, kc, vc, mask.cuda())
+    o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    ref = oracle.attention_grads(oracle.retention_parallel, q, k, v, dout, mask=mask, freeze_r=True)
+    _check_grads((qc.grad, kc.grad, vc.grad), ref, "engine retention")
+
+
+def test_retention_backward_needs_its_inputs():
+    hb = _hb()
+    q = torch.zeros(1, 64, 1, 256, device="cuda", dtype=torch.bfloat16)
+    v = torch.zeros(1, 64, 1, 512, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(hb.MetaAttentionError):
+        hb.attn_bwd(q, q, v, v, v, torch.ones(1, 1, 64, device="cuda"), family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0)
+
+
 def test_parallel_and_chunked_forms_agree_at_full_size():
     """B=8 H=16 S=2048 Dqk=256 Dv=512: the parallel operator (mask = gamma^(i-j)) times its
     row scale r is the un-normalised retention the chunked operator computes."""
