@@ -20,7 +20,10 @@ sigmoid_attention      element-wise closed form 1/(1+exp(-x)) brute force;
                        masked entries contribute exactly 0
 relu_attention         brute-force loops on tiny shapes
 retention_parallel     brute force fp64; clamp invariant (rows with
-                       sum|.|<1 stay un-normalised); all-ones mask special case
+                       sum|.|<1 stay un-normalised); all-ones mask special case;
+                       freeze_r (the gradient with the row scale held constant):
+                       autograd == the written-out dq, dk, dv; == the true
+                       gradient where the clamp holds r at 1
 retnet_chunked         3-way agreement: quadratic form == token recurrence
                        == chunked form for several chunk sizes (fp64)
 ssd_chunk_scan         3-way agreement: chunked reference == naive sequential
