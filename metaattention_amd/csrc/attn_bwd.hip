@@ -337,7 +337,10 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
   constexpr int BNW = 128, BMT = 32;   // keys per workgroup, query rows per tile
   constexpr int KS = DQK / 16, VS = DV / 16, QB = DQK / 32, VB = DV / 32;
   constexpr int QROW = DQK * 2, DOROW = DV * 2;
-  constexpr int QTILE = BMT * QROW, DOTILE = BMT * DOROW, STAGE = QTILE + DOTILE;
+  // a stage: the Q tile and the dO tile; behind both stages, lse and delta of each stage's 32 rows (softmax; 2 x 128
+  // bytes per stage -- not inside the stages: the swizzled reads address a tile as base XOR offset, which needs the
+  // tile bases aligned to the row size)
+  constexpr int QTILE = BMT * QROW, DOTILE = BMT * DOROW, STAGE = QTILE + DOTILE, ROWVALS = 2 * STAGE;
 
   extern __shared__ __align__(16) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
@@ -398,6 +401,14 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
     const char* dob = (const char*)((const T*)a.dout + (int64_t)b * a.dosb + (int64_t)h * a.dosh);
     dma_tile<QROW, 4>(qb, q_row_bytes, m0, a.Sq, lds0 + buf * STAGE, wave, lane);
     dma_tile<DOROW, 4>(dob, do_row_bytes, m0, a.Sq, lds0 + buf * STAGE + QTILE, wave, lane);
+    if constexpr (FAMILY == BF_SOFTMAX) {
+      // lse (lanes 0..31) and delta (lanes 32..63) of the tile's rows come with it: read from global memory inside
+      // the loop, their latency is not covered by the little work a tile is
+      if (wave == 0) {
+        const int64_t ri = ((int64_t)b * a.H + h) * a.Sq + min(m0 + (lane & 31), a.Sq - 1);
+        dma4((lane < 32 ? a.lse : (const float*)a.delta) + ri, lds0 + ROWVALS + buf * 256);
+      }
+    }
   };
 
   int step_next = next_step(0);
@@ -440,27 +451,16 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
     }
     // lse and delta of the rows this lane holds: m0 + 8q4 + 4g + {0..3}
     if constexpr (FAMILY == BF_SOFTMAX) {
-      const int64_t rbase = ((int64_t)b * a.H + h) * a.Sq;
-      if ((a.Sq & 3) == 0 && m0 + BMT <= a.Sq) {   // whole tile, 16-byte aligned groups of four rows
+      const uint32_t rv = lds0 + ROWVALS + buf * 256;
 #pragma unroll
-        for (int q4 = 0; q4 < 4; q4++) {
-          const f32x4 tl = *(const f32x4*)(a.lse + rbase + m0 + 8 * q4 + 4 * g);
-          const f32x4 td = *(const f32x4*)(a.delta + rbase + m0 + 8 * q4 + 4 * g);
+      for (int q4 = 0; q4 < 4; q4++) {
+        const f32x4 tl = lds_read<f32x4>(rv + (8 * q4 + 4 * g) * 4);
+        const f32x4 td = lds_read<f32x4>(rv + 128 + (8 * q4 + 4 * g) * 4);
 #pragma unroll
-          for (int i = 0; i < 4; i++) {
-            lse2[4 * q4 + i] = c_bias - tl[i] * kLog2e;   // what the row function adds to s * c_scale
-            dl[4 * q4 + i] = td[i];
-          }
+        for (int i = 0; i < 4; i++) {
+          lse2[4 * q4 + i] = c_bias - tl[i] * kLog2e;   // what the row function adds to s * c_scale
+          dl[4 * q4 + i] = td[i];
         }
-      } else {
-#pragma unroll
-        for (int q4 = 0; q4 < 4; q4++)
-#pragma unroll
-          for (int i = 0; i < 4; i++) {
-            const int m = min(m0 + 8 * q4 + 4 * g + i, a.Sq - 1);
-            lse2[4 * q4 + i] = c_bias - a.lse[rbase + m] * kLog2e;
-            dl[4 * q4 + i] = a.delta[rbase + m];
-          }
       }
     }
     const f32x16 s = mm_rows<T, DQK>(qbase, r, g, kf);     // S: lane = key n_lane, element jj = row m0 + 8(jj/4) + 4g + jj%4
@@ -528,7 +528,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
 template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
 static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   constexpr int DMAX = DQK > DV ? DQK : DV;
-  constexpr size_t tiles = 2 * (size_t)32 * (DQK + DV) * 2;
+  constexpr size_t tiles = 2 * ((size_t)32 * (DQK + DV) * 2 + 256);   // (+ the row values of the dk / dv kernels' stages)
   constexpr size_t ostage = 4 * 32 * (size_t)(DMAX + 16);
   constexpr size_t lds = tiles > ostage ? tiles : ostage;
   auto k1 = attn_bwd_dq_kernel<T, DQK, DV, FAMILY, CAUSAL>;

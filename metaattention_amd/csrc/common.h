@@ -100,6 +100,16 @@ __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
       : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr)
       : "memory");
 }
+// Direct-to-LDS load of 64 x 4 bytes (global_load_lds_dword): lane i's dword lands at lds_base + 4 i.
+__device__ __forceinline__ void dma4(const void* gptr, uint32_t lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dword %1, off\n\t"
+      :
+      : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(gptr)
+      : "memory");
+}
 // Same with a wave-uniform 64-bit base (scalar registers) plus a per-lane 32-bit byte offset.
 __device__ __forceinline__ void dma16_so(const void* base_uniform, uint32_t lane_off, uint32_t lds_base) {
   const uint64_t b = (uint64_t)(uintptr_t)base_uniform;
