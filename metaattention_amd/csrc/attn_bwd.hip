@@ -71,6 +71,23 @@ __device__ __forceinline__ void dma_tile(const char* src, int64_t row_stride, in
   }
 }
 
+// Retention: a wave's [32 rows x 32 columns] block of the score multiplier (64 bytes per row) by DMA into a 2 KB area of
+// its own, two instructions; the 16-byte chunk c of row r sits at position c ^ ((r >> 1) & 3) of the row, so that the
+// 8-byte reads of `mult_read` (lane: row r, columns 8 q4 + 4 g ..) spread over the banks.  `first` points at the wave's
+// first row and the block's first column; rows from `rows_left` on are clamped to the last one.
+template <typename T>
+__device__ __forceinline__ void mult_dma(const T* first, int64_t row_stride, int rows_left, uint32_t lds_base, int lane) {
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    const int row = (lane >> 2) + 16 * j, lc = (lane & 3) ^ ((row >> 1) & 3);
+    dma16(first + (int64_t)min(row, rows_left - 1) * row_stride + 8 * lc, lds_base + j * 1024);
+  }
+}
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::x4 mult_read(uint32_t lds_base, int r, int g, int q4) {
+  return lds_read<typename Elem<T>::x4>(lds_base + r * 64 + ((q4 ^ ((r >> 1) & 3)) << 4) + 8 * g);
+}
+
 // [32 x 32] += A B^T over DIM columns, A = the 32 rows of an LDS tile (row reads), B = fragments in registers
 template <typename T, int DIM>
 __device__ __forceinline__ f32x16 mm_rows(uint32_t tile, int r, int g, const typename Elem<T>::x8 (&bf)[DIM / 16]) {
@@ -222,9 +239,18 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
   int n_tiles = (a.Skv + BN - 1) / BN;
   if (CAUSAL) n_tiles = min(n_tiles, (mb * BM + BM + BN - 1) / BN);
 
+  // retention: whole tiles of the multiplier come with the K/V tile (a 2 KB area per wave and stage behind the stages);
+  // a partial last tile, or a tensor whose rows are not 16-byte aligned, is read from global memory as it is needed
+  constexpr int MULT = 2 * STAGE;
+  const bool mult_ok = FAMILY == BF_RETENTION && (a.sm_sq & 7) == 0 && (a.sm_sb & 7) == 0 && (a.sm_sh & 7) == 0 && ((uintptr_t)a.smask & 15) == 0;
   auto issue_tile = [&](int n0, int buf) {
     dma_tile<KROW, 4>(kb, k_row_bytes, n0, a.Skv, lds0 + buf * STAGE, wave, lane);
     dma_tile<VROW, 4>(vb, v_row_bytes, n0, a.Skv, lds0 + buf * STAGE + KTILE, wave, lane);
+    if constexpr (FAMILY == BF_RETENTION) {
+      if (mult_ok && n0 + BN <= a.Skv && m_wave < a.Sq)
+        mult_dma<T>((const T*)a.smask + (int64_t)b * a.sm_sb + (int64_t)h * a.sm_sh + (int64_t)m_wave * a.sm_sq + n0, a.sm_sq, a.Sq - m_wave,
+                    lds0 + MULT + (buf * 4 + wave) * 2048, lane);
+    }
   };
 
   f32x16 dq[QB];
@@ -260,14 +286,19 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
     // retention: the multipliers of this lane's 16 scores, requested before the products that hide their latency
     typename E::x4 mk[4];
     if constexpr (FAMILY == BF_RETENTION) {
+      if (mult_ok && n0 + BN <= a.Skv && m_wave < a.Sq) {
 #pragma unroll
-      for (int q4 = 0; q4 < 4; q4++) {
-        const int n = n0 + 8 * q4 + 4 * g;
-        if (n + 3 < a.Skv) {
-          mk[q4] = *(const typename E::x4*)(sm_row + n);
-        } else {
+        for (int q4 = 0; q4 < 4; q4++) mk[q4] = mult_read<T>(lds0 + MULT + (buf * 4 + wave) * 2048, r, g, q4);
+      } else {
 #pragma unroll
-          for (int i = 0; i < 4; i++) mk[q4][i] = n + i < a.Skv ? sm_row[n + i] : (T)0.f;
+        for (int q4 = 0; q4 < 4; q4++) {
+          const int n = n0 + 8 * q4 + 4 * g;
+          if (n + 3 < a.Skv) {
+            mk[q4] = *(const typename E::x4*)(sm_row + n);
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) mk[q4][i] = n + i < a.Skv ? sm_row[n + i] : (T)0.f;
+          }
         }
       }
     }
@@ -341,6 +372,8 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
   // bytes per stage -- not inside the stages: the swizzled reads address a tile as base XOR offset, which needs the
   // tile bases aligned to the row size)
   constexpr int QTILE = BMT * QROW, DOTILE = BMT * DOROW, STAGE = QTILE + DOTILE, ROWVALS = 2 * STAGE;
+  // retention: behind those, a 2 KB block of the transposed multiplier per wave and stage (see the dq kernel)
+  constexpr int MULT = ROWVALS + 512;
 
   extern __shared__ __align__(16) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
@@ -395,6 +428,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
       while (step < n_steps && !qbm[(int64_t)(hk * a.kv_group + step / t_count) * a.qbm_sh + t_first + step % t_count]) step++;
     return step;
   };
+  const bool mult_ok = FAMILY == BF_RETENTION && (a.smt_sk & 7) == 0 && (a.smt_sb & 7) == 0 && (a.smt_sh & 7) == 0 && ((uintptr_t)a.smask_t & 15) == 0;
   auto issue_step = [&](int step, int buf) {
     const int h = hk * a.kv_group + step / t_count, m0 = (t_first + step % t_count) * BMT;
     const char* qb = (const char*)((const T*)a.q + (int64_t)b * a.qsb + (int64_t)h * a.qsh);
@@ -408,6 +442,14 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
         const int64_t ri = ((int64_t)b * a.H + h) * a.Sq + min(m0 + (lane & 31), a.Sq - 1);
         dma4((lane < 32 ? a.lse : (const float*)a.delta) + ri, lds0 + ROWVALS + buf * 256);
       }
+    }
+    if constexpr (FAMILY == BF_RETENTION) {
+      // the row scales r of the tile's rows (twice: both halves of the wave fetch them) and, for whole tiles of an
+      // aligned tensor, each wave's block of the transposed multiplier
+      if (wave == 0) dma4(a.lse + ((int64_t)b * a.H + h) * a.Sq + min(m0 + (lane & 31), a.Sq - 1), lds0 + ROWVALS + buf * 256);
+      if (mult_ok && m0 + BMT <= a.Sq && n_wave < a.Skv)
+        mult_dma<T>((const T*)a.smask_t + (int64_t)b * a.smt_sb + (int64_t)h * a.smt_sh + (int64_t)n_wave * a.smt_sk + m0, a.smt_sk, a.Skv - n_wave,
+                    lds0 + MULT + (buf * 4 + wave) * 2048, lane);
     }
   };
 
@@ -430,23 +472,22 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
     // multiplier tensor: this key's row, indexed by query position)
     float lse2[16], dl[16];
     if constexpr (FAMILY == BF_RETENTION) {
-      const int64_t rbase = ((int64_t)b * a.H + h) * a.Sq;
+      const uint32_t rv = lds0 + ROWVALS + buf * 256;
       const T* smt_row = (const T*)a.smask_t + (int64_t)b * a.smt_sb + (int64_t)h * a.smt_sh + (int64_t)n_ld * a.smt_sk;
+      const bool staged = mult_ok && m0 + BMT <= a.Sq && n_wave < a.Skv;
 #pragma unroll
       for (int q4 = 0; q4 < 4; q4++) {
         const int m = m0 + 8 * q4 + 4 * g;
-        if ((a.Sq & 3) == 0 && m + 3 < a.Sq) {
-          const f32x4 tr = *(const f32x4*)(a.lse + rbase + m);
-          const typename E::x4 tm = *(const typename E::x4*)(smt_row + m);
-#pragma unroll
-          for (int i = 0; i < 4; i++) lse2[4 * q4 + i] = (float)tm[i] / tr[i];
+        const f32x4 tr = lds_read<f32x4>(rv + (8 * q4 + 4 * g) * 4);
+        typename E::x4 tm;
+        if (staged) {
+          tm = mult_read<T>(lds0 + MULT + (buf * 4 + wave) * 2048, r, g, q4);
         } else {
 #pragma unroll
-          for (int i = 0; i < 4; i++) {
-            const int mm = min(m + i, a.Sq - 1);
-            lse2[4 * q4 + i] = (float)smt_row[mm] / a.lse[rbase + mm];
-          }
+          for (int i = 0; i < 4; i++) tm[i] = smt_row[min(m + i, a.Sq - 1)];
         }
+#pragma unroll
+        for (int i = 0; i < 4; i++) lse2[4 * q4 + i] = (float)tm[i] * fast_rcp(tr[i]);
       }
     }
     // lse and delta of the rows this lane holds: m0 + 8q4 + 4g + {0..3}
@@ -528,7 +569,8 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
 template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
 static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   constexpr int DMAX = DQK > DV ? DQK : DV;
-  constexpr size_t tiles = 2 * ((size_t)32 * (DQK + DV) * 2 + 256);   // (+ the row values of the dk / dv kernels' stages)
+  // (+ the row values of the dk / dv kernels' stages and the retention family's multiplier blocks)
+  constexpr size_t tiles = 2 * (size_t)32 * (DQK + DV) * 2 + 512 + (FAMILY == BF_RETENTION ? 2 * 4 * 2048 : 0);
   constexpr size_t ostage = 4 * 32 * (size_t)(DMAX + 16);
   constexpr size_t lds = tiles > ostage ? tiles : ostage;
   auto k1 = attn_bwd_dq_kernel<T, DQK, DV, FAMILY, CAUSAL>;
