@@ -88,6 +88,15 @@ __device__ __forceinline__ typename Elem<T>::x4 mult_read(uint32_t lds_base, int
   return lds_read<typename Elem<T>::x4>(lds_base + r * 64 + ((q4 ^ ((r >> 1) & 3)) << 4) + 8 * g);
 }
 
+// Element-wise keep masks: a wave's [32 rows x 32 columns] block of mask bytes by DMA into a 1 KB area of its own (one
+// instruction: two lanes per row); lane (row r, half g) then reads the four bytes of columns 8 q4 + 4 g .. as one word.
+__device__ __forceinline__ void keep_dma(const uint8_t* first, int64_t row_stride, int rows_left, uint32_t lds_base, int lane) {
+  dma16(first + (int64_t)min(lane >> 1, rows_left - 1) * row_stride + 16 * (lane & 1), lds_base);
+}
+__device__ __forceinline__ uint32_t keep_read(uint32_t lds_base, int r, int g, int q4) {
+  return lds_read<uint32_t>(lds_base + r * 32 + 8 * q4 + 4 * g);
+}
+
 // [32 x 32] += A B^T over DIM columns, A = the 32 rows of an LDS tile (row reads), B = fragments in registers
 template <typename T, int DIM>
 __device__ __forceinline__ f32x16 mm_rows(uint32_t tile, int r, int g, const typename Elem<T>::x8 (&bf)[DIM / 16]) {
@@ -243,6 +252,7 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
   // a partial last tile, or a tensor whose rows are not 16-byte aligned, is read from global memory as it is needed
   constexpr int MULT = 2 * STAGE;
   const bool mult_ok = FAMILY == BF_RETENTION && (a.sm_sq & 7) == 0 && (a.sm_sb & 7) == 0 && (a.sm_sh & 7) == 0 && ((uintptr_t)a.smask & 15) == 0;
+  const bool keep_ok = FAMILY != BF_RETENTION && a.elem_mask && ((a.em_sq | a.em_sb | a.em_sh | (int64_t)(uintptr_t)a.elem_mask) & 15) == 0;
   auto issue_tile = [&](int n0, int buf) {
     dma_tile<KROW, 4>(kb, k_row_bytes, n0, a.Skv, lds0 + buf * STAGE, wave, lane);
     dma_tile<VROW, 4>(vb, v_row_bytes, n0, a.Skv, lds0 + buf * STAGE + KTILE, wave, lane);
@@ -250,6 +260,11 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
       if (mult_ok && n0 + BN <= a.Skv && m_wave < a.Sq)
         mult_dma<T>((const T*)a.smask + (int64_t)b * a.sm_sb + (int64_t)h * a.sm_sh + (int64_t)m_wave * a.sm_sq + n0, a.sm_sq, a.Sq - m_wave,
                     lds0 + MULT + (buf * 4 + wave) * 2048, lane);
+    } else {
+      // element-wise keep mask: whole tiles of a 16-byte aligned mask come with the K/V tile (same area, 1 KB per wave and stage)
+      if (keep_ok && n0 + BN <= a.Skv && m_wave < a.Sq)
+        keep_dma(a.elem_mask + (int64_t)b * a.em_sb + (int64_t)h * a.em_sh + (int64_t)m_wave * a.em_sq + n0, a.em_sq, a.Sq - m_wave,
+                 lds0 + MULT + (buf * 4 + wave) * 1024, lane);
     }
   };
 
@@ -314,7 +329,10 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
     // with an element-wise mask every tile does
     if ((CAUSAL && n0 + BN - 1 > m_wave) || n0 + BN > a.Skv || em_row) {
       uint32_t keep[4] = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};   // the bytes of this lane's four keys per group
-      if (em_row) {
+      if (keep_ok && n0 + BN <= a.Skv && m_wave < a.Sq) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) keep[q4] = keep_read(lds0 + MULT + (buf * 4 + wave) * 1024, r, g, q4);
+      } else if (em_row) {
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) {
           const int n = n0 + 8 * q4 + 4 * g;
@@ -428,6 +446,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
       while (step < n_steps && !qbm[(int64_t)(hk * a.kv_group + step / t_count) * a.qbm_sh + t_first + step % t_count]) step++;
     return step;
   };
+  const bool keep_ok = FAMILY != BF_RETENTION && a.elem_mask_t && ((a.emt_sk | a.emt_sb | a.emt_sh | (int64_t)(uintptr_t)a.elem_mask_t) & 15) == 0;
   const bool mult_ok = FAMILY == BF_RETENTION && (a.smt_sk & 7) == 0 && (a.smt_sb & 7) == 0 && (a.smt_sh & 7) == 0 && ((uintptr_t)a.smask_t & 15) == 0;
   auto issue_step = [&](int step, int buf) {
     const int h = hk * a.kv_group + step / t_count, m0 = (t_first + step % t_count) * BMT;
@@ -450,6 +469,11 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
       if (mult_ok && m0 + BMT <= a.Sq && n_wave < a.Skv)
         mult_dma<T>((const T*)a.smask_t + (int64_t)b * a.smt_sb + (int64_t)h * a.smt_sh + (int64_t)n_wave * a.smt_sk + m0, a.smt_sk, a.Skv - n_wave,
                     lds0 + MULT + (buf * 4 + wave) * 2048, lane);
+    } else {
+      // the transposed element-wise keep mask: whole tiles of a 16-byte aligned mask come with the Q/dO tile
+      if (keep_ok && m0 + BMT <= a.Sq && n_wave < a.Skv)
+        keep_dma(a.elem_mask_t + (int64_t)b * a.emt_sb + (int64_t)h * a.emt_sh + (int64_t)n_wave * a.emt_sk + m0, a.emt_sk, a.Skv - n_wave,
+                 lds0 + MULT + (buf * 4 + wave) * 1024, lane);
     }
   };
 
@@ -515,7 +539,10 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
     // with an element-wise mask every tile does
     if ((CAUSAL && n_wave + 31 > m0) || m0 + BMT > a.Sq || n_wave + 32 > a.Skv || a.elem_mask_t) {
       uint32_t keep[4] = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};   // the bytes of this lane's four rows per group
-      if (a.elem_mask_t) {
+      if (keep_ok && m0 + BMT <= a.Sq && n_wave < a.Skv) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) keep[q4] = keep_read(lds0 + MULT + (buf * 4 + wave) * 1024, r, g, q4);
+      } else if (a.elem_mask_t) {
         // the transposed mask: this key's row, indexed by query position
         const uint8_t* emt_row = a.elem_mask_t + (int64_t)b * a.emt_sb + (int64_t)h * a.emt_sh + (int64_t)n_ld * a.emt_sk;
 #pragma unroll
@@ -569,8 +596,8 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
 template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
 static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   constexpr int DMAX = DQK > DV ? DQK : DV;
-  // (+ the row values of the dk / dv kernels' stages and the retention family's multiplier blocks)
-  constexpr size_t tiles = 2 * (size_t)32 * (DQK + DV) * 2 + 512 + (FAMILY == BF_RETENTION ? 2 * 4 * 2048 : 0);
+  // (+ the row values of the dk / dv kernels' stages and the retention family's multiplier blocks / the keep-mask blocks)
+  constexpr size_t tiles = 2 * (size_t)32 * (DQK + DV) * 2 + 512 + (FAMILY == BF_RETENTION ? 2 * 4 * 2048 : 2 * 4 * 1024);
   constexpr size_t ostage = 4 * 32 * (size_t)(DMAX + 16);
   constexpr size_t lds = tiles > ostage ? tiles : ostage;
   auto k1 = attn_bwd_dq_kernel<T, DQK, DV, FAMILY, CAUSAL>;
