@@ -128,7 +128,7 @@ typedef struct ma_attn_bwd_params {
   const uint8_t* elem_mask;   int64_t em_stride_b, em_stride_h, em_stride_q;
   const uint8_t* elem_mask_t; int64_t emt_stride_b, emt_stride_h, emt_stride_k;
   /* optional tile masks for the masks above (0 = the tile keeps nothing and is skipped; a non-zero entry for a tile
-   * that keeps nothing is harmless), uint8/bool, strides in bytes, stride 0 broadcasts; give both or neither:
+   * that keeps nothing is harmless; 2 = the element mask keeps every score of the tile and is not consulted for it), uint8/bool, strides in bytes, stride 0 broadcasts; give both or neither:
    * kv_block_mask [1 or B, 1 or H, ceil(Sq/128), ceil(Skv/32)] (the forward pass's prefill form) for the dq kernel,
    * q_block_mask  [1 or B, 1 or H, ceil(Skv/128), ceil(Sq/32)] for the dk / dv kernels. */
   const uint8_t* kv_block_mask; int64_t kbm_stride_b, kbm_stride_h, kbm_stride_q;

@@ -303,10 +303,11 @@ class AttentionEngine:
         Bm, Hm = elem.shape[:2]
         elem_t = elem.transpose(2, 3)
 
-        def pool(m, r, c):                        # blocks of 128 rows x 32 columns, kept when any element is
+        def pool(m, r, c):                        # blocks of 128 rows x 32 columns: 0 nothing kept, 1 some, 2 every element
             rp = (r + 127) // 128 * 128
             m = torch.nn.functional.pad(m, (0, 0, 0, rp - r)) if rp != r else m
-            return m.reshape(Bm, Hm, rp // 128, 128, c // 32, 32).any(dim=5).any(dim=3).to(torch.uint8).contiguous()
+            m = m.reshape(Bm, Hm, rp // 128, 128, c // 32, 32)
+            return (m.any(dim=5).any(dim=3).to(torch.uint8) + m.all(dim=5).all(dim=3).to(torch.uint8)).contiguous()
 
         return dict(elem_mask=elem.to(torch.uint8).contiguous(), elem_mask_t=elem_t.to(torch.uint8).contiguous(),
                     kv_block_mask=pool(elem, Sq, Skv), q_block_mask=pool(elem_t, Skv, Sq))
@@ -327,8 +328,11 @@ class AttentionEngine:
             buf[..., :Skv] = dense
             pad = torch.zeros(Bm, Hm, sqp, nkp, dtype=torch.bool, device=device)
             pad[:, :, :Sq, :Skv] = dense
-            blocks = pad.view(Bm, Hm, sqp // 128, 128, nkp // 32, 32).any(dim=5).any(dim=3).to(torch.uint8).contiguous()
-            self._mask_tensors = [key, buf[..., :Skv], blocks, None]
+            tiles = pad.view(Bm, Hm, sqp // 128, 128, nkp // 32, 32)
+            blocks = tiles.any(dim=5).any(dim=3).to(torch.uint8).contiguous()
+            # for the backward kernels: 2 where the mask keeps every element of the tile (it is then not consulted there)
+            blocks_bwd = (blocks + tiles.all(dim=5).all(dim=3).to(torch.uint8)).contiguous()
+            self._mask_tensors = [key, buf[..., :Skv], blocks, None, blocks_bwd]
             if self._infer_blocks is not None:
                 # the attribute the reference keeps for operators whose mask is not the exact causal one
                 # (attn_engine.py:394-397): the mask_mod pooled to infer_mask_block_M x infer_mask_block_N blocks
@@ -345,9 +349,10 @@ class AttentionEngine:
                 skp, sqp = (Skv + 127) // 128 * 128, (Sq + 31) // 32 * 32
                 pad = torch.zeros(elem.shape[0], elem.shape[1], skp, sqp, dtype=torch.bool, device=device)
                 pad[:, :, :Skv, :Sq] = elem.transpose(2, 3) != 0
-                blocks_t = pad.view(elem.shape[0], elem.shape[1], skp // 128, 128, sqp // 32, 32).any(dim=5).any(dim=3)
-                self._mask_tensors[3] = (buf_t[..., :Sq], blocks_t.to(torch.uint8).contiguous())
-            return self._mask_tensors[1], self._mask_tensors[3][0], self._mask_tensors[2], self._mask_tensors[3][1]
+                tiles_t = pad.view(elem.shape[0], elem.shape[1], skp // 128, 128, sqp // 32, 32)
+                blocks_t = tiles_t.any(dim=5).any(dim=3).to(torch.uint8) + tiles_t.all(dim=5).all(dim=3).to(torch.uint8)
+                self._mask_tensors[3] = (buf_t[..., :Sq], blocks_t.contiguous())
+            return self._mask_tensors[1], self._mask_tensors[3][0], self._mask_tensors[4], self._mask_tensors[3][1]
         return self._mask_tensors[1], self._mask_tensors[2]
 
     # ------------------------------------------------------------------ MLA decode

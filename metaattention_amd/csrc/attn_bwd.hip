@@ -253,6 +253,8 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
   constexpr int MULT = 2 * STAGE;
   const bool mult_ok = FAMILY == BF_RETENTION && (a.sm_sq & 7) == 0 && (a.sm_sb & 7) == 0 && (a.sm_sh & 7) == 0 && ((uintptr_t)a.smask & 15) == 0;
   const bool keep_ok = FAMILY != BF_RETENTION && a.elem_mask && ((a.em_sq | a.em_sb | a.em_sh | (int64_t)(uintptr_t)a.elem_mask) & 15) == 0;
+  const uint8_t* bm_full = a.kv_block_mask ? a.kv_block_mask + (int64_t)b * a.kbm_sb + (int64_t)h * a.kbm_sh + (int64_t)mb * a.kbm_sq : nullptr;
+  auto tile_full = [&](int jt_) { return bm_full && bm_full[jt_] >= 2; };   // the element-wise mask keeps every score of the tile
   auto issue_tile = [&](int n0, int buf) {
     dma_tile<KROW, 4>(kb, k_row_bytes, n0, a.Skv, lds0 + buf * STAGE, wave, lane);
     dma_tile<VROW, 4>(vb, v_row_bytes, n0, a.Skv, lds0 + buf * STAGE + KTILE, wave, lane);
@@ -261,8 +263,9 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
         mult_dma<T>((const T*)a.smask + (int64_t)b * a.sm_sb + (int64_t)h * a.sm_sh + (int64_t)m_wave * a.sm_sq + n0, a.sm_sq, a.Sq - m_wave,
                     lds0 + MULT + (buf * 4 + wave) * 2048, lane);
     } else {
-      // element-wise keep mask: whole tiles of a 16-byte aligned mask come with the K/V tile (same area, 1 KB per wave and stage)
-      if (keep_ok && n0 + BN <= a.Skv && m_wave < a.Sq)
+      // element-wise keep mask: whole tiles of a 16-byte aligned mask come with the K/V tile (same area, 1 KB per wave and
+      // stage); a tile the block mask marks as kept in full (entry 2) needs none of it
+      if (keep_ok && n0 + BN <= a.Skv && m_wave < a.Sq && !tile_full(n0 / BN))
         keep_dma(a.elem_mask + (int64_t)b * a.em_sb + (int64_t)h * a.em_sh + (int64_t)m_wave * a.em_sq + n0, a.em_sq, a.Sq - m_wave,
                  lds0 + MULT + (buf * 4 + wave) * 1024, lane);
     }
@@ -327,9 +330,11 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
     }
     // only tiles that touch the diagonal or the end of the keys pay for the mask (the test is wave-uniform);
     // with an element-wise mask every tile does
-    if ((CAUSAL && n0 + BN - 1 > m_wave) || n0 + BN > a.Skv || em_row) {
+    const bool full = tile_full(n0 / BN);
+    if ((CAUSAL && n0 + BN - 1 > m_wave) || n0 + BN > a.Skv || (em_row && !full)) {
       uint32_t keep[4] = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};   // the bytes of this lane's four keys per group
-      if (keep_ok && n0 + BN <= a.Skv && m_wave < a.Sq) {
+      if (full) {
+      } else if (keep_ok && n0 + BN <= a.Skv && m_wave < a.Sq) {
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) keep[q4] = keep_read(lds0 + MULT + (buf * 4 + wave) * 1024, r, g, q4);
       } else if (em_row) {
@@ -441,6 +446,8 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
   const int64_t q_row_bytes = a.qss * 2, do_row_bytes = a.doss * 2;
   // tiles in which the mask keeps nothing for this workgroup's keys are never fetched
   const uint8_t* qbm = a.q_block_mask ? a.q_block_mask + (int64_t)b * a.qbm_sb + (int64_t)nb * a.qbm_sk : nullptr;
+  // (entry 2: the element-wise mask keeps every score of the tile)
+  auto step_full = [&](int step) { return qbm && qbm[(int64_t)(hk * a.kv_group + step / t_count) * a.qbm_sh + t_first + step % t_count] >= 2; };
   auto next_step = [&](int step) {
     if (qbm)
       while (step < n_steps && !qbm[(int64_t)(hk * a.kv_group + step / t_count) * a.qbm_sh + t_first + step % t_count]) step++;
@@ -471,7 +478,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
                     lds0 + MULT + (buf * 4 + wave) * 2048, lane);
     } else {
       // the transposed element-wise keep mask: whole tiles of a 16-byte aligned mask come with the Q/dO tile
-      if (keep_ok && m0 + BMT <= a.Sq && n_wave < a.Skv)
+      if (keep_ok && m0 + BMT <= a.Sq && n_wave < a.Skv && !step_full(step))
         keep_dma(a.elem_mask_t + (int64_t)b * a.emt_sb + (int64_t)h * a.emt_sh + (int64_t)n_wave * a.emt_sk + m0, a.emt_sk, a.Skv - n_wave,
                  lds0 + MULT + (buf * 4 + wave) * 1024, lane);
     }
@@ -537,9 +544,11 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
     x8 pf[2], dsf[2];
     // only tiles that touch the diagonal or an end of the sequences pay for the mask (the test is wave-uniform);
     // with an element-wise mask every tile does
-    if ((CAUSAL && n_wave + 31 > m0) || m0 + BMT > a.Sq || n_wave + 32 > a.Skv || a.elem_mask_t) {
+    const bool full = step_full(step);
+    if ((CAUSAL && n_wave + 31 > m0) || m0 + BMT > a.Sq || n_wave + 32 > a.Skv || (a.elem_mask_t && !full)) {
       uint32_t keep[4] = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};   // the bytes of this lane's four rows per group
-      if (keep_ok && m0 + BMT <= a.Sq && n_wave < a.Skv) {
+      if (full) {
+      } else if (keep_ok && m0 + BMT <= a.Sq && n_wave < a.Skv) {
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) keep[q4] = keep_read(lds0 + MULT + (buf * 4 + wave) * 1024, r, g, q4);
       } else if (a.elem_mask_t) {

@@ -261,11 +261,11 @@ def test_backward_tile_skipping_changes_nothing():
     g = torch.Generator().manual_seed(5)
     q, k, v, dout = (torch.randn(B, S, H, D, generator=g).bfloat16().cuda() for _ in range(4))
     i, j = torch.arange(S, device="cuda").view(S, 1), torch.arange(S, device="cuda").view(1, S)
-    keep = ((i >= j) & (i - j < 100)).to(torch.uint8).view(1, 1, S, S)
+    keep = ((i >= j) & (i - j < 300)).to(torch.uint8).view(1, 1, S, S)
     keep_t = keep.transpose(2, 3).contiguous()
     kbm = keep.view(1, 1, S // 128, 128, S // 32, 32).amax(dim=(3, 5)).contiguous()
     qbm = keep_t.view(1, 1, S // 128, 128, S // 32, 32).amax(dim=(3, 5)).contiguous()
-    assert int(kbm.sum()) < kbm.numel() // 3 and int(qbm.sum()) < qbm.numel() // 3
+    assert int(kbm.sum()) < kbm.numel() // 2 and int(qbm.sum()) < qbm.numel() // 2
     lse = torch.empty(B, H, S, device="cuda")
     o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=False, scale=D ** -0.5, row_scale=lse, elem_mask=keep)
     kw = dict(family=hb.MA_ATTN_SOFTMAX, causal=False, scale=D ** -0.5, elem_mask=keep, elem_mask_t=keep_t)
@@ -273,6 +273,14 @@ def test_backward_tile_skipping_changes_nothing():
     got = hb.attn_bwd(q, k, v, o, dout, lse, kv_block_mask=kbm, q_block_mask=qbm, **kw)
     torch.cuda.synchronize()
     for a, b_ in zip(got, ref):
+        assert torch.equal(a, b_)
+    # entry 2 = the mask keeps every score of the tile (the element mask is then not read for it): the same bits again
+    kbm2 = (kbm + keep.view(1, 1, S // 128, 128, S // 32, 32).amin(dim=(3, 5))).contiguous()
+    qbm2 = (qbm + keep_t.view(1, 1, S // 128, 128, S // 32, 32).amin(dim=(3, 5))).contiguous()
+    assert int((kbm2 == 2).sum()) > 0 and int((qbm2 == 2).sum()) > 0
+    got2 = hb.attn_bwd(q, k, v, o, dout, lse, kv_block_mask=kbm2, q_block_mask=qbm2, **kw)
+    torch.cuda.synchronize()
+    for a, b_ in zip(got2, ref):
         assert torch.equal(a, b_)
     with pytest.raises(hb.MetaAttentionError):
         hb.attn_bwd(q, k, v, o, dout, lse, kv_block_mask=kbm, q_block_mask=qbm, family=hb.MA_ATTN_SOFTMAX, causal=False, scale=D ** -0.5)
