@@ -35,8 +35,8 @@ sys.path.insert(0, os.path.join(ROOT, "metaattention_amd"))
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a
-# 1 GiB copy (profiles/attn_fwd_kernel_c2_softmax_sigmoid.md): 1290 MB read + 273 MB written
-ATTN_FWD_HBM_BYTES = 1.563e9
+# 1 GiB copy (profiles/attn_fwd_kernel_c2_softmax_sigmoid.md): 1291 MB read + 273 MB written
+ATTN_FWD_HBM_BYTES = 1.564e9
 
 
 def time_gpu(fn, steps, warmup, flush=None):
