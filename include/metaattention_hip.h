@@ -89,7 +89,8 @@ typedef struct ma_attn_params {
    * RETENTION.  With or without it, kv_block_mask may be the prefill form
    * [1 or B, 1 or heads, ceil(Sq/128), ceil(Skv/kv_block_size)] of the block-sparse prefill operator: set
    * kbm_stride_q (blocks of 128 query rows; strides 0 broadcast) and kbm_per_query_head = 1.  This form also goes
-   * with MA_MASK_CAUSAL. */
+   * with MA_MASK_CAUSAL.  Beside an elem_mask, a block entry of 2 says that the element mask keeps every score of the
+   * block: it is then not read for it (1, or any other non-zero value: read). */
   const uint8_t* elem_mask; int64_t em_stride_b, em_stride_h, em_stride_q;
   int64_t kbm_stride_q; int32_t kbm_per_query_head;
   /* optional; with ma_attn_workspace_bytes(&params) bytes, decode shapes (at most 32 query rows, SOFTMAX, no

@@ -227,12 +227,14 @@ class AttentionEngine:
             kw = dict(family=fam_code, causal=self.mask_kind == "causal", scale=form.scale, bias=form.bias,
                       bias_tensor=given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None)
             if self.mask_kind.startswith("other"):
-                elem, blocks = self._dense_mask(B, H, Sq, k.shape[1], q.device)
-                kw.update(elem_mask=elem, kv_block_mask=blocks, kv_block_size=32)
+                elem, _ = self._dense_mask(B, H, Sq, k.shape[1], q.device)
+                # (block entries 0 / 1 / 2: nothing, something, everything kept; the kernels skip the 0s and do not read
+                # the element mask for the 2s)
+                kw.update(elem_mask=elem, kv_block_mask=self._mask_tensors[4], kv_block_size=32)
             if prefill_blocks is not None:
                 ext = self._expand_block_mask(prefill_blocks, B, H, Sq, k.shape[1])
                 if "kv_block_mask" in kw:
-                    ext = ext & kw["kv_block_mask"]        # (the mask_mod's own block mask: broadcast over batch / heads)
+                    ext = ext * kw["kv_block_mask"]        # (the mask_mod's own block mask: broadcast over batch / heads)
                 kw.update(kv_block_mask=ext.contiguous(), kv_block_size=32)
             if sparse:
                 kw.update(kv_seqlens=cache_seqlens.to(torch.int32) if cache_seqlens is not None else None, kv_block_mask=block_mask,

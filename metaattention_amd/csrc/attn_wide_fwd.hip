@@ -126,6 +126,8 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
       while (jt < n_tiles && !bm_row[jt / tiles_per_block]) jt++;
     return jt;
   };
+  // (block mask entry 2, beside an element-wise mask: that mask keeps every score of the block and is not read for it)
+  auto tile_full = [&](int jt) { return em_row && bm_row && bm_row[jt / tiles_per_block] >= 2; };
 
   // DMA of one tile: each instruction moves 1 KB (1024 / row bytes tile rows); lane i fetches the
   // 16-byte chunk that belongs at physical position i of that KB.  Rows beyond the sequence are clamped
@@ -178,11 +180,13 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
 
   x4 mk_next[4];
   uint32_t keep_next[4] = {0, 0, 0, 0};
+  bool full_next = false;
   int jt = next_tile(t_begin);
   if (jt < n_tiles) {
     issue_tile(jt * BN, 0);
+    full_next = tile_full(jt);
     if constexpr (FAMILY == WF_RETENTION) load_mask(jt * BN, mk_next);
-    else if (em_row) load_keep(jt * BN, keep_next);
+    else if (em_row && !full_next) load_keep(jt * BN, keep_next);
   }
 
   for (int it = 0; jt < n_tiles; it++) {
@@ -198,9 +202,11 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
     uint32_t keep[4];
 #pragma unroll
     for (int q4 = 0; q4 < 4; q4++) keep[q4] = keep_next[q4];
+    const bool full = full_next;
     if (jt < n_tiles) {
+      full_next = tile_full(jt);
       if constexpr (FAMILY == WF_RETENTION) load_mask(jt * BN, mk_next);
-      else if (em_row) load_keep(jt * BN, keep_next);
+      else if (em_row && !full_next) load_keep(jt * BN, keep_next);
       issue_tile(jt * BN, buf ^ 1);
     }
     const uint32_t kbase = lds0 + buf * STAGE, vbase = kbase + KTILE;
@@ -241,7 +247,7 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
           if ((CAUSAL && n > m_lane) || n >= skv) s[jj] = -INFINITY;
         }
       }
-      if (em_row) {
+      if (em_row && !full) {
 #pragma unroll
         for (int jj = 0; jj < 16; jj++)
           if (((keep[jj >> 2] >> (8 * (jj & 3))) & 0xff) == 0) s[jj] = -INFINITY;

@@ -355,6 +355,25 @@ def test_engine_block_sparse_prefill(family, mask, D, S, bq, bk):
     oracle.assert_close(o1.float().cpu(), ref1, rtol=RTOL, atol=ATOL, mismatch_ratio=ratio)
 
 
+def test_blocks_kept_in_full_skip_the_element_mask():
+    """Beside an element-wise mask, a block entry of 2 means "every score of the block is kept": the mask is not read for
+    such blocks, and the output is the same bits as with entries of 1."""
+    hb = _hb()
+    B, H, S, D = 1, 2, 1024, 64
+    g = torch.Generator().manual_seed(9)
+    q, k, v = (torch.randn(B, S, H, D, generator=g).bfloat16().cuda() for _ in range(3))
+    i, j = torch.arange(S, device="cuda").view(S, 1), torch.arange(S, device="cuda").view(1, S)
+    keep = ((i >= j) & (i - j < 300)).to(torch.uint8).view(1, 1, S, S)
+    tiles = keep.view(1, 1, S // 128, 128, S // 32, 32)
+    any_, all_ = tiles.amax(dim=(3, 5)).contiguous(), tiles.amin(dim=(3, 5))
+    assert int(all_.sum()) > 0
+    kw = dict(family=hb.MA_ATTN_SOFTMAX, causal=False, scale=D ** -0.5, elem_mask=keep, kv_block_size=32)
+    o1 = hb.attn_fwd(q, k, v, kv_block_mask=any_, **kw)
+    o2 = hb.attn_fwd(q, k, v, kv_block_mask=(any_ + all_).contiguous(), **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2)
+
+
 def test_block_sparse_prefill_rejects_odd_blocks():
     mod = _sparse_prefill_engine("softmax", True, None, 1, 2, 512, 128)
     q = torch.zeros(1, 512, 2, 128, device="cuda", dtype=torch.bfloat16)
