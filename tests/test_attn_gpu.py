@@ -99,6 +99,26 @@ def test_softmax_work_distribution(B, H, S, causal):
         torch.testing.assert_close(lse[b:b + 1, h:h + 1].cpu(), lse_ref, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("B,H,S,causal", [(40, 16, 64, False), (40, 16, 96, True), (37, 9, 33, True), (40, 16, 128, False),
+                                          (40, 16, 160, True), (20, 16, 288, False), (24, 16, 300, True)])
+def test_softmax_many_short_items(B, H, S, causal):
+    """Several short work items per workgroup: the first sub-tiles of an item are fetched by the last steps of the item
+    before it (or, after an item of fewer than 4 sub-tiles, all at once), in every alignment of the ring; every row of
+    every item is checked."""
+    hb = _hb()
+    D = 128
+    g = torch.Generator().manual_seed(S + B)
+    q, k, v = (torch.randn(B, S, H, D, generator=g).bfloat16() for _ in range(3))
+    o = torch.full((B, S, H, D), float("nan"), device="cuda", dtype=torch.bfloat16)
+    lse = torch.full((B, H, S), float("nan"), device="cuda")
+    print(f"short items B{B} H{H} S{S} causal={causal}", flush=True)
+    hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_SOFTMAX, causal=causal, scale=1 / math.sqrt(D), out=o, row_scale=lse)
+    torch.cuda.synchronize()
+    ref, lse_ref = oracle.softmax_attention(q, k, v, causal=causal, return_lse=True)
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(lse.cpu(), lse_ref, rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_softmax_growing_and_jumping_scores(dtype):
     """Row maxima that keep growing along the kv axis (the reference point of the exponentials moves
