@@ -9,7 +9,7 @@
 // Mapping onto CDNA4 (wave64, v_mfma_f32_32x32x16):
 //   * a workgroup is 8 waves (two per SIMD, one workgroup per CU); each wave owns 32 query rows
 //     (block_M = 256) and every wave walks the same 32-row KV sub-tiles, which arrive in LDS by
-//     direct-to-LDS DMA through rings of 6 K and 6 V buffers (K runs 7, V 4 sub-tiles ahead; each wave
+//     direct-to-LDS DMA through rings of 6 K and 6 V buffers (K runs 6, V 4 sub-tiles ahead; each wave
 //     issues one K and one V instruction per sub-tile, spread between its MFMAs: a wave that issues a
 //     burst of loads stalls on the CU's vector memory path, so also the first sub-tiles of the NEXT work
 //     item are fetched one per step, by the last steps of the item before it);
@@ -23,18 +23,22 @@
 //     transposing LDS read (ds_read_b64_tr_b16);
 //   * both LDS tiles are XOR-swizzled at 16-byte granularity so the 128-bit K
 //     reads and the transposing V reads are bank-conflict free without padding;
-//   * software pipeline inside each wave, three sub-tiles deep.  Vector-ALU work overlaps matrix work only
-//     when the two are interleaved finely (about four VALU instructions fit behind one MFMA), and a wave
-//     that alternates long MFMA-only and VALU-only phases leaves the matrix pipe idle whenever its SIMD
-//     partner is in the same phase.  So step u of a wave runs, interleaved per MFMA pair,
-//         MFMAs   P(u-1) V(u-1)   and   K(u+2) Q^T
-//         VALU    exp / sum / convert of sub-tile u   and   running row maximum of sub-tile u+1,
-//     with the scores of three and the probabilities of two sub-tiles live in registers: by the time a
-//     sub-tile's exponentials start, its row maximum is already folded into the reference point, so the
-//     exponentials depend on nothing that the step itself computes and every wave's instruction stream
-//     looks the same at all times;
-//   * the reference point of the exponentials follows the running maximum lazily: it (and with it the
-//     accumulator) only moves when a row's maximum has grown by more than 2^8 (see `finish_step`).
+//   * two phases per sub-tile and wave, and the two waves of a SIMD in opposite phases.  Matrix phase of step u:
+//     the MFMAs of P(u-1) V(u-1) and K(u+1) Q^T back to back, their fragments read from LDS a few MFMAs ahead,
+//     nothing else.  Vector phase: the DMA instructions of the step, mask, exponentials, row sum, conversion of
+//     sub-tile u, and the first fragment requests of the next matrix phase.  There is one workgroup barrier per
+//     step; waves 0..3 pass it before their matrix phase, waves 4..7 between their matrix and their vector phase,
+//     so between two barriers one wave of every SIMD runs matrix-then-vector and the other vector-then-matrix.
+//     Timestamps inside the kernel: matrix phase 650 clocks (16 MFMAs), vector phase 850 (of them 200 in which the
+//     wave stands still while the CU's vector memory path takes its two DMA instructions, 480 of vector ALU: a
+//     v_exp_f32 holds the ALU for 16 clocks).  Interleaving both kinds of work inside each wave (one MFMA, a few
+//     vector instructions, ...) measured 4 % slower, a second barrier between the phases 2 % slower (the phases
+//     are not equally long, and every stall of one wave is then waited for by all);
+//   * scores and probabilities of two sub-tiles are live in registers (s[u & 1], p[u & 1]);
+//   * the reference point of the exponentials follows the running maximum lazily and optimistically: a
+//     step takes its exponentials relative to the reference as it stands and checks afterwards whether some
+//     row's scores exceeded it by more than 2^8; only then (rare) the reference moves, which is a cold path
+//     that rescales the accumulator and takes that sub-tile's exponentials again (see `move_ref`).
 #include "attn_fwd.h"
 
 #include <type_traits>
@@ -64,14 +68,14 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   using x4 = typename E::x4;
   using x2 = typename E::x2;
   constexpr int NW = 8, BM = 32 * NW, BN = 32, NBUF = ATTN_NBUF;
-  constexpr int DK_AHEAD = 7, DV_AHEAD = 4;   // step u issues the loads of K(u + 7) and V(u + 4)
+  constexpr int DK_AHEAD = 6, DV_AHEAD = 4;   // step u issues the loads of K(u + 6) and V(u + 4)
   constexpr int KS = DQK / 16;   // k-slices of the QK^T contraction
   constexpr int DB = DV / 32;    // 32-wide output column blocks
   constexpr int CPRK = DQK / 8, CPRV = DV / 8;  // 16-byte chunks per row
   constexpr int KROW = DQK * 2, VROW = DV * 2;
   constexpr int KTILE = BN * KROW, VTILE = BN * VROW;
   constexpr int NQK = KS, NPV = 2 * DB;                  // MFMAs per sub-tile
-  static_assert(NBUF == 6, "the step bodies are unrolled by ring slot, score buffer (3) and parity (2)");
+  static_assert(NBUF == 6, "the step bodies are unrolled by ring slot and by the parity of the score / probability buffers");
   static_assert(CPRK == 16 && CPRV == 16, "one DMA instruction (1 KB) covers 4 tile rows");
   static_assert(KTILE == NW * 1024 && VTILE == NW * 1024, "one K and one V DMA instruction per wave and sub-tile");
   static_assert(NQK == NPV && NQK + NPV == 16, "one MFMA pair per two score elements");
@@ -85,6 +89,7 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   // Waves w and w + 4 share a SIMD.  Their 32-row blocks are paired as (0,7) (1,6) (2,5) (3,4) so that under
   // a causal mask, where a block's work grows with its position, every SIMD gets the same amount.
   const int row_block = wave < 4 ? wave : 11 - wave;
+  const bool late = wave >= 4;   // passes the step's barrier between its two phases instead of before them
 
   // ---- per work item (one 256-row q block of one (batch, head)); see the item loop at the bottom
   int b = 0, h = 0, mb = 0, m_wave = 0, m_lane = 0;
@@ -111,15 +116,24 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   const uint32_t k_row_bytes = (uint32_t)(a.kss * 2), v_row_bytes = (uint32_t)(a.vss * 2);
   //      Positions from n_sub on fetch the next item's sub-tile `slot` (a position more than a turn of the ring past
   //      the end repeats an earlier one: the same bytes into the same slot).
-  auto issue_k_rt = [&](int su, uint32_t slot) __attribute__((always_inline)) {
+  const uint32_t k_lane_off = (uint32_t)tile_row * k_row_bytes + swz_lane, v_lane_off = (uint32_t)tile_row * v_row_bytes + swz_lane;
+  auto issue_rt = [&](int su, uint32_t slot, const char* cur, const char* nxt, uint32_t row_bytes, uint32_t lane_off, uint32_t lds_dst)
+      __attribute__((always_inline)) {
     const bool nx = su >= n_sub;
-    const uint32_t row = (uint32_t)min((nx ? (int)slot : su) * BN + tile_row, a.Skv - 1);
-    dma16_so(nx ? kbase_n : kbase, row * k_row_bytes + swz_lane, lds_k + slot * KTILE + wave * 1024);
+    const int row0 = (nx ? (int)slot : su) * BN;
+    const char* base = nx ? nxt : cur;
+    if (row0 + BN <= a.Skv) {   // (wave-uniform) whole sub-tile inside the sequence: scalar base, the lane's constant offset
+      dma16_so(base + (uint64_t)((uint32_t)row0 * row_bytes), lane_off, lds_dst);
+    } else {
+      const uint32_t row = (uint32_t)min(row0 + tile_row, a.Skv - 1);
+      dma16_so(base, row * row_bytes + swz_lane, lds_dst);
+    }
+  };
+  auto issue_k_rt = [&](int su, uint32_t slot) __attribute__((always_inline)) {
+    issue_rt(su, slot, kbase, kbase_n, k_row_bytes, k_lane_off, lds_k + slot * KTILE + wave * 1024);
   };
   auto issue_v_rt = [&](int su, uint32_t slot) __attribute__((always_inline)) {
-    const bool nx = su >= n_sub;
-    const uint32_t row = (uint32_t)min((nx ? (int)slot : su) * BN + tile_row, a.Skv - 1);
-    dma16_so(nx ? vbase_n : vbase, row * v_row_bytes + swz_lane, lds_v + slot * VTILE + wave * 1024);
+    issue_rt(su, slot, vbase, vbase_n, v_row_bytes, v_lane_off, lds_v + slot * VTILE + wave * 1024);
   };
 
   // ---- per-lane LDS read addresses: all lane-dependent parts, one register each; what is added per
@@ -148,14 +162,14 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   const float bias = a.bias + (a.bias_ptr ? *a.bias_ptr : 0.f);
   const float c_scale = a.scale * kLog2e;  // scores are handled in the log2 domain
   const float c_bias = bias * kLog2e;
-  float row_ref = -1e30f;  // reference point of the exponentials: a running max of (scale*s + bias) * log2e, moved lazily
+  float row_ref = 0.f;     // softmax: reference point of the exponentials, (scale * s + bias) * log2e of some earlier running max
   float row_sum = 0.f;     // this lane's share of the running sum (the other half lives in lane^32)
 
-  // scores s[u % 3] and probabilities p[u & 1] of sub-tile u.
+  // scores s[u & 1] and probabilities p[u & 1] of sub-tile u.
   // lane holds query row r; element jj of a sub-tile is kv row 8(jj/4) + 4g + jj%4.
   // p[par][sl] packs elements 8sl .. 8sl+7: the B operand of PV slice sl (k slot i of lane half g is
   // kv row 16sl + 8(i/4) + 4g + i%4, matched by the rows the transposing V reads fetch).
-  f32x16 s[3];
+  f32x16 s[2];
   u32x4 p[2][2];
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
@@ -173,11 +187,9 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
     }
   };
 
-  // one element of the sub-tile in s[SB]: score -> probability (and its contribution to the row sum)
-  auto prob_one = [&](auto sb_c, auto e_c, float sub, float& part) __attribute__((always_inline)) -> float {
+  // one score -> probability (and its contribution to the row sum); sub = c_bias - row_ref
+  auto prob_one = [&](float v, float sub, float& part) __attribute__((always_inline)) -> float {
 #pragma clang fp reassociate(off)   // keep the running sum a chain in element order
-    constexpr int SB = decltype(sb_c)::value, e = decltype(e_c)::value;
-    const float v = s[SB][e];
     if constexpr (FAMILY == FAM_SOFTMAX) {
       const float pe = fast_exp2(v * c_scale + sub);
       part += pe;
@@ -194,42 +206,47 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
     x2 pk;
     pk[0] = (T)pe0;
     pk[1] = (T)pe1;
-    p[PAR][e0 >> 3][(e0 & 7) >> 1] = __builtin_bit_cast(uint32_t, pk);
+    uint32_t w = __builtin_bit_cast(uint32_t, pk);
+    // (pinned where it stands: the cold path takes a step's probabilities again, and without this the compiler moves
+    // the first take, exponentials and all, from between the MFMAs to behind the branch around that path)
+    asm volatile("" : "+v"(w));
+    p[PAR][e0 >> 3][(e0 & 7) >> 1] = w;
   };
 
-  // Softmax bookkeeping once the raw maximum `mx` of a sub-tile is known, BEFORE that sub-tile's
-  // exponentials: the reference point only moves for rows whose maximum exceeds it by more than 2^8.
-  // Until then probabilities are taken relative to the stale reference (at most 256: exact in fp32, in
-  // range for bf16/fp16) and nothing needs rescaling; the final division by row_sum absorbs the offset.
-  // When rows move, everything accumulated relative to the old reference is rescaled: the accumulator,
-  // the row sum and the probabilities of the previous sub-tile, which are still waiting for their P V.
-  // Each row decides for itself (rows that stay multiply by exactly 1), so a row's result never depends
-  // on what other rows of its wave see.
-  auto fold_max = [&](auto pend_c, float mx) __attribute__((always_inline)) {
-    constexpr int PEND = decltype(pend_c)::value;   // parity of the pending probabilities
+  // Softmax, cold path.  A step takes the exponentials of its sub-tile relative to the reference point as it
+  // stands (at most 2^8 while the scores stay within 8 of it: exact in fp32, in range for bf16/fp16; the final
+  // division by row_sum absorbs the offset) and afterwards looks at the sub-tile's maximum `mx`.  Only if some
+  // row exceeded its reference by more than 8 does the step come here: such rows move their reference up to
+  // the new maximum, the accumulator and the row sum are rescaled, and the probabilities of this step's sub-tile
+  // (scores in s[SB], probabilities pending in p[PAR]) are taken again.  Each row decides for itself (rows that
+  // stay multiply by exactly 1), so a row's result never depends on what other rows of its wave see.
+  auto move_ref = [&](auto par_c, auto sb_c, float& part) __attribute__((always_inline)) {
+    constexpr int SB = decltype(sb_c)::value;
+    float mx = s[SB][0];
+#pragma unroll
+    for (int j = 1; j < 16; j++) mx = fmaxf(mx, s[SB][j]);
     float m_lo, m_hi;
     xhalf_pair(mx, m_lo, m_hi);
     const float cand = fmaxf(m_lo, m_hi) * c_scale + c_bias;
     const bool move = cand - row_ref > 8.f;
-    if (__builtin_expect(__any(move), 0)) {
-      const float corr = move ? fast_exp2(row_ref - cand) : 1.f;
-      row_ref = move ? cand : row_ref;
-      row_sum *= corr;
-      // In place by construction, and with the wait states that cover the longest MFMA-result-to-VALU
-      // hazard (only the compiler's own instructions get those for free).
-      asm volatile("s_nop 7\n s_nop 7\n s_nop 7");
+    const float corr = move ? fast_exp2(row_ref - cand) : 1.f;
+    row_ref = move ? cand : row_ref;
+    row_sum *= corr;
+    // In place by construction, and with the wait states that cover the longest MFMA-result-to-VALU
+    // hazard (only the compiler's own instructions get those for free).
+    asm volatile("s_nop 7\n s_nop 7\n s_nop 7");
 #pragma unroll
-      for (int i = 0; i < DB; i++)
+    for (int i = 0; i < DB; i++)
 #pragma unroll
-        for (int j = 0; j < 16; j++) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(o[i][j]) : "v"(corr));
-#pragma unroll
-      for (int sl = 0; sl < 2; sl++) {
-        x8 v = __builtin_bit_cast(x8, p[PEND][sl]);
-#pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = (T)((float)v[i] * corr);
-        p[PEND][sl] = __builtin_bit_cast(u32x4, v);
-      }
-    }
+      for (int j = 0; j < 16; j++) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(o[i][j]) : "v"(corr));
+    part = 0.f;
+    const float sub = c_bias - row_ref;
+    static_for<0, 8>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value;
+      const float pe0 = prob_one(s[SB][2 * i], sub, part);
+      const float pe1 = prob_one(s[SB][2 * i + 1], sub, part);
+      pack_pair(par_c, std::integral_constant<int, 2 * i>{}, pe0, pe1);
+    });
   };
 
   // K and V fragments travel through small register rings and are requested PF-1 MFMA pairs ahead, across
@@ -247,48 +264,47 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
     kf[I % PF] = lds_read<x8>(k_addr[I] + KSL * KTILE);
   };
 
-  // Step u of the software pipeline; SLOT = u % 6 is compile-time and fixes the ring slots, the score
-  // buffers (u % 3) and the probability buffers (u & 1):
+  // Step u of a wave, in two phases; SLOT = u % 6 is compile-time and fixes the ring slots and the score and
+  // probability buffers (u & 1).
+  // Matrix phase:
   //   O^T += V(u-1)^T P(u-1)^T   V ring slot SLOT-1, probabilities p[1-PAR]
-  //   s[(u+2) % 3] = K(u+2) Q^T  K ring slot SLOT+2
-  //   probabilities of sub-tile u from s[u % 3] into p[PAR]          (its maximum is already in row_ref)
-  //   mask and row maximum of sub-tile u+1 in s[(u+1) % 3], folded into row_ref at the end
-  // and, last, the first fragment requests of step u+1 (V(u), K(u+3)).
-  auto step = [&](auto slot_c, int u) __attribute__((always_inline)) {
+  //   s[1-PAR] = K(u+1) Q^T      K ring slot SLOT+1
+  auto g_phase = [&](auto slot_c) __attribute__((always_inline)) {
     constexpr int SLOT = decltype(slot_c)::value, PAR = SLOT & 1;
-    using ic = std::integral_constant<int, 0>;
-    constexpr auto par_c = std::integral_constant<int, PAR>{};
-    constexpr auto sb_exp_c = std::integral_constant<int, SLOT % 3>{};
-    constexpr auto sb_max_c = std::integral_constant<int, (SLOT + 1) % 3>{};
-    constexpr int SB_MAX = (SLOT + 1) % 3, SB_QK = (SLOT + 2) % 3;
     constexpr auto vs_c = std::integral_constant<int, (SLOT + NBUF - 1) % NBUF>{};
-    constexpr auto ks_c = std::integral_constant<int, (SLOT + 2) % NBUF>{};
-    constexpr auto vs_next_c = std::integral_constant<int, SLOT>{};
-    constexpr auto ks_next_c = std::integral_constant<int, (SLOT + 3) % NBUF>{};
-    (void)sizeof(ic);
-    if constexpr (FAMILY == FAM_SOFTMAX) apply_mask(sb_max_c, u + 1);
-    else apply_mask(sb_exp_c, u);
-    const float sub = c_bias - row_ref;
-    float part = 0.f, mx = -INFINITY;
+    constexpr auto ks_c = std::integral_constant<int, (SLOT + 1) % NBUF>{};
     static_for<0, NPV>([&](auto i_c) __attribute__((always_inline)) {
       constexpr int i = decltype(i_c)::value;
       if constexpr (i + PF - 1 < NPV) request(std::integral_constant<int, i + PF - 1>{}, vs_c, ks_c);
-      if constexpr (i == 1) issue_k_rt(u + DK_AHEAD, (SLOT + DK_AHEAD) % NBUF);
-      if constexpr (i == 5) issue_v_rt(u + DV_AHEAD, (SLOT + DV_AHEAD) % NBUF);
       __builtin_amdgcn_sched_barrier(0);
       x8 vf = __builtin_shufflevector(lo[i % PF], hi[i % PF], 0, 1, 2, 3, 4, 5, 6, 7);
       o[i % DB] = E::mfma32(vf, __builtin_bit_cast(x8, p[1 - PAR][i / DB]), o[i % DB]);
-      const float pe0 = prob_one(sb_exp_c, std::integral_constant<int, 2 * i>{}, sub, part);   // behind the PV MFMA
-      if constexpr (FAMILY == FAM_SOFTMAX) mx = fmaxf(fmaxf(mx, s[SB_MAX][2 * i]), s[SB_MAX][2 * i + 1]);
-      __builtin_amdgcn_sched_barrier(0);
-      s[SB_QK] = E::mfma32(kf[i % PF], qf[i], i == 0 ? zero16 : s[SB_QK]);
-      const float pe1 = prob_one(sb_exp_c, std::integral_constant<int, 2 * i + 1>{}, sub, part);   // behind the QK MFMA
-      pack_pair(par_c, std::integral_constant<int, 2 * i>{}, pe0, pe1);
+      s[1 - PAR] = E::mfma32(kf[i % PF], qf[i], i == 0 ? zero16 : s[1 - PAR]);
       __builtin_amdgcn_sched_barrier(0);
     });
+  };
+  // Vector phase: mask, probabilities and maximum of sub-tile u from s[PAR] into p[PAR]; the loads of K(u+6) and
+  // V(u+4); and, last, the first fragment requests of the next matrix phase (V(u), K(u+2)).
+  auto s_phase = [&](auto slot_c, int u) __attribute__((always_inline)) {
+    constexpr int SLOT = decltype(slot_c)::value, PAR = SLOT & 1;
+    constexpr auto par_c = std::integral_constant<int, PAR>{};
+    constexpr auto vs_next_c = std::integral_constant<int, SLOT>{};
+    constexpr auto ks_next_c = std::integral_constant<int, (SLOT + 2) % NBUF>{};
+    issue_k_rt(u + DK_AHEAD, (SLOT + DK_AHEAD) % NBUF);
+    issue_v_rt(u + DV_AHEAD, (SLOT + DV_AHEAD) % NBUF);
+    apply_mask(par_c, u);
+    float part = 0.f;
+    const float sub = c_bias - row_ref;
+    static_for<0, 8>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value;
+      const float pe0 = prob_one(s[PAR][2 * i], sub, part);
+      const float pe1 = prob_one(s[PAR][2 * i + 1], sub, part);
+      pack_pair(par_c, std::integral_constant<int, 2 * i>{}, pe0, pe1);
+    });
     if constexpr (FAMILY == FAM_SOFTMAX) {
+      asm volatile("" : "+v"(part));   // (as in pack_pair)
+      if (__builtin_expect(__any(!(part <= 4096.f)), 0)) move_ref(par_c, par_c, part);
       row_sum += part;
-      fold_max(par_c, mx);
     }
     static_for<0, PF - 1>([&](auto i_c) __attribute__((always_inline)) { request(i_c, vs_next_c, ks_next_c); });
   };
@@ -355,8 +371,8 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
     }
   };
 
-  // the Q rows as loaded by open_item -> fragments (lane: row r, columns 16ks + 8g ..), through this wave's rows of the
-  // output staging area (16-byte chunks XOR-swizzled by row, as the output uses it)
+  // the Q rows as loaded by open_item -> fragments (lane: row r, columns 16ks + 8g ..), through this
+  // wave's rows of the output staging area (16-byte chunks XOR-swizzled by row, as the output uses it)
   auto q_fragments = [&]() __attribute__((always_inline)) {
     static_assert(DQK == DV, "the staging rows hold one Q row each");
     const uint32_t qb = lds0 + NBUF * (KTILE + VTILE) + wave * 32 * VROW;
@@ -371,7 +387,7 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
 
   int stores_behind = 0;   // output stores this wave issued after the current item's first loads
   int t_cur = 2 * first;
-  // An item that nobody fetched ahead for (the first of the workgroup; the one after an item of fewer than 4 sub-tiles,
+  // An item that nobody fetched ahead for (the first of the workgroup; the one after an item of fewer than 5 sub-tiles,
   // whose few steps do not get round the ring): K(0..5) -> slots 0..5, V(0..3) -> slots 0..3.
   auto fetch_first = [&]() __attribute__((always_inline)) {
     static_for<0, NBUF>([&](auto t_c) __attribute__((always_inline)) {
@@ -392,15 +408,17 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
       for (int j = 0; j < 16; j++) o[i][j] = 0.f;
 #pragma unroll
     for (int i = 0; i < 2; i++) p[0][i] = p[1][i] = u32x4{0u, 0u, 0u, 0u};
-    row_ref = -1e30f;
     row_sum = 0.f;
 
-    // ---- schedule.  Step u (u = 0 .. last_sub + 1 for a wave) reads K(u+2), V(u-1) and the first fragments
-    //      of K(u+3), V(u).  The barrier at the top of step u therefore stands for: K(u+3) and V(u) have
-    //      landed for every wave, and every wave is done reading K(<=u+1) and V(<=u-2) -- the ring slots
-    //      that step u refills with K(u+7) and V(u+4).  A wave's loads complete in order and every step
-    //      issues K then V; K(u+3) and V(u) are the pair of step u-4, so at the top of step u the six
-    //      instructions of steps u-3 .. u-1 may still be in flight.
+    // ---- schedule.  Step u (u = 0 .. last_sub + 1 for a wave): the matrix phase reads K(u+1) and V(u-1), the vector
+    //      phase issues the loads of K(u+6) and V(u+4) and reads the first fragments of K(u+2) and V(u).  Barrier u
+    //      stands before the matrix phase of waves 0..3 and between the two phases of waves 4..7, so it has: every
+    //      matrix phase of step u-1 behind it (every wave is done reading K(<=u) and V(<=u-2), the ring slots that
+    //      the loads of step u refill), every vector phase of step u before it, and of the matrix phases of step u
+    //      those of waves 4..7 behind it.  What is read after it, K(u+1), K(u+2), V(u-1), V(u), must therefore have
+    //      landed for every wave: K(u+2) and V(u) are the pair of step u-4, a wave's loads complete in order, and at
+    //      barrier u every wave has issued the pairs of steps <= u-1, so the six instructions of steps u-3 .. u-1 may
+    //      still be in flight.
     // the item's first sub-tiles (fetched by the previous item's last steps) and Q rows must have landed; the previous
     // item's output stores, issued after them, need not
     if (stores_behind == 32 * CPRV / 64 + 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (32 * CPRV / 64 + 1));
@@ -415,29 +433,27 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
       const uint32_t row = (uint32_t)min(v_fix * BN + tile_row, a.Skv - 1);
       dma16_so(vbase, row * v_row_bytes + swz_lane, lds_v + (uint32_t)v_fix * VTILE + wave * 1024);
     }
-    {   // s[0] = K(0) Q^T with its maximum folded in, s[1] = K(1) Q^T; then K(6) may replace K(0)
+    {   // s[0] = K(0) Q^T.  Softmax: the row's first reference point is the maximum of this sub-tile (finite: every row
+        // sees key 0).
       x8 k0[KS];
   #pragma unroll
       for (int ks = 0; ks < KS; ks++) k0[ks] = lds_read<x8>(k_addr[ks]);
   #pragma unroll
       for (int ks = 0; ks < KS; ks++) s[0] = E::mfma32(k0[ks], qf[ks], ks == 0 ? zero16 : s[0]);
-  #pragma unroll
-      for (int ks = 0; ks < KS; ks++) k0[ks] = lds_read<x8>(k_addr[ks] + KTILE);
-  #pragma unroll
-      for (int ks = 0; ks < KS; ks++) s[1] = E::mfma32(k0[ks], qf[ks], ks == 0 ? zero16 : s[1]);
       if constexpr (FAMILY == FAM_SOFTMAX) {
         apply_mask(std::integral_constant<int, 0>{}, 0);
         float mx = s[0][0];
   #pragma unroll
         for (int j = 1; j < 16; j++) mx = fmaxf(mx, s[0][j]);
-        fold_max(std::integral_constant<int, 1>{}, mx);
+        float m_lo, m_hi;
+        xhalf_pair(mx, m_lo, m_hi);
+        row_ref = fmaxf(m_lo, m_hi) * c_scale + c_bias;
       }
     }
     wait_dma();
-    __syncthreads();   // every wave is done reading K(0), and V ring slot NBUF-1 is filled
-    issue_k_rt(NBUF, 0);
-    static_for<0, PF - 1>([&](auto i_c) __attribute__((always_inline)) {   // first fragments of step 0: zeros, K(2)
-      request(i_c, std::integral_constant<int, NBUF - 1>{}, std::integral_constant<int, 2>{});
+    __syncthreads();   // V ring slot NBUF-1 is filled (and every wave is done reading K(0): step 0 refills its slot)
+    static_for<0, PF - 1>([&](auto i_c) __attribute__((always_inline)) {   // first fragments of step 0: zeros, K(1)
+      request(i_c, std::integral_constant<int, NBUF - 1>{}, std::integral_constant<int, 1>{});
     });
     const int my_steps = last_sub + 2;   // steps 0 .. last_sub + 1
     for (int u0 = 0; u0 < my_steps; u0 += NBUF) {
@@ -445,11 +461,16 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
         constexpr int SLOT = decltype(slot_c)::value;
         const int u = u0 + SLOT;
         if (u < my_steps) {
-          if (u > 0) {
+          if (!late) {
             __builtin_amdgcn_s_waitcnt(0x0F70 | 6);   // vmcnt(6)
             __syncthreads();
           }
-          step(slot_c, u);
+          g_phase(slot_c);
+          if (late) {
+            __builtin_amdgcn_s_waitcnt(0x0F70 | 6);
+            __syncthreads();
+          }
+          s_phase(slot_c, u);
         }
       });
     }
@@ -473,7 +494,7 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
     const bool row_ok = m_lane < a.Sq;
     t_cur = t_next;
     if (t_cur < 2 * units) {
-      const bool unfetched = n_sub < 4;
+      const bool unfetched = n_sub < 5;
       open_item(t_cur);
       if (unfetched) {
         wait_dma();
