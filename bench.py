@@ -8,9 +8,11 @@ resident in HBM).  Prints ONE JSON line; `value` is algorithmic TFLOP/s
 carries the roofline of the dominant kernel, a CPU baseline (the oracle's
 restated PyTorch reference timed on this box's host cores over a bounded
 sample of the same workload) and, under "other_workloads", the remaining
-benchmark configurations, each with its own roofline fraction:
+benchmark configurations, each with its own roofline fraction (and, for C3, C4 and C5, the oracle timed on the host
+cores over a bounded sample as "cpu_baseline"):
 
   c2_sigmoid_causal   same shape, sigmoid(q.k*scale - log S) row function
+  c2_softmax_causal_operator  the headline workload through the operator AttentionEngine returns (with its allocations)
   c2_softmax_causal_bwd  backward of the headline workload (dq, dk, dv)
   c3_retnet_chunked   RetNet retention, chunked operator, B8 H16 S2048 Dqk256 Dv512
   c3_retnet_parallel  same shape, normalised parallel operator with a [1,H,S,S] decay mask
@@ -34,9 +36,21 @@ sys.path.insert(0, os.path.join(ROOT, "metaattention_amd"))
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a
-# 1 GiB copy (profiles/attn_fwd_kernel_c2_softmax_sigmoid.md): 1291 MB read + 273 MB written
-ATTN_FWD_HBM_BYTES = 1.564e9
+# HBM bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy: the
+# profile summary of that kernel holds the figure in a line "hbm_traffic_bytes_per_launch[<kernel>]: <bytes>"
+ATTN_FWD_PROFILE = os.path.join(ROOT, "profiles", "attn_fwd_kernel_c2_softmax_sigmoid.md")
+ATTN_FWD_KERNEL = "ma::attn_fwd_kernel<bf16, 128, 128, softmax, causal>"
+
+
+def profiled_traffic(path, kernel):
+    """(bytes per launch, file it was read from) from a profile summary, or (None, None)."""
+    try:
+        for ln in open(path):
+            if ln.startswith("hbm_traffic_bytes_per_launch[" + kernel + "]:"):
+                return float(ln.split(":", 3)[-1].strip()), os.path.relpath(path, ROOT)
+    except OSError:
+        pass
+    return None, None
 
 
 def time_gpu(fn, steps, warmup, flush=None):
@@ -92,6 +106,45 @@ def bench_softmax(steps, warmup, family="softmax"):
     ms = time_gpu(fn, steps, warmup)
     flops = 0.5 * 4.0 * B * H * S * S * D
     return dict(ms=ms, flops=flops, tflops=flops / ms / 1e9, shape=dict(B=B, H=H, S=S, D=D, DV=D, causal=True))
+
+
+def bench_softmax_operator(steps, warmup):
+    """The headline workload through the operator that AttentionEngine returns for the softmax spec (what a user of the
+    reference calls: it allocates its output and lse, reads the current stream, goes through ctypes)."""
+    import torch
+    from attn_engine import AttentionEngine, OnlineFunc
+    from core import CustomIO, SymbolicArray, SymbolScalar, Var, meta_tensor
+    B, H, S, D = 8, 32, 4096, 128
+
+    class OnlineSoftmax(OnlineFunc):   # the row function of examples/mha.py:21-71
+        def __init__(self):
+            super().__init__({"m": SymbolScalar("m", Var("-inf")), "r": SymbolScalar("r", Var("0.0"))},
+                             {"lse": SymbolScalar("lse", Var("0.0"))}, CustomIO())
+
+        @staticmethod
+        def online_fwd(scores, online_rowscales, b, h, q_idx):
+            m, r = online_rowscales["m"], online_rowscales["r"]
+            m_new = m.max(scores.get_reduce("max"))
+            scale_tmp = (m - m_new).exp()
+            r = r * scale_tmp
+            scores = (scores - m_new).exp()
+            r = r + scores.get_reduce("sum")
+            return scores, {"m": m_new, "r": r}, scale_tmp
+
+        @staticmethod
+        def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+            o_new = o / online_rowscales["r"]
+            lse = online_rowscales["r"].log() + online_rowscales["m"]
+            return o_new, {"lse": lse}
+
+    meta = tuple(meta_tensor(B, H, S, D, dtype=torch.bfloat16) for _ in range(3))
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=lambda s, io, b, h, q, k: s * (D ** -0.5),
+                          mask_mod=lambda b, h, q, k: q >= k, online_func=OnlineSoftmax())
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q, k, v = (torch.randn(B, S, H, D, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(3))
+    with torch.no_grad():
+        ms = time_gpu(lambda: mod(q, k, v), steps, warmup)
+    return _mfma_entry(ms, 0.5 * 4.0 * B * H * S * S * D, "the headline workload through the AttentionEngine operator (allocates o and lse per call)")
 
 
 def bench_softmax_bwd(steps, warmup):
@@ -153,7 +206,6 @@ def bench_retnet_chunked(steps, warmup):
 
 def bench_retnet_parallel(steps, warmup, backward=False):
     import torch
-    import oracle
     from metaattention_amd import hip_backend as hb
     B, H, S, D, DV = 8, 16, 2048, 256, 512
     g = torch.Generator(device="cuda").manual_seed(0)
@@ -239,6 +291,65 @@ def cpu_baseline_softmax():
                        f"os.cpu_count()={os.cpu_count()}")
 
 
+def _timed(fn):
+    t0 = time.perf_counter()
+    fn()
+    return time.perf_counter() - t0
+
+
+def cpu_baseline_retention_parallel():
+    """bench_utils.py:1158-1163 restated (oracle.retention_parallel), fp32, the whole workload."""
+    import torch
+    import oracle
+    B, H, S, D, DV = 8, 16, 2048, 256, 512
+    q, k, v, _ = oracle.inputs.retnet_inputs(B, H, S, D, DV, seed=0, layout="bshd")
+    mask = oracle.retention_decay_mask(H, S)
+    dt = _timed(lambda: oracle.retention_parallel(q, k, v, mask))
+    flops = 0.5 * 2.0 * B * H * S * S * (D + DV)
+    return dict(value=round(flops / dt / 1e12, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"B=8 of 8, H={H}, S={S}, Dqk={D}, Dv={DV}, fp32 oracle, {dt:.1f} s")
+
+
+def cpu_baseline_retnet_chunked():
+    """testing/test.py:738-747 restated (oracle.retnet_quadratic: what the reference's test checks the chunked operator
+    against), fp32, four batch entries of the 8; priced by the same chunk-64 FLOP convention as the GPU number."""
+    import torch
+    import oracle
+    B, H, T, Dk, Dv = 4, 16, 2048, 256, 512
+    q, k, v, _ = oracle.inputs.retnet_inputs(B, H, T, Dk, Dv, seed=0)
+    dt = _timed(lambda: oracle.retnet_quadratic(q, k, v))
+    flops = B * H * (2.0 * T * 64 * (Dk + Dv) + 4.0 * T * Dk * Dv)
+    return dict(value=round(flops / dt / 1e12, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"B=4 of 8, H={H}, S={T}, Dqk={Dk}, Dv={Dv}, fp32 oracle (quadratic form), {dt:.1f} s; credited with the chunk-64 "
+                       "algorithmic FLOPs of the GPU figure")
+
+
+def cpu_baseline_mamba2():
+    """testing/test.py:206-343 restated (oracle.ssd_chunk_scan_combined, chunk 256), fp32, four batch entries of the 8."""
+    import torch
+    import oracle
+    B, H, T, P, N, Lc = 4, 64, 2048, 64, 128, 256
+    Cm, Bm, x, dtt, A = oracle.inputs.mamba2_inputs(B, H, T, P, N, seed=0)
+    xs, dts = x.transpose(1, 2).contiguous(), dtt.transpose(1, 2).contiguous()
+    Bs, Cs = Bm.transpose(1, 2).contiguous(), Cm.transpose(1, 2).contiguous()
+    dt = _timed(lambda: oracle.ssd_chunk_scan_combined(xs, dts, A.view(-1), Bs, Cs, chunk_size=Lc))
+    flops = B * H * (2.0 * T * Lc * N + 2.0 * T * Lc * P + 4.0 * T * N * P)
+    return dict(value=round(flops / dt / 1e12, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"B=4 of 8, H={H}, S={T}, P={P}, N={N}, chunk {Lc}, fp32 oracle, {dt:.1f} s")
+
+
+def cpu_baseline_mla():
+    """testing/test.py:807-839 restated (oracle.mla_decode), fp32, the whole workload."""
+    import torch
+    import oracle
+    B, Hq, Skv, D, Dpe = 64, 128, 4096, 512, 64
+    q, q_pe, kv, k_pe = oracle.inputs.mla_inputs(B, Hq, Skv, D, Dpe, seed=0)
+    dt = _timed(lambda: oracle.mla_decode(q, q_pe, kv, k_pe))
+    nbytes = 2.0 * (kv.numel() + k_pe.numel() + q.numel() + q_pe.numel() + q.numel())
+    return dict(value=round(nbytes / dt / 1e9, 2), unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"B=64 of 64, Hq={Hq}, KV={Skv}, d={D}+{Dpe}, fp32 oracle, {dt:.1f} s; algorithmic bytes of the bf16 tensors over the time")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -273,6 +384,7 @@ def main():
     others = {}
     want = [w for w in args.only.split(",") if w]
     table = [("c2_sigmoid_causal", "sigmoid", lambda: (lambda r: _mfma_entry(r["ms"], r["flops"]))(bench_softmax(args.steps, args.warmup, "sigmoid"))),
+             ("c2_softmax_causal_operator", "operator", lambda: bench_softmax_operator(args.steps, args.warmup)),
              ("c2_softmax_causal_bwd", "bwd", lambda: bench_softmax_bwd(args.steps, args.warmup)),
              ("c3_retnet_chunked", "retnet", lambda: bench_retnet_chunked(args.steps, args.warmup)),
              ("c3_retnet_parallel", "retention", lambda: bench_retnet_parallel(args.steps, args.warmup)),
@@ -280,12 +392,17 @@ def main():
              ("c4_mamba2_ssd", "mamba", lambda: bench_mamba2(args.steps, args.warmup)),
              ("c5_mla_decode", "mla", lambda: bench_mla(args.steps, args.warmup)),
              ("gqa_decode", "decode", lambda: bench_decode(args.steps, args.warmup))]
+    cpu_legs = {"c3_retnet_chunked": cpu_baseline_retnet_chunked, "c3_retnet_parallel": cpu_baseline_retention_parallel,
+                "c4_mamba2_ssd": cpu_baseline_mamba2, "c5_mla_decode": cpu_baseline_mla}
     for name, key, fn in table:
         if want and (want == ["none"] or not any(key.startswith(w) or w in name for w in want)):
             continue
         others[name] = fn()
         torch.cuda.empty_cache()
+        if name in cpu_legs and not args.no_cpu_baseline:
+            others[name]["cpu_baseline"] = cpu_legs[name]()
 
+    traffic, traffic_from = profiled_traffic(ATTN_FWD_PROFILE, ATTN_FWD_KERNEL)
     line = {
         "metric": "fwd TFLOP/s + % bf16 MFMA peak (prefill/chunked); decode HBM GB/s % peak",
         "value": round(main_res["tflops"], 2),
@@ -297,9 +414,8 @@ def main():
         "config": {"workload": "causal softmax MHA forward, bf16 in / fp32 accumulate, B=8 H=32 S=4096 D=128",
                    **main_res["shape"]},
         "roofline": {"bound": "mfma", "achieved": round(main_res["tflops"], 2), "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(main_res["tflops"] / PEAK_BF16_TFLOPS, 4), "traffic": ATTN_FWD_HBM_BYTES,
-                     "kernel": "ma::attn_fwd_kernel<bf16, 128, 128, softmax, causal>",
-                     "flops_per_launch": main_res["flops"]},
+                     "unit": "TFLOP/s", "frac": round(main_res["tflops"] / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
+                     "traffic_from": traffic_from, "kernel": ATTN_FWD_KERNEL, "flops_per_launch": main_res["flops"]},
         "cpu_baseline": None,
         "other_workloads": others,
     }

@@ -8,7 +8,13 @@
  *   - plain pointers and sizes only; every pointer is a device pointer to
  *     memory the CALLER owns (inputs, outputs and workspace alike);
  *   - work is enqueued on the given hipStream_t and the call returns without
- *     synchronising; the library allocates nothing and keeps no state;
+ *     synchronising; the library allocates nothing.  The only state it keeps is what a first call caches per
+ *     device (raised LDS limits of its kernels, the number of CUs); concurrent first calls from several host
+ *     threads are safe, and so are concurrent calls afterwards;
+ *   - K and V (and the latent cache of the MLA operator) must be finite everywhere, also at positions a mask
+ *     hides: the kernels multiply masked positions by probabilities that are exactly 0 (and the first step of
+ *     a work item multiplies one resident V sub-tile of the same batch entry and head by zeros), and 0 x inf is
+ *     not 0.  The reference's kernels share this for every position inside a visited tile;
  *   - return value 0 on success, a negative MA_ERR_* code otherwise, in which
  *     case ma_last_error() (thread local) describes the problem;
  *   - strides are in ELEMENTS of the tensor's dtype; the innermost (feature)

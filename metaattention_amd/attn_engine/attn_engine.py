@@ -378,11 +378,13 @@ class AttentionEngine:
         from hip_backend import flash_mla_with_kvcache
         m = self.meta
         page = k_cache.shape[1]
-        pad = ((m["Skv"] + 255) // 256) * 256                     # as attn_engine.py:211-216
+        # The reference's table (attn_engine.py:211-216): sequence b owns pages b * pad / page .. of the pool, where pad is
+        # the cache length rounded up to 256, so the pool must hold B * pad / page pages.
+        pad = ((m["Skv"] + 255) // 256) * 256
+        if pad % page != 0 or k_cache.shape[0] < m["B"] * pad // page:
+            raise ValueError(f"paged MLA cache: expected a pool of at least {m['B']} x {pad} / {page} pages of {page} rows (cache length "
+                             f"{m['Skv']} rounded up to 256, as the reference lays it out), got {tuple(k_cache.shape)}")
         table = torch.arange(m["B"] * pad // page, dtype=torch.int32, device=q.device).view(m["B"], pad // page)
-        if pad != m["Skv"]:                                        # the pool holds Skv / page pages per sequence, in order
-            table = (torch.arange(m["B"], dtype=torch.int32, device=q.device).view(-1, 1) * (m["Skv"] // page)
-                     + torch.arange(pad // page, dtype=torch.int32, device=q.device).view(1, -1)).clamp_(max=k_cache.shape[0] - 1)
         lens = torch.full((m["B"],), m["Skv"], dtype=torch.int32, device=q.device)
         return flash_mla_with_kvcache(q, k_cache, table, lens, m["Dv"], softmax_scale=self.mla_scale)
 

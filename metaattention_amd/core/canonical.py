@@ -320,41 +320,68 @@ def _allclose(a, b) -> bool:
 # ---------------------------------------------------------------------------
 # mask_mod
 # ---------------------------------------------------------------------------
+class _IndexNotToBeRead:
+    """Stands in for the batch / head index of a mask_mod: any use of it raises."""
+
+    def _used(self, *a, **k):
+        raise _IndexWasRead()
+
+    __eq__ = __ne__ = __lt__ = __le__ = __gt__ = __ge__ = __add__ = __radd__ = __sub__ = __rsub__ = __mul__ = __rmul__ = _used
+    __truediv__ = __rtruediv__ = __floordiv__ = __rfloordiv__ = __mod__ = __rmod__ = __and__ = __rand__ = __or__ = __ror__ = _used
+    __xor__ = __rxor__ = __neg__ = __invert__ = __index__ = __int__ = __float__ = __bool__ = __getitem__ = __hash__ = _used
+    __torch_function__ = classmethod(lambda cls, *a, **k: (_ for _ in ()).throw(_IndexWasRead()))
+
+
+class _IndexWasRead(Exception):
+    pass
+
+
+# a mask_mod that reads its batch / head index is compared over every (batch, head) pair when the whole mask has at
+# most this many elements; beyond that it is taken to depend on them
+_MASK_COMPARE_LIMIT = 1 << 30
+
+
 def classify_mask(mask_mod, B, H, Sq, Skv, block_M=128, block_N=128) -> str:
     """"none" | "causal" | "other" | "other_bh".  Evaluates ``mask_mod`` densely on index grids on
-    the CPU (as the reference does at block granularity, lower.py:723-740) and compares with the
-    exact causal pattern on a sample of (batch, head) pairs.  "other": some other pattern, the same
-    for every sampled (batch, head); "other_bh": it depends on batch or head.  Both run through an
-    element-wise keep mask built by the caller (the reference generates the mask_mod's code into
-    its block-sparse kernel instead, blockattn_tl.py:176-190)."""
-    from .transform.core import create_mask
+    the CPU (as the reference does, over all of B and H, at block granularity: lower.py:723-740) and
+    compares with the exact causal pattern.  "other": some other pattern, the same for every (batch,
+    head); "other_bh": it depends on batch or head.  Both run through an element-wise keep mask built by
+    the caller (the reference generates the mask_mod's code into its block-sparse kernel instead,
+    blockattn_tl.py:176-190).
+
+    Whether the pattern depends on (batch, head) is decided, not sampled: a mask_mod that never touches
+    its b and h arguments (found by calling it with stand-ins that raise on any use) is evaluated once;
+    one that does is evaluated for every pair and compared with the first, and where that would be more
+    than 2^30 elements it counts as depending on them (always correct, possibly a larger keep mask than
+    needed)."""
     if mask_mod is None:
         return "none"
     qi = torch.arange(Sq).view(Sq, 1)
     kj = torch.arange(Skv).view(1, Skv)
-    causal = qi >= kj
-    kinds = set()
-    first, same = None, True
-    for b in sorted({0, B - 1}):
-        for h in sorted({0, H // 2, H - 1}):
-            m = mask_mod(torch.tensor(b), torch.tensor(h), qi, kj)
-            m = m if torch.is_tensor(m) else torch.full((Sq, Skv), bool(m))
-            m = m.expand(Sq, Skv)
-            if first is None:
-                first = m
-            elif not torch.equal(m, first):
-                same = False
-            if Sq == Skv and torch.equal(m, causal):
-                kinds.add("causal")
-            elif bool(m.all()):
-                kinds.add("none")
-            else:
-                kinds.add("other")
-    if kinds == {"causal"}:
+
+    def dense(b, h):
+        m = mask_mod(b, h, qi, kj)
+        m = m if torch.is_tensor(m) else torch.full((Sq, Skv), bool(m))
+        return m.to(torch.bool).expand(Sq, Skv)
+
+    try:
+        first = dense(_IndexNotToBeRead(), _IndexNotToBeRead())
+        reads_bh = False
+    except Exception:   # the stand-in was used (or handed to something that refuses it)
+        first = dense(torch.tensor(0), torch.tensor(0))
+        reads_bh = True
+    if reads_bh and B * H > 1:
+        if B * H * Sq * Skv > _MASK_COMPARE_LIMIT:
+            return "other_bh"
+        for b in range(B):
+            for h in range(H):
+                if (b or h) and not torch.equal(dense(torch.tensor(b), torch.tensor(h)), first):
+                    return "other_bh"
+    if Sq == Skv and torch.equal(first, qi >= kj):
         return "causal"
-    if kinds == {"none"}:
+    if bool(first.all()):
         return "none"
-    return "other" if same else "other_bh"
+    return "other"
 
 
 # ---------------------------------------------------------------------------

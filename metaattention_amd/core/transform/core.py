@@ -10,9 +10,9 @@ API surface of attention_engine/core/transform/core.py:36-349 and :352-506:
 A trace is the graph of ``SymbolScalar`` objects linked through ``prev``; each
 carries the op tag in ``code.type``.  Nothing here emits source text: the
 trace is consumed by the canonicaliser, which selects a pre-built kernel, and
-by the spec interpreter.  Forward only: the reverse-mode pass of the
-reference (:119-199) belongs to the backward kernels, which this package does
-not have.
+by the spec interpreter.  The backward kernels of the library hold each
+family's derivative themselves, so the reverse-mode pass the reference runs
+over the trace (:119-199) is not needed to build them.
 """
 from __future__ import annotations
 

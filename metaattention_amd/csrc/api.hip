@@ -107,7 +107,7 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
                                        (hipStream_t)stream);
   if (rc == -2)
     return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: no kernel for family %d, Dqk=%d, Dv=%d", p->family, p->dim_qk, p->dim_v);
-  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_attn_fwd: launch failed: %s", hipGetErrorString(hipGetLastError()));
+  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_attn_fwd: launch failed: %s", hipGetErrorString(ma::t_hip_error));
   return MA_OK;
 }
 
@@ -190,7 +190,7 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
   a.smask_t = p->score_mask_t; a.smt_sb = p->smt_stride_b; a.smt_sh = p->smt_stride_h; a.smt_sk = p->smt_stride_k;
   const int rc = ma::attn_bwd_dispatch(a, p->family, p->mask == MA_MASK_CAUSAL, p->dtype == MA_BF16, p->dim_qk, p->dim_v, (hipStream_t)stream);
   if (rc == -2) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: no kernel for family %d, Dqk=%d, Dv=%d", p->family, p->dim_qk, p->dim_v);
-  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_attn_bwd: launch failed: %s", hipGetErrorString(hipGetLastError()));
+  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_attn_bwd: launch failed: %s", hipGetErrorString(ma::t_hip_error));
   return MA_OK;
 }
 
@@ -240,17 +240,19 @@ int ma_linear_fwd(const ma_linear_params* p, ma_stream_t stream) {
   const int rc = ma::linear_fwd_dispatch(a, p->dim_k, p->segments, p->workspace, p->workspace_bytes, (hipStream_t)stream, nullptr);
   if (rc == -2)
     return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: no kernel for dim_k=%d (128 or 256) / dim_v=%d (multiple of 64)", p->dim_k, p->dim_v);
-  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_linear_fwd: launch failed: %s", hipGetErrorString(hipGetLastError()));
+  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_linear_fwd: launch failed: %s", hipGetErrorString(ma::t_hip_error));
   return MA_OK;
 }
 
-// Split count: enough workgroups to fill the 256 CUs once, each split a whole
-// number of 64-row tiles, and never more splits than tiles.
+// Split count: enough workgroups to fill the device's CUs once (256 assumed where no device can be asked), each split a
+// whole number of 64-row tiles, and never more splits than tiles.
 int ma_mla_choose_split(const ma_mla_params* p) {
   if (!p || p->batch <= 0 || p->heads_q <= 0 || p->seqlen_kv <= 0) return 1;
   const int head_blocks = (p->heads_q + 127) / 128;
   const int tiles = (p->seqlen_kv + 63) / 64;
-  int split = 256 / (p->batch * head_blocks);
+  int cus = ma::device_cus();
+  if (cus <= 0) cus = 256;
+  int split = cus / (p->batch * head_blocks);
   if (split < 1) split = 1;
   if (split > tiles) split = tiles;
   if (split > 64) split = 64;
@@ -263,9 +265,8 @@ static int mla_split_of(const ma_mla_params* p) { return p->num_split > 0 ? p->n
 // (flash_api.cpp:39 with this library's block of heads).
 int ma_mla_num_sm_parts(int heads_q) {
   if (heads_q <= 0) return 0;
-  int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-    cus = 256;
+  int cus = ma::device_cus();
+  if (cus <= 0) cus = 256;
   const int parts = cus / ((heads_q + 127) / 128);
   return parts < 1 ? 1 : parts;
 }
@@ -276,7 +277,7 @@ int ma_mla_get_metadata(const int32_t* kv_seqlens, int batch, int num_sm_parts, 
   if (batch <= 0 || num_sm_parts <= 0) return fail(MA_ERR_INVALID_ARG, "ma_mla_get_metadata: batch and num_sm_parts must be positive");
   // blocks of 64 tokens and 5 blocks of fixed cost per batch entry, as kernels/config.h:6,11
   if (ma::mla_plan_dispatch(kv_seqlens, batch, num_sm_parts, 64, 5, tile_scheduler_metadata, num_splits, (hipStream_t)stream) != 0)
-    return fail(MA_ERR_LAUNCH, "ma_mla_get_metadata: launch failed: %s", hipGetErrorString(hipGetLastError()));
+    return fail(MA_ERR_LAUNCH, "ma_mla_get_metadata: launch failed: %s", hipGetErrorString(ma::t_hip_error));
   return MA_OK;
 }
 
@@ -349,7 +350,7 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
   }
   const int rc = ma::mla_decode_dispatch(a, p->dtype == MA_BF16, p->dim, p->dim_pe, (hipStream_t)stream);
   if (rc == -2) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: only dim=512, dim_pe=64 is in the kernel library (got %d, %d)", p->dim, p->dim_pe);
-  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_mla_decode: launch failed: %s", hipGetErrorString(hipGetLastError()));
+  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_mla_decode: launch failed: %s", hipGetErrorString(ma::t_hip_error));
   return MA_OK;
 }
 

@@ -614,20 +614,15 @@ static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   constexpr bool SPLIT = DQK + DV >= 256 && (DQK + DV < 512 || DQK + DV > 512);
   auto k2 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL, SPLIT ? 1 : 3>;
   auto k3 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL, 2>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
-    if (hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
-    if (SPLIT && hipFuncSetAttribute((const void*)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (allow_lds(lds_ok, lds, k1, k2, k3) != 0) return -1;
   AttnBwdArgs args = a;
   args.num_blocks = (a.Sq + 127) / 128;
   hipLaunchKernelGGL(k1, dim3((unsigned)(args.num_blocks * a.B * a.H)), dim3(256), lds, stream, args);
   args.num_blocks = (a.Skv + 127) / 128;
   hipLaunchKernelGGL(k2, dim3((unsigned)(args.num_blocks * a.B * a.Hkv)), dim3(256), lds, stream, args);
   if (SPLIT) hipLaunchKernelGGL(k3, dim3((unsigned)(args.num_blocks * a.B * a.Hkv)), dim3(256), lds, stream, args);
-  return hipGetLastError() == hipSuccess ? 0 : -1;
+  return launch_status();
 }
 
 template <typename T, int DQK, int DV>

@@ -568,26 +568,18 @@ static int launch(const AttnArgs& a, hipStream_t stream) {
   constexpr size_t tiles = NBUF * (size_t)BN * (DQK + DV) * 2;
   constexpr size_t lds = tiles + 8 * 32 * (size_t)DV * 2;   // rings + output staging
   auto kern = attn_fwd_kernel<T, DQK, DV, FAMILY, CAUSAL>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (allow_lds(lds_ok, lds, kern) != 0) return -1;
   // the kernel addresses K and V rows with 32-bit byte offsets from the (batch, head) plane
   if ((uint64_t)a.Skv * (uint64_t)a.kss * 2 >= (1ull << 32) || (uint64_t)a.Skv * (uint64_t)a.vss * 2 >= (1ull << 32)) return -2;
   AttnArgs args = a;
   args.num_m_blocks = (a.Sq + BM - 1) / BM;
-  static int num_cus = 0;
-  if (num_cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -1;
-    num_cus = prop.multiProcessorCount;
-  }
+  const int num_cus = device_cus();
+  if (num_cus <= 0) return -1;
   const int n_items = args.num_m_blocks * a.B * a.H;
   const unsigned grid = (unsigned)(n_items < num_cus ? n_items : num_cus);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, stream, args);
-  return hipGetLastError() == hipSuccess ? 0 : -1;
+  return launch_status();
 }
 
 template <typename T, int DQK, int DV>

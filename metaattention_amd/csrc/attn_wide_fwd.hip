@@ -390,11 +390,8 @@ static int launch_wide(const AttnArgs& a, hipStream_t stream) {
   constexpr size_t ostage = NW * 32 * (size_t)(DV + 16);
   constexpr size_t lds = tiles > ostage ? tiles : ostage;
   auto kern = attn_wide_fwd_kernel<T, DQK, DV, FAMILY, CAUSAL, NW>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (allow_lds(lds_ok, lds, kern) != 0) return -1;
   AttnArgs args = a;
   if (args.n_split < 1) args.n_split = 1;
   args.num_m_blocks = (a.Sq + 32 * NW - 1) / (32 * NW);
@@ -403,7 +400,7 @@ static int launch_wide(const AttnArgs& a, hipStream_t stream) {
     const int64_t rows = (int64_t)a.B * a.H * a.Sq;
     hipLaunchKernelGGL((attn_split_combine_kernel<T, DV>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, args);
   }
-  return hipGetLastError() == hipSuccess ? 0 : -1;
+  return launch_status();
 }
 
 // Decode shapes: at most 32 query rows per (batch, head), softmax, no structural mask.  Splits are chosen

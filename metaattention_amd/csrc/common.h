@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "host_util.h"
+
 namespace ma {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;

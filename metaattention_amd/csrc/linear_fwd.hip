@@ -555,21 +555,21 @@ struct Config {
   static constexpr int64_t ws_wave_floats = (int64_t)(DK / 32) * 16 * 64;
 
   static bool prepare(int& resident, int& cus) {
-    static int s_resident = -1, s_cus = 0;
-    if (s_resident < 0) {
-      const void* kerns[3] = {(const void*)linear_fwd_kernel<DK, NWH, HG, 0>, (const void*)linear_fwd_kernel<DK, NWH, HG, 1>,
-                              (const void*)linear_fwd_kernel<DK, NWH, HG, 2>};
-      for (const void* kp : kerns)
-        if (hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return false;
-      int dev = 0, n = 0, r = 0;
-      if (hipGetDevice(&dev) != hipSuccess) return false;
-      if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return false;
-      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, linear_fwd_kernel<DK, NWH, HG, 2>, 64 * NW, lds) != hipSuccess) return false;
-      s_cus = n;
-      s_resident = r < 1 ? 1 : r;
+    // (threads that meet in a first call compute the same numbers; a device other than the first one asked is assumed to
+    // be of the same kind)
+    static std::atomic<uint64_t> lds_ok{0};
+    static std::atomic<int> s_resident{-1};
+    if (allow_lds(lds_ok, lds, linear_fwd_kernel<DK, NWH, HG, 0>, linear_fwd_kernel<DK, NWH, HG, 1>, linear_fwd_kernel<DK, NWH, HG, 2>) != 0)
+      return false;
+    cus = device_cus();
+    if (cus <= 0) return false;
+    int r = s_resident.load(std::memory_order_relaxed);
+    if (r < 0) {
+      if (hip_check(hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, linear_fwd_kernel<DK, NWH, HG, 2>, 64 * NW, lds)) != 0) return false;
+      r = r < 1 ? 1 : r;
+      s_resident.store(r, std::memory_order_relaxed);
     }
-    resident = s_resident;
-    cus = s_cus;
+    resident = r;
     return true;
   }
 
@@ -619,7 +619,7 @@ struct Config {
       hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 1>), dim3(groups * (args.nseg - 1)), dim3(64 * NW), lds, stream, args);
       hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 2>), dim3(groups * args.nseg), dim3(64 * NW), lds, stream, args);
     }
-    return hipGetLastError() == hipSuccess ? 0 : -1;
+    return launch_status();
   }
 };
 }  // namespace

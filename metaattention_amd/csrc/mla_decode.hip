@@ -380,14 +380,17 @@ __global__ __launch_bounds__(256) void mla_combine_kernel(const MlaArgs a) {
     for (int s2 = tid; s2 < ns; s2 += 64) mx = fmaxf(mx, lp[(int64_t)s2 * a.Hq]);
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+    // (every piece empty: mx = -inf; the weights are then 0, the output zeros and the lse -inf, as the unsplit launch gives)
+    const float mref = mx == -INFINITY ? 0.f : mx;
     float sum = 0.f;
-    for (int s2 = tid; s2 < ns; s2 += 64) sum += fast_exp2(lp[(int64_t)s2 * a.Hq] - mx);
+    for (int s2 = tid; s2 < ns; s2 += 64) sum += fast_exp2(lp[(int64_t)s2 * a.Hq] - mref);
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, 64);
+    const float inv = sum > 0.f ? 1.f / sum : 0.f;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const T* pp = (const T*)a.o_part + (first * a.Hq + head) * D + tid * 8;
     for (int s2 = 0; s2 < ns; s2++) {
-      const float w = fast_exp2(lp[(int64_t)s2 * a.Hq] - mx) / sum;
+      const float w = fast_exp2(lp[(int64_t)s2 * a.Hq] - mref) * inv;
       const x8 v = *(const x8*)(pp + (int64_t)s2 * a.Hq * D);
 #pragma unroll
       for (int i = 0; i < 8; i++) acc[i] += (float)v[i] * w;
@@ -396,7 +399,7 @@ __global__ __launch_bounds__(256) void mla_combine_kernel(const MlaArgs a) {
 #pragma unroll
     for (int i = 0; i < 8; i++) w[i] = (T)acc[i];
     *(x8*)((T*)a.o + (int64_t)b * a.osb + (int64_t)head * a.osh + tid * 8) = w;
-    if (a.lse && tid == 0) a.lse[(int64_t)b * a.Hq + head] = (mx + fast_log2(sum)) * kLn2;
+    if (a.lse && tid == 0) a.lse[(int64_t)b * a.Hq + head] = sum > 0.f ? (mx + fast_log2(sum)) * kLn2 : -INFINITY;
     return;
   }
   // lane s of the wave holds the log-sum-exp of split s (at most 64 splits here): one load, wave reductions
@@ -404,11 +407,12 @@ __global__ __launch_bounds__(256) void mla_combine_kernel(const MlaArgs a) {
   float mx = my;
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
-  const float e = tid < ns ? fast_exp2(my - mx) : 0.f;
+  // (every piece empty: mx = -inf; weights 0, output zeros, lse -inf, as the unsplit launch gives)
+  const float e = (tid < ns && mx != -INFINITY) ? fast_exp2(my - mx) : 0.f;
   float sum = e;
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, 64);
-  const float wgt = e / sum;
+  const float wgt = sum > 0.f ? e / sum : 0.f;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const T* pp = (const T*)a.o_part + (first * a.Hq + head) * D + tid * 8;
   int s0 = 0;
@@ -433,7 +437,7 @@ __global__ __launch_bounds__(256) void mla_combine_kernel(const MlaArgs a) {
 #pragma unroll
   for (int i = 0; i < 8; i++) w[i] = (T)acc[i];
   *(x8*)((T*)a.o + (int64_t)b * a.osb + (int64_t)head * a.osh + tid * 8) = w;
-  if (a.lse && tid == 0) a.lse[(int64_t)b * a.Hq + head] = (mx + fast_log2(sum)) * kLn2;
+  if (a.lse && tid == 0) a.lse[(int64_t)b * a.Hq + head] = sum > 0.f ? (mx + fast_log2(sum)) * kLn2 : -INFINITY;
 }
 
 // The work plan of get_mla_metadata.cu:8-75, one lane: cache blocks of block_n tokens plus a fixed overhead per batch
@@ -482,7 +486,7 @@ __global__ __launch_bounds__(64) void mla_plan_kernel(const int32_t* seqlens, in
 int mla_plan_dispatch(const int32_t* seqlens, int batch, int parts, int block_n, int overhead_blocks, int32_t* meta, int32_t* splits,
                       hipStream_t stream) {
   hipLaunchKernelGGL(mla_plan_kernel, dim3(1), dim3(64), 0, stream, seqlens, batch, parts, block_n, overhead_blocks, meta, splits);
-  return hipGetLastError() == hipSuccess ? 0 : -1;
+  return launch_status();
 }
 
 template <typename T>
@@ -490,26 +494,22 @@ static int launch_t(const MlaArgs& a, hipStream_t stream) {
   constexpr size_t lds = NSTAGE * (size_t)STAGE + NW * (size_t)XCHG;
   auto kern = mla_split_kernel<T, false>;
   auto kern_planned = mla_split_kernel<T, true>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
-    if (hipFuncSetAttribute((const void*)kern_planned, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return -1;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (allow_lds(lds_ok, lds, kern, kern_planned) != 0) return -1;
   MlaArgs args = a;
   args.head_blocks = (a.Hq + HB - 1) / HB;
   if (a.plan_meta) {
     hipLaunchKernelGGL(kern_planned, dim3((unsigned)(a.plan_parts * args.head_blocks)), dim3(64 * NW), lds, stream, args);
-    if (hipGetLastError() != hipSuccess) return -1;
+    if (launch_status() != 0) return -1;
     hipLaunchKernelGGL(mla_combine_kernel<T>, dim3((unsigned)(((int64_t)a.B * a.Hq + 3) / 4)), dim3(256), 0, stream, args);
-    return hipGetLastError() == hipSuccess ? 0 : -1;
+    return launch_status();
   }
   const unsigned grid = (unsigned)(a.B * a.num_split * args.head_blocks);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, args);
-  if (hipGetLastError() != hipSuccess) return -1;
+  if (launch_status() != 0) return -1;
   if (a.num_split > 1) {
     hipLaunchKernelGGL(mla_combine_kernel<T>, dim3((unsigned)(((int64_t)a.B * a.Hq + 3) / 4)), dim3(256), 0, stream, a);
-    if (hipGetLastError() != hipSuccess) return -1;
+    if (launch_status() != 0) return -1;
   }
   return 0;
 }

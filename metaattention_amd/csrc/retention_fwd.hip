@@ -249,15 +249,12 @@ __global__ __launch_bounds__(64 * RP_NW, 2) void retention_pair_fwd_kernel(const
 template <typename T, bool CAUSAL>
 static int launch_pair(const AttnArgs& a, hipStream_t stream) {
   auto kern = retention_pair_fwd_kernel<T, CAUSAL>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RP_LDS) != hipSuccess) return -1;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (allow_lds(lds_ok, RP_LDS, kern) != 0) return -1;
   AttnArgs args = a;
   args.num_m_blocks = (a.Sq + RP_BM - 1) / RP_BM;
   hipLaunchKernelGGL(kern, dim3((unsigned)(args.num_m_blocks * a.B * a.H)), dim3(64 * RP_NW), RP_LDS, stream, args);
-  return hipGetLastError() == hipSuccess ? 0 : -1;
+  return launch_status();
 }
 
 // returns 0 ok, -1 launch failure

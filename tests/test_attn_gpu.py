@@ -57,6 +57,24 @@ def test_softmax_full_size_property():
         oracle.assert_close(o[b:b + 1, :, h:h + 1].float().cpu(), ref, rtol=RTOL, atol=ATOL)
 
 
+def test_sigmoid_full_size():
+    """The sigmoid variant of the benchmark configuration at its full size (B8 H32 S4096 D128, causal,
+    sigmoid(q.k * scale - log S)): three (batch, head) slices against the oracle at atol 2e-2 / rtol 1e-2, every
+    output finite, and row 0 = sigmoid(score) * v[0] exactly as the oracle has it."""
+    hb = _hb()
+    B, H, S, D = 8, 32, 4096, 128
+    g = torch.Generator(device="cuda").manual_seed(1)
+    q, k, v = (torch.randn(B, S, H, D, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(3))
+    scale, bias = 1 / math.sqrt(D), -math.log(S)
+    o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SIGMOID, causal=True, scale=scale, bias=bias)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all()
+    for b, h in [(0, 0), (7, 31), (4, 13)]:
+        ref = oracle.sigmoid_attention(q[b:b + 1, :, h:h + 1].cpu(), k[b:b + 1, :, h:h + 1].cpu(), v[b:b + 1, :, h:h + 1].cpu(),
+                                       bias, causal=True, softmax_scale=scale)
+        oracle.assert_close(o[b:b + 1, :, h:h + 1].float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
 def test_causal_mask_is_exact():
     """Future keys must have exactly zero influence: poisoning k/v at positions
     > i must not change row i bit-for-bit."""

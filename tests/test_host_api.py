@@ -60,6 +60,21 @@ def test_classify_mask():
     assert classify_mask(lambda b, h, q, k: (q >= k) & (q - k < 16), 2, 4, 64, 64) == "other"  # sliding window
     assert classify_mask(lambda b, h, q, k: (q >= k) & (h > 0), 1, 2, 64, 64) == "other_bh"    # depends on the head
     assert classify_mask(lambda b, h, q, k: q >= k, 1, 1, 64, 128) == "other"                  # "causal" needs equal lengths
+    # a mask that is special for one head or one batch entry only, neither the first, the middle nor the last one
+    assert classify_mask(lambda b, h, q, k: (q >= k) & ((h != 1) | (k > 3)), 2, 8, 64, 64) == "other_bh"
+    assert classify_mask(lambda b, h, q, k: (q >= k) | (b == 1), 5, 2, 64, 64) == "other_bh"
+    doc = torch.tensor([[0] * 32 + [1] * 32, [0] * 20 + [1] * 44, [0] * 32 + [1] * 32])   # per-batch document ids, first == last
+    assert classify_mask(lambda b, h, q, k: doc[b, q] == doc[b, k], 3, 2, 64, 64) == "other_bh"
+    # reads b and h but does not depend on them: found by comparing every (batch, head)
+    assert classify_mask(lambda b, h, q, k: (q >= k) & (b >= 0) & (h * 0 == 0), 3, 5, 64, 64) == "causal"
+    # too large to compare: counts as depending on (batch, head)
+    import core.canonical as cn
+    lim, cn._MASK_COMPARE_LIMIT = cn._MASK_COMPARE_LIMIT, 1000
+    try:
+        assert classify_mask(lambda b, h, q, k: (q >= k) & (b >= 0), 3, 5, 64, 64) == "other_bh"
+        assert classify_mask(lambda b, h, q, k: q >= k, 3, 5, 64, 64) == "causal"   # never touches b, h: one evaluation decides
+    finally:
+        cn._MASK_COMPARE_LIMIT = lim
 
 
 def test_canonical_score_forms():

@@ -136,6 +136,31 @@ def test_engine_paged_mla_backend():
     torch.testing.assert_close(lse.cpu()[:, :, 0], lse_ref, rtol=1e-4, atol=1e-4)
 
 
+def test_engine_paged_mla_backend_ragged_length():
+    """A cache length that is not a multiple of 256: the reference's block table gives sequence b the pages from
+    b * pad / 64 on, pad = the length rounded up to 256 (attn_engine.py:211-216), so the pool is laid out that way;
+    a pool too small for that layout is refused."""
+    from attn_engine import AttentionEngine
+    from core import CustomIO, meta_tensor
+    import specs
+    B, Hq, Skv, pad = 3, 128, 200, 256
+    meta = (meta_tensor(B, Hq, 1, 576, dtype=torch.bfloat16), meta_tensor(B, 1, Skv, 576, dtype=torch.bfloat16),
+            meta_tensor(B, 1, Skv, 512, dtype=torch.bfloat16))
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=lambda s, io, b, h, q, k: s * (576 ** -0.5), mask_mod=None,
+                          online_func=specs.OnlineSoftmax(), kv_shared=True, backend="cute")
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn(B, 1, Hq, 576, generator=g).bfloat16()
+    cache = torch.randn(B * pad // 64, 64, 1, 576, generator=g).bfloat16()
+    out, lse = mod(q.cuda(), cache.cuda())
+    torch.cuda.synchronize()
+    rows = cache.view(B, pad, 1, 576)[:, :Skv]
+    ref, lse_ref = oracle.mla_decode(q[..., :512], q[..., 512:], rows[..., :512], rows[..., 512:], return_lse=True)
+    oracle.assert_close(out.float().cpu(), ref, rtol=1e-2, atol=2e-2)
+    torch.testing.assert_close(lse.cpu()[:, :, 0], lse_ref, rtol=1e-4, atol=1e-4)
+    with pytest.raises(ValueError):
+        mod(q.cuda(), cache[:B * Skv // 64].cuda())
+
+
 @pytest.mark.parametrize("seed", [0, 1, 2, 3])
 def test_mla_plan_kernel_matches_the_oracle(seed):
     """get_mla_metadata (cute_template_kvshared/kernels/get_mla_metadata.cu:8-75) is integer work: bit-exact."""
@@ -189,6 +214,27 @@ def test_planned_paged_mla_decode(B, Hq, parts, maxlen):
         ref, lse_ref = oracle.paged_mla_decode(q[b:b + 1], cache, table[b:b + 1], lens[b:b + 1])
         oracle.assert_close(out[b:b + 1].float().cpu(), ref, rtol=1e-2, atol=2e-2)
         torch.testing.assert_close(lse[b:b + 1].cpu(), lse_ref, rtol=1e-4, atol=1e-4)
-    keep = lens > 0
-    torch.testing.assert_close(out[keep.cuda()].float(), out_u[keep.cuda()].float(), rtol=2e-2, atol=2e-2)
-    torch.testing.assert_close(lse[keep.cuda()], lse_u[keep.cuda()], rtol=1e-4, atol=1e-4)
+    # the launch without a plan: same results, empty entries included (zeros and lse = -inf from its combine kernel too)
+    torch.testing.assert_close(out.float(), out_u.float(), rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(lse, lse_u, rtol=1e-4, atol=1e-4)
+    assert torch.isfinite(out_u.float()).all()
+
+
+@pytest.mark.parametrize("num_split", [0, 1, 3, 8])
+def test_mla_decode_with_an_empty_cache_entry(num_split):
+    """kv_seqlens with a zero in it through the uniform launch, unsplit and split: that batch entry gets zeros and
+    lse = -inf (every piece of it is empty, so the combine kernel has nothing to weigh), the others are unaffected."""
+    hb = _hb()
+    B, Hq, Skv = 4, 128, 640
+    q, q_pe, kv, k_pe = inputs.mla_inputs(B, Hq, Skv, 512, 64, seed=3)
+    lens = torch.tensor([Skv, 0, 37, 300], dtype=torch.int32)
+    lse = torch.full((B, Hq), float("nan"), device="cuda")
+    o = hb.mla_decode(q.cuda(), q_pe.cuda(), kv.cuda(), k_pe.cuda(), scale=SCALE, num_split=num_split, lse=lse,
+                      kv_seqlens=lens.cuda())
+    torch.cuda.synchronize()
+    assert torch.count_nonzero(o[1]) == 0 and torch.isinf(lse[1]).all() and (lse[1] < 0).all()
+    for b in (0, 2, 3):
+        n = int(lens[b])
+        ref, lse_ref = oracle.mla_decode(q[b:b + 1], q_pe[b:b + 1], kv[b:b + 1, :n], k_pe[b:b + 1, :n], return_lse=True)
+        oracle.assert_close(o[b:b + 1].float().cpu(), ref, rtol=1e-2, atol=2e-2)
+        torch.testing.assert_close(lse[b:b + 1].cpu(), lse_ref.view(1, Hq), rtol=1e-4, atol=1e-4)
