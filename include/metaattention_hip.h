@@ -235,6 +235,19 @@ int ma_mla_choose_split(const ma_mla_params* p);
 size_t ma_mla_workspace_bytes(const ma_mla_params* p);
 int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream);
 
+/* ma_mla_decode for callers that cannot allocate device memory and have no workspace at hand (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose operators
+ * allocate their partial results on every call.  Same arguments and results as ma_mla_decode, except that p->workspace is
+ * ignored: the partial results of the kv splits go to an array inside the library, ma_mla_noalloc_max_workspace() bytes
+ * (40 MiB) per GPU, held until the process ends.  A call whose ma_mla_workspace_bytes(p) exceeds that returns
+ * MA_ERR_WORKSPACE.  The call itself allocates nothing and synchronises nothing.  All calls on one GPU share the array:
+ * calls that overlap on one GPU (different streams, different threads) race; calls on one stream do not.  Every slot a
+ * call reads it has written before, so nothing needs clearing between calls.  The first call on a device looks the
+ * array's address up (and, if it is the library's first call, makes the runtime load the code object): make that call
+ * outside graph capture. */
+size_t ma_mla_noalloc_max_workspace(void);
+int ma_mla_decode_noalloc(const ma_mla_params* p, ma_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

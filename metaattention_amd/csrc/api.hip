@@ -6,6 +6,7 @@
 #include "linear_fwd.h"
 #include "mla_decode.h"
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -352,6 +353,49 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
   if (rc == -2) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: only dim=512, dim_pe=64 is in the kernel library (got %d, %d)", p->dim, p->dim_pe);
   if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_mla_decode: launch failed: %s", hipGetErrorString(ma::t_hip_error));
   return MA_OK;
+}
+
+// ---- ma_mla_decode_noalloc: ma_mla_decode with the library's own scratch array as the workspace ----
+// The array lives in the code object's global segment: each GPU the library runs on holds its own copy, at its own
+// address, until the process ends.  In host code the array's name is only a handle for hipGetSymbolAddress (passing it to
+// a kernel would hand the kernel a host-side address): the device address is looked up once per device, with that
+// device current, and everything else uses the looked-up pointer.
+#define MA_MLA_SCRATCH_BYTES (40u << 20)
+static __device__ __align__(256) unsigned char scratch[MA_MLA_SCRATCH_BYTES];
+static std::atomic<void*> g_scratch_ptr[64];   // by device ordinal
+
+static void* scratch_of_current_device() {
+  const int dev = ma::current_device();
+  if (dev < 0 || dev >= 64) return nullptr;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr) return ptr;
+  if (ma::hip_check(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) != 0 || !ptr) return nullptr;
+  g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // (threads that meet here store the same address)
+  return ptr;
+}
+
+size_t ma_mla_noalloc_max_workspace(void) { return MA_MLA_SCRATCH_BYTES; }
+
+int ma_mla_decode_noalloc(const ma_mla_params* p, ma_stream_t stream) {
+  if (!p) return fail(MA_ERR_INVALID_ARG, "ma_mla_decode_noalloc: params is NULL");
+  if (p->batch <= 0 || p->heads_q <= 0 || p->seqlen_kv <= 0)
+    return fail(MA_ERR_INVALID_ARG, "ma_mla_decode_noalloc: sizes must be positive (B=%d Hq=%d Skv=%d)", p->batch, p->heads_q, p->seqlen_kv);
+  if (p->tile_scheduler_metadata && p->num_sm_parts <= 0)
+    return fail(MA_ERR_INVALID_ARG, "ma_mla_decode_noalloc: a work plan needs num_sm_parts > 0");
+  const size_t need = ma_mla_workspace_bytes(p);
+  if (need > MA_MLA_SCRATCH_BYTES)
+    return fail(MA_ERR_WORKSPACE, "ma_mla_decode_noalloc: this call needs %zu bytes of scratch, the built-in array holds %u: use ma_mla_decode with a "
+                "workspace of the caller's, or fewer splits", need, (unsigned)MA_MLA_SCRATCH_BYTES);
+  ma_mla_params q = *p;
+  q.workspace = nullptr;
+  q.workspace_bytes = 0;
+  if (need > 0) {
+    void* s = scratch_of_current_device();
+    if (!s) return fail(MA_ERR_LAUNCH, "ma_mla_decode_noalloc: no address for the scratch array: %s", hipGetErrorString(ma::t_hip_error));
+    q.workspace = s;
+    q.workspace_bytes = MA_MLA_SCRATCH_BYTES;
+  }
+  return ma_mla_decode(&q, stream);
 }
 
 }  // extern "C"

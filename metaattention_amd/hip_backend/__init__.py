@@ -25,6 +25,7 @@ EXPORTED_SYMBOLS = (
     "ma_version", "ma_last_error", "ma_attn_workspace_bytes", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes", "ma_attn_bwd",
     "ma_linear_workspace_bytes", "ma_linear_fwd",
     "ma_mla_choose_split", "ma_mla_workspace_bytes", "ma_mla_decode", "ma_mla_num_sm_parts", "ma_mla_get_metadata",
+    "ma_mla_noalloc_max_workspace", "ma_mla_decode_noalloc",
 )
 
 
@@ -141,6 +142,10 @@ def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
     lib.ma_mla_workspace_bytes.argtypes = [POINTER(MlaParams)]
     lib.ma_mla_workspace_bytes.restype = c_size_t
     lib.ma_mla_decode.argtypes = [POINTER(MlaParams), c_void_p]
+    lib.ma_mla_decode_noalloc.argtypes = [POINTER(MlaParams), c_void_p]
+    lib.ma_mla_decode_noalloc.restype = c_int
+    lib.ma_mla_noalloc_max_workspace.argtypes = []
+    lib.ma_mla_noalloc_max_workspace.restype = c_size_t
     lib.ma_mla_num_sm_parts.argtypes = [c_int]
     lib.ma_mla_num_sm_parts.restype = c_int
     lib.ma_mla_get_metadata.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]
@@ -313,9 +318,12 @@ def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, 
     return dq, dk, dv
 
 
-def mla_decode(q, q_pe, kv, k_pe, *, scale: float, num_split: int = 0, out=None, lse=None, workspace=None, kv_seqlens=None):
+def mla_decode(q, q_pe, kv, k_pe, *, scale: float, num_split: int = 0, out=None, lse=None, workspace=None, kv_seqlens=None,
+               no_alloc: bool = False):
     """Absorbed MLA decode.  q [B,1,Hq,D], q_pe [B,1,Hq,Dpe], kv [B,Skv,1,D],
-    k_pe [B,Skv,1,Dpe] (the reference operator's layouts) -> [B,1,Hq,D]."""
+    k_pe [B,Skv,1,Dpe] (the reference operator's layouts) -> [B,1,Hq,D].
+    no_alloc=True goes through ma_mla_decode_noalloc: the partial results of the kv splits live in the library's own
+    scratch array instead of a workspace tensor (``out`` must then be given, so that this call allocates nothing)."""
     _require_gpu(q, q_pe, kv, k_pe, out, lse, workspace)
     B, one, Hq, D = q.shape
     Skv, Dpe = kv.shape[1], q_pe.shape[-1]
@@ -323,6 +331,7 @@ def mla_decode(q, q_pe, kv, k_pe, *, scale: float, num_split: int = 0, out=None,
     for t in (q, q_pe, kv, k_pe):
         assert t.stride(-1) == 1, "last dimension must be contiguous"
     if out is None:
+        assert not no_alloc, "no_alloc=True needs the output tensor"
         out = torch.empty(B, 1, Hq, D, dtype=q.dtype, device=q.device)
     p = MlaParams()
     p.dtype = _dtype_code(q.dtype)
@@ -340,6 +349,9 @@ def mla_decode(q, q_pe, kv, k_pe, *, scale: float, num_split: int = 0, out=None,
         assert kv_seqlens.dtype == torch.int32 and kv_seqlens.shape == (B,) and kv_seqlens.is_contiguous() and kv_seqlens.is_cuda
         p.kv_seqlens = kv_seqlens.data_ptr()
     lib = load_library()
+    if no_alloc:
+        _check(lib.ma_mla_decode_noalloc(ctypes.byref(p), _stream()))
+        return out
     need = lib.ma_mla_workspace_bytes(ctypes.byref(p))
     if need:
         if workspace is None:
