@@ -102,6 +102,17 @@ typedef struct ma_attn_params {
   /* optional; with ma_attn_workspace_bytes(&params) bytes, decode shapes (at most 32 query rows, SOFTMAX, no
    * structural mask) run as split-KV + combine (attn_decode_tl.py:63-206); without it they run unsplit */
   void* workspace; size_t workspace_bytes;
+  /* additive terms of the score function, for score_mods that add custom inputs to the score (the three custom-input
+   * classes of core/lower/lower.py:561-615: tensors without a seq_len_kv axis such as [batch, heads, seq_len], tiles
+   * [.., seq_len, seq_len_kv], and seq_len_kv vectors) or terms linear in the indices (ALiBi).  All optional, with the
+   * SOFTMAX / SIGMOID / RELU families:
+   *   x = s * scale + bias + score_add[b, h, q, kv] + pos_slope_q[h] * q + pos_slope_kv[h] * kv,
+   * score_add fp32 (score_add_fp32 != 0) or `dtype`, addressed with ELEMENT strides, 0 for an axis the tensor does not
+   * have; pos_slope_* fp32 [heads].  softcap > 0 (SOFTMAX only): x is replaced by softcap * tanh(x) before the row
+   * function.  The backward kernels do not take these. */
+  const void* score_add; int64_t sa_stride_b, sa_stride_h, sa_stride_q, sa_stride_kv; int32_t score_add_fp32;
+  const float* pos_slope_q; const float* pos_slope_kv;
+  float softcap;
 } ma_attn_params;
 
 /* Parallel attention backward for the SOFTMAX, SIGMOID, RELU and RETENTION families.  Replaces the backward of

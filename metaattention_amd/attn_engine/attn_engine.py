@@ -226,6 +226,7 @@ class AttentionEngine:
             grp = H // Hkv
             kw = dict(family=fam_code, causal=self.mask_kind == "causal", scale=form.scale, bias=form.bias,
                       bias_tensor=given[form.bias_tensor].to(torch.float32) if form.bias_tensor else None)
+            kw.update(self._additive_inputs(given, H, q.dtype, q.device))
             if self.mask_kind.startswith("other"):
                 elem, _ = self._dense_mask(B, H, Sq, k.shape[1], q.device)
                 # (block entries 0 / 1 / 2: nothing, something, everything kept; the kernels skip the 0s and do not read
@@ -263,6 +264,9 @@ class AttentionEngine:
             return run(q, k, v).squeeze(1)
 
         if any(t.requires_grad for t in (q, k, v)):
+            if form.extra or form.softcap is not None:
+                # (the backward kernels take the score as s * scale + bias: additive inputs and soft-capping are forward only)
+                return _ForwardOnly.apply(run, q, k, v)
             score_mask = None
             if self.family == "retention":
                 # the backward kernels of the retention operator exist for its own head size (examples/retention_parallel.py)
@@ -277,6 +281,43 @@ class AttentionEngine:
                 call_masks = lambda: self._block_mask_backward_masks(prefill_blocks, *shape)
             return _Attention.apply(self, run, fam_code, bias_t, call_masks, score_mask, q, k, v)
         return run(q, k, v)
+
+    def _additive_inputs(self, given, H, dtype, device):
+        """The score_mod's score-free terms as the kernel takes them: one tensor addressed [b, h, q, kv] with strides
+        (a single custom tensor is passed as it is, through a broadcasting view; several are summed once per call),
+        per-head slopes for the terms in q_idx / kv_idx, and the soft-capping constant."""
+        from core.eager import custom_tensor_view
+        form = self.score_form
+        kw = {}
+        if form.softcap is not None:
+            kw["softcap"] = form.softcap
+        syms = self.custom_fwd_inputs.input_tensors
+        adds, slopes = [], {"q_idx": None, "kv_idx": None}
+        for mono, coef in form.extra.items():
+            idx = [f[2:] for f in mono if f.startswith("i:")]
+            tens = [f[2:] for f in mono if not f.startswith("i:")]
+            if idx:
+                sl = torch.full((H,), float(coef), dtype=torch.float32, device=device)
+                if tens:
+                    sl = sl * given[tens[0]].to(torch.float32).reshape(-1).expand(H) if given[tens[0]].numel() in (1, H) else None
+                    if sl is None:
+                        raise ValueError(f"custom tensor '{tens[0]}' multiplying {idx[0]} must have one element or one per head")
+                slopes[idx[0]] = sl if slopes[idx[0]] is None else slopes[idx[0]] + sl
+            else:
+                adds.append((coef, custom_tensor_view(given[tens[0]], syms[tens[0]].shape_idx)))
+        if len(adds) == 1 and adds[0][0] == 1.0 and adds[0][1].dtype in (torch.float32, dtype):
+            kw["score_add"] = adds[0][1]
+        elif adds:
+            total = None
+            for coef, t in adds:
+                term = t.to(torch.float32) * coef
+                total = term if total is None else total + term
+            kw["score_add"] = total
+        if slopes["q_idx"] is not None:
+            kw["pos_slope_q"] = slopes["q_idx"].contiguous()
+        if slopes["kv_idx"] is not None:
+            kw["pos_slope_kv"] = slopes["kv_idx"].contiguous()
+        return kw
 
     @staticmethod
     def _expand_block_mask(block_mask, B, H, Sq, Skv):

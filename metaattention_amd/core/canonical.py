@@ -5,10 +5,14 @@ The reference prints every traced spec as kernel source
 package ships a fixed kernel library instead, so a traced spec is reduced to a
 small normal form and matched against the library:
 
-* ``score_mod`` is reduced algebraically to ``act(a * score [* T] + b + t)``
-  with ``act`` in {identity, sigmoid, relu}, ``a``/``b`` python constants, ``t``
-  an optional one-element custom tensor and ``T`` an optional
-  [.., seq_len, seq_len_kv] custom tensor (an element-wise score multiplier);
+* ``score_mod`` is reduced algebraically to ``act(a * score [* T] + b + t + e)``
+  with ``act`` in {identity, sigmoid, relu, cap * tanh}, ``a``/``b`` python
+  constants, ``t`` an optional one-element custom tensor, ``T`` an optional
+  [.., seq_len, seq_len_kv] custom tensor (an element-wise score multiplier)
+  and ``e`` a sum of score-free terms: custom tensors of any of the shape
+  classes of core/lower/lower.py:561-615 (additive [.., seq_len, seq_len_kv]
+  tiles, seq_len_kv vectors, per-row and per-head tensors) and terms linear
+  in ``q_idx`` / ``kv_idx`` (ALiBi: slope[h] * (kv_idx - q_idx));
 * the ``OnlineFunc`` is identified behaviourally: its traced ``online_fwd`` /
   ``online_fwd_epilogue`` are run by the spec interpreter on random tiles and
   compared with each library row function, so algebraically equivalent
@@ -39,20 +43,54 @@ SEQ_TOKENS = ("seq_len", "seq_len_kv")
 # ---------------------------------------------------------------------------
 @dataclass
 class Affine:
-    """a * score * [mask] + sum_t coef_t * t + c   (t: one-element tensors)"""
+    """a * score * [mask] + sum_t coef_t * t + c + sum_m coef_m * m   (t: one-element tensors; m: score-free
+    monomials, tuples of factors "t:<custom tensor>", "i:q_idx", "i:kv_idx", sorted)"""
     a: float = 0.0
     mask: Optional[str] = None
     tensors: Dict[str, float] = field(default_factory=dict)
     c: float = 0.0
-    tile: Optional[str] = None   # a bare [.., seq_len, seq_len_kv] tensor (not yet multiplied with the score)
+    tile: Optional[str] = None   # a bare [.., seq_len, seq_len_kv] tensor (not yet multiplied with the score, nor added to anything)
+    extra: Dict[tuple, float] = field(default_factory=dict)
 
     def is_const(self):
-        return self.a == 0.0 and not self.tensors and self.tile is None
+        return self.a == 0.0 and not self.tensors and self.tile is None and not self.extra
+
+    def settled(self):
+        """The same value with a bare tile counted as an additive term."""
+        if self.tile is None:
+            return self
+        extra = dict(self.extra)
+        extra[("t:" + self.tile,)] = extra.get(("t:" + self.tile,), 0.0) + 1.0
+        return Affine(self.a, self.mask, dict(self.tensors), self.c, None, extra)
 
     def scaled(self, f: float):
-        if self.tile is not None:
-            raise NotImplementedError("scaling a bare tile tensor")
-        return Affine(self.a * f, self.mask, {k: v * f for k, v in self.tensors.items()}, self.c * f)
+        x = self.settled()
+        return Affine(x.a * f, x.mask, {k: v * f for k, v in x.tensors.items()}, x.c * f, None, {k: v * f for k, v in x.extra.items()})
+
+    def score_free_poly(self):
+        """{monomial: coefficient} of a term without the score (one-element tensors as factors "o:<name>")."""
+        x = self.settled()
+        assert x.a == 0.0
+        poly = dict(x.extra)
+        if x.c != 0.0:
+            poly[()] = x.c
+        for k, v in x.tensors.items():
+            poly[("o:" + k,)] = v
+        return poly
+
+    @staticmethod
+    def from_poly(poly):
+        out = Affine()
+        for mono, coef in poly.items():
+            if coef == 0.0:
+                continue
+            if mono == ():
+                out.c += coef
+            elif len(mono) == 1 and mono[0].startswith("o:"):
+                out.tensors[mono[0][2:]] = out.tensors.get(mono[0][2:], 0.0) + coef
+            else:
+                out.extra[mono] = out.extra.get(mono, 0.0) + coef
+        return out
 
 
 @dataclass
@@ -71,6 +109,10 @@ class ScoreForm:
     bias: float
     bias_tensor: Optional[str]
     mask_tensor: Optional[str]
+    # score-free additive terms inside the activation: {monomial: coefficient}, see Affine
+    extra: Dict[tuple, float] = field(default_factory=dict)
+    # softcap: the activation's argument x is replaced by softcap * tanh(x) (identity activation only)
+    softcap: Optional[float] = None
 
 
 def _is_tile_tensor(sym) -> bool:
@@ -86,19 +128,22 @@ def _reduce_score(sym: SymbolScalar, score_id: int, custom: dict):
     if t == "Var" and not sym.prev:
         name = sym.varname
         if name in custom and custom[name] is sym:
-            if _is_tile_tensor(sym):
+            if _is_tile_tensor(sym) and "seq_len" in sym.shape_idx:
                 return Affine(tile=name)
             numel_tokens = [x for x in sym.shape_idx if x not in ("1",)]
             if numel_tokens:
-                raise NotImplementedError(
-                    f"score_mod: custom tensor '{name}' of shape {sym.shape_idx} is neither a one-element tensor nor a "
-                    f"[.., seq_len, seq_len_kv] tile")
+                for tok in numel_tokens:
+                    if tok not in ("batch", "heads", "seq_len", "seq_len_kv"):
+                        raise NotImplementedError(f"score_mod: custom tensor '{name}' of shape {sym.shape_idx}: literal sizes other than 1")
+                return Affine(extra={("t:" + name,): 1.0})
             return Affine(tensors={name: 1.0})
+        if name in ("q_idx", "kv_idx"):
+            return Affine(extra={("i:" + name,): 1.0})
         try:
             return Affine(c=float(sym.code.name))
         except ValueError:
             raise NotImplementedError(f"score_mod uses '{name}', which the kernel library does not provide "
-                                      f"(index-dependent score functions are not in the library)") from None
+                                      f"(of the index arguments only q_idx and kv_idx are)") from None
     ins = [_reduce_score(p, score_id, custom) for p in sym.prev]
     if t == "Neg":
         return _scale(ins[0], -1.0)
@@ -115,9 +160,18 @@ def _reduce_score(sym: SymbolScalar, score_id: int, custom: dict):
             return _scale(y, x.c)
         if isinstance(x, Affine) and isinstance(y, Affine):
             for u, w in ((x, y), (y, x)):
-                if w.tile is not None and u.tile is None and u.mask is None and not u.tensors and u.c == 0.0 and u.a != 0.0:
+                if (w.tile is not None and not w.extra and u.tile is None and u.mask is None and not u.tensors and u.c == 0.0
+                        and not u.extra and u.a != 0.0):
                     return Affine(a=u.a, mask=w.tile)
-        raise NotImplementedError("score_mod: product of two non-constant terms other than score * tile tensor")
+            if x.a == 0.0 and y.a == 0.0:   # two score-free terms: multiply out
+                poly = {}
+                for mx, cx in x.score_free_poly().items():
+                    for my, cy in y.score_free_poly().items():
+                        mono = tuple(sorted(mx + my))
+                        poly[mono] = poly.get(mono, 0.0) + cx * cy
+                return Affine.from_poly(poly)
+        raise NotImplementedError("score_mod: product of two non-constant terms other than score * tile tensor and products of "
+                                  "score-free terms")
     if t == "Div":
         x, y = ins
         if isinstance(y, Affine) and y.is_const():
@@ -128,15 +182,15 @@ def _reduce_score(sym: SymbolScalar, score_id: int, custom: dict):
         raise NotImplementedError("score_mod: division by a non-constant term")
     if t in ("Tanh", "Exp"):
         (x,) = ins
-        if not isinstance(x, Affine) or x.tile is not None:
+        if not isinstance(x, Affine):
             raise NotImplementedError(f"score_mod: {t} of a non-affine term")
-        return Activated(t.lower(), x)
+        return Activated(t.lower(), x.settled())
     if t == "Max":
         x, y = ins
         if isinstance(y, Affine) and y.is_const() and y.c == 0.0 and isinstance(x, Affine):
-            return Activated("relu", x)
+            return Activated("relu", x.settled())
         if isinstance(x, Affine) and x.is_const() and x.c == 0.0 and isinstance(y, Affine):
-            return Activated("relu", y)
+            return Activated("relu", y.settled())
         raise NotImplementedError("score_mod: max() other than max(affine, 0)")
     raise NotImplementedError(f"score_mod: op {t} is not in the kernel library")
 
@@ -149,14 +203,16 @@ def _scale(x, f: float):
 
 def _add(x, y):
     if isinstance(x, Affine) and isinstance(y, Affine):
-        if x.tile is not None or y.tile is not None:
-            raise NotImplementedError("score_mod: adding a tile tensor to the score (additive bias tiles are not in the library)")
+        x, y = x.settled(), y.settled()   # (a bare tile in a sum is an additive bias tile)
         if x.a != 0.0 and y.a != 0.0 and x.mask != y.mask:
             raise NotImplementedError("score_mod: score terms with different multipliers")
         tensors = dict(x.tensors)
         for k, v in y.tensors.items():
             tensors[k] = tensors.get(k, 0.0) + v
-        return Affine(x.a + y.a, x.mask if x.a != 0.0 else y.mask, tensors, x.c + y.c)
+        extra = dict(x.extra)
+        for k, v in y.extra.items():
+            extra[k] = extra.get(k, 0.0) + v
+        return Affine(x.a + y.a, x.mask if x.a != 0.0 else y.mask, tensors, x.c + y.c, None, {k: v for k, v in extra.items() if v != 0.0})
     if isinstance(x, Activated) and isinstance(y, Affine) and y.is_const():
         return Activated(x.fn, x.inner, x.p, x.q + y.c)
     if isinstance(y, Activated) and isinstance(x, Affine) and x.is_const():
@@ -173,10 +229,13 @@ def canonicalize_score_mod(score_mod, custom_fwd_inputs) -> ScoreForm:
     idx = [SymbolScalar(n, Var(n)) for n in ("b", "h", "q_idx", "kv_idx")]
     out = score_mod(score, custom_fwd_inputs, *idx) if score_mod is not None else score
     form = _reduce_score(out, id(score), custom_fwd_inputs.input_tensors)
+    softcap = None
     if isinstance(form, Activated):
         inner, act = form.inner, None
         if form.fn == "tanh" and _close(form.p, 0.5) and _close(form.q, 0.5):
             inner, act = inner.scaled(2.0), "sigmoid"      # (tanh(x)+1)/2 = sigmoid(2x)
+        elif form.fn == "tanh" and _close(form.q, 0.0) and form.p > 0:
+            act, softcap = "identity", float(form.p)        # soft-capping: cap * tanh(x), then the row function
         elif form.fn == "sigmoid" and _close(form.p, 1.0) and _close(form.q, 0.0):
             act = "sigmoid"
         elif form.fn == "relu" and _close(form.q, 0.0) and form.p > 0:
@@ -184,9 +243,20 @@ def canonicalize_score_mod(score_mod, custom_fwd_inputs) -> ScoreForm:
         if act is None:
             raise NotImplementedError(f"score_mod: {form.p}*{form.fn}(.)+{form.q} is not a library activation")
     else:
-        inner, act = form, "identity"
+        inner, act = form.settled(), "identity"
     if inner.tile is not None or inner.a == 0.0:
         raise NotImplementedError("score_mod does not depend linearly on the score")
+    for mono in inner.extra:
+        n_idx = sum(f.startswith("i:") for f in mono)
+        if n_idx > 1 or (n_idx == 1 and len(mono) > 2) or (n_idx == 0 and len(mono) > 1):
+            raise NotImplementedError(f"score_mod: the additive term {' * '.join(f[2:] for f in mono)} is not in the kernel library "
+                                      "(sums of custom tensors, and q_idx / kv_idx times a constant or a per-head tensor, are)")
+        if n_idx == 1 and len(mono) == 2:
+            other = [f for f in mono if not f.startswith("i:")][0]
+            sym = custom_fwd_inputs.input_tensors.get(other[2:])
+            toks = [x for x in (sym.shape_idx if sym is not None else []) if x != "1"]
+            if toks not in ([], ["heads"]):
+                raise NotImplementedError(f"score_mod: {mono}: an index may be multiplied by a constant, a one-element or a per-head tensor")
     bias_tensor = None
     if inner.tensors:
         if len(inner.tensors) > 1:
@@ -196,7 +266,9 @@ def canonicalize_score_mod(score_mod, custom_fwd_inputs) -> ScoreForm:
             raise NotImplementedError("score_mod: bias tensor with a coefficient other than 1")
     if act != "identity" and inner.mask is not None:
         raise NotImplementedError("score_mod: activation of a tile-multiplied score")
-    return ScoreForm(act, inner.a, inner.c, bias_tensor, inner.mask)
+    if inner.mask is not None and (inner.extra or softcap is not None):
+        raise NotImplementedError("score_mod: additive terms / soft-capping together with a tile-multiplied score")
+    return ScoreForm(act, inner.a, inner.c, bias_tensor, inner.mask, dict(inner.extra), softcap)
 
 
 # ---------------------------------------------------------------------------

@@ -104,6 +104,18 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
     }
   }
   a.scale = p->scale; a.bias = p->bias;
+  if (p->score_add || p->pos_slope_q || p->pos_slope_kv || p->softcap != 0.f) {
+    if (p->family == MA_ATTN_RETENTION)
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: score_add / pos_slope / softcap go with the softmax / sigmoid / relu families");
+    if (p->softcap < 0.f || (p->softcap > 0.f && p->family != MA_ATTN_SOFTMAX))
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: softcap must be >= 0 and goes with the softmax family");
+    if (p->score_add && (uintptr_t)p->score_add % (p->score_add_fp32 ? 4 : 2) != 0)
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: score_add must be aligned to its element size");
+    a.add = p->score_add; a.add_sb = p->sa_stride_b; a.add_sh = p->sa_stride_h; a.add_sq = p->sa_stride_q; a.add_sk = p->sa_stride_kv;
+    a.add_f32 = p->score_add_fp32 != 0;
+    a.slope_q = p->pos_slope_q; a.slope_kv = p->pos_slope_kv;
+    a.softcap = p->softcap;
+  }
   const int rc = ma::attn_fwd_dispatch(a, p->family, p->mask == MA_MASK_CAUSAL, p->dtype == MA_BF16, p->dim_qk, p->dim_v,
                                        (hipStream_t)stream);
   if (rc == -2)

@@ -29,6 +29,14 @@ struct AttnArgs {
   void* o_part;
   float* lse_part;
   float scale, bias;
+  // additive score terms (attn_wide_fwd_kernel only): x = s * scale + bias + add[b, h, q, kv] + slope_q[h] * q + slope_kv[h] * kv,
+  // then, with softcap > 0, x = softcap * tanh(x).  add: fp32 or the tensor dtype, element strides (0 broadcasts).
+  const void* add;
+  int64_t add_sb, add_sh, add_sq, add_sk;
+  int add_f32;
+  const float* slope_q;
+  const float* slope_kv;
+  float softcap;
 };
 
 int attn_wide_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);

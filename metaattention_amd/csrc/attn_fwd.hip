@@ -597,7 +597,8 @@ static int dispatch_family(const AttnArgs& a, int family, bool causal, hipStream
 
 // returns 0 ok, -1 launch failure, -2 unsupported
 int attn_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream) {
-  if (family != 3 && dqk == 128 && dv == 128 && !a.kv_lens && !a.kv_block_mask && !a.o_part && !a.elem_mask) {
+  if (family != 3 && dqk == 128 && dv == 128 && !a.kv_lens && !a.kv_block_mask && !a.o_part && !a.elem_mask && !a.add && !a.slope_q &&
+      !a.slope_kv && !(a.softcap > 0.f)) {
     return is_bf16 ? dispatch_family<__bf16, 128, 128>(a, family, causal, stream)
                    : dispatch_family<_Float16, 128, 128>(a, family, causal, stream);
   }

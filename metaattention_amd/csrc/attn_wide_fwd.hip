@@ -116,6 +116,23 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
       }
     }
   };
+  // additive score terms of this lane's row (the score_mod's custom inputs other than the multiplier; core/lower/
+  // lower.py:561-615 loads them per q tile, per kv step or as [block_M, block_N] tiles depending on their shape: here
+  // one strided tensor covers all of those shapes) and terms linear in the indices; folded into the raw score as
+  // extra / scale, so that everything after sees s * scale + bias + extra
+  const bool has_extra = a.add || a.slope_q || a.slope_kv;
+  const float inv_scale = 1.f / a.scale;
+  const float sl_q = a.slope_q ? a.slope_q[h] * (float)m_ld : 0.f, sl_kv = a.slope_kv ? a.slope_kv[h] : 0.f;
+  const int64_t add_row = (int64_t)b * a.add_sb + (int64_t)h * a.add_sh + (int64_t)m_ld * a.add_sq;
+  auto load_extra = [&](int n0, float (&ex)[16]) {
+#pragma unroll
+    for (int jj = 0; jj < 16; jj++) {
+      const int n = min(n0 + 8 * (jj >> 2) + 4 * g + (jj & 3), skv - 1);
+      float e = sl_q + sl_kv * (float)n;
+      if (a.add) e += a.add_f32 ? ((const float*)a.add)[add_row + (int64_t)n * a.add_sk] : (float)((const T*)a.add)[add_row + (int64_t)n * a.add_sk];
+      ex[jj] = e * inv_scale;
+    }
+  };
   const int tiles_per_block = a.kv_block / BN;
   // this workgroup's share of the tiles
   const int tiles_per_split = (n_tiles + a.n_split - 1) / a.n_split;
@@ -210,6 +227,10 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
       issue_tile(jt * BN, buf ^ 1);
     }
     const uint32_t kbase = lds0 + buf * STAGE, vbase = kbase + KTILE;
+    float ex[16];
+    if constexpr (FAMILY != WF_RETENTION) {
+      if (has_extra) load_extra(n0, ex);
+    }
 
     // ---- S^T = K Q^T
     f32x16 s;
@@ -238,6 +259,18 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
         pf[jj >> 3][jj & 7] = (T)p;
       }
     } else {
+      if (has_extra) {
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++) s[jj] += ex[jj];
+      }
+      if (a.softcap > 0.f) {   // x -> softcap * tanh(x), x = s * scale + bias;  tanh(x) = 1 - 2 / (1 + e^(2x))
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++) {
+          const float x = s[jj] * a.scale + bias;
+          const float th = 1.f - 2.f * fast_rcp(1.f + fast_exp2(x * (2.f * kLog2e)));
+          s[jj] = (a.softcap * th - bias) * inv_scale;
+        }
+      }
       // element-wise mask only on tiles that reach past the diagonal or the end of the sequence
       const bool edge = (CAUSAL && n0 + BN - 1 > m_wave) || n0 + BN > skv;
       if (edge) {

@@ -53,6 +53,8 @@ class AttnParams(Structure):
         ("elem_mask", c_void_p), ("em_stride_b", c_int64), ("em_stride_h", c_int64), ("em_stride_q", c_int64),
         ("kbm_stride_q", c_int64), ("kbm_per_query_head", c_int32),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+        ("score_add", c_void_p), ("sa_stride_b", c_int64), ("sa_stride_h", c_int64), ("sa_stride_q", c_int64), ("sa_stride_kv", c_int64),
+        ("score_add_fp32", c_int32), ("pos_slope_q", c_void_p), ("pos_slope_kv", c_void_p), ("softcap", c_float),
     ]
 
 
@@ -180,10 +182,14 @@ def _require_gpu(*tensors):
 
 def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None,
              score_mask=None, out=None, row_scale=None, kv_seqlens=None, kv_block_mask=None, kv_block_size: int = 0,
-             workspace=None, split_kv: bool = True, elem_mask=None):
+             workspace=None, split_kv: bool = True, elem_mask=None, score_add=None, pos_slope_q=None, pos_slope_kv=None,
+             softcap: float = 0.0):
     """Parallel attention forward on BSHD tensors.  Returns ``out`` ([B,Sq,H,Dv]).  k and v may
-    have fewer heads than q (grouped-query: query head h reads kv head h // (H // Hkv))."""
-    _require_gpu(q, k, v, bias_tensor, score_mask, out, row_scale, kv_seqlens, kv_block_mask)
+    have fewer heads than q (grouped-query: query head h reads kv head h // (H // Hkv)).
+    score_add: fp32 or q.dtype tensor broadcastable as [B|1, H|1, Sq|1, Skv|1] added to the scaled score;
+    pos_slope_q / pos_slope_kv: fp32 [H], the score gets slope_q[h] * q_idx + slope_kv[h] * kv_idx;
+    softcap > 0: softmax of softcap * tanh(x)."""
+    _require_gpu(q, k, v, bias_tensor, score_mask, out, row_scale, kv_seqlens, kv_block_mask, score_add, pos_slope_q, pos_slope_kv)
     B, Sq, H, Dqk = q.shape
     Skv, Hkv, Dv = k.shape[1], k.shape[2], v.shape[-1]
     assert k.shape == (B, Skv, Hkv, Dqk) and v.shape == (B, Skv, Hkv, Dv) and H % Hkv == 0, "q/k/v shapes disagree"
@@ -235,6 +241,18 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
         p.em_stride_b = elem_mask.stride(0) if elem_mask.shape[0] > 1 else 0
         p.em_stride_h = elem_mask.stride(1) if elem_mask.shape[1] > 1 else 0
         p.em_stride_q = elem_mask.stride(2)
+    if score_add is not None:
+        assert score_add.dim() == 4 and score_add.dtype in (torch.float32, q.dtype)
+        for ax, full in enumerate((B, H, Sq, Skv)):
+            assert score_add.shape[ax] in (1, full), f"score_add {tuple(score_add.shape)} does not broadcast to {(B, H, Sq, Skv)}"
+        st = [score_add.stride(ax) if score_add.shape[ax] > 1 else 0 for ax in range(4)]
+        p.score_add, p.score_add_fp32 = score_add.data_ptr(), int(score_add.dtype == torch.float32)
+        p.sa_stride_b, p.sa_stride_h, p.sa_stride_q, p.sa_stride_kv = st
+    for name, t in (("pos_slope_q", pos_slope_q), ("pos_slope_kv", pos_slope_kv)):
+        if t is not None:
+            assert t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous()
+            setattr(p, name, t.data_ptr())
+    p.softcap = float(softcap)
     lib = load_library()
     if split_kv:
         need = lib.ma_attn_workspace_bytes(ctypes.byref(p))

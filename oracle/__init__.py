@@ -40,6 +40,10 @@ masked_attention       SDPA with a boolean attn_mask (fp64); tril keep mask ==
                        softmax_attention(causal); a block mask == attention over
                        the gathered kept keys of each query block; rows without
                        keys are 0; sigmoid / relu by element-wise brute force
+biased_attention       SDPA with a float attn_mask (fp64), with and without the causal
+                       triangle; add = 0 == softmax_attention; a seq_len_kv vector equal for
+                       all keys leaves softmax unchanged and shifts lse by it; soft-capping,
+                       sigmoid and relu element by element
 attention_grads,       central differences of the pinned forward functions in
 linear_attention_grads fp64 along random directions; SDPA's own autograd
 (all of the above)     tests/golden/*.npz: the operators' definitions evaluated
@@ -59,6 +63,7 @@ from .attention_ref import (  # noqa: F401
     sparse_decode_attention,
     paged_mla_decode,
     masked_attention,
+    biased_attention,
 )
 from .linear_ref import (  # noqa: F401
     retnet_quadratic,

@@ -216,6 +216,46 @@ def masked_attention(q, k, v, keep=None, block_mask=None, family: str = "softmax
     return out
 
 
+def biased_attention(q, k, v, add=None, causal: bool = False, family: str = "softmax", softmax_scale: Optional[float] = None,
+                     bias: float = 0.0, softcap: Optional[float] = None, compute_dtype=torch.float32, return_lse: bool = False):
+    """Attention whose score function adds score-free terms to the scaled score, the general form a ``score_mod`` with
+    custom inputs takes: x = s * scale + bias + add[b, h, q, kv], then (``softcap``) x = softcap * tanh(x), then the row
+    function of ``family`` ("softmax", "sigmoid", "relu").  ``add`` is anything that broadcasts to [B, H, Sq, Skv]: the
+    reference's three custom-input classes (core/lower/lower.py:561-615: tensors without a seq_len_kv axis, [.., seq_len,
+    seq_len_kv] tiles, seq_len_kv vectors) and index terms such as ALiBi's slope[h] * (kv_idx - q_idx) all reduce to it.
+    The score_mod sits where the reference's kernel has it: after the -inf fill of masked scores and before the online
+    row function (tl_template/attn/attn_tl.py:140-169), so a masked element contributes exactly 0.
+    q,k [B,S,H,D], v [B,S,H,Dv] -> [B,Sq,H,Dv] (and the natural-log lse [B,H,Sq] for softmax)."""
+    B, Sq, H, D = q.shape
+    Skv, Dv = k.shape[1], v.shape[-1]
+    scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+    out = torch.empty(B, Sq, H, Dv, dtype=compute_dtype)
+    lse = torch.empty(B, H, Sq, dtype=compute_dtype)
+    if add is not None:
+        add = add.to(compute_dtype).expand(B, H, Sq, Skv)
+    keep = _causal_keep(Sq, Skv, q.device) if causal else None
+    for b in range(B):
+        for h in range(H):
+            x = (q[b, :, h].to(compute_dtype) @ k[b, :, h // (H // k.shape[2])].to(compute_dtype).T) * scale + bias
+            if add is not None:
+                x = x + add[b, h]
+            if softcap is not None:
+                x = softcap * torch.tanh(x)
+            if keep is not None:
+                x = x.masked_fill(~keep, float("-inf"))
+            if family == "softmax":
+                p = torch.softmax(x, dim=-1)
+                lse[b, h] = torch.logsumexp(x, dim=-1)
+            elif family == "sigmoid":
+                p = torch.sigmoid(x)
+            elif family == "relu":
+                p = torch.relu(x).masked_fill(torch.isinf(x), 0.0)
+            else:
+                raise ValueError(family)
+            out[b, :, h] = p @ v[b, :, h // (H // v.shape[2])].to(compute_dtype)
+    return (out, lse) if return_lse and family == "softmax" else out
+
+
 def paged_mla_decode(q, k_cache, block_table, cache_seqlens, head_dim_v: int = 512, compute_dtype=torch.float32):
     """flash_mla_with_kvcache semantics (cute_template_kvshared/flash_mla_interface.py:75-115) for one query
     token: q [B,1,Hq,d+dpe]; k_cache [pages, page_size, 1, d+dpe]; sequence b is the rows of pages

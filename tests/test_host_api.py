@@ -92,8 +92,31 @@ def test_canonical_score_forms():
     assert (f.activation, f.scale, f.mask_tensor) == ("identity", 1.0, "mask")
     f = canonicalize_score_mod(lambda s, c, b, h, q, k: t["mask"] * (s * 0.5), io)
     assert (f.scale, f.mask_tensor) == (0.5, "mask")
-    for bad in (lambda s, c, b, h, q, k: s * s, lambda s, c, b, h, q, k: s + q, lambda s, c, b, h, q, k: s.tanh(),
-                lambda s, c, b, h, q, k: s + t["mask"], lambda s, c, b, h, q, k: s.abs()):
+    for bad in (lambda s, c, b, h, q, k: s * s, lambda s, c, b, h, q, k: s + h, lambda s, c, b, h, q, k: s.tanh() * 2 + 1,
+                lambda s, c, b, h, q, k: s + q * k, lambda s, c, b, h, q, k: s.abs(), lambda s, c, b, h, q, k: s * t["mask"] + t["mask"]):
+        with pytest.raises(NotImplementedError):
+            canonicalize_score_mod(bad, io)
+
+
+def test_canonical_additive_score_terms():
+    """The custom-input classes of core/lower/lower.py:561-615 as additive terms, index terms (ALiBi), soft-capping."""
+    io = CustomIO({"rel": (1, "heads", "seq_len", "seq_len_kv"), "colv": ("seq_len_kv",), "rowt": ("batch", "heads", "seq_len"),
+                   "slopes": ("heads",), "b1": (1,)})
+    t = io.input_tensors
+    f = canonicalize_score_mod(lambda s, c, b, h, q, k: s * 0.125 + t["rel"], io)
+    assert (f.activation, f.scale, f.mask_tensor, f.extra) == ("identity", 0.125, None, {("t:rel",): 1.0})
+    f = canonicalize_score_mod(lambda s, c, b, h, q, k: (s + t["colv"]) * 0.125 + t["rowt"] + t["b1"], io)
+    assert f.bias_tensor == "b1" and f.extra == {("t:colv",): 0.125, ("t:rowt",): 1.0}
+    f = canonicalize_score_mod(lambda s, c, b, h, q, k: s * 0.125 - t["slopes"] * (q - k), io)
+    assert f.extra == {("i:q_idx", "t:slopes"): -1.0, ("i:kv_idx", "t:slopes"): 1.0}
+    f = canonicalize_score_mod(lambda s, c, b, h, q, k: s * 0.125 + (k - q) * 0.5, io)
+    assert f.extra == {("i:kv_idx",): 0.5, ("i:q_idx",): -0.5}
+    f = canonicalize_score_mod(lambda s, c, b, h, q, k: (s * (0.125 / 30)).tanh() * 30, io)
+    assert f.activation == "identity" and f.softcap == 30.0 and abs(f.scale - 0.125 / 30) < 1e-12
+    f = canonicalize_score_mod(lambda s, c, b, h, q, k: ((s * 0.1 + t["rel"]) * 0.5).tanh() * 0.5 + 0.5, io)
+    assert f.activation == "sigmoid" and f.extra == {("t:rel",): 1.0} and abs(f.scale - 0.1) < 1e-12
+    for bad in (lambda s, c, b, h, q, k: s + t["rel"] * t["colv"], lambda s, c, b, h, q, k: s + t["rowt"] * q,
+                lambda s, c, b, h, q, k: s * t["rel"] + t["colv"]):
         with pytest.raises(NotImplementedError):
             canonicalize_score_mod(bad, io)
 

@@ -422,3 +422,50 @@ def test_mla_work_plan_small_cases_and_invariants():
             assert all(e > s_ for s_, e in cover[b]) or lens[b] == 0
             assert splits[b + 1] - splits[b] == len(cover[b])
         assert all(v <= payload for v in load.values())
+
+
+def test_biased_attention_against_sdpa_and_special_cases():
+    g = torch.Generator().manual_seed(23)
+    B, H, S, D = 2, 3, 20, 8
+    q, k, v = (torch.randn(B, S, H, D, generator=g, dtype=torch.float64) for _ in range(3))
+    add = torch.randn(B, H, S, S, generator=g, dtype=torch.float64)
+    qt, kt, vt = (t.transpose(1, 2) for t in (q, k, v))
+    # a float attn_mask is added to the scaled scores by SDPA
+    got, lse = oracle.biased_attention(q, k, v, add=add, compute_dtype=torch.float64, return_lse=True)
+    sd = torch.nn.functional.scaled_dot_product_attention(qt, kt, vt, attn_mask=add).transpose(1, 2)
+    torch.testing.assert_close(got, sd)
+    x = torch.einsum("bqhd,bkhd->bhqk", q, k) / math.sqrt(D) + add
+    torch.testing.assert_close(lse, torch.logsumexp(x, dim=-1))
+    # with the causal triangle: the same as a float mask that also holds -inf above the diagonal
+    tri = torch.full((S, S), float("-inf"), dtype=torch.float64).triu(1)
+    got = oracle.biased_attention(q, k, v, add=add, causal=True, compute_dtype=torch.float64)
+    sd = torch.nn.functional.scaled_dot_product_attention(qt, kt, vt, attn_mask=add + tri).transpose(1, 2)
+    torch.testing.assert_close(got, sd)
+    # broadcast shapes: a [heads, 1, 1]-shaped slope times (kv - q) (ALiBi), a per-row tensor, a kv vector
+    idx = torch.arange(S, dtype=torch.float64)
+    alibi = torch.tensor([0.5, 0.25, 0.125], dtype=torch.float64).view(1, H, 1, 1) * (idx.view(1, 1, 1, S) - idx.view(1, 1, S, 1))
+    got = oracle.biased_attention(q, k, v, add=alibi, causal=True, compute_dtype=torch.float64)
+    sd = torch.nn.functional.scaled_dot_product_attention(qt, kt, vt, attn_mask=alibi.expand(B, H, S, S) + tri).transpose(1, 2)
+    torch.testing.assert_close(got, sd)
+    row = torch.randn(B, H, S, 1, generator=g, dtype=torch.float64)      # constant along the row: softmax ignores it, lse moves by it
+    base, lse0 = oracle.softmax_attention(q, k, v, causal=True, compute_dtype=torch.float64, return_lse=True)
+    got, lse = oracle.biased_attention(q, k, v, add=row, causal=True, compute_dtype=torch.float64, return_lse=True)
+    torch.testing.assert_close(got, base)
+    torch.testing.assert_close(lse, lse0 + row.squeeze(-1))
+    torch.testing.assert_close(oracle.biased_attention(q, k, v, causal=False, compute_dtype=torch.float64),
+                               oracle.softmax_attention(q, k, v, causal=False, compute_dtype=torch.float64))
+    # soft-capping, sigmoid, relu: element by element
+    colv = torch.randn(S, generator=g, dtype=torch.float64)
+    for family, cap in (("softmax", 2.5), ("sigmoid", None), ("relu", None)):
+        got = oracle.biased_attention(q[:1, :5, :1], k[:1, :5, :1], v[:1, :5, :1], add=colv[:5].view(1, 1, 1, 5), causal=True, family=family,
+                                      softmax_scale=0.7, bias=-0.2, softcap=cap, compute_dtype=torch.float64)
+        for i in range(5):
+            w = []
+            for j in range(i + 1):
+                x = float(q[0, i, 0] @ k[0, j, 0]) * 0.7 - 0.2 + float(colv[j])
+                if cap is not None:
+                    x = cap * math.tanh(x)
+                w.append(math.exp(x) if family == "softmax" else (1 / (1 + math.exp(-x)) if family == "sigmoid" else max(x, 0.0)))
+            tot = sum(w) if family == "softmax" else 1.0
+            ref = sum(wj / tot * v[0, j, 0] for j, wj in enumerate(w))
+            torch.testing.assert_close(got[0, i, 0], ref)
