@@ -30,8 +30,10 @@ class OnlineFunc:
     the updated statistics and the factor the output accumulator is rescaled
     by.  ``online_fwd_epilogue(o, online_rowscales, b, h, q_idx)`` returns
     ``(o', final_rowscales)``.  ``forward`` / ``backward`` describe the
-    recompute for a backward pass and ``combine`` the split-KV merge; they are
-    part of the contract but unused by the forward kernels here.
+    recompute for a backward pass and ``combine`` the split-KV merge.  The
+    kernel library holds one version of each per row function; where a spec
+    overrides them, its traced version is compared with the library's and a
+    spec that computes something else is refused (core/canonical.py).
     """
 
     def __init__(self, online_rowscales: dict, final_rowscales: dict, external_fwd_tensors: CustomIO):

@@ -16,7 +16,9 @@ small normal form and matched against the library:
 * the ``OnlineFunc`` is identified behaviourally: its traced ``online_fwd`` /
   ``online_fwd_epilogue`` are run by the spec interpreter on random tiles and
   compared with each library row function, so algebraically equivalent
-  spellings of the same row function are accepted;
+  spellings of the same row function are accepted; its ``forward``,
+  ``backward`` and ``combine`` are checked the same way against what the
+  backward and split-KV combine kernels compute;
 * the linear-attention mods are reduced to a q scale, a per-token v scale and
   a traced decay function.
 
@@ -369,11 +371,88 @@ def identify_online_func(online_func) -> str:
                 if not ok:
                     break
             if ok:
+                _check_recompute_and_combine(online_func, lib_name)
                 return lib_name
         tried.append(lib_name)
     raise NotImplementedError(
         f"OnlineFunc with row scales {names} (initial values {inits}) matches no library row function "
         f"(softmax, identity, retention); compared against: {tried or 'none with that many row scales'}")
+
+
+def _check_recompute_and_combine(online_func, lib_name: str):
+    """The other three methods of the contract, where the spec overrides them: ``forward`` (the probabilities again, from
+    the scores and the final row scale), ``backward`` (dscores from dp: both generated into the backward kernel by
+    core/lower/lower.py:425-438) and ``combine`` (the weight of every kv split, generated into the split-KV merge by
+    core/lower/lower_decode.py:287-313).  The library's backward and combine kernels hold ONE version of each per row
+    function; a spec whose traced version computes something else is refused instead of being silently replaced:
+        softmax    forward exp(s - lse)   backward (dp - doosum) * p   combine exp(lse_i - logsumexp_i(lse))  (or the same
+                   in base 2, as examples/mha_decode.py:72-80 spells it for its log2-domain lse)
+        identity   forward s              backward dp
+        retention  forward s / r          backward dp / r"""
+    from attn_engine import OnlineFunc          # (the base class: methods left at its defaults are not looked at)
+    from .transform.core import SymbolicColReduceArray
+    cls = type(online_func)
+    finals = list(online_func.final_rowscales)
+    if lib_name != "identity" and len(finals) != 1:
+        return
+    gen = torch.Generator().manual_seed(4321)
+    M, N, NS = 5, 7, 4
+    idx = [SymbolScalar(n, Var(n)) for n in ("b", "h", "q_idx", "kv_idx")]
+
+    def run(method, what, build):
+        try:
+            out_sym, env, like, expect = build()
+            got = evaluate([out_sym], env, like)[0]
+        except NotImplementedError:
+            raise
+        except Exception as e:
+            raise NotImplementedError(f"OnlineFunc.{method} could not be traced: {e!r}") from None
+        if not any(_allclose(got, e) for e in expect):
+            raise NotImplementedError(f"OnlineFunc.{method} computes something else than the library's {what} for the {lib_name} row "
+                                      "function; the kernel library holds one version of it and does not generate another")
+
+    fin = torch.randn(M, 1, generator=gen, dtype=torch.float64)
+    if lib_name == "retention":
+        fin = fin.abs() + 1.0
+    sc = torch.randn(M, N, generator=gen, dtype=torch.float64)
+    prob = {"softmax": lambda: torch.exp(sc - fin), "identity": lambda: sc, "retention": lambda: sc / fin}[lib_name]()
+
+    if getattr(cls, "forward", None) is not OnlineFunc.forward:
+        def build():
+            tile = SymbolicArray("scores_fwd", Var("scores_fwd"))
+            fsyms = {n: SymbolScalar(n, Var(n)) for n in finals}
+            out = online_func.forward(tile, fsyms, *idx)
+            env = {id(tile): sc, **{id(v): fin for v in fsyms.values()}}
+            return out, env, sc, [prob]
+        run("forward", "recomputation of the probabilities", build)
+
+    if getattr(cls, "backward", None) is not OnlineFunc.backward:
+        dp = torch.randn(M, N, generator=gen, dtype=torch.float64)
+        doosum = torch.randn(M, 1, generator=gen, dtype=torch.float64)
+        expect = {"softmax": (dp - doosum) * prob, "identity": dp, "retention": dp / fin}[lib_name]
+
+        def build():
+            dps, ps = SymbolicArray("dp", Var("dp")), SymbolicArray("p", Var("p"))
+            ds = SymbolScalar("doosum", Var("doosum"))
+            fsyms = {n: SymbolScalar(n, Var(n)) for n in finals}
+            try:     # the signature lower.py:437-438 calls; the base class declares it without the row sums
+                out = online_func.backward(dps, ps, fsyms, ds, *idx)
+            except TypeError:
+                out = online_func.backward(dps, ps, fsyms, *idx)
+            env = {id(dps): dp, id(ps): prob, id(ds): doosum, **{id(v): fin for v in fsyms.values()}}
+            return out, env, dp, [expect]
+        run("backward", "score gradient", build)
+
+    if getattr(cls, "combine", None) is not OnlineFunc.combine:
+        if lib_name != "softmax":
+            raise NotImplementedError("split-KV combine is only in the softmax operators of the kernel library")
+        lse = torch.randn(NS, M, generator=gen, dtype=torch.float64) * 3
+
+        def build():
+            fsyms = {finals[0]: SymbolicColReduceArray(finals[0], Var(finals[0]), shape_idx=["num_split", "block_M"])}
+            out = online_func.combine(fsyms)
+            return out, {id(fsyms[finals[0]]): lse}, lse, [torch.softmax(lse, dim=0), torch.softmax(lse * math.log(2.0), dim=0)]
+        run("combine", "log-sum-exp merge of the kv splits", build)
 
 
 def _same_init(a: float, b: float) -> bool:

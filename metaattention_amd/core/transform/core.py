@@ -84,7 +84,7 @@ class SymbolScalar:
         name = self.varname if varname_suffix is None else f"{self.varname}_{varname_suffix}"
         node = code(*[x.code for x in [self] + operands])
         out = SymbolScalar(f"{name}_{self.count}", node, [self] + operands, shape_idx)
-        if isinstance(self, SymbolicArray) and len(shape_idx) == len(self.shape_idx):
+        if isinstance(self, (SymbolicArray, SymbolicColReduceArray)) and len(shape_idx) == len(self.shape_idx):
             out.__class__ = self.__class__
         for x in [self] + operands:
             x.use_list.append(out)

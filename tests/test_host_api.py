@@ -236,3 +236,74 @@ def test_specs_on_cpu_match_oracle(block_n):
     ref, r = oracle.retention_parallel(q, k, v, mask, return_r=True)
     torch.testing.assert_close(o, ref, rtol=2e-5, atol=2e-5)
     torch.testing.assert_close(fin["r"], r, rtol=2e-5, atol=2e-5)
+
+
+def test_spec_forward_backward_combine_are_checked_against_the_library():
+    """forward / backward / combine of an OnlineFunc are traced and compared with the one version the kernel library
+    holds per row function (the spellings of examples/mha.py:73-83, examples/mha_decode.py:72-80 and
+    examples/retention_parallel.py:76-86 pass); a spec that defines another one is refused, not silently replaced."""
+    class Softmax(specs.OnlineSoftmax):
+        @staticmethod
+        def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
+            return (scores - final_rowscales["lse"]).exp()
+
+        @staticmethod
+        def backward(dp, scores, final_rowscales, doosum_rowscales, b, h, q_idx, kv_idx):
+            return (dp - doosum_rowscales) * scores
+
+        @staticmethod
+        def combine(final_rowscales):
+            lse = final_rowscales["lse"]
+            lse_max = lse.get_reduce("max")
+            row_sum = (lse - lse_max).exp2()
+            lse_sum = row_sum.get_reduce("sum").log2() + lse_max
+            return (lse - lse_sum).exp2()
+
+    assert identify_online_func(Softmax()) == "softmax"
+
+    class NaturalCombine(Softmax):
+        @staticmethod
+        def combine(final_rowscales):
+            lse = final_rowscales["lse"]
+            m = lse.get_reduce("max")
+            e = (lse - m).exp()
+            return e / e.get_reduce("sum")
+
+    assert identify_online_func(NaturalCombine()) == "softmax"
+
+    class Retention(specs.OnlineRetention):
+        @staticmethod
+        def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
+            return scores / final_rowscales["r"]
+
+        @staticmethod
+        def backward(dp, scores, final_rowscales, doosum_rowscales, b, h, q_idx, kv_idx):
+            return dp / final_rowscales["r"]
+
+    assert identify_online_func(Retention()) == "retention"
+
+    class WrongBackward(Softmax):
+        @staticmethod
+        def backward(dp, scores, final_rowscales, doosum_rowscales, b, h, q_idx, kv_idx):
+            return dp * scores
+
+    class WrongForward(Softmax):
+        @staticmethod
+        def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
+            return (scores - final_rowscales["lse"]).exp2()
+
+    class WrongCombine(Softmax):
+        @staticmethod
+        def combine(final_rowscales):
+            lse = final_rowscales["lse"]
+            return (lse - lse.get_reduce("max")).exp()
+
+    class RetentionTrueGradient(Retention):
+        @staticmethod
+        def backward(dp, scores, final_rowscales, doosum_rowscales, b, h, q_idx, kv_idx):
+            return (dp - doosum_rowscales) / final_rowscales["r"]
+
+    for bad, word in ((WrongBackward, "backward"), (WrongForward, "forward"), (WrongCombine, "combine"), (RetentionTrueGradient, "backward")):
+        with pytest.raises(NotImplementedError) as ei:
+            identify_online_func(bad())
+        assert word in str(ei.value)
