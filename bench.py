@@ -16,6 +16,7 @@ cores over a bounded sample as "cpu_baseline"):
   c2_softmax_causal_bwd  backward of the headline workload (dq, dk, dv)
   c3_retnet_chunked   RetNet retention, chunked operator, B8 H16 S2048 Dqk256 Dv512
   c3_retnet_parallel  same shape, normalised parallel operator with a [1,H,S,S] decay mask
+  c3_retnet_parallel_generated_mask  the same operator told the mask is gamma_h^(i-j) (decay_gamma): no mask tensor is read
   c3_retnet_parallel_bwd  backward of that operator (dq, dk, dv; the row scale held constant, as the reference defines it)
   c4_mamba2_ssd       Mamba2 SSD, B8 H64 S2048 P64 N128, one B/C group
   c5_mla_decode       absorbed MLA decode, B64 Hq128 KV4096 d512+64 (HBM bound)
@@ -204,7 +205,7 @@ def bench_retnet_chunked(steps, warmup):
     return _mfma_entry(ms, flops, "chunked form, chunk 64: 2*S*C*(Dqk+Dv) + 4*S*Dqk*Dv per (batch, head)")
 
 
-def bench_retnet_parallel(steps, warmup, backward=False):
+def bench_retnet_parallel(steps, warmup, backward=False, generated_mask=False):
     import torch
     from metaattention_amd import hip_backend as hb
     B, H, S, D, DV = 8, 16, 2048, 256, 512
@@ -226,9 +227,16 @@ def bench_retnet_parallel(steps, warmup, backward=False):
         ms = time_gpu(lambda: hb.attn_bwd(q, k, v, o, do, r, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mask,
                                           score_mask_t=mask_t), max(steps // 3, 3), 2)
         return _mfma_entry(ms, 2.5 * flops, "backward, 2.5 x the forward's algorithmic FLOPs (three kernels dq, dv, dk)")
+    if generated_mask:
+        gamma = gam.contiguous()
+        ms = time_gpu(lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, decay_gamma=gamma, out=o,
+                                          row_scale=r), steps, warmup)
+        return _mfma_entry(ms, flops, "parallel form, causal counted at one half; the decay mask gamma_h^(i-j) is generated by the kernel "
+                                      "from the per-head gamma (decay_gamma) instead of being read as a [1,H,S,S] tensor")
     ms = time_gpu(lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mask, out=o,
                                       row_scale=r), steps, warmup)
-    return _mfma_entry(ms, flops, "parallel form, causal counted at one half")
+    return _mfma_entry(ms, flops, "parallel form, causal counted at one half; the decay mask is a [1,H,S,S] bf16 tensor argument, as the "
+                                  "reference's operator takes it")
 
 
 def bench_mamba2(steps, warmup):
@@ -388,6 +396,7 @@ def main():
              ("c2_softmax_causal_bwd", "bwd", lambda: bench_softmax_bwd(args.steps, args.warmup)),
              ("c3_retnet_chunked", "retnet", lambda: bench_retnet_chunked(args.steps, args.warmup)),
              ("c3_retnet_parallel", "retention", lambda: bench_retnet_parallel(args.steps, args.warmup)),
+             ("c3_retnet_parallel_generated_mask", "retention_gamma", lambda: bench_retnet_parallel(args.steps, args.warmup, generated_mask=True)),
              ("c3_retnet_parallel_bwd", "retention_bwd", lambda: bench_retnet_parallel(args.steps, args.warmup, backward=True)),
              ("c4_mamba2_ssd", "mamba", lambda: bench_mamba2(args.steps, args.warmup)),
              ("c5_mla_decode", "mla", lambda: bench_mla(args.steps, args.warmup)),

@@ -113,6 +113,11 @@ typedef struct ma_attn_params {
   const void* score_add; int64_t sa_stride_b, sa_stride_h, sa_stride_q, sa_stride_kv; int32_t score_add_fp32;
   const float* pos_slope_q; const float* pos_slope_kv;
   float softcap;
+  /* RETENTION at Dqk 256 / Dv 512 under MA_MASK_CAUSAL, instead of score_mask: fp32 [heads].  Says that the multiplier is
+   * the geometric decay mask of RetNet, M[h, q, kv] = decay_gamma[h]^(q - kv) for kv <= q and 0 above the diagonal
+   * (examples/retention_parallel.py:11-23 builds that tensor on the host); the kernel then generates it in fp32 instead
+   * of reading a [1, H, Sq, Skv] tensor once per batch entry. */
+  const float* decay_gamma;
 } ma_attn_params;
 
 /* Parallel attention backward for the SOFTMAX, SIGMOID, RELU and RETENTION families.  Replaces the backward of

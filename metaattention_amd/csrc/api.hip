@@ -65,8 +65,10 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
     if ((uintptr_t)p->elem_mask % 4 != 0 || p->em_stride_q % 4 != 0 || p->em_stride_h % 4 != 0 || p->em_stride_b % 4 != 0)
       return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: elem_mask rows must be 4-byte aligned");
   }
-  if (p->family == MA_ATTN_RETENTION) {
-    if (!p->score_mask) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: RETENTION needs score_mask");
+  if (p->decay_gamma && (p->family != MA_ATTN_RETENTION || p->score_mask || p->mask != MA_MASK_CAUSAL || p->dim_qk != 256 || p->dim_v != 512))
+    return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: decay_gamma replaces score_mask in the RETENTION family at Dqk 256 / Dv 512 under MA_MASK_CAUSAL");
+  if (p->family == MA_ATTN_RETENTION && !p->decay_gamma) {
+    if (!p->score_mask) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: RETENTION needs score_mask (or decay_gamma)");
     if ((uintptr_t)p->score_mask % 8 != 0 || p->sm_stride_b % 4 != 0 || p->sm_stride_h % 4 != 0 || p->sm_stride_q % 4 != 0)
       return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: score_mask must be 8-byte aligned with strides that are multiples of 4 elements");
   }
@@ -104,6 +106,7 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
     }
   }
   a.scale = p->scale; a.bias = p->bias;
+  a.decay_gamma = p->decay_gamma;
   if (p->score_add || p->pos_slope_q || p->pos_slope_kv || p->softcap != 0.f) {
     if (p->family == MA_ATTN_RETENTION)
       return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: score_add / pos_slope / softcap go with the softmax / sigmoid / relu families");

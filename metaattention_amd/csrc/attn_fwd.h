@@ -37,13 +37,15 @@ struct AttnArgs {
   const float* slope_q;
   const float* slope_kv;
   float softcap;
+  // retention family at Dqk 256 / Dv 512, instead of smask: fp32 [H], the multiplier is gamma[h]^(q - kv) for kv <= q, else 0
+  const float* decay_gamma;
 };
 
 int attn_wide_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);
 // number of kv splits the decode path would use for these sizes (1: not a decode shape / nothing to gain)
 int attn_decode_splits(int family, bool causal, int B, int H, int Sq, int Skv, int dqk, int dv);
 int attn_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);
-// the retention family at Dqk 256 / Dv 512 (retention_fwd.hip); 0 ok, -1 launch failure
+// the retention family at Dqk 256 / Dv 512 (retention_fwd.hip); 0 ok, -1 launch failure, -2 unsupported
 int retention_pair_fwd_dispatch(const AttnArgs& a, bool causal, bool is_bf16, hipStream_t stream);
 
 }  // namespace ma

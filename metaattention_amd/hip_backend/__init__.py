@@ -55,6 +55,7 @@ class AttnParams(Structure):
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("score_add", c_void_p), ("sa_stride_b", c_int64), ("sa_stride_h", c_int64), ("sa_stride_q", c_int64), ("sa_stride_kv", c_int64),
         ("score_add_fp32", c_int32), ("pos_slope_q", c_void_p), ("pos_slope_kv", c_void_p), ("softcap", c_float),
+        ("decay_gamma", c_void_p),
     ]
 
 
@@ -183,12 +184,14 @@ def _require_gpu(*tensors):
 def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None,
              score_mask=None, out=None, row_scale=None, kv_seqlens=None, kv_block_mask=None, kv_block_size: int = 0,
              workspace=None, split_kv: bool = True, elem_mask=None, score_add=None, pos_slope_q=None, pos_slope_kv=None,
-             softcap: float = 0.0):
+             softcap: float = 0.0, decay_gamma=None):
     """Parallel attention forward on BSHD tensors.  Returns ``out`` ([B,Sq,H,Dv]).  k and v may
     have fewer heads than q (grouped-query: query head h reads kv head h // (H // Hkv)).
     score_add: fp32 or q.dtype tensor broadcastable as [B|1, H|1, Sq|1, Skv|1] added to the scaled score;
     pos_slope_q / pos_slope_kv: fp32 [H], the score gets slope_q[h] * q_idx + slope_kv[h] * kv_idx;
-    softcap > 0: softmax of softcap * tanh(x)."""
+    softcap > 0: softmax of softcap * tanh(x).
+    decay_gamma: fp32 [H], for the retention family at 256 / 512 instead of score_mask: the multiplier is
+    gamma[h]^(q - kv) below and on the diagonal, generated by the kernel."""
     _require_gpu(q, k, v, bias_tensor, score_mask, out, row_scale, kv_seqlens, kv_block_mask, score_add, pos_slope_q, pos_slope_kv)
     B, Sq, H, Dqk = q.shape
     Skv, Hkv, Dv = k.shape[1], k.shape[2], v.shape[-1]
@@ -253,6 +256,9 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
             assert t.dtype == torch.float32 and t.shape == (H,) and t.is_contiguous()
             setattr(p, name, t.data_ptr())
     p.softcap = float(softcap)
+    if decay_gamma is not None:
+        assert decay_gamma.dtype == torch.float32 and decay_gamma.shape == (H,) and decay_gamma.is_contiguous() and decay_gamma.is_cuda
+        p.decay_gamma = decay_gamma.data_ptr()
     lib = load_library()
     if split_kv:
         need = lib.ma_attn_workspace_bytes(ctypes.byref(p))

@@ -41,6 +41,31 @@ def test_retention_parallel(B, H, S, D, DV, causal):
     torch.testing.assert_close(rs.cpu(), r_ref, rtol=1e-3, atol=1e-3)
 
 
+@pytest.mark.parametrize("B,H,S", [(1, 2, 128), (2, 3, 200), (1, 16, 700), (1, 1, 5)])
+def test_retention_parallel_generated_decay_mask(B, H, S):
+    """decay_gamma [H] instead of the multiplier tensor: the kernel generates gamma_h^(i - j) [i >= j] itself.  Checked
+    against the oracle fed with that mask in fp32 (the tensor form rounds it to the tensor dtype first), and against the
+    tensor path of the same kernel within the rounding of the bf16 mask."""
+    hb = _hb()
+    D, DV = 256, 512
+    q, k, v, mask_bf16 = _inputs(B, H, S, D, DV, seed=S + 1)
+    mask = oracle.retention_decay_mask(H, S)                    # fp32
+    gamma = (1.0 - torch.exp2(-5.0 - torch.arange(H, dtype=torch.float64))).float()
+    ref, r_ref = oracle.retention_parallel(q, k, v, mask, return_r=True)
+    rs = torch.full((B, H, S), float("nan"), device="cuda")
+    o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, decay_gamma=gamma.cuda(),
+                    row_scale=rs)
+    torch.cuda.synchronize()
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(rs.cpu(), r_ref, rtol=1e-3, atol=1e-3)
+    if S % 4 == 0:   # (the tensor form wants 8-byte aligned mask rows)
+        o_t = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mask_bf16.cuda())
+        torch.cuda.synchronize()
+        oracle.assert_close(o.float().cpu(), o_t.float().cpu(), rtol=2 * RTOL, atol=2 * ATOL)
+    with pytest.raises(hb.MetaAttentionError):   # the generated mask is lower triangular: it goes with the causal structural mask
+        hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_RETENTION, causal=False, scale=1.0, decay_gamma=gamma.cuda())
+
+
 def test_clamp_branch_leaves_rows_unnormalised():
     """Tiny scores: every row sum is below 1, r = 1 everywhere, o = (qk * M) v exactly as un-normalised retention."""
     hb = _hb()
