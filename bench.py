@@ -40,7 +40,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy: the
 # profile summary of that kernel holds the figure in a line "hbm_traffic_bytes_per_launch[<kernel>]: <bytes>"
 ATTN_FWD_PROFILE = os.path.join(ROOT, "profiles", "attn_fwd_kernel_c2_softmax_sigmoid.md")
-ATTN_FWD_KERNEL = "ma::attn_fwd_kernel<bf16, 128, 128, softmax, causal>"
+ATTN_FWD_KERNEL = "ma::attn_fwd_kernel<bf16, 128, 128, 0, true>"   # (element type, Dqk, Dv, family 0 = softmax, causal)
 
 
 def profiled_traffic(path, kernel):
