@@ -62,7 +62,7 @@ def test_relu_other_head_sizes(B, H, S, D, DV):
     torch.cuda.synchronize()
     # outputs are un-normalised sums over S keys: the reference accepts rtol=atol=1e-1 with 1e-3 of the elements off (:623)
     oracle.assert_close(o.float().cpu(), ref, rtol=1e-1, atol=1e-1, mismatch_ratio=1e-3)
-    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=5e-2)
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=1e-3)
 
 
 def test_reference_softmax_test_shape_128_256():
@@ -143,7 +143,7 @@ def test_grouped_query_prefill(D, DV, H, Hkv, family):
         ref = oracle.relu_attention(q, k, v)
         o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_RELU, causal=False, scale=scale)
     torch.cuda.synchronize()
-    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=5e-2 if family == "relu" else 0.0)
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=1e-3 if family == "relu" else 0.0)
     o_rep = hb.attn_fwd(q.cuda(), k.repeat_interleave(H // Hkv, dim=2).cuda(), v.repeat_interleave(H // Hkv, dim=2).cuda(),
                         family={"softmax": hb.MA_ATTN_SOFTMAX, "sigmoid": hb.MA_ATTN_SIGMOID, "relu": hb.MA_ATTN_RELU}[family],
                         causal=family != "relu", scale=scale, bias=-3.0 if family == "sigmoid" else 0.0)
@@ -346,7 +346,7 @@ def test_engine_block_sparse_prefill(family, mask, D, S, bq, bk):
                   torch.arange(S).view(1, 1, 1, S)).expand(B, H, S, S)
     ref = oracle.masked_attention(q, k, v, keep=keep, block_mask=bm, family=family, softmax_scale=1 / math.sqrt(D), bias=-math.log(S))
     # (un-normalised relu sums: the rounding of the probabilities to bf16 alone is ~2.5e-2 rms at these sizes)
-    ratio = 5e-2 if family == "relu" else 0.0
+    ratio = 2e-2 if family == "relu" else 0.0
     oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=ratio)
     assert torch.count_nonzero(o[0, bq:2 * bq, 0]) == 0
     # a broadcast mask [1, 1, nq, nk], and the all-ones mask == the dense operator

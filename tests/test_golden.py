@@ -115,7 +115,7 @@ def _g_sigmoid(hb, d):
 def _g_relu(hb, d):
     o = hb.attn_fwd(d["q"].cuda(), d["k"].cuda(), d["v"].cuda(), family=hb.MA_ATTN_RELU, causal=False, scale=1 / math.sqrt(d["q"].shape[-1]))
     # un-normalised sums: the reference accepts rtol=atol=1e-1 with 1e-3 of the elements off (testing/test.py:623)
-    return {"out": (o, RTOL, ATOL, 5e-2), "out ": (o, 1e-1, 1e-1, 1e-3)}
+    return {"out": (o, RTOL, ATOL, 1e-3), "out ": (o, 1e-1, 1e-1, 1e-3)}
 
 
 def _g_retention(hb, d):

@@ -91,7 +91,7 @@ def test_engine_gated_retention():
     torch.cuda.synchronize()
     ref = oracle.simple_gla_chunked(q, k, v, g)
     oracle.assert_close(o.float().cpu(), ref, rtol=1e-1, atol=1e-1)
-    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=2e-2)   # outputs are O(10): bf16 output rounding
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=1e-3)   # outputs are O(10): bf16 output rounding
 
 
 def test_full_size_properties():
