@@ -188,7 +188,7 @@ def bench_decode(steps, warmup, B=64, H=32, Hkv=8, Skv=4096, D=128):
                 note="split-KV kernel + combine kernel per call; caches overwritten before every timed call")
 
 
-def bench_retnet_chunked(steps, warmup):
+def bench_retnet_chunked(steps, warmup, backward=False):
     import torch
     from metaattention_amd import hip_backend as hb
     B, H, T, Dk, Dv = 8, 16, 2048, 256, 512
@@ -197,11 +197,17 @@ def bench_retnet_chunked(steps, warmup):
     k = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 16).bfloat16()
     v = torch.randn(B, H, T, Dv, device="cuda", generator=g).bfloat16()
     ld = torch.log(1 - torch.exp2(-5 - torch.arange(H, device="cuda").float())).view(1, H, 1).expand(B, H, T).contiguous()
+    C = 64
+    flops = B * H * (2.0 * T * C * (Dk + Dv) + 4.0 * T * Dk * Dv)
+    if backward:
+        do = torch.randn(B, H, T, Dv, device="cuda", generator=g).bfloat16()
+        ws = torch.empty(_linear_bwd_workspace(hb, B, H, H, H, T, Dk, Dv), dtype=torch.uint8, device="cuda")
+        ms = time_gpu(lambda: hb.linear_bwd(q, k, v, ld, do, q_scale=Dk ** -0.5, workspace=ws), max(steps // 3, 3), 2)
+        return _mfma_entry(ms, 2.5 * flops, "backward (dq, dk, dv, dlog_decay), 2.5 x the forward's algorithmic FLOPs; five scans of the "
+                                            "forward kernel (the two 512-wide contractions in two pieces) + packing + epilogue")
     o = torch.empty_like(v)
     ws = torch.empty(max(hb.linear_workspace_bytes(B, H, H, H, T, Dk, Dv), 16), dtype=torch.uint8, device="cuda")
     ms = time_gpu(lambda: hb.linear_fwd(q, k, v, ld, q_scale=Dk ** -0.5, out=o, workspace=ws), steps, warmup)
-    C = 64
-    flops = B * H * (2.0 * T * C * (Dk + Dv) + 4.0 * T * Dk * Dv)
     return _mfma_entry(ms, flops, "chunked form, chunk 64: 2*S*C*(Dqk+Dv) + 4*S*Dqk*Dv per (batch, head)")
 
 
@@ -239,7 +245,14 @@ def bench_retnet_parallel(steps, warmup, backward=False, generated_mask=False):
                                   "reference's operator takes it")
 
 
-def bench_mamba2(steps, warmup):
+def _linear_bwd_workspace(hb, B, H, Hq, Hk, T, Dk, Dv):
+    import ctypes
+    p = hb.LinearBwdParams()
+    p.dtype, p.batch, p.heads, p.heads_q, p.heads_k, p.seqlen, p.dim_k, p.dim_v = hb.MA_BF16, B, H, Hq, Hk, T, Dk, Dv
+    return max(hb.load_library().ma_linear_bwd_workspace_bytes(ctypes.byref(p)), 16)
+
+
+def bench_mamba2(steps, warmup, backward=False):
     import torch
     from metaattention_amd import hip_backend as hb
     B, H, T, P, N = 8, 64, 2048, 64, 128
@@ -250,11 +263,17 @@ def bench_mamba2(steps, warmup):
     dt = torch.nn.functional.softplus(torch.randn(B, H, T, device="cuda", generator=g) - 2)
     A = -torch.exp(torch.rand(1, H, device="cuda", generator=g) * math.log(16))
     ld = (dt * A.view(1, H, 1)).contiguous()
+    Lc = 256
+    flops = B * H * (2.0 * T * Lc * N + 2.0 * T * Lc * P + 4.0 * T * N * P)
+    if backward:
+        do = torch.randn(B, H, T, P, device="cuda", generator=g).bfloat16()
+        ws = torch.empty(_linear_bwd_workspace(hb, B, H, 1, 1, T, N, P), dtype=torch.uint8, device="cuda")
+        ms = time_gpu(lambda: hb.linear_bwd(Cm, Bm, x, ld, do, v_scale=dt, workspace=ws), max(steps // 3, 3), 2)
+        return _mfma_entry(ms, 2.5 * flops, "backward (dC, dB, dx, dlog_decay, ddt-scale), 2.5 x the forward's algorithmic FLOPs; three scans "
+                                            "of the forward kernel + packing + epilogue")
     o = torch.empty_like(x)
     ws = torch.empty(max(hb.linear_workspace_bytes(B, H, 1, 1, T, N, P), 16), dtype=torch.uint8, device="cuda")
     ms = time_gpu(lambda: hb.linear_fwd(Cm, Bm, x, ld, v_scale=dt, out=o, workspace=ws), steps, warmup)
-    Lc = 256
-    flops = B * H * (2.0 * T * Lc * N + 2.0 * T * Lc * P + 4.0 * T * N * P)
     return _mfma_entry(ms, flops, "chunk 256, C.B^T counted per head: 2*S*L*N + 2*S*L*P + 4*S*N*P per (batch, head); "
                                   "the kernel itself uses 32-token chunks and executes fewer FLOPs")
 
@@ -443,10 +462,12 @@ def main():
              ("c2_softmax_causal_operator", "operator", lambda: bench_softmax_operator(args.steps, args.warmup)),
              ("c2_softmax_causal_bwd", "bwd", lambda: bench_softmax_bwd(args.steps, args.warmup)),
              ("c3_retnet_chunked", "retnet", lambda: bench_retnet_chunked(args.steps, args.warmup)),
+             ("c3_retnet_chunked_bwd", "retnet_bwd", lambda: bench_retnet_chunked(args.steps, args.warmup, backward=True)),
              ("c3_retnet_parallel", "retention", lambda: bench_retnet_parallel(args.steps, args.warmup)),
              ("c3_retnet_parallel_generated_mask", "retention_gamma", lambda: bench_retnet_parallel(args.steps, args.warmup, generated_mask=True)),
              ("c3_retnet_parallel_bwd", "retention_bwd", lambda: bench_retnet_parallel(args.steps, args.warmup, backward=True)),
              ("c4_mamba2_ssd", "mamba", lambda: bench_mamba2(args.steps, args.warmup)),
+             ("c4_mamba2_bwd", "mamba_bwd", lambda: bench_mamba2(args.steps, args.warmup, backward=True)),
              ("c5_mla_decode", "mla", lambda: bench_mla(args.steps, args.warmup)),
              ("gqa_decode", "decode", lambda: bench_decode(args.steps, args.warmup))]
     cpu_legs = {"c3_retnet_chunked": cpu_baseline_retnet_chunked, "c3_retnet_parallel": cpu_baseline_retention_parallel,

@@ -185,6 +185,27 @@ typedef struct ma_linear_params {
   void* workspace; size_t workspace_bytes; /* see ma_linear_workspace_bytes; may be NULL (then single pass) */
 } ma_linear_params;
 
+/* Chunked linear / stateful attention backward.  Replaces LinearAttention.backward
+ * (tl_template/linear/linear_tl.py:1268-1340: chunk_bwd_kernel_dh :461, chunk_bwd_dqkg :606, chunk_bwd_kernel_dv :876,
+ * compute_final_dg :64-76): gradients of ma_linear_fwd's o with respect to q, k, v, log_decay and v_scale, given dout.
+ * Tensors as in ma_linear_params (bf16, BHSD, contiguous, 16-byte aligned); dout [B,H,T,Dv] bf16; dq, dk, dv are bf16
+ * with the shapes of q, k, v (heads that share a q / k head have their gradients summed, :1300-1303); dlog_decay fp32
+ * [B,H,T]; dv_scale fp32 [B,H,T], written when v_scale is given (may then still be NULL to skip it).  dim_k 128 or 256,
+ * dim_v a multiple of 64.  The workspace (ma_linear_bwd_workspace_bytes, 256-byte aligned) holds the fp32 per-head
+ * gradients the decay gradient is formed from, and is required. */
+typedef struct ma_linear_bwd_params {
+  int32_t dtype;
+  int32_t batch, heads, heads_q, heads_k, seqlen, dim_k, dim_v;
+  const void* q; const void* k; const void* v; const void* dout;
+  const float* log_decay;
+  const float* v_scale;
+  float q_scale;
+  void* dq; void* dk; void* dv;
+  float* dlog_decay;
+  float* dv_scale;
+  void* workspace; size_t workspace_bytes;
+} ma_linear_bwd_params;
+
 /* Absorbed MLA decode forward.  Replaces flash_attn_split + combine
  * (tl_template/attn/mla_decode_tl.py:154-290, wrapper :450-459):
  *   o = softmax((q.kv^T + q_pe.k_pe^T) * scale) . kv
@@ -245,6 +266,10 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream);
 /* linear_tl.py:1240-1269 */
 size_t ma_linear_workspace_bytes(const ma_linear_params* p);
 int ma_linear_fwd(const ma_linear_params* p, ma_stream_t stream);
+
+/* linear_tl.py:1268-1340 */
+size_t ma_linear_bwd_workspace_bytes(const ma_linear_bwd_params* p);
+int ma_linear_bwd(const ma_linear_bwd_params* p, ma_stream_t stream);
 
 /* mla_decode_tl.py:293-303 (`main_split`) */
 int ma_mla_choose_split(const ma_mla_params* p);

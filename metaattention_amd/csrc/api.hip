@@ -4,6 +4,7 @@
 #include "attn_fwd.h"
 #include "attn_bwd.h"
 #include "linear_fwd.h"
+#include "linear_bwd.h"
 #include "mla_decode.h"
 
 #include <atomic>
@@ -227,7 +228,7 @@ static ma::LinArgs linear_args(const ma_linear_params* p) {
   ma::LinArgs a{};
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.log_decay = p->log_decay; a.v_scale = p->v_scale;
   a.q_scale = p->q_scale;
-  a.out_f32 = p->out_fp32 != 0;
+  a.out_f32 = p->out_fp32 != 0 ? 1 : 0;
   a.B = p->batch; a.H = p->heads; a.Hq = p->heads_q; a.Hk = p->heads_k; a.T = p->seqlen; a.Dv = p->dim_v;
   return a;
 }
@@ -257,6 +258,55 @@ int ma_linear_fwd(const ma_linear_params* p, ma_stream_t stream) {
   if (rc == -2)
     return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: no kernel for dim_k=%d (128 or 256) / dim_v=%d (multiple of 64)", p->dim_k, p->dim_v);
   if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_linear_fwd: launch failed: %s", hipGetErrorString(ma::t_hip_error));
+  return MA_OK;
+}
+
+static int check_linear_bwd(const ma_linear_bwd_params* p, const char* who) {
+  if (!p) return fail(MA_ERR_INVALID_ARG, "%s: params is NULL", who);
+  if (p->batch <= 0 || p->heads <= 0 || p->heads_q <= 0 || p->heads_k <= 0 || p->seqlen <= 0 || p->dim_k <= 0 || p->dim_v <= 0)
+    return fail(MA_ERR_INVALID_ARG, "%s: sizes must be positive", who);
+  if (p->dtype != MA_BF16) return fail(MA_ERR_UNSUPPORTED, "%s: only bf16 (the reference's linear kernels are bf16 only)", who);
+  if (p->heads % p->heads_q != 0 || p->heads % p->heads_k != 0)
+    return fail(MA_ERR_INVALID_ARG, "%s: heads (%d) must be a multiple of heads_q (%d) and heads_k (%d)", who, p->heads, p->heads_q, p->heads_k);
+  if ((p->dim_k != 128 && p->dim_k != 256) || p->dim_v % 64 != 0 || p->dim_v > 4096)
+    return fail(MA_ERR_UNSUPPORTED, "%s: dim_k=%d must be 128 or 256 and dim_v=%d a multiple of 64 (at most 4096)", who, p->dim_k, p->dim_v);
+  if ((int64_t)p->batch * p->heads * p->seqlen * (int64_t)(p->dim_k > p->dim_v ? p->dim_k : p->dim_v) / 8 > 0x7fffffffll * 256)
+    return fail(MA_ERR_UNSUPPORTED, "%s: grid too large", who);
+  return MA_OK;
+}
+
+static ma::LinBwdArgs linear_bwd_args(const ma_linear_bwd_params* p) {
+  ma::LinBwdArgs a{};
+  a.q = p->q; a.k = p->k; a.v = p->v; a.dout = p->dout; a.log_decay = p->log_decay; a.v_scale = p->v_scale;
+  a.dq = p->dq; a.dk = p->dk; a.dv = p->dv; a.dlog_decay = p->dlog_decay; a.dv_scale = p->v_scale ? p->dv_scale : nullptr;
+  a.q_scale = p->q_scale;
+  a.B = p->batch; a.H = p->heads; a.Hq = p->heads_q; a.Hk = p->heads_k; a.T = p->seqlen; a.Dk = p->dim_k; a.Dv = p->dim_v;
+  return a;
+}
+
+// Returns 0 for arguments ma_linear_bwd would refuse.
+size_t ma_linear_bwd_workspace_bytes(const ma_linear_bwd_params* p) {
+  if (!p || p->batch <= 0 || p->heads <= 0 || p->heads_q <= 0 || p->heads_k <= 0 || p->seqlen <= 0 || p->heads % p->heads_q != 0 ||
+      p->heads % p->heads_k != 0)
+    return 0;
+  size_t bytes = 0;
+  if (ma::linear_bwd_run(linear_bwd_args(p), nullptr, 0, nullptr, &bytes) != 0) return 0;
+  return bytes;
+}
+
+int ma_linear_bwd(const ma_linear_bwd_params* p, ma_stream_t stream) {
+  if (const int rc0 = check_linear_bwd(p, "ma_linear_bwd")) return rc0;
+  if (!p->q || !p->k || !p->v || !p->dout || !p->log_decay || !p->dq || !p->dk || !p->dv || !p->dlog_decay)
+    return fail(MA_ERR_INVALID_ARG, "ma_linear_bwd: q/k/v/dout/log_decay/dq/dk/dv/dlog_decay must be non-NULL");
+  const uintptr_t ptrs[] = {(uintptr_t)p->q, (uintptr_t)p->k, (uintptr_t)p->v, (uintptr_t)p->dout, (uintptr_t)p->dq, (uintptr_t)p->dk, (uintptr_t)p->dv};
+  for (uintptr_t x : ptrs)
+    if (x % 16 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_linear_bwd: q/k/v/dout/dq/dk/dv must be 16-byte aligned");
+  const int rc = ma::linear_bwd_run(linear_bwd_args(p), p->workspace, p->workspace_bytes, (hipStream_t)stream, nullptr);
+  if (rc == -3)
+    return fail(MA_ERR_WORKSPACE, "ma_linear_bwd: workspace missing, smaller than ma_linear_bwd_workspace_bytes (%zu) or not 256-byte aligned",
+                ma_linear_bwd_workspace_bytes(p));
+  if (rc == -2) return fail(MA_ERR_UNSUPPORTED, "ma_linear_bwd: no kernel for dim_k=%d / dim_v=%d", p->dim_k, p->dim_v);
+  if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_linear_bwd: launch failed: %s", hipGetErrorString(ma::t_hip_error));
   return MA_OK;
 }
 

@@ -1,0 +1,289 @@
+// Chunked linear / stateful attention backward (RetNet retention, Mamba2 SSD, gated retention) for gfx950.
+//
+// Replaces LinearAttention.backward of attention_engine/core/template/tl_template/linear/linear_tl.py:1268-1340
+// (chunk_bwd_kernel_dh :461, chunk_bwd_dqkg :606, chunk_bwd_kernel_dv :876, compute_final_dg :64-76).  The reference
+// materialises the forward state h and its gradient dh per chunk in HBM (bf16) and then visits the chunks in parallel.
+// Here no state ever leaves the chip.  With
+//   A_ts = q_scale (q_t . k_s) exp(G_t - G_s) [s <= t],   u = v * v_scale,   o = A u,   G = cumsum(log_decay)
+// the three gradients
+//   dq_t = q_scale sum_{s<=t} exp(G_t - G_s) (do_t . u_s) k_s
+//   du_s = sum_{t>=s} A_ts do_t
+//   dk_s = q_scale sum_{t>=s} exp(G_t - G_s) (do_t . u_s) q_t
+// are the forward operator LA(q, k, v) itself on permuted operands, the two sums over LATER tokens on the time-reversed
+// sequence with the log decay shifted by one token:
+//   dq = LA(do, v, k; v_scale)      du = R LA(R k, R q, R do)      dk = v_scale * R LA(R v, R do, R q)      (R reverses time)
+// so the backward pass is three scans of the forward kernel (linear_fwd.hip: state in accumulator registers, fp32
+// outputs), each contraction cut into the 128 / 256 wide pieces that kernel takes (their fp32 outputs add up), plus the
+// small kernels of this file: operand packing (time reversal, column slices, zero padding, head expansion), the shifted
+// reversed log decay, and the epilogue that forms dv, dv_scale, the per-token decay gradient
+//   dG_t = q_t . dq_t - k_t . dk_t        (fp32 products of the fp32 scan outputs)
+// sums the heads that share a q / k head (:1300-1303), converts, and turns dG into dlog_decay by a reversed running sum
+// in fp32 (compute_final_dg).
+#include "linear_bwd.h"
+
+#include "linear_fwd.h"
+
+namespace ma {
+
+namespace {
+
+// dst [B, Hd, T, W] bf16 <- src [B, Hs, T, Ws] columns c0 .. c0 + W (zeros beyond Ws), head hd reads source head
+// hd / (Hd / Hs), row t reads row T - 1 - t when rev.  One thread per 16 bytes of dst.
+__global__ __launch_bounds__(256) void pack_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, int Hd, int Hs, int T, int W, int Ws,
+                                                  int c0, int rev, int64_t n_chunks) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n_chunks) return;
+  const int cpr = W / 8;
+  const int c = (int)(i % cpr);
+  const int64_t row = i / cpr;
+  const int t = (int)(row % T);
+  const int64_t bh = row / T;
+  const int hd = (int)(bh % Hd);
+  const int64_t b = bh / Hd;
+  const int col = c0 + 8 * c;
+  uint4 val = {0u, 0u, 0u, 0u};
+  if (col < Ws) {
+    const int ts = rev ? T - 1 - t : t;
+    val = src[(((b * Hs + hd / (Hd / Hs)) * T + ts) * (int64_t)Ws + col) / 8];
+  }
+  dst[i] = val;
+}
+
+// g_rev[b, h, t'] = log_decay[b, h, T - t'] for t' >= 1, 0 for t' = 0: the decay between reversed tokens t' - 1 and t'
+__global__ __launch_bounds__(256) void shift_rev_kernel(float* __restrict__ dst, const float* __restrict__ src, int T, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int t = (int)(i % T);
+  dst[i] = t >= 1 ? src[i - t + (T - t)] : 0.f;
+}
+
+// sum over the LPT lanes (a power of two) that share a token
+template <int LPT>
+__device__ __forceinline__ float lanes_sum(float x) {
+#pragma unroll
+  for (int off = LPT / 2; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);
+  return x;
+}
+
+// LPT lanes per (batch, head, token), four columns per lane and round.  dqh [B,H,T,Dk] fp32 (time order), dkh_rev [B,H,T,Dk]
+// and du_rev [B,H,T,Dv] fp32 (reversed time order, dk before its v_scale factor).  Writes dG, dv, dv_scale and, where every
+// head has its own q / k head, dq / dk.
+template <int LPT>
+__global__ __launch_bounds__(256) void grads_kernel(LinBwdArgs a, const float* __restrict__ dqh, const float* __restrict__ dkh_rev,
+                                                   const float* __restrict__ du_rev, float* __restrict__ dG) {
+  const int sub = threadIdx.x % LPT;
+  const int64_t tok = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPT;
+  const bool live = tok < (int64_t)a.B * a.H * a.T;   // (dead lanes take part in the shuffles with zeros)
+  const int64_t tk = live ? tok : 0;
+  const int t = (int)(tk % a.T);
+  const int64_t bh = tk / a.T;
+  const int h = (int)(bh % a.H);
+  const int64_t b = bh / a.H;
+  const int64_t rtok = bh * a.T + (a.T - 1 - t);
+  const float vs = a.v_scale ? a.v_scale[tk] : 1.f;
+  const int hq = h / (a.H / a.Hq), hk = h / (a.H / a.Hk);
+  const __bf16* qrow = (const __bf16*)a.q + ((b * a.Hq + hq) * a.T + t) * (int64_t)a.Dk;
+  const __bf16* krow = (const __bf16*)a.k + ((b * a.Hk + hk) * a.T + t) * (int64_t)a.Dk;
+  float acc = 0.f, acc_vs = 0.f;
+  if (live) {
+    for (int c = 4 * sub; c < a.Dk; c += 4 * LPT) {
+      const f32x4 gq = *(const f32x4*)(dqh + tk * a.Dk + c);
+      f32x4 gk = *(const f32x4*)(dkh_rev + rtok * a.Dk + c);
+      const bf16x4 qv = *(const bf16x4*)(qrow + c), kv = *(const bf16x4*)(krow + c);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        gk[i] *= vs;
+        acc += (float)qv[i] * gq[i] - (float)kv[i] * gk[i];
+      }
+      if (a.Hq == a.H) {
+        bf16x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (__bf16)gq[i];
+        *(bf16x4*)((__bf16*)a.dq + tk * a.Dk + c) = w;
+      }
+      if (a.Hk == a.H) {
+        bf16x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (__bf16)gk[i];
+        *(bf16x4*)((__bf16*)a.dk + tk * a.Dk + c) = w;
+      }
+    }
+    for (int c = 4 * sub; c < a.Dv; c += 4 * LPT) {
+      const f32x4 gu = *(const f32x4*)(du_rev + rtok * a.Dv + c);
+      const bf16x4 vv = *(const bf16x4*)((const __bf16*)a.v + tk * a.Dv + c);
+      bf16x4 w;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        acc_vs += (float)vv[i] * gu[i];
+        w[i] = (__bf16)(gu[i] * vs);
+      }
+      *(bf16x4*)((__bf16*)a.dv + tk * a.Dv + c) = w;
+    }
+  }
+  acc = lanes_sum<LPT>(acc);
+  acc_vs = lanes_sum<LPT>(acc_vs);
+  if (live && sub == 0) {
+    dG[tk] = acc;
+    if (a.dv_scale) a.dv_scale[tk] = acc_vs;
+  }
+}
+
+// dst [B, Hg, T, D] bf16 = sum over the G = H / Hg heads of a group of src [B, H, T, D] fp32 (row T - 1 - t when rev),
+// each times scale[b, h, t] when scale is given.  One thread per 4 columns.
+__global__ __launch_bounds__(256) void group_sum_kernel(__bf16* __restrict__ dst, const float* __restrict__ src, const float* __restrict__ scale,
+                                                       int H, int Hg, int T, int D, int rev, int64_t n4) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n4) return;
+  const int cpr = D / 4;
+  const int c = 4 * (int)(i % cpr);
+  const int64_t row = i / cpr;
+  const int t = (int)(row % T);
+  const int64_t bg = row / T;
+  const int g = (int)(bg % Hg);
+  const int64_t b = bg / Hg;
+  const int G = H / Hg, ts = rev ? T - 1 - t : t;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < G; j++) {
+    const int64_t bh = b * H + g * G + j;
+    const f32x4 x = *(const f32x4*)(src + (bh * T + ts) * (int64_t)D + c);
+    const float s = scale ? scale[bh * T + t] : 1.f;
+#pragma unroll
+    for (int k = 0; k < 4; k++) acc[k] += x[k] * s;
+  }
+  bf16x4 w;
+#pragma unroll
+  for (int k = 0; k < 4; k++) w[k] = (__bf16)acc[k];
+  *(bf16x4*)(dst + row * D + c) = w;
+}
+
+// dlog_decay[b, h, t] = sum_{t' >= t} dG[b, h, t']: one wave per (batch, head), blocks of 64 tokens from the end
+__global__ __launch_bounds__(64) void suffix_sum_kernel(float* __restrict__ dst, const float* __restrict__ dG, int T) {
+  const int lane = threadIdx.x;
+  const float* src = dG + (int64_t)blockIdx.x * T;
+  float* out = dst + (int64_t)blockIdx.x * T;
+  float carry = 0.f;
+  for (int t0 = (T - 1) / 64 * 64; t0 >= 0; t0 -= 64) {
+    const int t = t0 + lane;
+    float x = t < T ? src[t] : 0.f;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const float y = __shfl_down(x, off, 64);
+      if (lane + off < 64) x += y;
+    }
+    if (t < T) out[t] = x + carry;
+    carry += __shfl(x, 0, 64);
+  }
+}
+
+inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// the widths the scan kernel contracts over: pieces of 256 columns, a remainder (or a narrow operand) as 128 or 256
+struct Slices {
+  int n = 0, c0[16], w[16];
+  explicit Slices(int width) {
+    for (int c = 0; c < width && n < 16;) {
+      const int rest = width - c;
+      w[n] = rest > 128 ? 256 : 128;
+      c0[n] = c;
+      c += w[n];
+      n++;
+    }
+  }
+};
+
+}  // namespace
+
+int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t stream, size_t* query) {
+  if ((a.Dk != 128 && a.Dk != 256) || a.Dv % 64 != 0 || a.Dv > 16 * 256) return -2;
+  const int64_t BHT = (int64_t)a.B * a.H * a.T;
+  const Slices sl(a.Dv);   // contraction of the dq and dk scans
+  const bool direct_a = a.Dv == 128 || a.Dv == 256;   // the dq scan reads do and v as they are
+
+  // workspace: fp32 scan outputs, dG, reversed log decay, packed operands, the scan kernel's own workspace
+  size_t off = 0;
+  auto take = [&](size_t bytes) { const size_t o = off; off += align256(bytes); return o; };
+  const size_t o_dqh = take((size_t)BHT * a.Dk * 4), o_dkh = take((size_t)BHT * a.Dk * 4), o_du = take((size_t)BHT * a.Dv * 4);
+  const size_t o_dG = take((size_t)BHT * 4), o_grev = take((size_t)BHT * 4);
+  const size_t o_pa = take((size_t)BHT * 256 * 2), o_pb = take((size_t)BHT * 256 * 2);   // q and k operands of a scan
+  const size_t o_pv = take((size_t)BHT * (a.Dk > a.Dv ? a.Dk : a.Dv) * 2);                // v operand of a scan
+  // the scan kernel's workspace (sequence segments): the largest any of the scans asks for
+  size_t scan_ws = 0;
+  {
+    LinArgs la{};
+    la.B = a.B; la.H = a.H; la.T = a.T;
+    size_t need = 0;
+    la.Hq = la.Hk = a.H; la.Dv = a.Dk;
+    for (int s = 0; s < sl.n; s++)
+      if (linear_fwd_dispatch(la, sl.w[s], 0, nullptr, 0, nullptr, &need) == 0 && need > scan_ws) scan_ws = need;
+    la.Hq = a.Hk; la.Hk = a.Hq; la.Dv = a.Dv;
+    if (linear_fwd_dispatch(la, a.Dk, 0, nullptr, 0, nullptr, &need) == 0 && need > scan_ws) scan_ws = need;
+  }
+  const size_t o_scan = take(scan_ws);
+  if (query) { *query = off; return 0; }
+  if (!ws || ws_bytes < off || ((uintptr_t)ws & 255) != 0) return -3;
+  char* base = (char*)ws;
+  float *dqh = (float*)(base + o_dqh), *dkh = (float*)(base + o_dkh), *du = (float*)(base + o_du), *dG = (float*)(base + o_dG), *grev = (float*)(base + o_grev);
+  void *pa = base + o_pa, *pb = base + o_pb, *pv = base + o_pv, *scan = scan_ws ? base + o_scan : nullptr;
+
+  auto pack = [&](void* dst, const void* src, int Hd, int Hs, int W, int Ws, int c0, bool rev) {
+    const int64_t n = (int64_t)a.B * Hd * a.T * (W / 8);
+    hipLaunchKernelGGL(pack_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, (uint4*)dst, (const uint4*)src, Hd, Hs, a.T, W, Ws, c0,
+                       rev ? 1 : 0, n);
+  };
+  auto scan_launch = [&](const void* q, int Hq, const void* k, int Hk, const void* v, int dk, int dv, const float* g, const float* vs, float* out,
+                         bool accumulate) -> int {
+    LinArgs la{};
+    la.q = q; la.k = k; la.v = v; la.o = out; la.log_decay = g; la.v_scale = vs; la.q_scale = a.q_scale;
+    la.B = a.B; la.H = a.H; la.Hq = Hq; la.Hk = Hk; la.T = a.T; la.Dv = dv;
+    la.out_f32 = accumulate ? 2 : 1;
+    return linear_fwd_dispatch(la, dk, 0, scan, scan_ws, stream, nullptr);
+  };
+
+  hipLaunchKernelGGL(shift_rev_kernel, dim3((unsigned)((BHT + 255) / 256)), dim3(256), 0, stream, grev, a.log_decay, a.T, BHT);
+
+  // dq (per head) = LA(do, v, k; v_scale), contraction over the value columns
+  const void* k_heads = a.k;
+  if (a.Hk != a.H) { pack(pv, a.k, a.H, a.Hk, a.Dk, a.Dk, 0, false); k_heads = pv; }
+  for (int s = 0; s < sl.n; s++) {
+    const void *qs = a.dout, *ks = a.v;
+    if (!direct_a) {
+      pack(pa, a.dout, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], false);
+      pack(pb, a.v, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], false);
+      qs = pa; ks = pb;
+    }
+    if (const int rc = scan_launch(qs, a.H, ks, a.H, k_heads, sl.w[s], a.Dk, a.log_decay, a.v_scale, dqh, s > 0)) return rc;
+  }
+
+  // du (reversed) = LA(R k, R q, R do), contraction over the key columns
+  pack(pa, a.k, a.Hk, a.Hk, a.Dk, a.Dk, 0, true);
+  pack(pb, a.q, a.Hq, a.Hq, a.Dk, a.Dk, 0, true);
+  pack(pv, a.dout, a.H, a.H, a.Dv, a.Dv, 0, true);
+  if (const int rc = scan_launch(pa, a.Hk, pb, a.Hq, pv, a.Dk, a.Dv, grev, nullptr, du, false)) return rc;
+
+  // dk (per head, reversed, before its v_scale factor) = LA(R v, R do, R q), contraction over the value columns
+  pack(pv, a.q, a.H, a.Hq, a.Dk, a.Dk, 0, true);
+  for (int s = 0; s < sl.n; s++) {
+    pack(pa, a.v, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], true);
+    pack(pb, a.dout, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], true);
+    if (const int rc = scan_launch(pa, a.H, pb, a.H, pv, sl.w[s], a.Dk, grev, nullptr, dkh, s > 0)) return rc;
+  }
+
+  if ((a.Dk > a.Dv ? a.Dk : a.Dv) >= 256)
+    hipLaunchKernelGGL(grads_kernel<64>, dim3((unsigned)((BHT + 3) / 4)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh, (const float*)du, dG);
+  else
+    hipLaunchKernelGGL(grads_kernel<32>, dim3((unsigned)((BHT + 7) / 8)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh, (const float*)du, dG);
+  if (a.Hq != a.H) {
+    const int64_t n4 = (int64_t)a.B * a.Hq * a.T * (a.Dk / 4);
+    hipLaunchKernelGGL(group_sum_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (__bf16*)a.dq, (const float*)dqh, (const float*)nullptr,
+                       a.H, a.Hq, a.T, a.Dk, 0, n4);
+  }
+  if (a.Hk != a.H) {
+    const int64_t n4 = (int64_t)a.B * a.Hk * a.T * (a.Dk / 4);
+    hipLaunchKernelGGL(group_sum_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (__bf16*)a.dk, (const float*)dkh, a.v_scale, a.H, a.Hk,
+                       a.T, a.Dk, 1, n4);
+  }
+  hipLaunchKernelGGL(suffix_sum_kernel, dim3((unsigned)(a.B * a.H)), dim3(64), 0, stream, a.dlog_decay, (const float*)dG, a.T);
+  return launch_status();
+}
+
+}  // namespace ma

@@ -13,7 +13,7 @@ struct LinArgs {
   // sequence segments (see linear_fwd.hip): nseg segments of seg_chunks 32-token chunks; local end
   // states [group][segment][wave][registers][lane] fp32 and per-(batch*head, segment) log decays
   int nseg, seg_chunks;
-  int out_f32;   // o is fp32 [B,H,T,Dv] instead of bf16
+  int out_f32;   // 1: o is fp32 [B,H,T,Dv] instead of bf16; 2: fp32, and the result is added to what o holds
   float* ws_state;
   float* ws_decay;
 };

@@ -510,7 +510,12 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
           const int ci = ln + 64 * it, row = ci >> 2, cc = ci & 3;
           const u32x4 w = ALIAS_OST ? lds_read<u32x4>(vbase + row * RBV + (uint32_t)(((4 * wave + cc) ^ swz_tile<CPRV>(row)) << 4))
                                     : lds_read<u32x4>(lds_ost + row * OROW + cc * 16);
-          if (t0 + row < Tn) *(u32x4*)(ob32 + (int64_t)(t0 + row) * a.Dv + 16 * half + cc * 4) = w;
+          if (t0 + row < Tn) {
+            f32x4* dst = (f32x4*)(ob32 + (int64_t)(t0 + row) * a.Dv + 16 * half + cc * 4);
+            f32x4 val = __builtin_bit_cast(f32x4, w);
+            if (a.out_f32 == 2) val += *dst;   // (a contraction cut into pieces: the pieces' outputs add up)
+            *dst = val;
+          }
         }
       }
     } else if constexpr (MODE != 1) {

@@ -23,7 +23,7 @@ MA_MASK_NONE, MA_MASK_CAUSAL = 0, 1
 
 EXPORTED_SYMBOLS = (
     "ma_version", "ma_last_error", "ma_attn_workspace_bytes", "ma_attn_fwd", "ma_attn_bwd_workspace_bytes", "ma_attn_bwd",
-    "ma_linear_workspace_bytes", "ma_linear_fwd",
+    "ma_linear_workspace_bytes", "ma_linear_fwd", "ma_linear_bwd_workspace_bytes", "ma_linear_bwd",
     "ma_mla_choose_split", "ma_mla_workspace_bytes", "ma_mla_decode", "ma_mla_num_sm_parts", "ma_mla_get_metadata",
     "ma_mla_noalloc_max_workspace", "ma_mla_decode_noalloc",
 )
@@ -95,6 +95,20 @@ class LinearParams(Structure):
     ]
 
 
+class LinearBwdParams(Structure):
+    _fields_ = [
+        ("dtype", c_int32),
+        ("batch", c_int32), ("heads", c_int32), ("heads_q", c_int32), ("heads_k", c_int32),
+        ("seqlen", c_int32), ("dim_k", c_int32), ("dim_v", c_int32),
+        ("q", c_void_p), ("k", c_void_p), ("v", c_void_p), ("dout", c_void_p),
+        ("log_decay", c_void_p), ("v_scale", c_void_p),
+        ("q_scale", c_float),
+        ("dq", c_void_p), ("dk", c_void_p), ("dv", c_void_p),
+        ("dlog_decay", c_void_p), ("dv_scale", c_void_p),
+        ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+    ]
+
+
 class MlaParams(Structure):
     _fields_ = [
         ("dtype", c_int32),
@@ -140,6 +154,10 @@ def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
     lib.ma_linear_workspace_bytes.restype = c_size_t
     lib.ma_linear_fwd.argtypes = [POINTER(LinearParams), c_void_p]
     lib.ma_linear_fwd.restype = c_int
+    lib.ma_linear_bwd_workspace_bytes.argtypes = [POINTER(LinearBwdParams)]
+    lib.ma_linear_bwd_workspace_bytes.restype = c_size_t
+    lib.ma_linear_bwd.argtypes = [POINTER(LinearBwdParams), c_void_p]
+    lib.ma_linear_bwd.restype = c_int
     lib.ma_mla_choose_split.argtypes = [POINTER(MlaParams)]
     lib.ma_mla_choose_split.restype = c_int
     lib.ma_mla_workspace_bytes.argtypes = [POINTER(MlaParams)]
@@ -499,63 +517,42 @@ def linear_fwd(q, k, v, log_decay, *, q_scale: float = 1.0, v_scale=None, chunk=
     return out
 
 
-def _linear_any_width(q, k, v, log_decay, q_scale, v_scale=None):
-    """linear_fwd with fp32 outputs for any key width: the kernels contract over 128 or 256 key columns;
-    narrower keys are zero-padded, wider ones are cut into slices of 256 whose results add (the operator
-    is linear in q.k)."""
-    D = q.shape[-1]
-    if D in (128, 256):
-        return linear_fwd(q, k, v, log_decay, q_scale=q_scale, v_scale=v_scale, out_fp32=True)
-    if D < 256:
-        W = 128 if D < 128 else 256
-        pad = lambda t: torch.nn.functional.pad(t, (0, W - D))
-        return linear_fwd(pad(q), pad(k), v, log_decay, q_scale=q_scale, v_scale=v_scale, out_fp32=True)
-    acc = None
-    for c0 in range(0, D, 256):
-        part = _linear_any_width(q[..., c0:c0 + 256].contiguous(), k[..., c0:c0 + 256].contiguous(), v, log_decay, q_scale, v_scale)
-        acc = part if acc is None else acc + part
-    return acc
-
-
-def linear_bwd(q, k, v, log_decay, dout, *, q_scale: float = 1.0, v_scale=None):
-    """Gradients of linear_fwd with respect to q, k, v, log_decay and v_scale (None when no v_scale).
-
-    With A_ts = q_scale (q_t.k_s) exp(G_t - G_s) [s <= t] and u = v * v_scale, o = A u and
-        dq_t = q_scale sum_{s<=t} exp(G_t-G_s) (do_t.u_s) k_s
-        du_s = sum_{t>=s} A_ts do_t,      dk_s = q_scale sum_{t>=s} exp(G_t-G_s) (do_t.u_s) q_t
-    are the SAME operator on permuted (and, for the two sums over later tokens, time-reversed) inputs:
-        dq = LA(do, v, k; v_scale),   du = flip LA(flip k, flip q, flip do),   dk = v_scale * flip LA(flip v, flip do, flip q)
-    with the reversed log decay shifted by one token.  So the backward pass is three launches of the
-    parity-tested forward kernel plus element-wise glue; heads that share a q / k head have their
-    gradients summed, as LinearAttention.backward does (linear_tl.py:1300-1303).  The decay gradient
-    follows from dG_t = q_t.dq_t - k_t.dk_t and G = cumsum(log_decay) (a reversed cumulative sum,
-    compute_final_dg of the reference)."""
-    _require_gpu(q, k, v, log_decay, dout, v_scale)
+def linear_bwd(q, k, v, log_decay, dout, *, q_scale: float = 1.0, v_scale=None, workspace=None):
+    """Gradients of linear_fwd with respect to q, k, v, log_decay and v_scale (None when no v_scale):
+    (dq, dk, dv, dlog_decay, dv_scale) with dq, dk, dv in the tensors' dtype (the gradients of heads that share a
+    q / k head summed, as LinearAttention.backward does, linear_tl.py:1300-1303) and the two per-token gradients in
+    fp32 [B,H,T].  One call of ma_linear_bwd; the workspace it needs is allocated here unless one is passed."""
+    _require_gpu(q, k, v, log_decay, dout, v_scale, workspace)
     B, H, T, Dv = v.shape
     Hq, Hk, Dk = q.shape[1], k.shape[1], q.shape[-1]
-    g = log_decay.to(torch.float32).contiguous()
-    vs = v_scale.to(torch.float32).contiguous() if v_scale is not None else None
+    assert q.shape == (B, Hq, T, Dk) and k.shape == (B, Hk, T, Dk) and dout.shape == v.shape, "q/k/v/dout shapes disagree"
+    assert log_decay.shape == (B, H, T), "log_decay must be [B,H,T]"
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     dout = dout.to(v.dtype).contiguous()
-    flip = lambda t: torch.flip(t, dims=(2,)).contiguous()
-    expand = lambda t, h: t if t.shape[1] == H else t.repeat_interleave(H // h, dim=1)
-    qe, ke = expand(q, Hq), expand(k, Hk)
-    g_rev = torch.zeros_like(g)
-    if T > 1:
-        g_rev[:, :, 1:] = torch.flip(g, dims=(2,))[:, :, :-1]          # g_rev[t'] = g[T - t'], t' >= 1
-    dq_h = _linear_any_width(dout, v, ke, g, q_scale, vs)                                     # [B,H,T,Dk]
-    du = flip(_linear_any_width(flip(k), flip(q), flip(dout), g_rev, q_scale))                # [B,H,T,Dv]
-    dk_h = flip(_linear_any_width(flip(v), flip(dout), flip(qe), g_rev, q_scale))             # [B,H,T,Dk], before the v_scale factor
-    # (dq_h, du, dk_h are fp32 from here on)
-    if vs is not None:
-        dk_h = dk_h * vs.unsqueeze(-1)
-        dv = (du * vs.unsqueeze(-1)).to(v.dtype)
-        dvs = (v.float() * du).sum(-1)
-    else:
-        dv, dvs = du.to(v.dtype), None
-    dG = (qe.float() * dq_h).sum(-1) - (ke.float() * dk_h).sum(-1)                            # [B,H,T]
-    dld = torch.flip(torch.cumsum(torch.flip(dG, dims=(2,)), dim=2), dims=(2,))
-    dq = (dq_h if Hq == H else dq_h.view(B, Hq, H // Hq, T, Dk).sum(2)).to(q.dtype)
-    dk = (dk_h if Hk == H else dk_h.view(B, Hk, H // Hk, T, Dk).sum(2)).to(k.dtype)
+    g = log_decay.to(torch.float32).contiguous()
+    vs = None
+    if v_scale is not None:
+        assert v_scale.shape == (B, H, T)
+        vs = v_scale.to(torch.float32).contiguous()
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dld = torch.empty(B, H, T, dtype=torch.float32, device=v.device)
+    dvs = torch.empty(B, H, T, dtype=torch.float32, device=v.device) if vs is not None else None
+    p = LinearBwdParams()
+    p.dtype = _dtype_code(v.dtype)
+    p.batch, p.heads, p.heads_q, p.heads_k, p.seqlen, p.dim_k, p.dim_v = B, H, Hq, Hk, T, Dk, Dv
+    p.q, p.k, p.v, p.dout = q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr()
+    p.log_decay = g.data_ptr()
+    p.v_scale = vs.data_ptr() if vs is not None else None
+    p.q_scale = float(q_scale)
+    p.dq, p.dk, p.dv, p.dlog_decay = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dld.data_ptr()
+    p.dv_scale = dvs.data_ptr() if dvs is not None else None
+    lib = load_library()
+    need = lib.ma_linear_bwd_workspace_bytes(ctypes.byref(p))
+    if need > 0:
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=v.device)
+        p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()   # (a small one is refused by the library)
+    _check(lib.ma_linear_bwd(ctypes.byref(p), _stream()))
     return dq, dk, dv, dld, dvs
 
 

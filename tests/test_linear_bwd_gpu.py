@@ -4,7 +4,7 @@ q, k, v gradients at atol 2e-2 / rtol 1e-2 with a small allowance for the bf16 r
 intermediate gradients (the reference's own checks: rtol = atol = 1e-1, testing/test.py:364-385,
 488-505, which is also asserted); the decay and value-scale gradients, which the reference's tests
 leave unchecked (:386-397, :506-511), are sums of bf16-rounded products over the head dimension and
-are held to 5 % of their largest magnitude (at least 1e-2)."""
+are held to 3 % of their largest magnitude (at least 1e-2; the runs show at most 2.1 %)."""
 import math
 
 import pytest
@@ -35,7 +35,7 @@ def _check(got, ref, what):
             oracle.assert_close(a, b, rtol=1e-1, atol=1e-1, mismatch_ratio=1e-2, msg=f"{what}:{name} (reference acceptance)")
             oracle.assert_close(a, b, rtol=RTOL, atol=ATOL, mismatch_ratio=5e-3, msg=f"{what}:{name}")
         else:
-            tol = max(0.05 * float(b.abs().max()), 1e-2)
+            tol = max(0.03 * float(b.abs().max()), 1e-2)
             assert float((a - b).abs().max()) <= tol, f"{what}:{name}: {float((a - b).abs().max())} > {tol}"
 
 
@@ -82,7 +82,7 @@ def test_engine_mamba2_backward():
                                           compute_dtype=torch.float64)
     out.backward(dout.double())
     _check((Cc.grad, Bc.grad, xc.grad), (q64.grad, k64.grad, v64.grad), "mamba2")
-    tol = max(0.05 * float(dt64.grad.abs().max()), 1e-2)
+    tol = max(0.03 * float(dt64.grad.abs().max()), 1e-2)
     err = float((dtc.grad.double().cpu() - dt64.grad).abs().max())
     assert err <= tol, f"ddt: {err} > {tol}"
     # dA_h = sum_t dlog_decay_t dt_t = sum_j dG_j C_j with C_j = sum_{t<=j} dt_t (up to ~40 here): a residual of T large terms
@@ -111,3 +111,44 @@ def test_engine_retnet_backward():
     torch.cuda.synchronize()
     ref = oracle.linear_attention_grads(q, k, v, torch.log(decay), dout, q_scale=Dk ** -0.5)
     _check((qc.grad, kc.grad, vc.grad), ref[:3], "retnet")
+
+
+def test_linear_backward_full_size_properties():
+    """The RetNet benchmark shape (B8 H16 T2048 Dk256 Dv512) through ma_linear_bwd.  Size-independent properties: the
+    first token's log decay does not reach the output (G_0 cancels in every G_t - G_s), so its gradient, the sum of all
+    per-token decay gradients, vanishes against their magnitude; the gradients are linear in dout.  And one (batch,
+    head) against the gradient oracle."""
+    hb = _hb()
+    B, H, T, Dk, Dv = 8, 16, 2048, 256, 512
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 16).bfloat16()
+    k = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 16).bfloat16()
+    v = torch.randn(B, H, T, Dv, device="cuda", generator=g).bfloat16()
+    ld = torch.log(1 - torch.exp2(-5 - torch.arange(H, device="cuda").float())).view(1, H, 1).expand(B, H, T).contiguous()
+    dout = (0.5 * torch.randn(B, H, T, Dv, device="cuda", generator=g)).bfloat16()
+    print("linear bwd full size B8 H16 T2048 Dk256 Dv512", flush=True)
+    dq, dk, dv, dld, dvs = hb.linear_bwd(q, k, v, ld, dout, q_scale=Dk ** -0.5)
+    dq2, dk2, dv2, dld2, _ = hb.linear_bwd(q, k, v, ld, (dout.float() * 2).bfloat16(), q_scale=Dk ** -0.5)
+    torch.cuda.synchronize()
+    assert dvs is None
+    for a, b in ((dq, dq2), (dk, dk2), (dv, dv2)):
+        assert torch.isfinite(a.float()).all()
+        torch.testing.assert_close(b.float(), 2 * a.float(), rtol=1e-2, atol=1e-3)   # (bf16 rounding of the doubled result)
+    torch.testing.assert_close(dld2, 2 * dld, rtol=1e-3, atol=1e-3 * float(dld.abs().max()))
+    step = (dld[:, :, :-1] - dld[:, :, 1:]).abs().sum(dim=2)    # sum_t |dG_t|
+    assert float((dld[:, :, 0].abs() / step).max()) < 1e-2
+    b, h = 5, 9
+    ref = oracle.linear_attention_grads(q[b:b + 1, h:h + 1].cpu(), k[b:b + 1, h:h + 1].cpu(), v[b:b + 1, h:h + 1].cpu(), ld[b:b + 1, h:h + 1].cpu(),
+                                        dout[b:b + 1, h:h + 1].cpu(), q_scale=Dk ** -0.5)
+    _check((dq[b:b + 1, h:h + 1], dk[b:b + 1, h:h + 1], dv[b:b + 1, h:h + 1], dld[b:b + 1, h:h + 1], None), ref, "full size")
+
+
+def test_linear_backward_refuses_a_small_workspace():
+    hb = _hb()
+    B, H, T, Dk, Dv = 1, 2, 64, 128, 64
+    q = torch.randn(B, H, T, Dk, device="cuda").bfloat16()
+    v = torch.randn(B, H, T, Dv, device="cuda").bfloat16()
+    ld = -torch.rand(B, H, T, device="cuda")
+    with pytest.raises(hb.MetaAttentionError) as err:
+        hb.linear_bwd(q, q, v, ld, v, workspace=torch.empty(4096, dtype=torch.uint8, device="cuda"))
+    assert err.value.code == -3
