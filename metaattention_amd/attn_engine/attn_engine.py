@@ -271,8 +271,9 @@ class AttentionEngine:
                 return _ForwardOnly.apply(run, q, k, v)
             score_mask = None
             if self.family == "retention":
-                # the backward kernels of the retention operator exist for its own head size (examples/retention_parallel.py)
-                if (q.shape[-1], v.shape[-1]) != (256, 512) or not form.mask_tensor:
+                # head sizes the backward kernels of the retention operator are built for (256 / 512 is its own,
+                # examples/retention_parallel.py)
+                if (q.shape[-1], v.shape[-1]) not in ((256, 512), (128, 128), (64, 64), (128, 256), (256, 256)) or not form.mask_tensor:
                     return _ForwardOnly.apply(run, q, k, v)
                 score_mask = given[form.mask_tensor]
                 score_mask = score_mask if score_mask.dtype == q.dtype else score_mask.to(q.dtype)

@@ -640,13 +640,21 @@ static int bwd_family(const AttnBwdArgs& a, int family, bool causal, hipStream_t
 
 template <typename T>
 static int bwd_dims(const AttnBwdArgs& a, int family, bool causal, int dqk, int dv, hipStream_t stream) {
-  if (family == BF_RETENTION) {   // the head size of the retention operator (examples/retention_parallel.py: 256 / 512)
-    if (dqk != 256 || dv != 512) return -2;
-    return causal ? launch_bwd<T, 256, 512, BF_RETENTION, true>(a, stream) : launch_bwd<T, 256, 512, BF_RETENTION, false>(a, stream);
+  if (family == BF_RETENTION) {   // 256 / 512 is the head size of the retention operator itself (examples/retention_parallel.py)
+#define MA_RET_BWD(DQ, DVV) \
+  if (dqk == DQ && dv == DVV) return causal ? launch_bwd<T, DQ, DVV, BF_RETENTION, true>(a, stream) : launch_bwd<T, DQ, DVV, BF_RETENTION, false>(a, stream);
+    MA_RET_BWD(256, 512)
+    MA_RET_BWD(128, 128)
+    MA_RET_BWD(64, 64)
+    MA_RET_BWD(128, 256)
+    MA_RET_BWD(256, 256)
+#undef MA_RET_BWD
+    return -2;
   }
   if (dqk == 128 && dv == 128) return bwd_family<T, 128, 128>(a, family, causal, stream);
   if (dqk == 64 && dv == 64) return bwd_family<T, 64, 64>(a, family, causal, stream);
   if (dqk == 128 && dv == 256) return bwd_family<T, 128, 256>(a, family, causal, stream);
+  if (dqk == 256 && dv == 256) return bwd_family<T, 256, 256>(a, family, causal, stream);
   return -2;
 }
 

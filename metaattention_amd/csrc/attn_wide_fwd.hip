@@ -469,8 +469,13 @@ template <typename T>
 static int wide_dims(const AttnArgs& a, int family, bool causal, int dqk, int dv, hipStream_t stream) {
   if (family == WF_RETENTION) {
     if (dqk == 256 && dv == 512) return retention_pair_fwd_dispatch(a, causal, std::is_same<T, __bf16>::value, stream);   // retention_fwd.hip
-    if (dqk == 128 && dv == 128)
-      return causal ? launch_wide<T, 128, 128, WF_RETENTION, true>(a, stream) : launch_wide<T, 128, 128, WF_RETENTION, false>(a, stream);
+#define MA_RET_FWD(DQ, DVV) \
+  if (dqk == DQ && dv == DVV) return causal ? launch_wide<T, DQ, DVV, WF_RETENTION, true>(a, stream) : launch_wide<T, DQ, DVV, WF_RETENTION, false>(a, stream);
+    MA_RET_FWD(128, 128)
+    MA_RET_FWD(64, 64)
+    MA_RET_FWD(128, 256)
+    MA_RET_FWD(256, 256)
+#undef MA_RET_FWD
     return -2;
   }
   if (dqk == 128 && dv == 128) return wide_family<T, 128, 128>(a, family, causal, stream);   // (only with kv selection: see attn_fwd_dispatch)

@@ -46,7 +46,7 @@ def _run(hb, family, q, k, v, dout, causal, scale, bias=0.0):
     return got, ref
 
 
-@pytest.mark.parametrize("D,DV", [(128, 128), (64, 64), (128, 256)])
+@pytest.mark.parametrize("D,DV", [(128, 128), (64, 64), (128, 256), (256, 256)])
 @pytest.mark.parametrize("B,H,Hkv,S,causal", [(1, 2, 2, 256, True), (2, 3, 3, 200, True), (1, 2, 2, 333, False), (1, 4, 2, 129, True), (1, 1, 1, 1, True)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_softmax_backward(D, DV, B, H, Hkv, S, causal, dtype):
@@ -130,16 +130,32 @@ def test_engine_sigmoid_backward_with_bias_tensor():
     _check((qc.grad, kc.grad, vc.grad), ref, "engine sigmoid")
 
 
-def test_retention_backward_at_other_head_sizes_still_raises():
-    """The retention backward kernels exist for the operator's own head size (256 / 512); elsewhere backward raises."""
-    B, H, S = 1, 2, 128
+def test_engine_retention_backward_at_another_head_size():
+    """The retention operator at 128 / 128 (not its own 256 / 512): o.backward(do) through the operator built from the spec."""
+    B, H, S = 1, 2, 136
     mod = specs.retention_parallel(B, H, S, 128, 128)
     q, k, v, _ = inputs.retnet_inputs(B, H, S, 128, 128, seed=1, layout="bshd")
+    q = (q.float() * 4.0).bfloat16()
+    mask = oracle.retention_decay_mask(H, S).bfloat16()
+    dout = (0.5 * torch.randn(B, S, H, 128, generator=torch.Generator().manual_seed(2))).bfloat16()
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = mod(qc, kc, vc, mask.cuda())
+    o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    ref = oracle.attention_grads(oracle.retention_parallel, q, k, v, dout, mask=mask, freeze_r=True)
+    _check((qc.grad, kc.grad, vc.grad), ref, "engine retention 128/128")
+
+
+def test_retention_backward_at_an_unbuilt_head_size_raises():
+    """Head sizes without backward kernels (here 256 / 128): the forward runs, backward raises."""
+    hb = _hb()
+    B, H, S = 1, 2, 128
+    q = torch.randn(B, S, H, 256, device="cuda").bfloat16()
+    v = torch.randn(B, S, H, 128, device="cuda").bfloat16()
     mask = oracle.retention_decay_mask(H, S).bfloat16().cuda()
-    qc = q.cuda().requires_grad_(True)
-    o = mod(qc, k.cuda(), v.cuda(), mask)
-    with pytest.raises(NotImplementedError):
-        o.sum().backward()
+    with pytest.raises(hb.MetaAttentionError):
+        hb.attn_bwd(q, q, v, v, v, torch.ones(B, H, S, device="cuda"), family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mask,
+                    score_mask_t=mask.transpose(2, 3).contiguous())
 
 
 MASKS = {

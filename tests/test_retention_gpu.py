@@ -97,15 +97,16 @@ def _check_grads(got, ref, what):
         oracle.assert_close(a.float().cpu(), b.float(), rtol=RTOL, atol=ATOL, mismatch_ratio=1e-3, msg=f"{what}:{name}")
 
 
-@pytest.mark.parametrize("B,H,S,causal,dtype", [(1, 2, 128, True, torch.bfloat16), (2, 3, 200, True, torch.bfloat16),
-                                                (1, 2, 132, False, torch.bfloat16), (1, 1, 4, True, torch.bfloat16),
-                                                (1, 2, 260, True, torch.float16)])
-def test_retention_backward(B, H, S, causal, dtype):
+@pytest.mark.parametrize("B,H,S,causal,dtype,D,DV", [(1, 2, 128, True, torch.bfloat16, 256, 512), (2, 3, 200, True, torch.bfloat16, 256, 512),
+                                                     (1, 2, 132, False, torch.bfloat16, 256, 512), (1, 1, 4, True, torch.bfloat16, 256, 512),
+                                                     (1, 2, 260, True, torch.float16, 256, 512),
+                                                     (1, 2, 200, True, torch.bfloat16, 128, 128), (2, 2, 136, True, torch.bfloat16, 64, 64),
+                                                     (1, 2, 160, False, torch.bfloat16, 128, 256), (1, 2, 144, True, torch.bfloat16, 256, 256)])
+def test_retention_backward(B, H, S, causal, dtype, D, DV):
     """dq, dk, dv of the retention operator through the C ABI: the row scale r of the forward pass is a constant of the
     backward (examples/retention_parallel.py:82-86).  Oracle: autograd over oracle.retention_parallel(freeze_r=True)
     in fp64."""
     hb = _hb()
-    D, DV = 256, 512
     q, k, v, mask = _inputs(B, H, S, D, DV, seed=S)
     q, k, v, mask = (t.to(dtype) for t in (q, k, v, mask))
     dout = (0.5 * torch.randn(B, S, H, DV, generator=torch.Generator().manual_seed(S))).to(dtype)
@@ -113,7 +114,7 @@ def test_retention_backward(B, H, S, causal, dtype):
         mask = (mask.float() + mask.float().transpose(2, 3)).to(dtype)     # a full multiplier: decay on both sides of the diagonal
     qc, kc, vc, mc = q.cuda(), k.cuda(), v.cuda(), mask.cuda()
     rs = torch.empty(B, H, S, device="cuda")
-    print(f"retention bwd B{B} H{H} S{S} causal={causal} {dtype}", flush=True)
+    print(f"retention bwd B{B} H{H} S{S} D{D} DV{DV} causal={causal} {dtype}", flush=True)
     o = hb.attn_fwd(qc, kc, vc, family=hb.MA_ATTN_RETENTION, causal=causal, scale=1.0, score_mask=mc, row_scale=rs)
     got = hb.attn_bwd(qc, kc, vc, o, dout.cuda(), rs, family=hb.MA_ATTN_RETENTION, causal=causal, scale=1.0,
                       score_mask=mc, score_mask_t=mc.transpose(2, 3).contiguous())
