@@ -152,3 +152,25 @@ def test_linear_backward_refuses_a_small_workspace():
     with pytest.raises(hb.MetaAttentionError) as err:
         hb.linear_bwd(q, q, v, ld, v, workspace=torch.empty(4096, dtype=torch.uint8, device="cuda"))
     assert err.value.code == -3
+
+
+@pytest.mark.parametrize("T,Dk,Dv,rtol,atol,ratio", [(32, 128, 64, RTOL, ATOL, 0.0), (64, 128, 64, RTOL, ATOL, 0.0), (64, 256, 256, RTOL, ATOL, 1e-2),
+                                                     (128, 128, 128, 2e-2, 5e-2, 0.0)])
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_decay_gradient_per_element_on_short_sequences(T, Dk, Dv, rtol, atol, ratio, seed):
+    """dlog_decay element by element where the running sum is short: inside 2e-2 / 1e-2 up to 64 tokens (at most 1 % of the
+    elements outside at the wide head size), inside 5e-2 / 2e-2 at 128.  Its error grows with the length of the sum, which
+    is why the long-sequence tests bound it against its largest magnitude instead."""
+    hb = _hb()
+    g = torch.Generator().manual_seed(seed)
+    B, H = 1, 2
+    q = torch.randn(B, H, T, Dk, generator=g).bfloat16()
+    k = (0.1 * torch.randn(B, H, T, Dk, generator=g)).bfloat16()
+    v = torch.randn(B, H, T, Dv, generator=g).bfloat16()
+    ld = torch.nn.functional.logsigmoid(torch.randn(B, H, T, generator=g) + 3.0)
+    dout = (0.5 * torch.randn(B, H, T, Dv, generator=g)).bfloat16()
+    print(f"decay gradient T{T} Dk{Dk} Dv{Dv} seed {seed}", flush=True)
+    got = hb.linear_bwd(q.cuda(), k.cuda(), v.cuda(), ld.cuda(), dout.cuda(), q_scale=Dk ** -0.5)
+    torch.cuda.synchronize()
+    ref = oracle.linear_attention_grads(q, k, v, ld, dout, q_scale=Dk ** -0.5)
+    oracle.assert_close(got[3].float().cpu(), ref[3].float(), rtol=rtol, atol=atol, mismatch_ratio=ratio, msg="dlog_decay")
