@@ -383,7 +383,8 @@ def run_probes():
     `attention_step`: 8 waves per CU run the per-step work of the 128/128 forward kernel (16 MFMAs of 32x32x16 per wave and
     32-key sub-tile) in a loop, with more and more of what surrounds the MFMAs in the real kernel switched on, once with
     constant and once with pseudo-random operands.  `tflops` is what the same step rate would mean for the whole chip.
-    `stream_to_lds`: direct-to-LDS streaming rate of the whole chip from windows that fit L2 / the last-level cache / HBM."""
+    `stream_to_lds`: direct-to-LDS streaming rate of the whole chip from windows that fit L2 / the last-level cache / HBM.
+    `issue_hold`: cycles a direct-to-LDS instruction holds its wave at issue, by how many waves of the CU issue at once."""
     import ctypes
     lib_path = os.path.join(ROOT, "metaattention_amd", "lib", "libmetaattention_probe.so")
     if not os.path.exists(lib_path):
@@ -415,7 +416,20 @@ def run_probes():
                 raise RuntimeError(f"ma_probe_stream_to_lds({region_mb} MB, {depth}) returned {rc}")
             streams.append({"region_mb": region_mb, "region": what, "kb_in_flight_per_cu": 8 * depth, "gb_per_s": round(gbs.value, 1),
                             "frac_of_hbm_peak": round(gbs.value / PEAK_HBM_GBS, 4)})
-    return {"probe": "ceilings", "attention_step": steps, "stream_to_lds": streams}
+    lib.ma_probe_issue_hold.argtypes = [ctypes.c_int, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+    holds = []
+    kinds = {0: "global_load_lds_dwordx4 (1 KB)", 1: "global_load_lds_dword (256 B)", 2: "global_load_dwordx4 to registers (1 KB)"}
+    for kind, kname in kinds.items():
+        for region_mb, what in ((16, "L2"), (2048, "HBM")):
+            for nwaves, per_round in ((1, 1), (1, 8), (8, 1), (8, 2), (8, 4), (8, 8)):
+                ci, ct = ctypes.c_double(), ctypes.c_double()
+                rc = lib.ma_probe_issue_hold(kind, region_mb << 20, nwaves, per_round, ctypes.byref(ci), ctypes.byref(ct))
+                if rc != 0:
+                    raise RuntimeError(f"ma_probe_issue_hold({kind}, {region_mb} MB, {nwaves}, {per_round}) returned {rc}")
+                holds.append({"instruction": kname, "from": what, "waves_issuing_per_cu": nwaves, "instructions_per_burst": per_round,
+                              "kb_per_burst_and_cu": nwaves * per_round * (0.25 if kind == 1 else 1.0),
+                              "issue_cycles_per_instruction": round(ci.value, 1), "cycles_per_instruction_with_wait": round(ct.value, 1)})
+    return {"probe": "ceilings", "attention_step": steps, "stream_to_lds": streams, "issue_hold": holds}
 
 
 def main():

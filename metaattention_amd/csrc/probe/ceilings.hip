@@ -11,6 +11,9 @@
 // instruction stream is the same, the switching activity is not, and the chip's power management answers the latter
 // with a lower clock.  The cycle counter of one wave and the wall time of the launch are both returned.
 //
+// probe 3 (ma_probe_issue_hold): how many cycles a direct-to-LDS load instruction holds the wave that issues it, by the number
+// of waves of the CU issuing at the same time, the number of instructions per burst and where the data comes from.
+//
 // probe 2 (ma_probe_stream_to_lds): 8 waves per CU stream a window of global memory into LDS with direct-to-LDS loads,
 // `depth` instructions (1 KB each) in flight per wave; the window is chosen to fit L2, the last-level cache, or neither.
 #include "../common.h"
@@ -149,6 +152,56 @@ __global__ __launch_bounds__(512) void stream_kernel(const char* src, size_t reg
   if (v[0] == 0x12345678u) sink[0] = v[1];
 }
 
+// probe 3: how long does a direct-to-LDS load instruction hold the wave that issues it?  `nwaves` of the 8 waves of every
+// workgroup (one workgroup per CU) issue `per_round` instructions (1 KB each) back to back, then wait for them, `rounds`
+// times, walking a window of global memory; the cycle counter brackets the issue alone.  clk[0] = cycles wave 0 of
+// workgroup 0 spent issuing, clk[1] = its cycles in all (issue + wait).
+// KIND 0: global_load_lds_dwordx4 (1 KB per instruction), 1: global_load_lds_dword (256 B), 2: global_load_dwordx4 into
+// registers (1 KB; the registers are stored to LDS with ds_write_b128 after the wait, outside the bracket).  A burst is NB
+// instructions, fully unrolled, each at the address of the one before plus 8 KB (one 64-bit add between them); the window
+// wrap is handled between the rounds, outside the bracket.
+template <int KIND, int NB>
+__global__ __launch_bounds__(512) void issue_hold_kernel(const char* src, size_t region_bytes, int nwaves, int rounds, long long* clk) {
+  extern __shared__ __align__(16) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (wave >= nwaves) return;
+  const size_t window = region_bytes / gridDim.x / 8192 * 8192;
+  const char* base = src + (size_t)blockIdx.x * window + (size_t)wave * 1024 + lane * (KIND == 1 ? 4 : 16);
+  size_t off = 0;
+  long long t_issue = 0;
+  u32x4 regs[NB];
+#pragma unroll
+  for (int i = 0; i < NB; i++) regs[i] = u32x4{0u, 0u, 0u, 0u};
+  const long long t0 = __builtin_readcyclecounter();
+  for (int r = 0; r < rounds; r++) {
+    const char* p = base + off;
+    uint32_t m0v = lds0 + (uint32_t)(wave * 1024);
+    asm volatile("" : "+v"(p));
+    const long long a0 = __builtin_readcyclecounter();
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+      if constexpr (KIND == 2) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(regs[i]) : "v"(p) : "memory");
+      else if constexpr (KIND == 0) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0v), "v"(p) : "memory");
+      else asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(m0v), "v"(p) : "memory");
+      p += 8192;
+    }
+    t_issue += __builtin_readcyclecounter() - a0;
+    off += (size_t)NB * 8192;
+    if (off + (size_t)NB * 8192 > window) off = 0;
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    if constexpr (KIND == 2) {
+#pragma unroll
+      for (int i = 0; i < NB; i++) {
+        asm volatile("" : "+v"(regs[i]));
+        lds_write<u32x4>(lds0 + (uint32_t)(((i & 7) * 8 + wave) * 1024 + lane * 16), regs[i]);
+      }
+    }
+  }
+  const long long t1 = __builtin_readcyclecounter();
+  if (blockIdx.x == 0 && wave == 0 && lane == 0) { clk[0] = t_issue; clk[1] = t1 - t0; }
+}
+
 struct Buffers {
   float* out = nullptr;
   long long* clk = nullptr;
@@ -240,6 +293,32 @@ int ma_probe_stream_to_lds(size_t region_bytes, int depth, int iters, double* gb
     if (rc != 0) return rc;
   }
   *gb_per_s = 256.0 * iters * depth * 8192.0 / ((double)ms * 1e-3) / 1e9;
+  return 0;
+}
+
+// `nwaves` (1..8) waves per CU issue `per_round` (1, 2, 4 or 8) load instructions back to back per round, 200 rounds, from a region
+// of `region_bytes`; kind 0: global_load_lds_dwordx4 (1 KB), 1: global_load_lds_dword (256 B), 2: global_load_dwordx4 into
+// registers (1 KB); the bracket of a burst of 1 also holds the two cycle-counter reads (subtract the 1-instruction figure
+// from 8 x the 8-instruction figure and divide by 7 for the cost of one more instruction); returns the cycles one instruction holds its wave at issue and the cycles per
+// instruction including the wait for the round's data (wave 0 of workgroup 0).
+int ma_probe_issue_hold(int kind, size_t region_bytes, int nwaves, int per_round, double* issue_cycles_per_instr, double* total_cycles_per_instr) {
+  if (kind < 0 || kind > 2 || nwaves < 1 || nwaves > 8 || (per_round != 1 && per_round != 2 && per_round != 4 && per_round != 8) || region_bytes < ((size_t)256 << 16) || ensure(region_bytes) != 0)
+    return -1;
+  float ms = 0.f;
+  const int rounds = 200;
+  auto go = [&](auto kern) { return timed(kern, dim3(256), dim3(512), (size_t)65536, &ms, (const char*)g_buf.gbuf, region_bytes, nwaves, rounds, g_buf.clk); };
+  for (int rep = 0; rep < 2; rep++) {
+    int rc;
+    if (per_round == 1) rc = kind == 0 ? go(issue_hold_kernel<0, 1>) : kind == 1 ? go(issue_hold_kernel<1, 1>) : go(issue_hold_kernel<2, 1>);
+    else if (per_round == 2) rc = kind == 0 ? go(issue_hold_kernel<0, 2>) : kind == 1 ? go(issue_hold_kernel<1, 2>) : go(issue_hold_kernel<2, 2>);
+    else if (per_round == 4) rc = kind == 0 ? go(issue_hold_kernel<0, 4>) : kind == 1 ? go(issue_hold_kernel<1, 4>) : go(issue_hold_kernel<2, 4>);
+    else rc = kind == 0 ? go(issue_hold_kernel<0, 8>) : kind == 1 ? go(issue_hold_kernel<1, 8>) : go(issue_hold_kernel<2, 8>);
+    if (rc != 0) return -1;
+  }
+  long long c[2] = {0, 0};
+  if (hipMemcpy(c, g_buf.clk, sizeof(c), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+  *issue_cycles_per_instr = (double)c[0] / ((double)rounds * per_round);
+  *total_cycles_per_instr = (double)c[1] / ((double)rounds * per_round);
   return 0;
 }
 
