@@ -393,7 +393,8 @@ def run_probes():
     lib.ma_probe_attention_step.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     lib.ma_probe_stream_to_lds.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
     names = {0: "mfma only", 1: "+ vector work", 2: "+ LDS fragment reads", 3: "+ vector work + LDS reads",
-             7: "+ vector + LDS + barrier per step", 15: "+ vector + LDS + barrier + direct-to-LDS loads"}
+             7: "+ vector + LDS + barrier per step", 15: "+ vector + LDS + barrier + direct-to-LDS loads",
+             31: "the same with the two loads behind the 3rd and 6th MFMA pair instead of at the start of the step"}
     flop_per_step = 256 * 8 * 16 * 2 * 32 * 32 * 16        # CUs x waves x MFMAs x flop of one 32x32x16
     steps = []
     for mode, name in names.items():

@@ -22,7 +22,7 @@ using namespace ma;
 
 namespace {
 
-enum { PROBE_VECTOR = 1, PROBE_LDS = 2, PROBE_BARRIER = 4, PROBE_DMA = 8 };
+enum { PROBE_VECTOR = 1, PROBE_LDS = 2, PROBE_BARRIER = 4, PROBE_DMA = 8, PROBE_DMA_MID = 16 };
 
 template <int MODE, bool RANDOM>
 __global__ __launch_bounds__(512, 2) void attention_step_kernel(float* out, int iters, float cs, float sub, long long* clk, const char* gbuf) {
@@ -74,11 +74,14 @@ __global__ __launch_bounds__(512, 2) void attention_step_kernel(float* out, int 
     float part = 0.f;
     if (MODE & PROBE_DMA) __builtin_amdgcn_s_waitcnt(0x0F70 | 6);
     if (MODE & PROBE_BARRIER) __syncthreads();
-    if (MODE & PROBE_DMA) {   // the next sub-tile: 16 KB per workgroup, into a ring of 4 slots behind the two tiles that are read
-      dma16_so(gwin + goff, (uint32_t)(wave * 1024 + lane * 16), lds0 + 16384 + ring * 16384 + wave * 1024);
-      dma16_so(gwin + goff + 8192, (uint32_t)(wave * 1024 + lane * 16), lds0 + 16384 + ring * 16384 + 8192 + wave * 1024);
-      goff = (goff + 16384) & (1048576 - 1);
-      ring = ring == 3 ? 0 : ring + 1;
+    // the next sub-tile: 16 KB per workgroup, into a ring of 4 slots behind the two tiles that are read; both instructions of
+    // a wave at the start of the step, or (PROBE_DMA_MID) one behind the third and one behind the sixth MFMA pair
+    auto load_part = [&](int part) __attribute__((always_inline)) {
+      dma16_so(gwin + goff + part * 8192, (uint32_t)(wave * 1024 + lane * 16), lds0 + 16384 + ring * 16384 + part * 8192 + wave * 1024);
+    };
+    if ((MODE & PROBE_DMA) && !(MODE & PROBE_DMA_MID)) {
+      load_part(0);
+      load_part(1);
     }
     uint32_t ka = k_addr, va = v_addr;
     asm volatile("" : "+v"(ka), "+v"(va));   // (the addresses are the same every step; keep the reads inside the loop)
@@ -107,7 +110,12 @@ __global__ __launch_bounds__(512, 2) void attention_step_kernel(float* out, int 
         asm volatile("" : "+v"(w));
         p[PAR][i >> 2][i & 3] = w;
       }
+      if ((MODE & PROBE_DMA) && (MODE & PROBE_DMA_MID) && (i == 2 || i == 5)) load_part(i == 5);
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if (MODE & PROBE_DMA) {
+      goff = (goff + 16384) & (1048576 - 1);
+      ring = ring == 3 ? 0 : ring + 1;
     }
     row_sum += part;
   };
@@ -250,8 +258,8 @@ int run_step(int random_operands, int iters, float* ms) {
 
 extern "C" {
 
-// mode: bit mask of 1 (vector work), 2 (LDS fragment reads), 4 (barrier per step), 8 (direct-to-LDS loads); only the masks
-// 0, 1, 2, 3, 7 and 15 are built.  Runs `iters` steps per wave on 256 workgroups twice (the first run is a warm-up) and
+// mode: bit mask of 1 (vector work), 2 (LDS fragment reads), 4 (barrier per step), 8 (direct-to-LDS loads), 16 (those loads
+// between the MFMAs of the step instead of at its start); only the masks 0, 1, 2, 3, 7, 15 and 31 are built.  Runs `iters` steps per wave on 256 workgroups twice (the first run is a warm-up) and
 // returns the wall time per step in nanoseconds and the cycle count per step seen by wave 0 of workgroup 0.  Returns 0
 // on success, -1 on a HIP failure, -2 for a mask that is not built.
 int ma_probe_attention_step(int mode, int random_operands, int iters, double* ns_per_step, double* cycles_per_step) {
@@ -268,6 +276,7 @@ int ma_probe_attention_step(int mode, int random_operands, int iters, double* ns
       case 3: rc = run_step<3>(random_operands, n, &ms); break;
       case 7: rc = run_step<7>(random_operands, n, &ms); break;
       case 15: rc = run_step<15>(random_operands, n, &ms); break;
+      case 31: rc = run_step<31>(random_operands, n, &ms); break;
       default: return -2;
     }
     if (rc != 0) return rc;
