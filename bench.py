@@ -91,22 +91,22 @@ def _mfma_entry(ms, flops, note=None, **extra):
     return d
 
 
-def bench_softmax(steps, warmup, family="softmax"):
+def bench_softmax(steps, warmup, family="softmax", B=8, S=4096, causal=True):
     import torch
     from metaattention_amd import hip_backend as hb
-    B, H, S, D = 8, 32, 4096, 128
+    H, D = 32, 128
     g = torch.Generator(device="cuda").manual_seed(0)
     q, k, v = (torch.randn(B, S, H, D, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(3))
     o = torch.empty_like(q)
     lse = torch.empty(B, H, S, device="cuda", dtype=torch.float32)
     scale = 1.0 / math.sqrt(D)
     if family == "softmax":
-        fn = lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale, out=o, row_scale=lse)
+        fn = lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=causal, scale=scale, out=o, row_scale=lse)
     else:  # sigmoid(q.k*scale - log S)
-        fn = lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SIGMOID, causal=True, scale=scale, bias=-math.log(S), out=o)
+        fn = lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SIGMOID, causal=causal, scale=scale, bias=-math.log(S), out=o)
     ms = time_gpu(fn, steps, warmup)
-    flops = 0.5 * 4.0 * B * H * S * S * D
-    return dict(ms=ms, flops=flops, tflops=flops / ms / 1e9, shape=dict(B=B, H=H, S=S, D=D, DV=D, causal=True))
+    flops = (0.5 if causal else 1.0) * 4.0 * B * H * S * S * D
+    return dict(ms=ms, flops=flops, tflops=flops / ms / 1e9, shape=dict(B=B, H=H, S=S, D=D, DV=D, causal=causal))
 
 
 def bench_softmax_operator(steps, warmup):
@@ -474,6 +474,11 @@ def main():
     others = {}
     want = [w for w in args.only.split(",") if w]
     table = [("c2_sigmoid_causal", "sigmoid", lambda: (lambda r: _mfma_entry(r["ms"], r["flops"]))(bench_softmax(args.steps, args.warmup, "sigmoid"))),
+             # the same kernel where an item is longer: how much of the headline's distance to the ceiling is the shape
+             ("softmax_noncausal_s4096", "noncausal", lambda: (lambda r: _mfma_entry(r["ms"], r["flops"], "non-causal, B8 H32 S4096 D128"))(
+                 bench_softmax(max(args.steps // 2, 3), 2, "softmax", causal=False))),
+             ("softmax_causal_s16384", "s16384", lambda: (lambda r: _mfma_entry(r["ms"], r["flops"], "causal, B2 H32 S16384 D128"))(
+                 bench_softmax(max(args.steps // 3, 3), 2, "softmax", B=2, S=16384))),
              ("c2_softmax_causal_operator", "operator", lambda: bench_softmax_operator(args.steps, args.warmup)),
              ("c2_softmax_causal_bwd", "bwd", lambda: bench_softmax_bwd(args.steps, args.warmup)),
              ("c3_retnet_chunked", "retnet", lambda: bench_retnet_chunked(args.steps, args.warmup)),
