@@ -22,11 +22,16 @@
 //                        operands) and walks the query rows of every query head of its group; here
 //                        S = Q K^T and dP = dO V^T are NOT transposed (lane = key), so P and dS are
 //                        directly the B operands of dV^T += dO^T P and dK^T += Q^T dS; lse and delta of
-//                        the 16 rows a lane holds come from global memory.
-// The scores are recomputed in both (7 tile products instead of 5), which is what avoiding the fp32
-// atomics and the post-pass costs.  Tiles of 32 rows arrive by direct-to-LDS DMA, double buffered,
-// one barrier per tile, XOR-swizzled like the forward tiles; the column-side operands (K^T, dO^T,
-// Q^T) come from the same tiles through the transposing LDS read.
+//                        a tile's rows come with the tile.  dk and dv in one launch or in two (then the
+//                        scores are computed once more), whichever lets two waves share a SIMD.
+//   attn_bwd_dkv_fused_kernel  the same work for the structural masks (none, causal) at head sizes up to
+//                        128 / 128: dk and dv in one launch, one wave per SIMD with the 512-register
+//                        budget, persistent, the loop pipelined inside the wave (see there).
+// The scores are recomputed in both kernels (7 tile products instead of 5; 8 where dk and dv take two
+// launches), which is what avoiding the fp32 atomics and the post-pass costs.  Tiles of 32 rows arrive by
+// direct-to-LDS DMA (a wave-uniform base in scalar registers plus 32-bit lane offsets computed once),
+// through a ring of stages, one barrier per tile, XOR-swizzled like the forward tiles; the column-side
+// operands (K^T, dO^T, Q^T) come from the same tiles through the transposing LDS read.
 #include "attn_bwd.h"
 
 namespace ma {
@@ -58,6 +63,20 @@ __device__ __forceinline__ void row_fn_bwd(float s, float dp, bool masked, float
   }
 }
 
+// The same in two parts, for the pipelined kernel: p of a kept score, and ds / scale from p.
+template <int FAMILY>
+__device__ __forceinline__ float row_p(float s, float c_scale, float c_bias, float scale, float bias, float lse2) {
+  if constexpr (FAMILY == BF_SOFTMAX) return fast_exp2(s * c_scale + lse2);
+  else if constexpr (FAMILY == BF_SIGMOID) return fast_rcp(1.f + fast_exp2(-(s * c_scale + c_bias)));
+  else return fmaxf(s * scale + bias, 0.f);
+}
+template <int FAMILY>
+__device__ __forceinline__ float row_ds(float p, float dp, float delta) {
+  if constexpr (FAMILY == BF_SOFTMAX) return p * (dp - delta);
+  else if constexpr (FAMILY == BF_SIGMOID) return dp * p * (1.f - p);
+  else return p > 0.f ? dp : 0.f;
+}
+
 // DMA of a [32 x ROWB bytes] tile whose rows are `row_stride` bytes apart in memory: each instruction
 // moves 1 KB; lane i fetches the 16-byte chunk that belongs at physical position i of that KB.  Rows
 // beyond `limit` are clamped to the last one (whatever is computed from them is masked).
@@ -70,6 +89,38 @@ __device__ __forceinline__ void dma_tile(const char* src, int64_t row_stride, in
     dma16(src + grow * row_stride + ((c ^ swz_tile<CPR>(row)) << 4), lds_base + ii * 1024);
   }
 }
+
+// The same tile when all of its 32 rows lie inside the tensor: the byte offsets of a lane (tile row * row stride + swizzled
+// chunk) are computed once, and a tile's DMA is then its wave-uniform first-row address in scalar registers plus those
+// 32-bit offsets -- no per-lane 64-bit address arithmetic inside the loops.  Where every instruction of a wave has the
+// same swizzle term (rows 16 apart) one offset serves them all and the row distance goes into the scalar base.
+template <int ROWB, int NWAVES>
+struct TileDma {
+  static constexpr int CPR = ROWB / 16, RPI = 1024 / ROWB, NI = 32 * ROWB / 1024, NJ = NI / NWAVES;
+  static constexpr bool SAME = NJ == 1 || (NWAVES * RPI) % 16 == 0;
+  static_assert(NI % NWAVES == 0, "a tile is a whole number of instructions per wave");
+  uint32_t off[SAME ? 1 : NJ];
+  uint32_t stride;
+  __device__ __forceinline__ void init(uint32_t row_stride, int wave, int lane) {
+    stride = row_stride;
+#pragma unroll
+    for (int j = 0; j < (SAME ? 1 : NJ); j++) {
+      const int row = (wave + NWAVES * j) * RPI + lane / CPR, c = lane % CPR;
+      off[j] = (uint32_t)row * row_stride + (uint32_t)((c ^ swz_tile<CPR>(row)) << 4);
+    }
+  }
+  __device__ __forceinline__ void issue(const char* first_row, uint32_t lds_base, int wave) const {
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+      dma16_so(SAME ? first_row + (uint64_t)((uint32_t)(j * NWAVES * RPI) * stride) : first_row, off[SAME ? 0 : j], lds_base + (wave + NWAVES * j) * 1024);
+  }
+};
+
+// Stages of the pipelined dk / dv kernel's tile ring: eight (tiles arrive four steps ahead) where they fit the LDS, else four.
+constexpr int fused_stages(int dqk, int dv) { return 8 * (32 * (dqk + dv) * 2 + 512) <= 150 * 1024 ? 8 : 4; }
+// Waits until at most N of this wave's vector-memory loads are outstanding (they complete in order).
+template <int N>
+__device__ __forceinline__ void wait_dma_but() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }
 
 // Retention: a wave's [32 rows x 32 columns] block of the score multiplier (64 bytes per row) by DMA into a 2 KB area of
 // its own, two instructions; the 16-byte chunk c of row r sits at position c ^ ((r >> 1) & 3) of the row, so that the
@@ -124,8 +175,10 @@ __device__ __forceinline__ f32x16 mm_rows(uint32_t tile, int r, int g, const typ
 // acc[DIM/32 blocks of 32 columns] += (tile columns)^T . pf, where pf holds a [32 x 32] factor in
 // accumulator order rounded to T (k slot i of slice s for lane half g is tile row 16s + 8(i/4) + 4g + i%4,
 // which is the row order the transposing reads below fetch)
-template <typename T, int DIM>
-__device__ __forceinline__ void mm_cols(uint32_t tile, int lane, const typename Elem<T>::x8 (&pf)[2], f32x16 (&acc)[DIM / 32]) {
+struct NoHook { __device__ __forceinline__ void operator()(int, int) const {} };
+// `between(idx, n)` runs behind MFMA idx of n: vector work that the matrix pipe covers
+template <typename T, int DIM, typename Hook = NoHook>
+__device__ __forceinline__ void mm_cols(uint32_t tile, int lane, const typename Elem<T>::x8 (&pf)[2], f32x16 (&acc)[DIM / 32], Hook between = Hook()) {
   using E = Elem<T>;
   using x8 = typename E::x8;
   using x4 = typename E::x4;
@@ -147,6 +200,7 @@ __device__ __forceinline__ void mm_cols(uint32_t tile, int lane, const typename 
     __builtin_amdgcn_sched_barrier(0);
     x8 af = __builtin_shufflevector(lo[idx % PF], hi[idx % PF], 0, 1, 2, 3, 4, 5, 6, 7);
     acc[idx >> 1] = E::mfma32(af, pf[idx & 1], acc[idx >> 1]);
+    between(idx, 2 * NB);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
@@ -255,9 +309,18 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
   const bool keep_ok = FAMILY != BF_RETENTION && a.elem_mask && ((a.em_sq | a.em_sb | a.em_sh | (int64_t)(uintptr_t)a.elem_mask) & 15) == 0;
   const uint8_t* bm_full = a.kv_block_mask ? a.kv_block_mask + (int64_t)b * a.kbm_sb + (int64_t)h * a.kbm_sh + (int64_t)mb * a.kbm_sq : nullptr;
   auto tile_full = [&](int jt_) { return bm_full && bm_full[jt_] >= 2; };   // the element-wise mask keeps every score of the tile
+  TileDma<KROW, 4> k_dma;
+  TileDma<VROW, 4> v_dma;
+  k_dma.init((uint32_t)k_row_bytes, wave, lane);
+  v_dma.init((uint32_t)v_row_bytes, wave, lane);
   auto issue_tile = [&](int n0, int buf) {
-    dma_tile<KROW, 4>(kb, k_row_bytes, n0, a.Skv, lds0 + buf * STAGE, wave, lane);
-    dma_tile<VROW, 4>(vb, v_row_bytes, n0, a.Skv, lds0 + buf * STAGE + KTILE, wave, lane);
+    if (n0 + BN <= a.Skv) {   // (wave-uniform)
+      k_dma.issue(kb + (int64_t)n0 * k_row_bytes, lds0 + buf * STAGE, wave);
+      v_dma.issue(vb + (int64_t)n0 * v_row_bytes, lds0 + buf * STAGE + KTILE, wave);
+    } else {
+      dma_tile<KROW, 4>(kb, k_row_bytes, n0, a.Skv, lds0 + buf * STAGE, wave, lane);
+      dma_tile<VROW, 4>(vb, v_row_bytes, n0, a.Skv, lds0 + buf * STAGE + KTILE, wave, lane);
+    }
     if constexpr (FAMILY == BF_RETENTION) {
       if (mult_ok && n0 + BN <= a.Skv && m_wave < a.Sq)
         mult_dma<T>((const T*)a.smask + (int64_t)b * a.sm_sb + (int64_t)h * a.sm_sh + (int64_t)m_wave * a.sm_sq + n0, a.sm_sq, a.Sq - m_wave,
@@ -396,7 +459,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
   // tile bases aligned to the row size)
   constexpr int QTILE = BMT * QROW, DOTILE = BMT * DOROW, STAGE = QTILE + DOTILE, ROWVALS = 2 * STAGE;
   // retention: behind those, a 2 KB block of the transposed multiplier per wave and stage (see the dq kernel)
-  constexpr int MULT = ROWVALS + 512;
+  constexpr int MULT = ROWVALS + 1024;
 
   extern __shared__ __align__(16) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
@@ -447,32 +510,50 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
   // tiles in which the mask keeps nothing for this workgroup's keys are never fetched
   const uint8_t* qbm = a.q_block_mask ? a.q_block_mask + (int64_t)b * a.qbm_sb + (int64_t)nb * a.qbm_sk : nullptr;
   // (entry 2: the element-wise mask keeps every score of the tile)
-  auto step_full = [&](int step) { return qbm && qbm[(int64_t)(hk * a.kv_group + step / t_count) * a.qbm_sh + t_first + step % t_count] >= 2; };
-  auto next_step = [&](int step) {
+  // a step = (query head of the group, tile of that head's rows), counted without divisions
+  struct Pos { int step, hg, t; };
+  auto advance = [&](Pos& p) {
+    p.step++;
+    if (++p.t == t_count) { p.t = 0; p.hg++; }
+  };
+  auto qbm_at = [&](const Pos& p) { return qbm[(int64_t)(hk * a.kv_group + p.hg) * a.qbm_sh + t_first + p.t]; };
+  auto step_full = [&](const Pos& p) { return qbm && qbm_at(p) >= 2; };
+  auto skip_empty = [&](Pos& p) {
     if (qbm)
-      while (step < n_steps && !qbm[(int64_t)(hk * a.kv_group + step / t_count) * a.qbm_sh + t_first + step % t_count]) step++;
-    return step;
+      while (p.step < n_steps && !qbm_at(p)) advance(p);
   };
   const bool keep_ok = FAMILY != BF_RETENTION && a.elem_mask_t && ((a.emt_sk | a.emt_sb | a.emt_sh | (int64_t)(uintptr_t)a.elem_mask_t) & 15) == 0;
   const bool mult_ok = FAMILY == BF_RETENTION && (a.smt_sk & 7) == 0 && (a.smt_sb & 7) == 0 && (a.smt_sh & 7) == 0 && ((uintptr_t)a.smask_t & 15) == 0;
-  auto issue_step = [&](int step, int buf) {
-    const int h = hk * a.kv_group + step / t_count, m0 = (t_first + step % t_count) * BMT;
+  TileDma<QROW, 4> q_dma;
+  TileDma<DOROW, 4> do_dma;
+  q_dma.init((uint32_t)q_row_bytes, wave, lane);
+  do_dma.init((uint32_t)do_row_bytes, wave, lane);
+  auto issue_step = [&](const Pos& step, int buf) {
+    const int h = hk * a.kv_group + step.hg, m0 = (t_first + step.t) * BMT;
     const char* qb = (const char*)((const T*)a.q + (int64_t)b * a.qsb + (int64_t)h * a.qsh);
     const char* dob = (const char*)((const T*)a.dout + (int64_t)b * a.dosb + (int64_t)h * a.dosh);
-    dma_tile<QROW, 4>(qb, q_row_bytes, m0, a.Sq, lds0 + buf * STAGE, wave, lane);
-    dma_tile<DOROW, 4>(dob, do_row_bytes, m0, a.Sq, lds0 + buf * STAGE + QTILE, wave, lane);
+    if (m0 + BMT <= a.Sq) {   // (wave-uniform)
+      q_dma.issue(qb + (int64_t)m0 * q_row_bytes, lds0 + buf * STAGE, wave);
+      do_dma.issue(dob + (int64_t)m0 * do_row_bytes, lds0 + buf * STAGE + QTILE, wave);
+    } else {
+      dma_tile<QROW, 4>(qb, q_row_bytes, m0, a.Sq, lds0 + buf * STAGE, wave, lane);
+      dma_tile<DOROW, 4>(dob, do_row_bytes, m0, a.Sq, lds0 + buf * STAGE + QTILE, wave, lane);
+    }
     if constexpr (FAMILY == BF_SOFTMAX) {
       // lse (lanes 0..31) and delta (lanes 32..63) of the tile's rows come with it: read from global memory inside
       // the loop, their latency is not covered by the little work a tile is
-      if (wave == 0) {
-        const int64_t ri = ((int64_t)b * a.H + h) * a.Sq + min(m0 + (lane & 31), a.Sq - 1);
-        dma4((lane < 32 ? a.lse : (const float*)a.delta) + ri, lds0 + ROWVALS + buf * 256);
+      // (wave 0 fetches lse, wave 1 delta: a scalar base and the lane's row; the upper lanes repeat the lower ones into
+      // the other half of the wave's 256 bytes)
+      if (wave < 2) {
+        const float* src = (wave == 0 ? a.lse : (const float*)a.delta) + ((int64_t)b * a.H + h) * a.Sq + m0;
+        dma4_so(src, (uint32_t)(min(m0 + (lane & 31), a.Sq - 1) - m0) * 4u, lds0 + ROWVALS + buf * 512 + wave * 256);
       }
     }
     if constexpr (FAMILY == BF_RETENTION) {
       // the row scales r of the tile's rows (twice: both halves of the wave fetch them) and, for whole tiles of an
       // aligned tensor, each wave's block of the transposed multiplier
-      if (wave == 0) dma4(a.lse + ((int64_t)b * a.H + h) * a.Sq + min(m0 + (lane & 31), a.Sq - 1), lds0 + ROWVALS + buf * 256);
+      if (wave == 0)
+        dma4_so(a.lse + ((int64_t)b * a.H + h) * a.Sq + m0, (uint32_t)(min(m0 + (lane & 31), a.Sq - 1) - m0) * 4u, lds0 + ROWVALS + buf * 512);
       if (mult_ok && m0 + BMT <= a.Sq && n_wave < a.Skv)
         mult_dma<T>((const T*)a.smask_t + (int64_t)b * a.smt_sb + (int64_t)h * a.smt_sh + (int64_t)n_wave * a.smt_sk + m0, a.smt_sk, a.Skv - n_wave,
                     lds0 + MULT + (buf * 4 + wave) * 2048, lane);
@@ -484,15 +565,18 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
     }
   };
 
-  int step_next = next_step(0);
-  if (step_next < n_steps) issue_step(step_next, 0);
-  for (int it = 0; step_next < n_steps; it++) {
-    const int buf = it & 1, step = step_next;
-    const int h = hk * a.kv_group + step / t_count, m0 = (t_first + step % t_count) * BMT;
+  Pos step_next = {0, 0, 0};
+  skip_empty(step_next);
+  if (step_next.step < n_steps) issue_step(step_next, 0);
+  for (int it = 0; step_next.step < n_steps; it++) {
+    const int buf = it & 1;
+    const Pos step = step_next;
+    const int h = hk * a.kv_group + step.hg, m0 = (t_first + step.t) * BMT;
     wait_dma();
     __syncthreads();
-    step_next = next_step(step + 1);
-    if (step_next < n_steps) issue_step(step_next, buf ^ 1);
+    advance(step_next);
+    skip_empty(step_next);
+    if (step_next.step < n_steps) issue_step(step_next, buf ^ 1);
     // (a wave whose keys all lie behind this tile's rows has nothing to add; it still takes part in the barriers.  With
     // the large accumulators of the 256 / 512 head size the second way round the loop costs register copies that spill,
     // and the few such tiles are computed instead: every element of them is masked)
@@ -503,7 +587,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
     // multiplier tensor: this key's row, indexed by query position)
     float lse2[16], dl[16];
     if constexpr (FAMILY == BF_RETENTION) {
-      const uint32_t rv = lds0 + ROWVALS + buf * 256;
+      const uint32_t rv = lds0 + ROWVALS + buf * 512;
       const T* smt_row = (const T*)a.smask_t + (int64_t)b * a.smt_sb + (int64_t)h * a.smt_sh + (int64_t)n_ld * a.smt_sk;
       const bool staged = mult_ok && m0 + BMT <= a.Sq && n_wave < a.Skv;
 #pragma unroll
@@ -523,11 +607,11 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
     }
     // lse and delta of the rows this lane holds: m0 + 8q4 + 4g + {0..3}
     if constexpr (FAMILY == BF_SOFTMAX) {
-      const uint32_t rv = lds0 + ROWVALS + buf * 256;
+      const uint32_t rv = lds0 + ROWVALS + buf * 512;
 #pragma unroll
       for (int q4 = 0; q4 < 4; q4++) {
         const f32x4 tl = lds_read<f32x4>(rv + (8 * q4 + 4 * g) * 4);
-        const f32x4 td = lds_read<f32x4>(rv + 128 + (8 * q4 + 4 * g) * 4);
+        const f32x4 td = lds_read<f32x4>(rv + 256 + (8 * q4 + 4 * g) * 4);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           lse2[4 * q4 + i] = c_bias - tl[i] * kLog2e;   // what the row function adds to s * c_scale
@@ -601,12 +685,284 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
   if constexpr (DO_DV) store_rows<T, DV>(dv, 1.f, stage, dvb, a.dvss, n_wave, a.Skv, lane);
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// dk and dv in one launch: one wave per SIMD, software pipelined
+// ------------------------------------------------------------------------------------------------
+// Where the K and V fragments and both [D x 32] accumulators of a wave's 32 keys fit the 512 registers of a wave that has its
+// SIMD to itself, dk and dv share the recomputed scores (7 tile products in all instead of 8).  With no second wave on the
+// SIMD to fill the matrix pipe while one evaluates the row function or waits for LDS, the loop is pipelined inside the
+// wave.  A step is ONE sequence of MFMAs:
+//   phase F  S(u+1) = Q(u+1) K^T and dP(u+1) = dO(u+1) V^T of the NEXT tile, with p of the current step's 16 score elements
+//            spread behind them,
+//   phase V  dV^T += dO(u)^T P(u), with ds of the 16 elements behind them,
+//   phase K  dK^T += Q(u)^T dS(u),
+// whose LDS operand fragments travel through one ring of registers, requested AH MFMAs ahead across the phases and across
+// steps (the last MFMAs of phase K request the first fragments of the next step).  Tiles come through a ring of stages, LA
+// steps ahead; the step's single barrier sits between phases V and K: behind it tile u+2 is visible to every wave, and
+// every wave is done with tile u-1, whose stage takes tile u+LA.  lse and delta of a tile's rows come with it.  The loop
+// body is written for two steps (the registers of "this" and "the next" step swap roles) so that nothing is copied; an odd
+// number of steps is padded with a step in which everything is masked.  Masked scores are set to -inf (times the sign
+// of scale) before the row function, in the few tiles that touch the diagonal or an end of the sequences: p = 0 and so
+// ds = 0 follow.  Structural masks only (none, causal): element-wise and tile masks, and the retention family, take the
+// two-launch kernels above.
+template <int I>
+struct IntC { static constexpr int value = I; };
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {   // f(IntC<I>()), ..., f(IntC<N - 1>()): indices that are constants by construction
+  if constexpr (I < N) {
+    f(IntC<I>());
+    static_for<I + 1, N>(f);
+  }
+}
+
+template <typename T>
+struct FusedStepRegs {
+  f32x16 s, dp;        // S and dP of the step's tile (lane = key, element jj = row 8(jj/4) + 4g + jj%4 of the tile)
+  f32x4 tl[4], td[4];  // lse and delta of those rows (softmax)
+};
+
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
+__global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBwdArgs a) {
+  using E = Elem<T>;
+  using x8 = typename E::x8;
+  using x4 = typename E::x4;
+  constexpr int BNW = 128, BMT = 32;
+  constexpr int KS = DQK / 16, VS = DV / 16, QB = DQK / 32, VB = DV / 32;
+  constexpr int QROW = DQK * 2, DOROW = DV * 2;
+  // a stage: the Q tile and the dO tile; behind the stages, 512 bytes per stage: lse (first 128) and delta (at 256) of its rows
+  constexpr int QTILE = BMT * QROW, DOTILE = BMT * DOROW, STAGE = QTILE + DOTILE;
+  constexpr int NST = fused_stages(DQK, DV), LA = NST == 8 ? 4 : 3, ROWVALS = NST * STAGE;
+  // the MFMAs of a step and the fragment ring
+  constexpr int NF = KS + VS, NV = 2 * VB, NK = 2 * QB, NTOT = NF + NV + NK;
+  constexpr int RING = 8, AH = NK < 6 ? NK : 6;
+  static_assert(NTOT % RING == 0 && AH < RING && AH <= NK && AH <= NF, "fragment ring");
+  static_assert(KS == VS, "phase F alternates the k slices of S and dP");
+
+  extern __shared__ __align__(16) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, g = lane >> 5;
+
+  // Persistent: the grid is one workgroup per CU, and every workgroup walks items  item = blockIdx.x, + gridDim.x, ...  An
+  // item is a (batch, kv head) and, under a causal mask, the PAIR of key blocks (k, n - 1 - k), which together see the
+  // same number of query tiles whatever k is: every item weighs the same.  Items that follow each other on an XCD
+  // (item % 8) belong to the same (batch, kv head) pairs, whose Q and dO tiles then come from that XCD's L2.
+  const int nnb = a.num_blocks, BHK = a.B * a.Hkv;
+  const int per_bh = CAUSAL ? (nnb + 1) / 2 : nnb, n_items = BHK * per_bh;
+  for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
+  int bhk, ki;
+  if ((BHK & 7) == 0) {
+    const int slot = item >> 3;
+    bhk = (slot / per_bh) * 8 + (item & 7);
+    ki = slot % per_bh;
+  } else {
+    bhk = item / per_bh;
+    ki = item % per_bh;
+  }
+  const int b = bhk / a.Hkv, hk = bhk % a.Hkv;
+  for (int part = 0; part < (CAUSAL && ki != nnb - 1 - ki ? 2 : 1); part++) {
+  const int nb = part == 0 ? ki : nnb - 1 - ki;
+  const int n_wave = nb * BNW + wave * 32, n_lane = n_wave + r;
+  const int n_ld = min(n_lane, a.Skv - 1);
+
+  x8 kf[KS], vf[VS];
+  {
+    const T* kp = (const T*)a.k + (int64_t)b * a.ksb + (int64_t)n_ld * a.kss + (int64_t)hk * a.ksh + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) kf[ks] = *(const x8*)(kp + 16 * ks);
+    const T* vp = (const T*)a.v + (int64_t)b * a.vsb + (int64_t)n_ld * a.vss + (int64_t)hk * a.vsh + 8 * g;
+#pragma unroll
+    for (int sl = 0; sl < VS; sl++) vf[sl] = *(const x8*)(vp + 16 * sl);
+  }
+  f32x16 dk[QB], dv[VB];
+#pragma unroll
+  for (int i = 0; i < QB; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) dk[i][j] = 0.f;
+#pragma unroll
+  for (int i = 0; i < VB; i++)
+#pragma unroll
+    for (int j = 0; j < 16; j++) dv[i][j] = 0.f;
+  const float bias = a.bias + (a.bias_ptr ? *a.bias_ptr : 0.f);
+  const float c_scale = a.scale * kLog2e, c_bias = bias * kLog2e;
+  const float s_masked = a.scale >= 0.f ? -__builtin_inff() : __builtin_inff();   // a score whose p is 0
+
+  // steps: for every query head of the kv head's group, the 32-row tiles that can see this workgroup's keys
+  const int t_first = CAUSAL ? (nb * BNW) / BMT : 0;
+  const int t_count = (a.Sq + BMT - 1) / BMT - t_first;
+  const int n_steps = t_count > 0 ? t_count * a.kv_group : 0;
+  const int64_t q_row_bytes = a.qss * 2, do_row_bytes = a.doss * 2;
+  TileDma<QROW, 4> q_dma;
+  TileDma<DOROW, 4> do_dma;
+  q_dma.init((uint32_t)q_row_bytes, wave, lane);
+  do_dma.init((uint32_t)do_row_bytes, wave, lane);
+  constexpr int TILE_DMAS = TileDma<QROW, 4>::NJ + TileDma<DOROW, 4>::NJ;   // what a wave issues per tile at least
+  auto issue_tile = [&](int hg, int t, int st) {
+    const int h = hk * a.kv_group + hg, m0 = (t_first + t) * BMT;
+    const char* qb = (const char*)((const T*)a.q + (int64_t)b * a.qsb + (int64_t)h * a.qsh);
+    const char* dob = (const char*)((const T*)a.dout + (int64_t)b * a.dosb + (int64_t)h * a.dosh);
+    if (m0 + BMT <= a.Sq) {   // (wave-uniform)
+      q_dma.issue(qb + (int64_t)m0 * q_row_bytes, lds0 + st * STAGE, wave);
+      do_dma.issue(dob + (int64_t)m0 * do_row_bytes, lds0 + st * STAGE + QTILE, wave);
+    } else {
+      dma_tile<QROW, 4>(qb, q_row_bytes, m0, a.Sq, lds0 + st * STAGE, wave, lane);
+      dma_tile<DOROW, 4>(dob, do_row_bytes, m0, a.Sq, lds0 + st * STAGE + QTILE, wave, lane);
+    }
+    if constexpr (FAMILY == BF_SOFTMAX) {
+      if (wave < 2) {   // wave 0 fetches lse, wave 1 delta (the upper lanes repeat the lower ones)
+        const float* src = (wave == 0 ? a.lse : (const float*)a.delta) + ((int64_t)b * a.H + h) * a.Sq + m0;
+        dma4_so(src, (uint32_t)(min(m0 + (lane & 31), a.Sq - 1) - m0) * 4u, lds0 + ROWVALS + st * 512 + wave * 256);
+      }
+    }
+  };
+  auto rowvals = [&](int st, FusedStepRegs<T>& x) {
+    if constexpr (FAMILY == BF_SOFTMAX) {
+      const uint32_t rv = lds0 + ROWVALS + st * 512;
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        x.tl[q4] = lds_read<f32x4>(rv + (8 * q4 + 4 * g) * 4);
+        x.td[q4] = lds_read<f32x4>(rv + 256 + (8 * q4 + 4 * g) * 4);
+      }
+    }
+  };
+
+  // the lane's part of the fragment addresses, relative to a tile: row reads (A operands of S and dP) and
+  // transposing reads (A operands of dV^T and dK^T: the tile's columns)
+  const uint32_t aq_l = (uint32_t)(r * QROW) + (uint32_t)((g ^ swz_tile<DQK / 8>(r)) << 4);
+  const uint32_t ad_l = (uint32_t)(r * DOROW) + (uint32_t)((g ^ swz_tile<DV / 8>(r)) << 4);
+  const int jr = (lane & 15) >> 2, lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
+  const uint32_t bq_l = (uint32_t)((4 * g + jr) * QROW + (lane & 1) * 8) + (uint32_t)((lc ^ swz_tile<DQK / 8>(4 * g + jr)) << 4);
+  const uint32_t bd_l = (uint32_t)((4 * g + jr) * DOROW + (lane & 1) * 8) + (uint32_t)((lc ^ swz_tile<DV / 8>(4 * g + jr)) << 4);
+  // the fragment of MFMA j of a step whose current tile sits at `cur` and whose next tile at `nxt` (LDS addresses)
+  auto fragment = [&](auto jc, uint32_t cur, uint32_t nxt) __attribute__((always_inline)) -> x8 {
+    constexpr int j = decltype(jc)::value;
+    // (consecutive MFMAs go to different accumulators: with one wave on the SIMD a dependent MFMA waits for the result
+    // of the one before it.  Phase F alternates S and dP; phases V and K walk the column blocks before the k slices)
+    if constexpr (j < NF && j % 2 == 0) {
+      return lds_read<x8>((nxt + aq_l) ^ (uint32_t)((j / 2) * 32));
+    } else if constexpr (j < NF) {
+      return lds_read<x8>((nxt + QTILE + ad_l) ^ (uint32_t)((j / 2) * 32));
+    } else {
+      constexpr bool is_v = j < NF + NV;
+      constexpr int idx = is_v ? j - NF : j - NF - NV, db = idx % (is_v ? VB : QB), sl = idx / (is_v ? VB : QB);
+      constexpr int rowb = is_v ? DOROW : QROW;
+      const uint32_t b0 = is_v ? cur + QTILE + bd_l : cur + bq_l;
+      const x4 lo = lds_read_tr4<T>((b0 ^ (uint32_t)((4 * db) << 4)) + 16 * sl * rowb);
+      const x4 hi = lds_read_tr4<T>((b0 ^ (uint32_t)(((4 * db) ^ 2) << 4)) + (16 * sl + 8) * rowb);
+      return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  };
+
+  if (n_steps > 0) {
+    // the next tile to fetch
+    int i_hg = 0, i_t = 0, i_n = 0;
+    auto issue_next = [&]() {
+      issue_tile(i_hg, i_t, i_n & (NST - 1));
+      i_n++;
+      if (++i_t == t_count) { i_t = 0; i_hg++; }
+    };
+#pragma unroll
+    for (int i = 0; i < LA; i++)
+      if (i_n < n_steps) issue_next();
+    // (the padding step of an odd number of steps evaluates S, dP, lse and delta of the stage behind the last tile's:
+    // where no earlier tile has been there, tile 0 goes there, so that what it computes is finite)
+    if ((n_steps & 1) && n_steps < NST) issue_tile(0, 0, n_steps);
+    wait_dma();
+    __syncthreads();
+    FusedStepRegs<T> ra, rb;
+    ra.s = mm_rows<T, DQK>(lds0, r, g, kf);
+    ra.dp = mm_rows<T, DV>(lds0 + QTILE, r, g, vf);
+    rowvals(0, ra);
+    x8 fr[RING];
+    static_for<0, AH>([&](auto jc) __attribute__((always_inline)) { fr[decltype(jc)::value] = fragment(jc, lds0, lds0 + STAGE); });   // (of step 0)
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    int c_t = 0;   // the current step's tile within its head
+    auto body = [&](int u, FusedStepRegs<T>& cur, FusedStepRegs<T>& nxt) __attribute__((always_inline)) {
+      const bool real = u < n_steps;                 // (the padding step: the last tile once more, everything masked)
+      const uint32_t cur_tile = lds0 + (uint32_t)(((real ? u : n_steps - 1) & (NST - 1)) * STAGE);
+      const uint32_t nxt_tile = lds0 + (uint32_t)(((u + 1) & (NST - 1)) * STAGE);
+      const uint32_t nn_tile = lds0 + (uint32_t)(((u + 2) & (NST - 1)) * STAGE);
+      const int m0 = real ? (t_first + c_t) * BMT : a.Sq;
+      if (++c_t == t_count) c_t = 0;
+      rowvals((u + 1) & (NST - 1), nxt);             // (requested here, needed in the next step)
+      // the few tiles that touch the diagonal or an end of the sequences (the test is wave-uniform)
+      if ((CAUSAL && n_wave + 31 > m0) || m0 + BMT > a.Sq || n_wave + 32 > a.Skv) {
+        // (m0 through an empty asm statement: the compiler would otherwise evaluate the 32 compares in every step, ahead
+        // of the branch, and turn the assignments into selects)
+        int m0e = m0;
+        asm volatile("; a tile that touches a mask" : "+s"(m0e));
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++) {
+          const int m = m0e + 8 * (jj >> 2) + 4 * g + (jj & 3);
+          if ((CAUSAL && n_lane > m) || m >= a.Sq || n_lane >= a.Skv) cur.s[jj] = s_masked;
+        }
+      }
+      x8 pf[2], dsf[2];
+      float p32[16];
+      static_for<0, NTOT>([&](auto jc) __attribute__((always_inline)) {
+        constexpr int j = decltype(jc)::value;
+        if constexpr (j == NF + NV) {
+          // tile u + 2 has landed (what may still be in flight: the tiles behind it) and every wave is done with
+          // tile u - 1, whose stage takes tile u + LA
+          if (LA > 3 && u + LA - 1 < n_steps) wait_dma_but<(LA - 3) * TILE_DMAS>();
+          else wait_dma();
+          asm volatile("" ::: "memory");
+          __builtin_amdgcn_s_barrier();
+          asm volatile("" ::: "memory");
+          if (i_n < n_steps) issue_next();
+        }
+        // the fragment of the MFMA AH places on (the last ones of the step: of the next step's first MFMAs)
+        if constexpr (j + AH < NTOT) fr[(j + AH) % RING] = fragment(IntC<j + AH>(), cur_tile, nxt_tile);
+        else fr[(j + AH) % RING] = fragment(IntC<j + AH - NTOT>(), nxt_tile, nn_tile);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (j < NF && j % 2 == 0) nxt.s = E::mfma32(fr[j % RING], kf[j / 2], j == 0 ? zero16 : nxt.s);
+        else if constexpr (j < NF) nxt.dp = E::mfma32(fr[j % RING], vf[j / 2], j == 1 ? zero16 : nxt.dp);
+        else if constexpr (j < NF + NV) dv[(j - NF) % VB] = E::mfma32(fr[j % RING], pf[(j - NF) / VB], dv[(j - NF) % VB]);
+        else dk[(j - NF - NV) % QB] = E::mfma32(fr[j % RING], dsf[(j - NF - NV) / QB], dk[(j - NF - NV) % QB]);
+        // vector work behind the MFMA: p of the step's 16 elements in phase F, ds in phase V
+        if constexpr (j < NF) {
+#pragma unroll
+          for (int jj = j * 16 / NF; jj < (j + 1) * 16 / NF; jj++) {
+            p32[jj] = row_p<FAMILY>(cur.s[jj], c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX ? fmaf(cur.tl[jj >> 2][jj & 3], -kLog2e, c_bias) : 0.f);
+            pf[jj >> 3][jj & 7] = (T)p32[jj];
+          }
+        } else if constexpr (j < NF + NV) {
+#pragma unroll
+          for (int jj = (j - NF) * 16 / NV; jj < (j - NF + 1) * 16 / NV; jj++)
+            dsf[jj >> 3][jj & 7] = (T)row_ds<FAMILY>(p32[jj], cur.dp[jj], FAMILY == BF_SOFTMAX ? cur.td[jj >> 2][jj & 3] : 0.f);
+          // (evaluated here, behind this MFMA: left alone the compiler moves it down to its use behind the barrier)
+          asm volatile("" : "+v"(dsf[((j - NF) * 16 / NV) >> 3]));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    };
+    for (int u = 0; u < n_steps; u += 2) {
+      body(u, ra, rb);
+      body(u + 1, rb, ra);
+    }
+  }
+  wait_dma();
+  __syncthreads();   // every wave is done with the tiles: they become output staging
+
+  constexpr int DMAX = DQK > DV ? DQK : DV, OROW = DMAX + 16;
+  const uint32_t stage = lds0 + wave * 32 * OROW;
+  T* dkb = (T*)a.dk + (int64_t)b * a.dksb + (int64_t)hk * a.dksh;
+  T* dvb = (T*)a.dv + (int64_t)b * a.dvsb + (int64_t)hk * a.dvsh;
+  store_rows<T, DQK>(dk, a.scale, stage, dkb, a.dkss, n_wave, a.Skv, lane);
+  store_rows<T, DV>(dv, 1.f, stage, dvb, a.dvss, n_wave, a.Skv, lane);
+  __syncthreads();   // the staged output has left the stages: the next key block's tiles may arrive
+  }   // the item's key blocks
+  }   // items
+}
+
 // ------------------------------------------------------------------------------------------------
 template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
 static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   constexpr int DMAX = DQK > DV ? DQK : DV;
   // (+ the row values of the dk / dv kernels' stages and the retention family's multiplier blocks / the keep-mask blocks)
-  constexpr size_t tiles = 2 * (size_t)32 * (DQK + DV) * 2 + 512 + (FAMILY == BF_RETENTION ? 2 * 4 * 2048 : 2 * 4 * 1024);
+  constexpr size_t tiles = 2 * (size_t)32 * (DQK + DV) * 2 + 1024 + (FAMILY == BF_RETENTION ? 2 * 4 * 2048 : 2 * 4 * 1024);
   constexpr size_t ostage = 4 * 32 * (size_t)(DMAX + 16);
   constexpr size_t lds = tiles > ostage ? tiles : ostage;
   auto k1 = attn_bwd_dq_kernel<T, DQK, DV, FAMILY, CAUSAL>;
@@ -620,6 +976,21 @@ static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   args.num_blocks = (a.Sq + 127) / 128;
   hipLaunchKernelGGL(k1, dim3((unsigned)(args.num_blocks * a.B * a.H)), dim3(256), lds, stream, args);
   args.num_blocks = (a.Skv + 127) / 128;
+  if constexpr (FAMILY != BF_RETENTION && DQK + DV <= 256) {
+    // structural masks only: dk and dv by the pipelined single launch
+    if (!a.elem_mask_t && !a.q_block_mask && a.scale != 0.f) {
+      constexpr size_t ftiles = fused_stages(DQK, DV) * ((size_t)32 * (DQK + DV) * 2 + 512);
+      constexpr size_t flds = ftiles > ostage ? ftiles : ostage;
+      auto kf = attn_bwd_dkv_fused_kernel<T, DQK, DV, FAMILY, CAUSAL>;
+      static std::atomic<uint64_t> flds_ok{0};
+      if (allow_lds(flds_ok, flds, kf) != 0) return -1;
+      const int cus = device_cus();
+      if (cus <= 0) return -1;
+      const int items = (CAUSAL ? (args.num_blocks + 1) / 2 : args.num_blocks) * a.B * a.Hkv;
+      hipLaunchKernelGGL(kf, dim3((unsigned)(items < cus ? items : cus)), dim3(256), flds, stream, args);
+      return launch_status();
+    }
+  }
   hipLaunchKernelGGL(k2, dim3((unsigned)(args.num_blocks * a.B * a.Hkv)), dim3(256), lds, stream, args);
   if (SPLIT) hipLaunchKernelGGL(k3, dim3((unsigned)(args.num_blocks * a.B * a.Hkv)), dim3(256), lds, stream, args);
   return launch_status();
@@ -660,6 +1031,9 @@ static int bwd_dims(const AttnBwdArgs& a, int family, bool causal, int dqk, int 
 
 // returns 0 ok, -1 launch failure, -2 unsupported
 int attn_bwd_dispatch(const AttnBwdArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream) {
+  // (the tile DMA addresses a tile's 32 rows with 32-bit byte offsets from its first row)
+  for (int64_t row_stride : {a.qss, a.kss, a.vss, a.doss})
+    if (row_stride < 0 || row_stride * 2 * 32 >= ((int64_t)1 << 32)) return -2;
   return is_bf16 ? bwd_dims<__bf16>(a, family, causal, dqk, dv, stream) : bwd_dims<_Float16>(a, family, causal, dqk, dv, stream);
 }
 

@@ -125,6 +125,18 @@ __device__ __forceinline__ void dma16_so(const void* base_uniform, uint32_t lane
       : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(lane_off), "s"(sb)
       : "memory");
 }
+__device__ __forceinline__ void dma4_so(const void* base_uniform, uint32_t lane_off, uint32_t lds_base) {
+  const uint64_t b = (uint64_t)(uintptr_t)base_uniform;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b), hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+  const uint64_t sb = ((uint64_t)hi << 32) | lo;
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dword %1, %2\n\t"
+      :
+      : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(lane_off), "s"(sb)
+      : "memory");
+}
 // vmcnt(0), other counters untouched.  The builtin (rather than asm) also tells the
 // compiler's own wait-count bookkeeping that no vector-memory load is pending any more.
 __device__ __forceinline__ void wait_dma() { __builtin_amdgcn_s_waitcnt(0x0F70); }

@@ -61,6 +61,21 @@ def test_softmax_backward(D, DV, B, H, Hkv, S, causal, dtype):
     _check(got, ref, "softmax")
 
 
+@pytest.mark.parametrize("D,H,Hkv,S,causal", [(128, 4, 2, 1100, True), (64, 2, 2, 1060, True), (128, 2, 1, 1100, False)])
+def test_softmax_backward_many_tiles(D, H, Hkv, S, causal):
+    """Longer sequences: the tile ring of the dk / dv kernel wraps several times, a workgroup takes a pair of key blocks
+    (an odd number of blocks leaves the middle one alone), the last tile and the last key block are partial."""
+    hb = _hb()
+    g = torch.Generator().manual_seed(S + D)
+    q = torch.randn(1, S, H, D, generator=g).bfloat16()
+    k = torch.randn(1, S, Hkv, D, generator=g).bfloat16()
+    v = torch.randn(1, S, Hkv, D, generator=g).bfloat16()
+    dout = torch.randn(1, S, H, D, generator=g).bfloat16()
+    print(f"softmax bwd many tiles D{D} H{H} Hkv{Hkv} S{S} causal={causal}", flush=True)
+    got, ref = _run(hb, "softmax", q, k, v, dout, causal, 1 / math.sqrt(D))
+    _check(got, ref, "softmax")
+
+
 @pytest.mark.parametrize("family", ["sigmoid", "relu"])
 @pytest.mark.parametrize("D,DV,S,causal", [(128, 128, 256, True), (64, 64, 200, False), (128, 128, 130, True)])
 def test_sigmoid_relu_backward(family, D, DV, S, causal):
