@@ -173,7 +173,7 @@ def bench_softmax_bwd(steps, warmup):
     o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale, row_scale=lse)
     ms = time_gpu(lambda: hb.attn_bwd(q, k, v, o, do, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale), max(steps // 3, 3), 2)
     flops = 2.5 * 0.5 * 4.0 * B * H * S * S * D
-    return _mfma_entry(ms, flops, "backward, 2.5 x the forward's algorithmic FLOPs (5 tile products; the three kernels dq, dv, dk execute 8: each recomputes the scores)")
+    return _mfma_entry(ms, flops, "backward, 2.5 x the forward's algorithmic FLOPs (5 tile products; the dq kernel and the fused dk/dv kernel execute 7: each recomputes the scores)")
 
 
 def bench_decode(steps, warmup, B=64, H=32, Hkv=8, Skv=4096, D=128):

@@ -125,7 +125,8 @@ typedef struct ma_attn_params {
  * dQ post-pass.  Tensors and strides as in ma_attn_params; o and lse are the forward pass's output and
  * fp32 [B,H,Sq] row scale (SOFTMAX only; may be NULL otherwise), dout is the gradient of o; dq [B,Sq,H,Dqk],
  * dk [B,Skv,Hkv,Dqk], dv [B,Skv,Hkv,Dv] are written (not accumulated into), in `dtype`.  The workspace
- * (ma_attn_bwd_workspace_bytes: fp32 [B,H,Sq]) carries delta = sum_d dout*o between the two kernels. */
+ * (ma_attn_bwd_workspace_bytes: fp32 [B,H,Sq]) carries delta = sum_d dout*o between the two kernels.  Sequence
+ * strides of q, k, v and dout must be non-negative and below 2^26 elements (MA_ERR_UNSUPPORTED otherwise). */
 typedef struct ma_attn_bwd_params {
   int32_t family; /* ma_attn_family: SOFTMAX, SIGMOID, RELU or RETENTION (Dqk 256, Dv 512) */
   int32_t dtype;
