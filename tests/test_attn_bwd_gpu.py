@@ -76,6 +76,43 @@ def test_softmax_backward_many_tiles(D, H, Hkv, S, causal):
     _check(got, ref, "softmax")
 
 
+@pytest.mark.parametrize("D,Sq,Skv", [(128, 200, 333), (128, 333, 200), (64, 70, 520), (128, 1, 300)])
+def test_softmax_backward_cross_lengths(D, Sq, Skv):
+    """Different numbers of queries and keys (no mask): the dq kernel walks Skv, the dk / dv kernel Sq."""
+    hb = _hb()
+    g = torch.Generator().manual_seed(Sq + Skv)
+    q = torch.randn(2, Sq, 2, D, generator=g).bfloat16()
+    k = torch.randn(2, Skv, 2, D, generator=g).bfloat16()
+    v = torch.randn(2, Skv, 2, D, generator=g).bfloat16()
+    dout = torch.randn(2, Sq, 2, D, generator=g).bfloat16()
+    print(f"softmax bwd cross D{D} Sq{Sq} Skv{Skv}", flush=True)
+    got, ref = _run(hb, "softmax", q, k, v, dout, False, 1 / math.sqrt(D))
+    _check(got, ref, "softmax")
+
+
+def test_backward_random_shapes():
+    """A seeded sweep over batch, heads, group size, length, head size, family and mask."""
+    hb = _hb()
+    rng = torch.Generator().manual_seed(1234)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=rng))
+    for case in range(14):
+        D = (64, 128)[ri(0, 1)]
+        Hkv = ri(1, 3)
+        H = Hkv * ri(1, 2)
+        B, S = ri(1, 2), ri(1, 420)
+        family = ("softmax", "softmax", "sigmoid", "relu")[ri(0, 3)]
+        causal = bool(ri(0, 1)) and family != "relu"
+        g = torch.Generator().manual_seed(case)
+        q = torch.randn(B, S, H, D, generator=g).bfloat16()
+        k = (0.7 * torch.randn(B, S, Hkv, D, generator=g)).bfloat16()
+        v = (0.7 * torch.randn(B, S, Hkv, D, generator=g)).bfloat16()
+        dout = (0.3 * torch.randn(B, S, H, D, generator=g)).bfloat16()
+        print(f"random bwd case {case}: {family} B{B} H{H} Hkv{Hkv} S{S} D{D} causal={causal}", flush=True)
+        got, ref = _run(hb, family, q, k, v, dout, causal, 1 / math.sqrt(D), bias=-1.0 if family == "sigmoid" else 0.0)
+        for name, a, b in zip(("dq", "dk", "dv"), got, ref):
+            oracle.assert_close(a.float().cpu(), b.float(), rtol=RTOL, atol=ATOL, mismatch_ratio=2e-3, msg=f"case {case} {family}:{name}")
+
+
 @pytest.mark.parametrize("family", ["sigmoid", "relu"])
 @pytest.mark.parametrize("D,DV,S,causal", [(128, 128, 256, True), (64, 64, 200, False), (128, 128, 130, True)])
 def test_sigmoid_relu_backward(family, D, DV, S, causal):
