@@ -1026,6 +1026,7 @@ static int bwd_dims(const AttnBwdArgs& a, int family, bool causal, int dqk, int 
   if (dqk == 64 && dv == 64) return bwd_family<T, 64, 64>(a, family, causal, stream);
   if (dqk == 128 && dv == 256) return bwd_family<T, 128, 256>(a, family, causal, stream);
   if (dqk == 256 && dv == 256) return bwd_family<T, 256, 256>(a, family, causal, stream);
+  if (dqk == 256 && dv == 512) return bwd_family<T, 256, 512>(a, family, causal, stream);
   return -2;
 }
 

@@ -482,9 +482,19 @@ static int wide_dims(const AttnArgs& a, int family, bool causal, int dqk, int dv
   if (dqk == 64 && dv == 64) return wide_family<T, 64, 64>(a, family, causal, stream);
   if (dqk == 128 && dv == 256) return wide_family<T, 128, 256>(a, family, causal, stream);
   if (dqk == 256 && dv == 256) return wide_family<T, 256, 256>(a, family, causal, stream);
-  // (softmax is left out at 256/512: rescaling a 256-register accumulator that lives in the MFMA
-  // accumulation registers makes the compiler spill it)
   if (dqk == 256 && dv == 512 && family != WF_SOFTMAX) return wide_family<T, 256, 512>(a, family, causal, stream);
+  // Softmax at 256/512: rescaling a 256-register accumulator that lives in the MFMA accumulation registers makes the
+  // compiler spill it.  Given the probabilities the value columns are independent, so the two halves of V and of the
+  // output go through the 256/256 kernel one after the other (the scores are computed twice; both launches write the
+  // same row scales).
+  if (dqk == 256 && dv == 512) {
+    AttnArgs half = a;
+    const int rc = wide_family<T, 256, 256>(half, family, causal, stream);
+    if (rc != 0) return rc;
+    half.v = (const T*)a.v + 256;
+    half.o = (T*)a.o + 256;
+    return wide_family<T, 256, 256>(half, family, causal, stream);
+  }
   return -2;
 }
 

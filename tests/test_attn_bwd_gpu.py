@@ -46,7 +46,7 @@ def _run(hb, family, q, k, v, dout, causal, scale, bias=0.0):
     return got, ref
 
 
-@pytest.mark.parametrize("D,DV", [(128, 128), (64, 64), (128, 256), (256, 256)])
+@pytest.mark.parametrize("D,DV", [(128, 128), (64, 64), (128, 256), (256, 256), (256, 512)])
 @pytest.mark.parametrize("B,H,Hkv,S,causal", [(1, 2, 2, 256, True), (2, 3, 3, 200, True), (1, 2, 2, 333, False), (1, 4, 2, 129, True), (1, 1, 1, 1, True)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_softmax_backward(D, DV, B, H, Hkv, S, causal, dtype):

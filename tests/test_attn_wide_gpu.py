@@ -21,7 +21,7 @@ def _hb():
     return hb
 
 
-@pytest.mark.parametrize("D,DV", [(64, 64), (128, 256), (256, 256)])
+@pytest.mark.parametrize("D,DV", [(64, 64), (128, 256), (256, 256), (256, 512)])
 @pytest.mark.parametrize("B,H,S,causal", [(1, 2, 256, True), (2, 3, 200, True), (1, 2, 333, False), (1, 1, 1, True), (1, 2, 129, True)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_softmax_other_head_sizes(D, DV, B, H, S, causal, dtype):
