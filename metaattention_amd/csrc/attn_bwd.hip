@@ -24,9 +24,9 @@
 //                        directly the B operands of dV^T += dO^T P and dK^T += Q^T dS; lse and delta of
 //                        a tile's rows come with the tile.  dk and dv in one launch or in two (then the
 //                        scores are computed once more), whichever lets two waves share a SIMD.
-//   attn_bwd_dkv_fused_kernel  the same work for the structural masks (none, causal) at head sizes up to
-//                        128 / 128: dk and dv in one launch, one wave per SIMD with the 512-register
-//                        budget, persistent, the loop pipelined inside the wave (see there).
+//   attn_bwd_dkv_fused_kernel  the same work at head sizes up to 128 / 128 (any mask): dk and dv in one launch,
+//                        one wave per SIMD with the 512-register budget, persistent, the loop pipelined
+//                        inside the wave (see there).
 // The scores are recomputed in both kernels (7 tile products instead of 5; 8 where dk and dv take two
 // launches), which is what avoiding the fp32 atomics and the post-pass costs.  Tiles of 32 rows arrive by
 // direct-to-LDS DMA (a wave-uniform base in scalar registers plus 32-bit lane offsets computed once),
@@ -704,8 +704,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
 // body is written for two steps (the registers of "this" and "the next" step swap roles) so that nothing is copied; an odd
 // number of steps is padded with a step in which everything is masked.  Masked scores are set to -inf (times the sign
 // of scale) before the row function, in the few tiles that touch the diagonal or an end of the sequences: p = 0 and so
-// ds = 0 follow.  Structural masks only (none, causal): element-wise and tile masks, and the retention family, take the
-// two-launch kernels above.
+// ds = 0 follow.  The retention family and the larger head sizes take the two-launch kernels above.
 template <int I>
 struct IntC { static constexpr int value = I; };
 template <int I, int N, typename F>
@@ -722,7 +721,13 @@ struct FusedStepRegs {
   f32x4 tl[4], td[4];  // lse and delta of those rows (softmax)
 };
 
-template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
+// MASKS: with an element-wise keep mask (its transpose: a lane walks a key's column) and / or a tile mask.  The steps of a
+// key block are then a list in LDS, built by wave 0 before the loop: the (query head, tile) pairs whose tile-mask entry is
+// not 0, each with the flag "kept in full" (entry 2: the element mask is not consulted).  A wave's [32 x 32] block of mask
+// bytes comes with the tile (whole tiles of a 16-byte aligned mask; others are read from global memory), and the
+// masked scores are set to -inf in the same place as for the structural masks.
+constexpr int FUSED_LIST_MAX = 2048;   // steps of a key block that the list holds (the launcher checks)
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL, bool MASKS>
 __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBwdArgs a) {
   using E = Elem<T>;
   using x8 = typename E::x8;
@@ -732,7 +737,9 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBw
   constexpr int QROW = DQK * 2, DOROW = DV * 2;
   // a stage: the Q tile and the dO tile; behind the stages, 512 bytes per stage: lse (first 128) and delta (at 256) of its rows
   constexpr int QTILE = BMT * QROW, DOTILE = BMT * DOROW, STAGE = QTILE + DOTILE;
-  constexpr int NST = fused_stages(DQK, DV), LA = NST == 8 ? 4 : 3, ROWVALS = NST * STAGE;
+  constexpr int NST = MASKS ? 4 : fused_stages(DQK, DV), LA = NST == 8 ? 4 : 3, ROWVALS = NST * STAGE;
+  // (MASKS) behind the row values: 1 KB of mask bytes per stage and wave, then the step list and its length
+  constexpr int KEEP = ROWVALS + NST * 512, LIST = KEEP + NST * 4 * 1024, LIST_N = LIST + FUSED_LIST_MAX * 4;
   // the MFMAs of a step and the fragment ring
   constexpr int NF = KS + VS, NV = 2 * VB, NK = 2 * QB, NTOT = NF + NV + NK;
   constexpr int RING = 8, AH = NK < 6 ? NK : 6;
@@ -756,9 +763,13 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBw
     const int slot = item >> 3;
     bhk = (slot / per_bh) * 8 + (item & 7);
     ki = slot % per_bh;
+    // (without the causal pairing a key block's work depends on the mask: a workgroup, whose items are a whole number of
+    // (batch, kv head) pairs apart, takes another key block each time round instead of the same one)
+    if (!CAUSAL) ki = (ki + slot / per_bh) % per_bh;
   } else {
     bhk = item / per_bh;
     ki = item % per_bh;
+    if (!CAUSAL) ki = (ki + bhk) % per_bh;
   }
   const int b = bhk / a.Hkv, hk = bhk % a.Hkv;
   for (int part = 0; part < (CAUSAL && ki != nnb - 1 - ki ? 2 : 1); part++) {
@@ -791,15 +802,50 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBw
   // steps: for every query head of the kv head's group, the 32-row tiles that can see this workgroup's keys
   const int t_first = CAUSAL ? (nb * BNW) / BMT : 0;
   const int t_count = (a.Sq + BMT - 1) / BMT - t_first;
-  const int n_steps = t_count > 0 ? t_count * a.kv_group : 0;
+  int n_steps = t_count > 0 ? t_count * a.kv_group : 0;
+  const bool keep_ok = MASKS && a.elem_mask_t && ((a.emt_sk | a.emt_sb | a.emt_sh | (int64_t)(uintptr_t)a.elem_mask_t) & 15) == 0;
+  if constexpr (MASKS) {
+    // the step list: entry = tile | head of the group << 16 | kept in full << 31
+    const uint8_t* qbm = a.q_block_mask ? a.q_block_mask + (int64_t)b * a.qbm_sb + (int64_t)nb * a.qbm_sk : nullptr;
+    if (wave == 0) {
+      int count = 0;
+      for (int i0 = 0; i0 < n_steps; i0 += 64) {
+        const int i = i0 + lane;
+        bool keep = false;
+        uint32_t entry = 0;
+        if (i < n_steps) {
+          const int hg = i / t_count, t = i - hg * t_count;
+          const uint8_t e = qbm ? qbm[(int64_t)(hk * a.kv_group + hg) * a.qbm_sh + t_first + t] : (uint8_t)1;
+          keep = e != 0;
+          entry = (uint32_t)t | ((uint32_t)hg << 16) | (e >= 2 || !a.elem_mask_t ? 0x80000000u : 0u);
+        }
+        const uint64_t votes = __ballot(keep);
+        if (keep) lds_write<uint32_t>(lds0 + LIST + 4 * (count + __popcll(votes & ((1ull << lane) - 1ull))), entry);
+        count += __popcll(votes);
+      }
+      if (lane == 0) lds_write<uint32_t>(lds0 + LIST_N, (uint32_t)count);
+    }
+    __syncthreads();
+    n_steps = __builtin_amdgcn_readfirstlane((int)lds_read<uint32_t>(lds0 + LIST_N));
+  }
+  // (list entries are requested a step before they are used and made wave-uniform only then: a read that is waited for
+  // at once would drain the ring of operand fragments)
+  auto list_request = [&](int i) { return lds_read<uint32_t>(lds0 + LIST + 4 * (i < n_steps ? i : 0)); };
+  auto uniform = [&](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
   const int64_t q_row_bytes = a.qss * 2, do_row_bytes = a.doss * 2;
   TileDma<QROW, 4> q_dma;
   TileDma<DOROW, 4> do_dma;
   q_dma.init((uint32_t)q_row_bytes, wave, lane);
   do_dma.init((uint32_t)do_row_bytes, wave, lane);
   constexpr int TILE_DMAS = TileDma<QROW, 4>::NJ + TileDma<DOROW, 4>::NJ;   // what a wave issues per tile at least
-  auto issue_tile = [&](int hg, int t, int st) {
+  auto issue_tile = [&](int hg, int t, int st, bool full = true) {
     const int h = hk * a.kv_group + hg, m0 = (t_first + t) * BMT;
+    if constexpr (MASKS) {
+      // the transposed element-wise keep mask: whole tiles of a 16-byte aligned mask come with the Q / dO tile
+      if (keep_ok && !full && m0 + BMT <= a.Sq && n_wave < a.Skv)
+        keep_dma(a.elem_mask_t + (int64_t)b * a.emt_sb + (int64_t)h * a.emt_sh + (int64_t)n_wave * a.emt_sk + m0, a.emt_sk, a.Skv - n_wave,
+                 lds0 + KEEP + (st * 4 + wave) * 1024, lane);
+    }
     const char* qb = (const char*)((const T*)a.q + (int64_t)b * a.qsb + (int64_t)h * a.qsh);
     const char* dob = (const char*)((const T*)a.dout + (int64_t)b * a.dosb + (int64_t)h * a.dosh);
     if (m0 + BMT <= a.Sq) {   // (wave-uniform)
@@ -857,17 +903,32 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBw
   if (n_steps > 0) {
     // the next tile to fetch
     int i_hg = 0, i_t = 0, i_n = 0;
+    uint32_t i_next = MASKS ? list_request(0) : 0u;   // (MASKS) the list entry of the next tile to fetch
     auto issue_next = [&]() {
-      issue_tile(i_hg, i_t, i_n & (NST - 1));
-      i_n++;
-      if (++i_t == t_count) { i_t = 0; i_hg++; }
+      if constexpr (MASKS) {
+        const uint32_t e = uniform(i_next);
+        issue_tile((int)((e >> 16) & 0x7fffu), (int)(e & 0xffffu), i_n & (NST - 1), (e >> 31) != 0);
+        i_n++;
+        i_next = list_request(i_n);
+      } else {
+        issue_tile(i_hg, i_t, i_n & (NST - 1));
+        i_n++;
+        if (++i_t == t_count) { i_t = 0; i_hg++; }
+      }
     };
 #pragma unroll
     for (int i = 0; i < LA; i++)
       if (i_n < n_steps) issue_next();
     // (the padding step of an odd number of steps evaluates S, dP, lse and delta of the stage behind the last tile's:
     // where no earlier tile has been there, tile 0 goes there, so that what it computes is finite)
-    if ((n_steps & 1) && n_steps < NST) issue_tile(0, 0, n_steps);
+    if ((n_steps & 1) && n_steps < NST) {
+      if constexpr (MASKS) {
+        const uint32_t e = uniform(list_request(0));
+        issue_tile((int)((e >> 16) & 0x7fffu), (int)(e & 0xffffu), n_steps);
+      } else {
+        issue_tile(0, 0, n_steps);
+      }
+    }
     wait_dma();
     __syncthreads();
     FusedStepRegs<T> ra, rb;
@@ -879,24 +940,53 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBw
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     int c_t = 0;   // the current step's tile within its head
+    uint32_t c_next = MASKS ? list_request(0) : 0u;   // (MASKS) the list entry of the step about to begin, requested a step ahead
     auto body = [&](int u, FusedStepRegs<T>& cur, FusedStepRegs<T>& nxt) __attribute__((always_inline)) {
       const bool real = u < n_steps;                 // (the padding step: the last tile once more, everything masked)
+      const uint32_t c_entry = MASKS ? uniform(c_next) : 0u;
+      if constexpr (MASKS) c_next = list_request(u + 1);
       const uint32_t cur_tile = lds0 + (uint32_t)(((real ? u : n_steps - 1) & (NST - 1)) * STAGE);
       const uint32_t nxt_tile = lds0 + (uint32_t)(((u + 1) & (NST - 1)) * STAGE);
       const uint32_t nn_tile = lds0 + (uint32_t)(((u + 2) & (NST - 1)) * STAGE);
-      const int m0 = real ? (t_first + c_t) * BMT : a.Sq;
+      const int m0 = real ? (t_first + (MASKS ? (int)(c_entry & 0xffffu) : c_t)) * BMT : a.Sq;
       if (++c_t == t_count) c_t = 0;
       rowvals((u + 1) & (NST - 1), nxt);             // (requested here, needed in the next step)
-      // the few tiles that touch the diagonal or an end of the sequences (the test is wave-uniform)
-      if ((CAUSAL && n_wave + 31 > m0) || m0 + BMT > a.Sq || n_wave + 32 > a.Skv) {
+      // the tiles that touch the diagonal, an end of the sequences or an element-wise mask (the test is wave-uniform)
+      const bool by_elem = MASKS && real && a.elem_mask_t && (c_entry >> 31) == 0;
+      if ((CAUSAL && n_wave + 31 > m0) || m0 + BMT > a.Sq || n_wave + 32 > a.Skv || by_elem) {
         // (m0 through an empty asm statement: the compiler would otherwise evaluate the 32 compares in every step, ahead
         // of the branch, and turn the assignments into selects)
         int m0e = m0;
         asm volatile("; a tile that touches a mask" : "+s"(m0e));
+        uint32_t keep[4] = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};   // the bytes of this lane's four rows per group
+        if constexpr (MASKS) {
+          if (by_elem) {
+            if (keep_ok && m0e + BMT <= a.Sq && n_wave < a.Skv) {
+#pragma unroll
+              for (int q4 = 0; q4 < 4; q4++) keep[q4] = keep_read(lds0 + KEEP + ((u & (NST - 1)) * 4 + wave) * 1024, r, g, q4);
+            } else {
+              // this key's row of the transposed mask, indexed by query position
+              const int h = hk * a.kv_group + (int)((c_entry >> 16) & 0x7fffu);
+              const uint8_t* emt_row = a.elem_mask_t + (int64_t)b * a.emt_sb + (int64_t)h * a.emt_sh + (int64_t)n_ld * a.emt_sk;
+#pragma unroll
+              for (int q4 = 0; q4 < 4; q4++) {
+                const int m = m0e + 8 * q4 + 4 * g;
+                keep[q4] = 0;
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                  if (m + i < a.Sq) keep[q4] |= (uint32_t)emt_row[m + i] << (8 * i);
+              }
+            }
+          }
+        }
 #pragma unroll
         for (int jj = 0; jj < 16; jj++) {
           const int m = m0e + 8 * (jj >> 2) + 4 * g + (jj & 3);
-          if ((CAUSAL && n_lane > m) || m >= a.Sq || n_lane >= a.Skv) cur.s[jj] = s_masked;
+          if ((CAUSAL && n_lane > m) || m >= a.Sq || n_lane >= a.Skv || (MASKS && ((keep[jj >> 2] >> (8 * (jj & 3))) & 0xffu) == 0)) {
+            cur.s[jj] = s_masked;
+            // (a row without any kept key has lse = -inf: its masked scores must still give p = 0)
+            if constexpr (FAMILY == BF_SOFTMAX) cur.tl[jj >> 2][jj & 3] = 0.f;
+          }
         }
       }
       x8 pf[2], dsf[2];
@@ -977,17 +1067,21 @@ static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL(k1, dim3((unsigned)(args.num_blocks * a.B * a.H)), dim3(256), lds, stream, args);
   args.num_blocks = (a.Skv + 127) / 128;
   if constexpr (FAMILY != BF_RETENTION && DQK + DV <= 256) {
-    // structural masks only: dk and dv by the pipelined single launch
-    if (!a.elem_mask_t && !a.q_block_mask && a.scale != 0.f) {
+    // dk and dv by the pipelined single launch (with masks: as long as a key block's steps fit its list)
+    const bool masks = a.elem_mask_t || a.q_block_mask;
+    if (a.scale != 0.f && (!masks || (int64_t)((a.Sq + 31) / 32) * a.kv_group <= FUSED_LIST_MAX)) {
       constexpr size_t ftiles = fused_stages(DQK, DV) * ((size_t)32 * (DQK + DV) * 2 + 512);
-      constexpr size_t flds = ftiles > ostage ? ftiles : ostage;
-      auto kf = attn_bwd_dkv_fused_kernel<T, DQK, DV, FAMILY, CAUSAL>;
+      constexpr size_t mtiles = 4 * ((size_t)32 * (DQK + DV) * 2 + 512 + 4 * 1024) + FUSED_LIST_MAX * 4 + 16;
+      constexpr size_t fmax = ftiles > mtiles ? ftiles : mtiles, flds = fmax > ostage ? fmax : ostage;
+      auto kf = attn_bwd_dkv_fused_kernel<T, DQK, DV, FAMILY, CAUSAL, false>;
+      auto km = attn_bwd_dkv_fused_kernel<T, DQK, DV, FAMILY, CAUSAL, true>;
       static std::atomic<uint64_t> flds_ok{0};
-      if (allow_lds(flds_ok, flds, kf) != 0) return -1;
+      if (allow_lds(flds_ok, flds, kf, km) != 0) return -1;
       const int cus = device_cus();
       if (cus <= 0) return -1;
       const int items = (CAUSAL ? (args.num_blocks + 1) / 2 : args.num_blocks) * a.B * a.Hkv;
-      hipLaunchKernelGGL(kf, dim3((unsigned)(items < cus ? items : cus)), dim3(256), flds, stream, args);
+      if (masks) hipLaunchKernelGGL(km, dim3((unsigned)(items < cus ? items : cus)), dim3(256), flds, stream, args);
+      else hipLaunchKernelGGL(kf, dim3((unsigned)(items < cus ? items : cus)), dim3(256), flds, stream, args);
       return launch_status();
     }
   }
