@@ -461,14 +461,20 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
         constexpr int SLOT = decltype(slot_c)::value;
         const int u = u0 + SLOT;
         if (u < my_steps) {
+          // (s_barrier alone: __syncthreads would also wait for the LDS reads in flight, the fragments that the vector
+          // phase has requested for the matrix phase behind the barrier)
           if (!late) {
             __builtin_amdgcn_s_waitcnt(0x0F70 | 6);   // vmcnt(6)
-            __syncthreads();
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
           }
           g_phase(slot_c);
           if (late) {
             __builtin_amdgcn_s_waitcnt(0x0F70 | 6);
-            __syncthreads();
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
           }
           s_phase(slot_c, u);
         }
