@@ -90,32 +90,6 @@ __device__ __forceinline__ void dma_tile(const char* src, int64_t row_stride, in
   }
 }
 
-// The same tile when all of its 32 rows lie inside the tensor: the byte offsets of a lane (tile row * row stride + swizzled
-// chunk) are computed once, and a tile's DMA is then its wave-uniform first-row address in scalar registers plus those
-// 32-bit offsets -- no per-lane 64-bit address arithmetic inside the loops.  Where every instruction of a wave has the
-// same swizzle term (rows 16 apart) one offset serves them all and the row distance goes into the scalar base.
-template <int ROWB, int NWAVES>
-struct TileDma {
-  static constexpr int CPR = ROWB / 16, RPI = 1024 / ROWB, NI = 32 * ROWB / 1024, NJ = NI / NWAVES;
-  static constexpr bool SAME = NJ == 1 || (NWAVES * RPI) % 16 == 0;
-  static_assert(NI % NWAVES == 0, "a tile is a whole number of instructions per wave");
-  uint32_t off[SAME ? 1 : NJ];
-  uint32_t stride;
-  __device__ __forceinline__ void init(uint32_t row_stride, int wave, int lane) {
-    stride = row_stride;
-#pragma unroll
-    for (int j = 0; j < (SAME ? 1 : NJ); j++) {
-      const int row = (wave + NWAVES * j) * RPI + lane / CPR, c = lane % CPR;
-      off[j] = (uint32_t)row * row_stride + (uint32_t)((c ^ swz_tile<CPR>(row)) << 4);
-    }
-  }
-  __device__ __forceinline__ void issue(const char* first_row, uint32_t lds_base, int wave) const {
-#pragma unroll
-    for (int j = 0; j < NJ; j++)
-      dma16_so(SAME ? first_row + (uint64_t)((uint32_t)(j * NWAVES * RPI) * stride) : first_row, off[SAME ? 0 : j], lds_base + (wave + NWAVES * j) * 1024);
-  }
-};
-
 // Stages of the pipelined dk / dv kernel's tile ring: eight (tiles arrive four steps ahead) where they fit the LDS, else four.
 constexpr int fused_stages(int dqk, int dv) { return 8 * (32 * (dqk + dv) * 2 + 512) <= 150 * 1024 ? 8 : 4; }
 // Waits until at most N of this wave's vector-memory loads are outstanding (they complete in order).

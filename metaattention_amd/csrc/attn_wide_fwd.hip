@@ -149,8 +149,17 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
   // DMA of one tile: each instruction moves 1 KB (1024 / row bytes tile rows); lane i fetches the
   // 16-byte chunk that belongs at physical position i of that KB.  Rows beyond the sequence are clamped
   // to its last row (their scores are masked, or multiplied by a zero of M).
+  TileDma<KROW, NW> k_dma;
+  TileDma<VROW, NW> v_dma;
+  k_dma.init((uint32_t)k_row_bytes, wave, lane);
+  v_dma.init((uint32_t)v_row_bytes, wave, lane);
   auto issue_tile = [&](int n0, int buf) {
     const uint32_t base = lds0 + buf * STAGE;
+    if (n0 + BN <= skv) {   // (wave-uniform) a whole tile: scalar bases, the lane offsets computed once
+      k_dma.issue(kb + (int64_t)n0 * k_row_bytes, base, wave);
+      v_dma.issue(vb + (int64_t)n0 * v_row_bytes, base + KTILE, wave);
+      return;
+    }
     for (int ii = wave; ii < NIK + NIV; ii += NW) {
       if (ii < NIK) {
         const int row = ii * (1024 / KROW) + lane / CPRK, c = lane % CPRK;
@@ -500,6 +509,9 @@ static int wide_dims(const AttnArgs& a, int family, bool causal, int dqk, int dv
 
 // returns 0 ok, -1 launch failure, -2 unsupported
 int attn_wide_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream) {
+  // (the tile DMA addresses a tile's 32 rows with 32-bit byte offsets from its first row)
+  for (int64_t row_stride : {a.kss, a.vss})
+    if (row_stride < 0 || row_stride * 2 * 32 >= ((int64_t)1 << 32)) return -2;
   return is_bf16 ? wide_dims<__bf16>(a, family, causal, dqk, dv, stream) : wide_dims<_Float16>(a, family, causal, dqk, dv, stream);
 }
 

@@ -155,6 +155,35 @@ __device__ __forceinline__ int swz_tile(int row) {
   return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
 }
 
+// DMA of a [32 rows x ROWB bytes] tile, XOR-swizzled in 16-byte chunks, whose 32 rows all lie inside the tensor (NWAVES
+// waves share the tile's instructions of 1 KB each: lane i fetches the chunk that belongs at physical position i of that
+// KB).  The byte offsets of a lane (tile row * row stride + swizzled chunk) are computed once, and a tile's DMA is then
+// its wave-uniform first-row address in scalar registers plus those 32-bit offsets: no per-lane 64-bit address
+// arithmetic inside the loops.  The swizzle term repeats every 16 rows, so instructions of a wave that are a multiple
+// of 16 rows apart share an offset and the row distance goes into the scalar base.
+template <int ROWB, int NWAVES>
+struct TileDma {
+  static constexpr int CPR = ROWB / 16, RPI = 1024 / ROWB, NI = 32 * ROWB / 1024, NJ = NI / NWAVES;
+  static constexpr int RPJ = NWAVES * RPI;   // rows between consecutive instructions of a wave
+  static constexpr int NOFF = RPJ % 16 == 0 ? 1 : (16 % RPJ == 0 && 16 / RPJ < NJ ? 16 / RPJ : NJ);
+  static_assert(NI % NWAVES == 0, "a tile is a whole number of instructions per wave");
+  uint32_t off[NOFF];
+  uint32_t stride;
+  __device__ __forceinline__ void init(uint32_t row_stride, int wave, int lane) {
+    stride = row_stride;
+#pragma unroll
+    for (int j = 0; j < NOFF; j++) {
+      const int row = (wave + NWAVES * j) * RPI + lane / CPR, c = lane % CPR;
+      off[j] = (uint32_t)row * row_stride + (uint32_t)((c ^ swz_tile<CPR>(row)) << 4);
+    }
+  }
+  __device__ __forceinline__ void issue(const char* first_row, uint32_t lds_base, int wave) const {
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+      dma16_so(first_row + (uint64_t)((uint32_t)((j / NOFF) * NOFF * RPJ) * stride), off[j % NOFF], lds_base + (wave + NWAVES * j) * 1024);
+  }
+};
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
