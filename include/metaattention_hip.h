@@ -64,7 +64,8 @@ typedef struct ma_attn_params {
   int32_t batch, heads, seqlen_q, seqlen_kv, dim_qk, dim_v;
   /* q [B,Sq,H,Dqk], k [B,Skv,Hkv,Dqk], v [B,Skv,Hkv,Dv], o [B,Sq,H,Dv]; BSHD is the
    * layout the reference operator takes (attn_tl.py:69-70) but any strides
-   * with a contiguous last dimension are accepted. */
+   * with a contiguous last dimension are accepted (sequence strides of k and v
+   * non-negative and below 2^26 elements). */
   const void* q; int64_t q_stride_b, q_stride_s, q_stride_h;
   const void* k; int64_t k_stride_b, k_stride_s, k_stride_h;
   const void* v; int64_t v_stride_b, v_stride_s, v_stride_h;
