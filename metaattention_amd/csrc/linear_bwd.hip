@@ -13,9 +13,10 @@
 // sequence with the log decay shifted by one token:
 //   dq = LA(do, v, k; v_scale)      du = R LA(R k, R q, R do)      dk = v_scale * R LA(R v, R do, R q)      (R reverses time)
 // so the backward pass is three scans of the forward kernel (linear_fwd.hip: state in accumulator registers, fp32
-// outputs), each contraction cut into the 128 / 256 wide pieces that kernel takes (their fp32 outputs add up), plus the
-// small kernels of this file: operand packing (time reversal, column slices, zero padding, head expansion), the shifted
-// reversed log decay, and the epilogue that forms dv, dv_scale, the per-token decay gradient
+// outputs), each contraction cut into the 128 / 256 wide pieces that kernel takes (their fp32 outputs add up); the scans
+// read their operands in place (reversed time, column slices and shared heads are the scan kernel's general operand
+// addressing), except a piece that needs zero padding, which pack_kernel copies.  Plus the small kernels of this file:
+// the shifted reversed log decay, and the epilogue that forms dv, dv_scale, the per-token decay gradient
 //   dG_t = q_t . dq_t - k_t . dk_t        (fp32 products of the fp32 scan outputs)
 // sums the heads that share a q / k head (:1300-1303), converts, and turns dG into dlog_decay by a reversed running sum
 // in fp32 (compute_final_dg).
@@ -197,7 +198,6 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   if ((a.Dk != 128 && a.Dk != 256) || a.Dv % 64 != 0 || a.Dv > 16 * 256) return -2;
   const int64_t BHT = (int64_t)a.B * a.H * a.T;
   const Slices sl(a.Dv);   // contraction of the dq and dk scans
-  const bool direct_a = a.Dv == 128 || a.Dv == 256;   // the dq scan reads do and v as they are
 
   // workspace: fp32 scan outputs, dG, reversed log decay, packed operands, the scan kernel's own workspace
   size_t off = 0;
@@ -230,42 +230,55 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
     hipLaunchKernelGGL(pack_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, (uint4*)dst, (const uint4*)src, Hd, Hs, a.T, W, Ws, c0,
                        rev ? 1 : 0, n);
   };
-  auto scan_launch = [&](const void* q, int Hq, const void* k, int Hk, const void* v, int dk, int dv, const float* g, const float* vs, float* out,
+  // an operand of a scan as the scan kernel reads it in place: heads, elements between its tokens (the pointer carries a
+  // column offset)
+  struct Operand { const void* p; int heads; int64_t row; };
+  auto scan_launch = [&](Operand q, Operand k, Operand v, bool reversed, int dk, int dv, const float* g, const float* vs, float* out,
                          bool accumulate) -> int {
     LinArgs la{};
-    la.q = q; la.k = k; la.v = v; la.o = out; la.log_decay = g; la.v_scale = vs; la.q_scale = a.q_scale;
-    la.B = a.B; la.H = a.H; la.Hq = Hq; la.Hk = Hk; la.T = a.T; la.Dv = dv;
+    la.q = q.p; la.k = k.p; la.v = v.p; la.o = out; la.log_decay = g; la.v_scale = vs; la.q_scale = a.q_scale;
+    la.B = a.B; la.H = a.H; la.Hq = q.heads; la.Hk = k.heads; la.Hv = v.heads; la.T = a.T; la.Dv = dv;
+    la.q_row = q.row; la.k_row = k.row; la.v_row = v.row; la.rev = reversed ? 1 : 0;
     la.out_f32 = accumulate ? 2 : 1;
     return linear_fwd_dispatch(la, dk, 0, scan, scan_ws, stream, nullptr);
   };
+  const __bf16 *q_p = (const __bf16*)a.q, *k_p = (const __bf16*)a.k, *v_p = (const __bf16*)a.v, *do_p = (const __bf16*)a.dout;
+  // a piece of the value columns is read in place when it lies inside them whole and the row is a multiple of its width
+  // (the scan kernel's condition); else it is packed (zero padded)
+  auto in_place = [&](int s) { return sl.c0[s] + sl.w[s] <= a.Dv && a.Dv % sl.w[s] == 0; };
 
   hipLaunchKernelGGL(shift_rev_kernel, dim3((unsigned)((BHT + 255) / 256)), dim3(256), 0, stream, grev, a.log_decay, a.T, BHT);
 
-  // dq (per head) = LA(do, v, k; v_scale), contraction over the value columns
-  const void* k_heads = a.k;
-  if (a.Hk != a.H) { pack(pv, a.k, a.H, a.Hk, a.Dk, a.Dk, 0, false); k_heads = pv; }
+  // dq (per head) = LA(do, v, k; v_scale), contraction over the value columns; k is read with its own heads
   for (int s = 0; s < sl.n; s++) {
-    const void *qs = a.dout, *ks = a.v;
-    if (!direct_a) {
+    Operand qs{do_p + sl.c0[s], a.H, a.Dv}, ks{v_p + sl.c0[s], a.H, a.Dv};
+    if (!in_place(s)) {
       pack(pa, a.dout, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], false);
       pack(pb, a.v, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], false);
-      qs = pa; ks = pb;
+      qs = Operand{pa, a.H, sl.w[s]};
+      ks = Operand{pb, a.H, sl.w[s]};
     }
-    if (const int rc = scan_launch(qs, a.H, ks, a.H, k_heads, sl.w[s], a.Dk, a.log_decay, a.v_scale, dqh, s > 0)) return rc;
+    if (const int rc = scan_launch(qs, ks, Operand{k_p, a.Hk, a.Dk}, false, sl.w[s], a.Dk, a.log_decay, a.v_scale, dqh, s > 0)) return rc;
   }
 
-  // du (reversed) = LA(R k, R q, R do), contraction over the key columns
-  pack(pa, a.k, a.Hk, a.Hk, a.Dk, a.Dk, 0, true);
-  pack(pb, a.q, a.Hq, a.Hq, a.Dk, a.Dk, 0, true);
-  pack(pv, a.dout, a.H, a.H, a.Dv, a.Dv, 0, true);
-  if (const int rc = scan_launch(pa, a.Hk, pb, a.Hq, pv, a.Dk, a.Dv, grev, nullptr, du, false)) return rc;
+  // du (reversed) = LA(R k, R q, R do), contraction over the key columns: the operands are read in reversed time in place
+  if (const int rc = scan_launch(Operand{k_p, a.Hk, a.Dk}, Operand{q_p, a.Hq, a.Dk}, Operand{do_p, a.H, a.Dv}, true, a.Dk, a.Dv, grev, nullptr, du, false))
+    return rc;
 
   // dk (per head, reversed, before its v_scale factor) = LA(R v, R do, R q), contraction over the value columns
-  pack(pv, a.q, a.H, a.Hq, a.Dk, a.Dk, 0, true);
   for (int s = 0; s < sl.n; s++) {
-    pack(pa, a.v, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], true);
-    pack(pb, a.dout, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], true);
-    if (const int rc = scan_launch(pa, a.H, pb, a.H, pv, sl.w[s], a.Dk, grev, nullptr, dkh, s > 0)) return rc;
+    Operand qs{v_p + sl.c0[s], a.H, a.Dv}, ks{do_p + sl.c0[s], a.H, a.Dv};
+    bool reversed = true;
+    if (!in_place(s)) {   // (packed in reversed order)
+      pack(pa, a.v, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], true);
+      pack(pb, a.dout, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], true);
+      qs = Operand{pa, a.H, sl.w[s]};
+      ks = Operand{pb, a.H, sl.w[s]};
+      pack(pv, a.q, a.H, a.Hq, a.Dk, a.Dk, 0, true);
+      if (const int rc = scan_launch(qs, ks, Operand{pv, a.H, a.Dk}, false, sl.w[s], a.Dk, grev, nullptr, dkh, s > 0)) return rc;
+      continue;
+    }
+    if (const int rc = scan_launch(qs, ks, Operand{q_p, a.Hq, a.Dk}, reversed, sl.w[s], a.Dk, grev, nullptr, dkh, s > 0)) return rc;
   }
 
   if ((a.Dk > a.Dv ? a.Dk : a.Dv) >= 256)

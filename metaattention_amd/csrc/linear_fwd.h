@@ -14,6 +14,12 @@ struct LinArgs {
   // states [group][segment][wave][registers][lane] fp32 and per-(batch*head, segment) log decays
   int nseg, seg_chunks;
   int out_f32;   // 1: o is fp32 [B,H,T,Dv] instead of bf16; 2: fp32, and the result is added to what o holds
+  // General operand addressing (the backward's scans; all zero: q [B,Hq,T,Dk], k [B,Hk,T,Dk], v [B,H,T,Dv] as they
+  // are): rev = the operands are read in reversed time order (token T-1-t at position t); q_row / k_row / v_row = elements
+  // between consecutive tokens of an operand (a column slice of a wider tensor: the pointer carries the column offset);
+  // Hv = heads of v (dividing H: head h reads v head h / (H / Hv)).
+  int rev, Hv;
+  int64_t q_row, k_row, v_row;
   float* ws_state;
   float* ws_decay;
 };

@@ -61,7 +61,9 @@ __device__ __forceinline__ X8 scale_bf16x8(X8 v, const float (&w)[8]) {
 template <int DK, int NWH, int HG>
 constexpr int min_waves_per_simd() { return HG > 1 ? 3 : (NWH == 4 ? 1 : 2); }
 
-template <int DK, int NWH, int HG, int MODE>
+// GEN: the operands' general addressing (reversed time, row strides, v head broadcast) of LinArgs; without it the
+// addressing is the plain one, with compile-time row sizes.
+template <int DK, int NWH, int HG, int MODE, bool GEN = false>
 __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>())) void linear_fwd_kernel(const LinArgs a) {
   constexpr int NW = NWH * HG;
   constexpr bool ALIAS_OST = HG > 1;     // output staging block inside the wave's own (already consumed) V columns
@@ -123,14 +125,17 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
   const int b = bh0 / a.H, h0 = bh0 % a.H;        // (HG divides H, and the heads of a group share hq and hk)
   const int hq = h0 / (a.H / a.Hq), hk = h0 / (a.H / a.Hk);
   const int Tn = a.T;
-  const char* qb = (const char*)a.q + ((int64_t)(b * a.Hq + hq) * Tn) * RBQ;
-  const char* kb = (const char*)a.k + ((int64_t)(b * a.Hk + hk) * Tn) * RBQ;
-  const char* vb = (const char*)a.v + ((int64_t)bh0 * Tn * a.Dv + dvb * (32 * NWH)) * 2;
-  const int64_t v_head_bytes = (int64_t)Tn * a.Dv * 2;
+  const bool rev = GEN && a.rev != 0;
+  const int64_t q_rb = GEN ? a.q_row * 2 : (int64_t)RBQ, k_rb = GEN ? a.k_row * 2 : (int64_t)RBQ;   // bytes between an operand's rows in memory
+  const int64_t v_row_bytes = (GEN ? a.v_row : (int64_t)a.Dv) * 2;
+  const int64_t bh0_v = GEN ? (int64_t)b * a.Hv + h0 / (a.H / a.Hv) : (int64_t)bh0;
+  const char* qb = (const char*)a.q + ((int64_t)(b * a.Hq + hq) * Tn) * q_rb;
+  const char* kb = (const char*)a.k + ((int64_t)(b * a.Hk + hk) * Tn) * k_rb;
+  const char* vb = (const char*)a.v + bh0_v * Tn * v_row_bytes + (int64_t)dvb * (32 * NWH) * 2;
+  const int64_t v_head_bytes = (int64_t)Tn * v_row_bytes;
   T* ob = (T*)a.o + (int64_t)bh * Tn * a.Dv + dvb * (32 * NWH) + 32 * (wave % NWH);
   const float* ldp = a.log_decay + (int64_t)bh * Tn;
   const float* vsp = a.v_scale ? a.v_scale + (int64_t)bh * Tn : nullptr;
-  const int64_t v_row_bytes = (int64_t)a.Dv * 2;
   const int n_chunks_all = (Tn + L - 1) / L;
   const int c_begin = MODE == 0 ? 0 : seg * a.seg_chunks;
   const int c_end = MODE == 0 ? n_chunks_all : min(c_begin + a.seg_chunks, n_chunks_all);
@@ -157,9 +162,13 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
       int ln2 = lane;
       asm volatile("" : "+v"(ln2));   // rebuilt per chunk: kept live across the chunk these would cost registers
       const int lrq = ln2 / CPRQ, lrv = ln2 / CPRV;
-      const uint32_t aq = lrq * RBQ + (uint32_t)(((ln2 % CPRQ) ^ swz_tile<CPRQ>(lrq)) << 4);
+      // (reversed time: an instruction's rows lie behind each other in memory the other way round; its base is then
+      // its LAST row's address, the lowest, and the lane's row offset counts from there)
+      const uint32_t aq_c = (uint32_t)(((ln2 % CPRQ) ^ swz_tile<CPRQ>(lrq)) << 4);
+      const uint32_t aq = (uint32_t)(rev ? RQ - 1 - lrq : lrq) * (uint32_t)q_rb + aq_c;
+      const uint32_t ak = GEN ? (uint32_t)(rev ? RQ - 1 - lrq : lrq) * (uint32_t)k_rb + aq_c : aq;
       const uint32_t lc0 = (ln2 % CPRV) ^ swz_tile<CPRV>(lrv);       // logical chunk: head lc / (4 NWH), then its columns
-      uint32_t av = lrv * (uint32_t)v_row_bytes + ((lc0 % (4 * NWH)) << 4);
+      uint32_t av = (uint32_t)(rev ? RV - 1 - lrv : lrv) * (uint32_t)v_row_bytes + ((lc0 % (4 * NWH)) << 4);
       if (HG > 1) av += (lc0 / (4 * NWH)) * (uint32_t)v_head_bytes;
 #pragma unroll (DK <= 128 ? 16 : 1)   // (with a 256-wide key the state leaves no registers for an unrolled burst)
       for (int it = 0; it < (NQK + NIV + NW - 1) / NW; it++) {
@@ -167,11 +176,13 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
         if ((NQK + NIV) % NW != 0 && ii >= NQK + NIV) break;
         if (ii < NQK) {
           const int which = MODE == 1 ? 1 : ii >= NIQ, i2 = (MODE != 1 && which) ? ii - NIQ : ii;
-          const char* sb = (which ? kb : qb) + (int64_t)(t0 + i2 * RQ) * RBQ;
-          dma16_so(sb, aq ^ (uint32_t)(swz_tile<CPRQ>(i2 * RQ) << 4), base + which * QT + i2 * 1024);
+          const int64_t row0 = rev ? Tn - t0 - (i2 + 1) * RQ : t0 + i2 * RQ;
+          const char* sb = (which ? kb + row0 * k_rb : qb + row0 * q_rb);
+          dma16_so(sb, (which ? ak : aq) ^ (uint32_t)(swz_tile<CPRQ>(i2 * RQ) << 4), base + which * QT + i2 * 1024);
         } else {
           const int i2 = ii - NQK;
-          const char* sb = vb + (int64_t)(t0 + i2 * RV) * v_row_bytes;
+          const int64_t row0 = rev ? Tn - t0 - (i2 + 1) * RV : t0 + i2 * RV;
+          const char* sb = vb + row0 * v_row_bytes;
           dma16_so(sb, av ^ (uint32_t)(swz_tile<CPRV>(i2 * RV) << 4), base + 2 * QT + i2 * 1024);
         }
       }
@@ -185,13 +196,13 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
       if (ii < NQK) {
         const int which = MODE == 1 ? 1 : ii >= NIQ, i2 = (MODE != 1 && which) ? ii - NIQ : ii;
         const int row = i2 * RQ + lane / CPRQ, c = lane % CPRQ;
-        const int trow = min(t0 + row, Tn - 1);
-        const char* src = (which ? kb : qb) + (int64_t)trow * RBQ + ((c ^ swz_tile<CPRQ>(row)) << 4);
+        const int tpos = min(t0 + row, Tn - 1), trow = rev ? Tn - 1 - tpos : tpos;
+        const char* src = (which ? kb + (int64_t)trow * k_rb : qb + (int64_t)trow * q_rb) + ((c ^ swz_tile<CPRQ>(row)) << 4);
         dma16(src, base + which * QT + i2 * 1024);
       } else {
         const int i2 = ii - NQK;
         const int row = i2 * RV + lane / CPRV, c = lane % CPRV;
-        const int trow = min(t0 + row, Tn - 1);
+        const int tpos = min(t0 + row, Tn - 1), trow = rev ? Tn - 1 - tpos : tpos;
         const int lc = c ^ swz_tile<CPRV>(row);          // logical 16-byte chunk: head lc / (4 NWH), then its columns
         const char* src = vb + (int64_t)trow * v_row_bytes + ((lc % (4 * NWH)) << 4);
         if (HG > 1) src += (lc / (4 * NWH)) * v_head_bytes;
@@ -564,7 +575,8 @@ struct Config {
     // be of the same kind)
     static std::atomic<uint64_t> lds_ok{0};
     static std::atomic<int> s_resident{-1};
-    if (allow_lds(lds_ok, lds, linear_fwd_kernel<DK, NWH, HG, 0>, linear_fwd_kernel<DK, NWH, HG, 1>, linear_fwd_kernel<DK, NWH, HG, 2>) != 0)
+    if (allow_lds(lds_ok, lds, linear_fwd_kernel<DK, NWH, HG, 0>, linear_fwd_kernel<DK, NWH, HG, 1>, linear_fwd_kernel<DK, NWH, HG, 2>,
+                  linear_fwd_kernel<DK, NWH, HG, 0, true>, linear_fwd_kernel<DK, NWH, HG, 1, true>, linear_fwd_kernel<DK, NWH, HG, 2, true>) != 0)
       return false;
     cus = device_cus();
     if (cus <= 0) return false;
@@ -611,18 +623,35 @@ struct Config {
     }
     LinArgs args = a;
     args.dv_blocks = a.Dv / (32 * NWH);
+    // general operand addressing: defaults for what is left at zero; the row distances must be multiples of the tile
+    // rows (the kernel XORs the swizzle of an instruction's first row onto the finished lane offset)
+    const bool gen = a.rev != 0 || a.q_row != 0 || a.k_row != 0 || a.v_row != 0 || (a.Hv != 0 && a.Hv != a.H);
+    if (gen) {
+      if (args.q_row == 0) args.q_row = DK;
+      if (args.k_row == 0) args.k_row = DK;
+      if (args.v_row == 0) args.v_row = a.Dv;
+      if (args.Hv == 0) args.Hv = a.H;
+      if (args.q_row % DK != 0 || args.k_row % DK != 0 || args.v_row % (32 * NWH) != 0 || args.Hv <= 0 || a.H % args.Hv != 0) return -2;
+      if (HG > 1 && args.Hv != a.H) return -2;
+    }
     plan(a, want_segments, resident, cus, args.nseg, args.seg_chunks);
     if (query) { *query = ws_bytes(a, args.nseg); return 0; }
     if (args.nseg > 1 && (!ws || ws_size < ws_bytes(a, args.nseg) || ((uintptr_t)ws & 3) != 0)) args.nseg = 1;   // no workspace: single pass
     const unsigned groups = (unsigned)((int64_t)a.B * a.H / HG * args.dv_blocks);
     if (args.nseg <= 1) {
       args.nseg = 1;
-      hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 0>), dim3(groups), dim3(64 * NW), lds, stream, args);
+      if (gen) hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 0, true>), dim3(groups), dim3(64 * NW), lds, stream, args);
+      else hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 0>), dim3(groups), dim3(64 * NW), lds, stream, args);
     } else {
       args.ws_state = (float*)ws;
       args.ws_decay = args.ws_state + (int64_t)groups * (args.nseg - 1) * NW * ws_wave_floats;
-      hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 1>), dim3(groups * (args.nseg - 1)), dim3(64 * NW), lds, stream, args);
-      hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 2>), dim3(groups * args.nseg), dim3(64 * NW), lds, stream, args);
+      if (gen) {
+        hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 1, true>), dim3(groups * (args.nseg - 1)), dim3(64 * NW), lds, stream, args);
+        hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 2, true>), dim3(groups * args.nseg), dim3(64 * NW), lds, stream, args);
+      } else {
+        hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 1>), dim3(groups * (args.nseg - 1)), dim3(64 * NW), lds, stream, args);
+        hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 2>), dim3(groups * args.nseg), dim3(64 * NW), lds, stream, args);
+      }
     }
     return launch_status();
   }
@@ -634,7 +663,7 @@ struct Config {
 int linear_fwd_dispatch(const LinArgs& a, int dk, int want_segments, void* ws, size_t ws_size, hipStream_t stream, size_t* query) {
   const int dv = a.Dv;
   // two heads per workgroup when they share their q and k heads (Mamba2: all heads of a batch entry do)
-  const bool pairable = a.H % 2 == 0 && (a.H / a.Hq) % 2 == 0 && (a.H / a.Hk) % 2 == 0;
+  const bool pairable = a.H % 2 == 0 && (a.H / a.Hq) % 2 == 0 && (a.H / a.Hk) % 2 == 0 && (a.Hv == 0 || a.Hv == a.H);
   if (dk == 256) {
     if (dv % 256 == 0) return Config<256, 8, 1>::run(a, want_segments, ws, ws_size, stream, query);
     if (dv % 128 == 0) return Config<256, 4, 1>::run(a, want_segments, ws, ws_size, stream, query);
