@@ -69,9 +69,11 @@ __device__ __forceinline__ float lanes_sum(float x) {
 // LPT lanes per (batch, head, token), four columns per lane and round.  dqh [B,H,T,Dk] fp32 (time order), dkh_rev [B,H,T,Dk]
 // and du_rev [B,H,T,Dv] fp32 (reversed time order, dk before its v_scale factor).  Writes dG, dv, dv_scale and, where every
 // head has its own q / k head, dq / dk.
+// With np > 1 the scan outputs dqh and dkh_rev are np pieces (partial sums over slices of the contraction), piece_stride
+// floats apart, which are added up here.
 template <int LPT>
 __global__ __launch_bounds__(256) void grads_kernel(LinBwdArgs a, const float* __restrict__ dqh, const float* __restrict__ dkh_rev,
-                                                   const float* __restrict__ du_rev, float* __restrict__ dG) {
+                                                   const float* __restrict__ du_rev, float* __restrict__ dG, int np, int64_t piece_stride) {
   const int sub = threadIdx.x % LPT;
   const int64_t tok = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPT;
   const bool live = tok < (int64_t)a.B * a.H * a.T;   // (dead lanes take part in the shuffles with zeros)
@@ -88,8 +90,12 @@ __global__ __launch_bounds__(256) void grads_kernel(LinBwdArgs a, const float* _
   float acc = 0.f, acc_vs = 0.f;
   if (live) {
     for (int c = 4 * sub; c < a.Dk; c += 4 * LPT) {
-      const f32x4 gq = *(const f32x4*)(dqh + tk * a.Dk + c);
+      f32x4 gq = *(const f32x4*)(dqh + tk * a.Dk + c);
       f32x4 gk = *(const f32x4*)(dkh_rev + rtok * a.Dk + c);
+      for (int p = 1; p < np; p++) {
+        gq += *(const f32x4*)(dqh + p * piece_stride + tk * a.Dk + c);
+        gk += *(const f32x4*)(dkh_rev + p * piece_stride + rtok * a.Dk + c);
+      }
       const bf16x4 qv = *(const bf16x4*)(qrow + c), kv = *(const bf16x4*)(krow + c);
 #pragma unroll
       for (int i = 0; i < 4; i++) {
@@ -131,8 +137,9 @@ __global__ __launch_bounds__(256) void grads_kernel(LinBwdArgs a, const float* _
 
 // dst [B, Hg, T, D] bf16 = sum over the G = H / Hg heads of a group of src [B, H, T, D] fp32 (row T - 1 - t when rev),
 // each times scale[b, h, t] when scale is given.  One thread per 4 columns.
+// (np pieces of src, piece_stride floats apart, are added up as well)
 __global__ __launch_bounds__(256) void group_sum_kernel(__bf16* __restrict__ dst, const float* __restrict__ src, const float* __restrict__ scale,
-                                                       int H, int Hg, int T, int D, int rev, int64_t n4) {
+                                                       int H, int Hg, int T, int D, int rev, int64_t n4, int np, int64_t piece_stride) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n4) return;
   const int cpr = D / 4;
@@ -146,7 +153,8 @@ __global__ __launch_bounds__(256) void group_sum_kernel(__bf16* __restrict__ dst
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int j = 0; j < G; j++) {
     const int64_t bh = b * H + g * G + j;
-    const f32x4 x = *(const f32x4*)(src + (bh * T + ts) * (int64_t)D + c);
+    f32x4 x = *(const f32x4*)(src + (bh * T + ts) * (int64_t)D + c);
+    for (int p = 1; p < np; p++) x += *(const f32x4*)(src + p * piece_stride + (bh * T + ts) * (int64_t)D + c);
     const float s = scale ? scale[bh * T + t] : 1.f;
 #pragma unroll
     for (int k = 0; k < 4; k++) acc[k] += x[k] * s;
@@ -202,7 +210,11 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   // workspace: fp32 scan outputs, dG, reversed log decay, packed operands, the scan kernel's own workspace
   size_t off = 0;
   auto take = [&](size_t bytes) { const size_t o = off; off += align256(bytes); return o; };
-  const size_t o_dqh = take((size_t)BHT * a.Dk * 4), o_dkh = take((size_t)BHT * a.Dk * 4), o_du = take((size_t)BHT * a.Dv * 4);
+  // (a contraction of equal pieces that are all read in place runs its pieces side by side, each with an output of its own)
+  const bool side_by_side = sl.n > 1 && a.Dv % sl.w[0] == 0 && sl.w[sl.n - 1] == sl.w[0];
+  const int np = side_by_side ? sl.n : 1;
+  const int64_t piece_stride = BHT * a.Dk;
+  const size_t o_dqh = take((size_t)np * BHT * a.Dk * 4), o_dkh = take((size_t)np * BHT * a.Dk * 4), o_du = take((size_t)BHT * a.Dv * 4);
   const size_t o_dG = take((size_t)BHT * 4), o_grev = take((size_t)BHT * 4);
   const size_t o_pa = take((size_t)BHT * 256 * 2), o_pb = take((size_t)BHT * 256 * 2);   // q and k operands of a scan
   const size_t o_pv = take((size_t)BHT * (a.Dk > a.Dv ? a.Dk : a.Dv) * 2);                // v operand of a scan
@@ -234,12 +246,13 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   // column offset)
   struct Operand { const void* p; int heads; int64_t row; };
   auto scan_launch = [&](Operand q, Operand k, Operand v, bool reversed, int dk, int dv, const float* g, const float* vs, float* out,
-                         bool accumulate) -> int {
+                         bool accumulate, int pieces = 1) -> int {
     LinArgs la{};
     la.q = q.p; la.k = k.p; la.v = v.p; la.o = out; la.log_decay = g; la.v_scale = vs; la.q_scale = a.q_scale;
     la.B = a.B; la.H = a.H; la.Hq = q.heads; la.Hk = k.heads; la.Hv = v.heads; la.T = a.T; la.Dv = dv;
     la.q_row = q.row; la.k_row = k.row; la.v_row = v.row; la.rev = reversed ? 1 : 0;
     la.out_f32 = accumulate ? 2 : 1;
+    if (pieces > 1) { la.n_pieces = pieces; la.piece_qk = dk; la.piece_o = piece_stride; }
     return linear_fwd_dispatch(la, dk, 0, scan, scan_ws, stream, nullptr);
   };
   const __bf16 *q_p = (const __bf16*)a.q, *k_p = (const __bf16*)a.k, *v_p = (const __bf16*)a.v, *do_p = (const __bf16*)a.dout;
@@ -250,7 +263,12 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   hipLaunchKernelGGL(shift_rev_kernel, dim3((unsigned)((BHT + 255) / 256)), dim3(256), 0, stream, grev, a.log_decay, a.T, BHT);
 
   // dq (per head) = LA(do, v, k; v_scale), contraction over the value columns; k is read with its own heads
-  for (int s = 0; s < sl.n; s++) {
+  if (side_by_side) {
+    if (const int rc = scan_launch(Operand{do_p, a.H, a.Dv}, Operand{v_p, a.H, a.Dv}, Operand{k_p, a.Hk, a.Dk}, false, sl.w[0], a.Dk, a.log_decay, a.v_scale,
+                                   dqh, false, np))
+      return rc;
+  }
+  for (int s = 0; s < sl.n && !side_by_side; s++) {
     Operand qs{do_p + sl.c0[s], a.H, a.Dv}, ks{v_p + sl.c0[s], a.H, a.Dv};
     if (!in_place(s)) {
       pack(pa, a.dout, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], false);
@@ -266,7 +284,11 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
     return rc;
 
   // dk (per head, reversed, before its v_scale factor) = LA(R v, R do, R q), contraction over the value columns
-  for (int s = 0; s < sl.n; s++) {
+  if (side_by_side) {
+    if (const int rc = scan_launch(Operand{v_p, a.H, a.Dv}, Operand{do_p, a.H, a.Dv}, Operand{q_p, a.Hq, a.Dk}, true, sl.w[0], a.Dk, grev, nullptr, dkh, false, np))
+      return rc;
+  }
+  for (int s = 0; s < sl.n && !side_by_side; s++) {
     Operand qs{v_p + sl.c0[s], a.H, a.Dv}, ks{do_p + sl.c0[s], a.H, a.Dv};
     bool reversed = true;
     if (!in_place(s)) {   // (packed in reversed order)
@@ -282,18 +304,20 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   }
 
   if ((a.Dk > a.Dv ? a.Dk : a.Dv) >= 256)
-    hipLaunchKernelGGL(grads_kernel<64>, dim3((unsigned)((BHT + 3) / 4)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh, (const float*)du, dG);
+    hipLaunchKernelGGL(grads_kernel<64>, dim3((unsigned)((BHT + 3) / 4)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh, (const float*)du, dG,
+                       np, piece_stride);
   else
-    hipLaunchKernelGGL(grads_kernel<32>, dim3((unsigned)((BHT + 7) / 8)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh, (const float*)du, dG);
+    hipLaunchKernelGGL(grads_kernel<32>, dim3((unsigned)((BHT + 7) / 8)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh, (const float*)du, dG,
+                       np, piece_stride);
   if (a.Hq != a.H) {
     const int64_t n4 = (int64_t)a.B * a.Hq * a.T * (a.Dk / 4);
     hipLaunchKernelGGL(group_sum_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (__bf16*)a.dq, (const float*)dqh, (const float*)nullptr,
-                       a.H, a.Hq, a.T, a.Dk, 0, n4);
+                       a.H, a.Hq, a.T, a.Dk, 0, n4, np, piece_stride);
   }
   if (a.Hk != a.H) {
     const int64_t n4 = (int64_t)a.B * a.Hk * a.T * (a.Dk / 4);
     hipLaunchKernelGGL(group_sum_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (__bf16*)a.dk, (const float*)dkh, a.v_scale, a.H, a.Hk,
-                       a.T, a.Dk, 1, n4);
+                       a.T, a.Dk, 1, n4, np, piece_stride);
   }
   hipLaunchKernelGGL(suffix_sum_kernel, dim3((unsigned)(a.B * a.H)), dim3(64), 0, stream, a.dlog_decay, (const float*)dG, a.T);
   return launch_status();

@@ -129,8 +129,9 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
   const int64_t q_rb = GEN ? a.q_row * 2 : (int64_t)RBQ, k_rb = GEN ? a.k_row * 2 : (int64_t)RBQ;   // bytes between an operand's rows in memory
   const int64_t v_row_bytes = (GEN ? a.v_row : (int64_t)a.Dv) * 2;
   const int64_t bh0_v = GEN ? (int64_t)b * a.Hv + h0 / (a.H / a.Hv) : (int64_t)bh0;
-  const char* qb = (const char*)a.q + ((int64_t)(b * a.Hq + hq) * Tn) * q_rb;
-  const char* kb = (const char*)a.k + ((int64_t)(b * a.Hk + hk) * Tn) * k_rb;
+  const int64_t piece = GEN ? (int64_t)blockIdx.y : 0;   // (pieces of a contraction side by side: see LinArgs)
+  const char* qb = (const char*)a.q + ((int64_t)(b * a.Hq + hq) * Tn) * q_rb + piece * a.piece_qk * 2;
+  const char* kb = (const char*)a.k + ((int64_t)(b * a.Hk + hk) * Tn) * k_rb + piece * a.piece_qk * 2;
   const char* vb = (const char*)a.v + bh0_v * Tn * v_row_bytes + (int64_t)dvb * (32 * NWH) * 2;
   const int64_t v_head_bytes = (int64_t)Tn * v_row_bytes;
   T* ob = (T*)a.o + (int64_t)bh * Tn * a.Dv + dvb * (32 * NWH) + 32 * (wave % NWH);
@@ -503,7 +504,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
       // fp32 outputs (used by the backward pass, whose decay gradient is a difference of sums over these
       // values): the same staging block, 16 columns at a time
       const int sw_r = swz_tile<CPRV>(r);
-      float* ob32 = (float*)a.o + (int64_t)bh * Tn * a.Dv + dvb * (32 * NWH) + 32 * (wave % NWH);
+      float* ob32 = (float*)a.o + piece * a.piece_o + (int64_t)bh * Tn * a.Dv + dvb * (32 * NWH) + 32 * (wave % NWH);
 #pragma unroll
       for (int half = 0; half < 2; half++) {
 #pragma unroll
@@ -595,6 +596,7 @@ struct Config {
   static void plan(const LinArgs& a, int want, int resident, int cus, int& nseg, int& seg_chunks) {
     const int n_chunks = (a.T + L - 1) / L;
     const int64_t groups = (int64_t)a.B * a.H / HG * (a.Dv / (32 * NWH));
+    if (a.n_pieces > 1) want = 1;   // (pieces side by side run the single pass)
     int n;
     if (want >= 1) n = want;
     else {
@@ -633,14 +635,18 @@ struct Config {
       if (args.Hv == 0) args.Hv = a.H;
       if (args.q_row % DK != 0 || args.k_row % DK != 0 || args.v_row % (32 * NWH) != 0 || args.Hv <= 0 || a.H % args.Hv != 0) return -2;
       if (HG > 1 && args.Hv != a.H) return -2;
+      if (a.n_pieces > 1 && !a.out_f32) return -2;
+    } else if (a.n_pieces > 1) {
+      return -2;
     }
+    const unsigned pieces = a.n_pieces > 1 ? (unsigned)a.n_pieces : 1u;
     plan(a, want_segments, resident, cus, args.nseg, args.seg_chunks);
     if (query) { *query = ws_bytes(a, args.nseg); return 0; }
     if (args.nseg > 1 && (!ws || ws_size < ws_bytes(a, args.nseg) || ((uintptr_t)ws & 3) != 0)) args.nseg = 1;   // no workspace: single pass
     const unsigned groups = (unsigned)((int64_t)a.B * a.H / HG * args.dv_blocks);
     if (args.nseg <= 1) {
       args.nseg = 1;
-      if (gen) hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 0, true>), dim3(groups), dim3(64 * NW), lds, stream, args);
+      if (gen) hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 0, true>), dim3(groups, pieces), dim3(64 * NW), lds, stream, args);
       else hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 0>), dim3(groups), dim3(64 * NW), lds, stream, args);
     } else {
       args.ws_state = (float*)ws;
