@@ -216,7 +216,7 @@ def bench_retnet_chunked(steps, warmup, backward=False):
         ws = torch.empty(_linear_bwd_workspace(hb, B, H, H, H, T, Dk, Dv), dtype=torch.uint8, device="cuda")
         ms = time_gpu(lambda: hb.linear_bwd(q, k, v, ld, do, q_scale=Dk ** -0.5, workspace=ws), max(steps // 3, 3), 2)
         return _mfma_entry(ms, 2.5 * flops, "backward (dq, dk, dv, dlog_decay), 2.5 x the forward's algorithmic FLOPs; five scans of the "
-                                            "forward kernel (the two 512-wide contractions in two pieces) + packing + epilogue")
+                                            "forward kernel on operands read in place (the two 512-wide contractions as two pieces side by side) + epilogue")
     o = torch.empty_like(v)
     ws = torch.empty(max(hb.linear_workspace_bytes(B, H, H, H, T, Dk, Dv), 16), dtype=torch.uint8, device="cuda")
     ms = time_gpu(lambda: hb.linear_fwd(q, k, v, ld, q_scale=Dk ** -0.5, out=o, workspace=ws), steps, warmup)
@@ -282,7 +282,7 @@ def bench_mamba2(steps, warmup, backward=False):
         ws = torch.empty(_linear_bwd_workspace(hb, B, H, 1, 1, T, N, P), dtype=torch.uint8, device="cuda")
         ms = time_gpu(lambda: hb.linear_bwd(Cm, Bm, x, ld, do, v_scale=dt, workspace=ws), max(steps // 3, 3), 2)
         return _mfma_entry(ms, 2.5 * flops, "backward (dC, dB, dx, dlog_decay, ddt-scale), 2.5 x the forward's algorithmic FLOPs; three scans "
-                                            "of the forward kernel + packing + epilogue")
+                                            "of the forward kernel on operands read in place + epilogue")
     o = torch.empty_like(x)
     ws = torch.empty(max(hb.linear_workspace_bytes(B, H, 1, 1, T, N, P), 16), dtype=torch.uint8, device="cuda")
     ms = time_gpu(lambda: hb.linear_fwd(Cm, Bm, x, ld, v_scale=dt, out=o, workspace=ws), steps, warmup)

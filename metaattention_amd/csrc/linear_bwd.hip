@@ -14,8 +14,8 @@
 //   dq = LA(do, v, k; v_scale)      du = R LA(R k, R q, R do)      dk = v_scale * R LA(R v, R do, R q)      (R reverses time)
 // so the backward pass is three scans of the forward kernel (linear_fwd.hip: state in accumulator registers, fp32
 // outputs), each contraction cut into the 128 / 256 wide pieces that kernel takes (their fp32 outputs add up); the scans
-// read their operands in place (reversed time, column slices and shared heads are the scan kernel's general operand
-// addressing), except a piece that needs zero padding, which pack_kernel copies.  Plus the small kernels of this file:
+// read their operands in place (reversed time, column slices, shared heads and the zero padding of a narrow piece are
+// the scan kernel's general operand addressing).  Plus the small kernels of this file:
 // the shifted reversed log decay, and the epilogue that forms dv, dv_scale, the per-token decay gradient
 //   dG_t = q_t . dq_t - k_t . dk_t        (fp32 products of the fp32 scan outputs)
 // sums the heads that share a q / k head (:1300-1303), converts, and turns dG into dlog_decay by a reversed running sum
@@ -27,28 +27,6 @@
 namespace ma {
 
 namespace {
-
-// dst [B, Hd, T, W] bf16 <- src [B, Hs, T, Ws] columns c0 .. c0 + W (zeros beyond Ws), head hd reads source head
-// hd / (Hd / Hs), row t reads row T - 1 - t when rev.  One thread per 16 bytes of dst.
-__global__ __launch_bounds__(256) void pack_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, int Hd, int Hs, int T, int W, int Ws,
-                                                  int c0, int rev, int64_t n_chunks) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n_chunks) return;
-  const int cpr = W / 8;
-  const int c = (int)(i % cpr);
-  const int64_t row = i / cpr;
-  const int t = (int)(row % T);
-  const int64_t bh = row / T;
-  const int hd = (int)(bh % Hd);
-  const int64_t b = bh / Hd;
-  const int col = c0 + 8 * c;
-  uint4 val = {0u, 0u, 0u, 0u};
-  if (col < Ws) {
-    const int ts = rev ? T - 1 - t : t;
-    val = src[(((b * Hs + hd / (Hd / Hs)) * T + ts) * (int64_t)Ws + col) / 8];
-  }
-  dst[i] = val;
-}
 
 // g_rev[b, h, t'] = log_decay[b, h, T - t'] for t' >= 1, 0 for t' = 0: the decay between reversed tokens t' - 1 and t'
 __global__ __launch_bounds__(256) void shift_rev_kernel(float* __restrict__ dst, const float* __restrict__ src, int T, int64_t n) {
@@ -216,8 +194,6 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   const int64_t piece_stride = BHT * a.Dk;
   const size_t o_dqh = take((size_t)np * BHT * a.Dk * 4), o_dkh = take((size_t)np * BHT * a.Dk * 4), o_du = take((size_t)BHT * a.Dv * 4);
   const size_t o_dG = take((size_t)BHT * 4), o_grev = take((size_t)BHT * 4);
-  const size_t o_pa = take((size_t)BHT * 256 * 2), o_pb = take((size_t)BHT * 256 * 2);   // q and k operands of a scan
-  const size_t o_pv = take((size_t)BHT * (a.Dk > a.Dv ? a.Dk : a.Dv) * 2);                // v operand of a scan
   // the scan kernel's workspace (sequence segments): the largest any of the scans asks for
   size_t scan_ws = 0;
   {
@@ -235,30 +211,24 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   if (!ws || ws_bytes < off || ((uintptr_t)ws & 255) != 0) return -3;
   char* base = (char*)ws;
   float *dqh = (float*)(base + o_dqh), *dkh = (float*)(base + o_dkh), *du = (float*)(base + o_du), *dG = (float*)(base + o_dG), *grev = (float*)(base + o_grev);
-  void *pa = base + o_pa, *pb = base + o_pb, *pv = base + o_pv, *scan = scan_ws ? base + o_scan : nullptr;
-
-  auto pack = [&](void* dst, const void* src, int Hd, int Hs, int W, int Ws, int c0, bool rev) {
-    const int64_t n = (int64_t)a.B * Hd * a.T * (W / 8);
-    hipLaunchKernelGGL(pack_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, (uint4*)dst, (const uint4*)src, Hd, Hs, a.T, W, Ws, c0,
-                       rev ? 1 : 0, n);
-  };
+  void* scan = scan_ws ? base + o_scan : nullptr;
   // an operand of a scan as the scan kernel reads it in place: heads, elements between its tokens (the pointer carries a
   // column offset)
   struct Operand { const void* p; int heads; int64_t row; };
   auto scan_launch = [&](Operand q, Operand k, Operand v, bool reversed, int dk, int dv, const float* g, const float* vs, float* out,
-                         bool accumulate, int pieces = 1) -> int {
+                         bool accumulate, int pieces = 1, int qk_cols = 0) -> int {
     LinArgs la{};
     la.q = q.p; la.k = k.p; la.v = v.p; la.o = out; la.log_decay = g; la.v_scale = vs; la.q_scale = a.q_scale;
     la.B = a.B; la.H = a.H; la.Hq = q.heads; la.Hk = k.heads; la.Hv = v.heads; la.T = a.T; la.Dv = dv;
     la.q_row = q.row; la.k_row = k.row; la.v_row = v.row; la.rev = reversed ? 1 : 0;
     la.out_f32 = accumulate ? 2 : 1;
     if (pieces > 1) { la.n_pieces = pieces; la.piece_qk = dk; la.piece_o = piece_stride; }
+    la.qk_cols = qk_cols;
     return linear_fwd_dispatch(la, dk, 0, scan, scan_ws, stream, nullptr);
   };
   const __bf16 *q_p = (const __bf16*)a.q, *k_p = (const __bf16*)a.k, *v_p = (const __bf16*)a.v, *do_p = (const __bf16*)a.dout;
-  // a piece of the value columns is read in place when it lies inside them whole and the row is a multiple of its width
-  // (the scan kernel's condition); else it is packed (zero padded)
-  auto in_place = [&](int s) { return sl.c0[s] + sl.w[s] <= a.Dv && a.Dv % sl.w[s] == 0; };
+  // the columns of piece s that exist (a last piece may reach beyond the value columns: the scan kernel pads with zeros)
+  auto piece_cols = [&](int s) { return sl.c0[s] + sl.w[s] <= a.Dv ? 0 : a.Dv - sl.c0[s]; };
 
   hipLaunchKernelGGL(shift_rev_kernel, dim3((unsigned)((BHT + 255) / 256)), dim3(256), 0, stream, grev, a.log_decay, a.T, BHT);
 
@@ -270,13 +240,7 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   }
   for (int s = 0; s < sl.n && !side_by_side; s++) {
     Operand qs{do_p + sl.c0[s], a.H, a.Dv}, ks{v_p + sl.c0[s], a.H, a.Dv};
-    if (!in_place(s)) {
-      pack(pa, a.dout, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], false);
-      pack(pb, a.v, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], false);
-      qs = Operand{pa, a.H, sl.w[s]};
-      ks = Operand{pb, a.H, sl.w[s]};
-    }
-    if (const int rc = scan_launch(qs, ks, Operand{k_p, a.Hk, a.Dk}, false, sl.w[s], a.Dk, a.log_decay, a.v_scale, dqh, s > 0)) return rc;
+    if (const int rc = scan_launch(qs, ks, Operand{k_p, a.Hk, a.Dk}, false, sl.w[s], a.Dk, a.log_decay, a.v_scale, dqh, s > 0, 1, piece_cols(s))) return rc;
   }
 
   // du (reversed) = LA(R k, R q, R do), contraction over the key columns: the operands are read in reversed time in place
@@ -290,17 +254,7 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   }
   for (int s = 0; s < sl.n && !side_by_side; s++) {
     Operand qs{v_p + sl.c0[s], a.H, a.Dv}, ks{do_p + sl.c0[s], a.H, a.Dv};
-    bool reversed = true;
-    if (!in_place(s)) {   // (packed in reversed order)
-      pack(pa, a.v, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], true);
-      pack(pb, a.dout, a.H, a.H, sl.w[s], a.Dv, sl.c0[s], true);
-      qs = Operand{pa, a.H, sl.w[s]};
-      ks = Operand{pb, a.H, sl.w[s]};
-      pack(pv, a.q, a.H, a.Hq, a.Dk, a.Dk, 0, true);
-      if (const int rc = scan_launch(qs, ks, Operand{pv, a.H, a.Dk}, false, sl.w[s], a.Dk, grev, nullptr, dkh, s > 0)) return rc;
-      continue;
-    }
-    if (const int rc = scan_launch(qs, ks, Operand{q_p, a.Hq, a.Dk}, reversed, sl.w[s], a.Dk, grev, nullptr, dkh, s > 0)) return rc;
+    if (const int rc = scan_launch(qs, ks, Operand{q_p, a.Hq, a.Dk}, true, sl.w[s], a.Dk, grev, nullptr, dkh, s > 0, 1, piece_cols(s))) return rc;
   }
 
   if ((a.Dk > a.Dv ? a.Dk : a.Dv) >= 256)

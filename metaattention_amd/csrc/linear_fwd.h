@@ -20,6 +20,10 @@ struct LinArgs {
   // Hv = heads of v (dividing H: head h reads v head h / (H / Hv)).
   int rev, Hv;
   int64_t q_row, k_row, v_row;
+  // qk_cols (general addressing only; 0: all Dk): the q and k operands hold only this many columns (a multiple of 8); the
+  // rest of the Dk-wide contraction is zeros that are never loaded (the tiles' LDS is cleared once, the loads of the missing
+  // columns are switched off).
+  int qk_cols;
   // pieces (general addressing only; 0 or 1: none): the launch runs n_pieces independent scans side by side, piece p with
   // its q and k pointers moved on by p * piece_qk elements (the next slice of the contraction's columns) and its output
   // (fp32) by p * piece_o elements; the caller adds the pieces' outputs up.  Single pass only (no sequence segments).

@@ -150,6 +150,15 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
   //      the 16-byte chunk that belongs at physical position i of that KB.
   //      (Spreading a chunk's instructions over the chunk's phases instead of issuing them together behind the
   //      barrier was measured: no gain at the RetNet shape, 5 % slower at the Mamba2 shape.)
+  const uint32_t qk_chunks = GEN && a.qk_cols > 0 ? (uint32_t)a.qk_cols / 8 : (uint32_t)CPRQ;   // 16-byte chunks of a q / k row that exist
+  if (GEN && qk_chunks < (uint32_t)CPRQ) {
+    // the Q and K tiles of both stages start as zeros: the missing columns are never written
+    for (uint32_t off = (uint32_t)tid * 16; off < (uint32_t)(2 * QT); off += 64 * NW * 16) {
+      lds_write<u32x4>(lds0 + off, u32x4{0u, 0u, 0u, 0u});
+      lds_write<u32x4>(lds0 + STAGE + off, u32x4{0u, 0u, 0u, 0u});
+    }
+    __syncthreads();
+  }
   auto issue_chunk = [&](int t0, int buf) {
     const uint32_t base = lds0 + buf * STAGE;
     constexpr int NQK = MODE == 1 ? NIQ : 2 * NIQ;      // (the state-only pass needs no Q)
@@ -165,9 +174,12 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
       const int lrq = ln2 / CPRQ, lrv = ln2 / CPRV;
       // (reversed time: an instruction's rows lie behind each other in memory the other way round; its base is then
       // its LAST row's address, the lowest, and the lane's row offset counts from there)
-      const uint32_t aq_c = (uint32_t)(((ln2 % CPRQ) ^ swz_tile<CPRQ>(lrq)) << 4);
-      const uint32_t aq = (uint32_t)(rev ? RQ - 1 - lrq : lrq) * (uint32_t)q_rb + aq_c;
-      const uint32_t ak = GEN ? (uint32_t)(rev ? RQ - 1 - lrq : lrq) * (uint32_t)k_rb + aq_c : aq;
+      // With the general addressing a row distance need not be a multiple of the tile's row size, so the instruction's
+      // part of the swizzle goes onto the chunk index before the row offset is added; chunks beyond the operand's columns
+      // are not loaded (their LDS stays zero).
+      const uint32_t cq = (uint32_t)((ln2 % CPRQ) ^ swz_tile<CPRQ>(lrq));
+      const uint32_t aq = (uint32_t)(rev ? RQ - 1 - lrq : lrq) * (uint32_t)q_rb + (GEN ? 0u : cq << 4);
+      const uint32_t ak = GEN ? (uint32_t)(rev ? RQ - 1 - lrq : lrq) * (uint32_t)k_rb : aq;
       const uint32_t lc0 = (ln2 % CPRV) ^ swz_tile<CPRV>(lrv);       // logical chunk: head lc / (4 NWH), then its columns
       uint32_t av = (uint32_t)(rev ? RV - 1 - lrv : lrv) * (uint32_t)v_row_bytes + ((lc0 % (4 * NWH)) << 4);
       if (HG > 1) av += (lc0 / (4 * NWH)) * (uint32_t)v_head_bytes;
@@ -179,7 +191,12 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
           const int which = MODE == 1 ? 1 : ii >= NIQ, i2 = (MODE != 1 && which) ? ii - NIQ : ii;
           const int64_t row0 = rev ? Tn - t0 - (i2 + 1) * RQ : t0 + i2 * RQ;
           const char* sb = (which ? kb + row0 * k_rb : qb + row0 * q_rb);
-          dma16_so(sb, (which ? ak : aq) ^ (uint32_t)(swz_tile<CPRQ>(i2 * RQ) << 4), base + which * QT + i2 * 1024);
+          if constexpr (GEN) {
+            const uint32_t lc = cq ^ (uint32_t)swz_tile<CPRQ>(i2 * RQ);
+            if (lc < qk_chunks) dma16_so(sb, (which ? ak : aq) + (lc << 4), base + which * QT + i2 * 1024);
+          } else {
+            dma16_so(sb, aq ^ (uint32_t)(swz_tile<CPRQ>(i2 * RQ) << 4), base + which * QT + i2 * 1024);
+          }
         } else {
           const int i2 = ii - NQK;
           const int64_t row0 = rev ? Tn - t0 - (i2 + 1) * RV : t0 + i2 * RV;
@@ -198,8 +215,9 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
         const int which = MODE == 1 ? 1 : ii >= NIQ, i2 = (MODE != 1 && which) ? ii - NIQ : ii;
         const int row = i2 * RQ + lane / CPRQ, c = lane % CPRQ;
         const int tpos = min(t0 + row, Tn - 1), trow = rev ? Tn - 1 - tpos : tpos;
-        const char* src = (which ? kb + (int64_t)trow * k_rb : qb + (int64_t)trow * q_rb) + ((c ^ swz_tile<CPRQ>(row)) << 4);
-        dma16(src, base + which * QT + i2 * 1024);
+        const uint32_t lc = (uint32_t)(c ^ swz_tile<CPRQ>(row));
+        const char* src = (which ? kb + (int64_t)trow * k_rb : qb + (int64_t)trow * q_rb) + (lc << 4);
+        if (!GEN || lc < qk_chunks) dma16(src, base + which * QT + i2 * 1024);
       } else {
         const int i2 = ii - NQK;
         const int row = i2 * RV + lane / CPRV, c = lane % CPRV;
@@ -627,13 +645,14 @@ struct Config {
     args.dv_blocks = a.Dv / (32 * NWH);
     // general operand addressing: defaults for what is left at zero; the row distances must be multiples of the tile
     // rows (the kernel XORs the swizzle of an instruction's first row onto the finished lane offset)
-    const bool gen = a.rev != 0 || a.q_row != 0 || a.k_row != 0 || a.v_row != 0 || (a.Hv != 0 && a.Hv != a.H);
+    const bool gen = a.rev != 0 || a.q_row != 0 || a.k_row != 0 || a.v_row != 0 || (a.Hv != 0 && a.Hv != a.H) || a.qk_cols != 0 || a.n_pieces > 1;
     if (gen) {
       if (args.q_row == 0) args.q_row = DK;
       if (args.k_row == 0) args.k_row = DK;
       if (args.v_row == 0) args.v_row = a.Dv;
       if (args.Hv == 0) args.Hv = a.H;
-      if (args.q_row % DK != 0 || args.k_row % DK != 0 || args.v_row % (32 * NWH) != 0 || args.Hv <= 0 || a.H % args.Hv != 0) return -2;
+      if (args.q_row % 8 != 0 || args.k_row % 8 != 0 || args.v_row % (32 * NWH) != 0 || args.Hv <= 0 || a.H % args.Hv != 0) return -2;
+      if (a.qk_cols < 0 || a.qk_cols > DK || a.qk_cols % 8 != 0) return -2;
       if (HG > 1 && args.Hv != a.H) return -2;
       if (a.n_pieces > 1 && !a.out_f32) return -2;
     } else if (a.n_pieces > 1) {
