@@ -44,7 +44,9 @@ def _check(got, ref, what):
     (1, 2, 2, 200, 256, 512, False),    # RetNet head sizes: the dq / dk launches contract over 512 = 2 x 256
     (2, 1, 4, 256, 128, 64, True),      # Mamba2: one q/k head for all heads, value scale, 64-wide contraction padded
     (1, 2, 4, 100, 128, 128, True),
-    (1, 1, 2, 96, 128, 384, True),      # pieces of unequal width (256 + 128): one after the other, the first one copied
+    (1, 1, 2, 96, 128, 384, True),      # pieces of unequal width (256 + 128), one after the other
+    (1, 1, 2, 77, 128, 64, True),       # a partial last chunk with the narrow (zero-padded) contraction
+    (1, 2, 2, 50, 256, 192, False),     # 192 value columns as one 256-wide piece
     (1, 2, 2, 130, 256, 768, False),    # three equal pieces side by side in one launch
     (1, 1, 1, 1, 128, 64, False),
 ])
