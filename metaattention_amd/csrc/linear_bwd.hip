@@ -113,6 +113,76 @@ __global__ __launch_bounds__(256) void grads_kernel(LinBwdArgs a, const float* _
   }
 }
 
+// The same for heads that share their q and k heads in groups of G = H / Hq (Hq == Hk < H): LPT lanes per (batch, shared
+// head, token) walk the G heads of the group, so that dq and dk of the shared head -- the sums over the group
+// (linear_tl.py:1300-1303) -- are formed while the per-head scan outputs pass through once.
+template <int LPT>
+__global__ __launch_bounds__(256) void grads_shared_kernel(LinBwdArgs a, const float* __restrict__ dqh, const float* __restrict__ dkh_rev,
+                                                          const float* __restrict__ du_rev, float* __restrict__ dG, int np, int64_t piece_stride) {
+  const int sub = threadIdx.x % LPT;
+  const int64_t tok = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPT;
+  const bool live = tok < (int64_t)a.B * a.Hq * a.T;   // (dead lanes take part in the shuffles with zeros)
+  const int64_t tg = live ? tok : 0;
+  const int t = (int)(tg % a.T);
+  const int64_t bg = tg / a.T;
+  const int g = (int)(bg % a.Hq), G = a.H / a.Hq;
+  const int64_t b = bg / a.Hq;
+  const int c = 4 * sub;                               // (4 LPT >= Dk: one group of four key columns per lane)
+  const bool has_c = live && c < a.Dk;
+  f32x4 qv = {0.f, 0.f, 0.f, 0.f}, kv = {0.f, 0.f, 0.f, 0.f}, sq = {0.f, 0.f, 0.f, 0.f}, sk = {0.f, 0.f, 0.f, 0.f};
+  if (has_c) {
+    const bf16x4 q4 = *(const bf16x4*)((const __bf16*)a.q + tg * a.Dk + c), k4 = *(const bf16x4*)((const __bf16*)a.k + tg * a.Dk + c);
+#pragma unroll
+    for (int i = 0; i < 4; i++) { qv[i] = (float)q4[i]; kv[i] = (float)k4[i]; }
+  }
+  for (int j = 0; j < G; j++) {
+    const int64_t bh = b * a.H + (int64_t)g * G + j, tk = bh * a.T + t, rtok = bh * a.T + (a.T - 1 - t);
+    const float vs = a.v_scale ? a.v_scale[tk] : 1.f;
+    float acc = 0.f, acc_vs = 0.f;
+    if (has_c) {
+      f32x4 gq = *(const f32x4*)(dqh + tk * a.Dk + c);
+      f32x4 gk = *(const f32x4*)(dkh_rev + rtok * a.Dk + c);
+      for (int p = 1; p < np; p++) {
+        gq += *(const f32x4*)(dqh + p * piece_stride + tk * a.Dk + c);
+        gk += *(const f32x4*)(dkh_rev + p * piece_stride + rtok * a.Dk + c);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        gk[i] *= vs;
+        acc += qv[i] * gq[i] - kv[i] * gk[i];
+        sq[i] += gq[i];
+        sk[i] += gk[i];
+      }
+    }
+    if (live) {
+      for (int cv = 4 * sub; cv < a.Dv; cv += 4 * LPT) {
+        const f32x4 gu = *(const f32x4*)(du_rev + rtok * a.Dv + cv);
+        const bf16x4 vv = *(const bf16x4*)((const __bf16*)a.v + tk * a.Dv + cv);
+        bf16x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          acc_vs += (float)vv[i] * gu[i];
+          w[i] = (__bf16)(gu[i] * vs);
+        }
+        *(bf16x4*)((__bf16*)a.dv + tk * a.Dv + cv) = w;
+      }
+    }
+    acc = lanes_sum<LPT>(acc);
+    acc_vs = lanes_sum<LPT>(acc_vs);
+    if (live && sub == 0) {
+      dG[tk] = acc;
+      if (a.dv_scale) a.dv_scale[tk] = acc_vs;
+    }
+  }
+  if (has_c) {
+    bf16x4 wq, wk;
+#pragma unroll
+    for (int i = 0; i < 4; i++) { wq[i] = (__bf16)sq[i]; wk[i] = (__bf16)sk[i]; }
+    *(bf16x4*)((__bf16*)a.dq + tg * a.Dk + c) = wq;
+    *(bf16x4*)((__bf16*)a.dk + tg * a.Dk + c) = wk;
+  }
+}
+
 // dst [B, Hg, T, D] bf16 = sum over the G = H / Hg heads of a group of src [B, H, T, D] fp32 (row T - 1 - t when rev),
 // each times scale[b, h, t] when scale is given.  One thread per 4 columns.
 // (np pieces of src, piece_stride floats apart, are added up as well)
@@ -257,6 +327,18 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
     if (const int rc = scan_launch(qs, ks, Operand{q_p, a.Hq, a.Dk}, true, sl.w[s], a.Dk, grev, nullptr, dkh, s > 0, 1, piece_cols(s))) return rc;
   }
 
+  if (a.Hq == a.Hk && a.Hq != a.H) {
+    // heads in groups that share q and k: gradients, group sums and conversions in one pass over the scan outputs
+    const int64_t n_tok = (int64_t)a.B * a.Hq * a.T;
+    if (a.Dk > 128)
+      hipLaunchKernelGGL(grads_shared_kernel<64>, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh,
+                         (const float*)du, dG, np, piece_stride);
+    else
+      hipLaunchKernelGGL(grads_shared_kernel<32>, dim3((unsigned)((n_tok + 7) / 8)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh,
+                         (const float*)du, dG, np, piece_stride);
+    hipLaunchKernelGGL(suffix_sum_kernel, dim3((unsigned)(a.B * a.H)), dim3(64), 0, stream, a.dlog_decay, (const float*)dG, a.T);
+    return launch_status();
+  }
   if ((a.Dk > a.Dv ? a.Dk : a.Dv) >= 256)
     hipLaunchKernelGGL(grads_kernel<64>, dim3((unsigned)((BHT + 3) / 4)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh, (const float*)du, dG,
                        np, piece_stride);
