@@ -151,6 +151,8 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
   //      (Spreading a chunk's instructions over the chunk's phases instead of issuing them together behind the
   //      barrier was measured: no gain at the RetNet shape, 5 % slower at the Mamba2 shape.)
   const uint32_t qk_chunks = GEN && a.qk_cols > 0 ? (uint32_t)a.qk_cols / 8 : (uint32_t)CPRQ;   // 16-byte chunks of a q / k row that exist
+  // (columns beyond the operand's are zeros: the 16- and 32-wide slices of the contraction that hold nothing else are skipped)
+  const int qk_used = GEN && a.qk_cols > 0 ? a.qk_cols : DK;
   if (GEN && qk_chunks < (uint32_t)CPRQ) {
     // the Q and K tiles of both stages start as zeros: the missing columns are never written
     for (uint32_t off = (uint32_t)tid * 16; off < (uint32_t)(2 * QT); off += 64 * NW * 16) {
@@ -296,8 +298,10 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
         const uint32_t ka = kbase + (16 * (slot >> 1) + rr) * RBQ + c0, qa = qbase + (16 * (slot > 0) + rr) * RBQ + c0;
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s2 = 0; s2 < NS16; s2++)
+        for (int s2 = 0; s2 < NS16; s2++) {
+          if (GEN && (kp * NS16 + s2) * 32 >= qk_used) break;
           acc = E::mfma16(lds_read<x8>(ka ^ (uint32_t)(s2 * 64)), lds_read<x8>(qa ^ (uint32_t)(s2 * 64)), acc);
+        }
         lds_write<f32x4>(lds_apart + wave * 1024 + la * 16, acc);
       }
     }
@@ -386,6 +390,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
       for (int ks = 0; ks < AH; ks++) request(ks);
 #pragma unroll
       for (int ks = 0; ks < NS; ks++) {
+        if (GEN && ks * 16 >= qk_used) break;
         if (ks + AH < NS) request(ks + AH);
         __builtin_amdgcn_sched_barrier(0);
         if (TWO_CHAINS && (ks & 1)) sacc2 = E::mfma32(kf[ks % RING], qf[ks % RING], ks == 1 ? zero16 : sacc2);
@@ -483,6 +488,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
       if (AHEAD) request(0);
 #pragma unroll
       for (int bb = 0; bb < KB; bb++) {
+        if (GEN && bb * 32 >= qk_used) break;
         if (!AHEAD) request(bb);
         else if (bb + 1 < KB) request(bb + 1);
         __builtin_amdgcn_sched_barrier(0);
