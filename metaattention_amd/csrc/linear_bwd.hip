@@ -46,7 +46,7 @@ __device__ __forceinline__ float lanes_sum(float x) {
 
 // LPT lanes per (batch, head, token), four columns per lane and round.  dqh [B,H,T,Dk] fp32 (time order), dkh_rev [B,H,T,Dk]
 // and du_rev [B,H,T,Dv] fp32 (reversed time order, dk before its v_scale factor).  Writes dG, dv, dv_scale and, where every
-// head has its own q / k head, dq / dk.
+// head has its own q / k head, dq / dk.  du_rev null: dv has been written by the scan itself (no v_scale: dv = du).
 // With np > 1 the scan outputs dqh and dkh_rev are np pieces (partial sums over slices of the contraction), piece_stride
 // floats apart, which are added up here.
 template <int LPT>
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(256) void grads_kernel(LinBwdArgs a, const float* _
         *(bf16x4*)((__bf16*)a.dk + tk * a.Dk + c) = w;
       }
     }
-    for (int c = 4 * sub; c < a.Dv; c += 4 * LPT) {
+    for (int c = 4 * sub; du_rev && c < a.Dv; c += 4 * LPT) {
       const f32x4 gu = *(const f32x4*)(du_rev + rtok * a.Dv + c);
       const bf16x4 vv = *(const bf16x4*)((const __bf16*)a.v + tk * a.Dv + c);
       bf16x4 w;
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(256) void grads_shared_kernel(LinBwdArgs a, const f
         sk[i] += gk[i];
       }
     }
-    if (live) {
+    if (live && du_rev) {
       for (int cv = 4 * sub; cv < a.Dv; cv += 4 * LPT) {
         const f32x4 gu = *(const f32x4*)(du_rev + rtok * a.Dv + cv);
         const bf16x4 vv = *(const bf16x4*)((const __bf16*)a.v + tk * a.Dv + cv);
@@ -285,13 +285,15 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   // an operand of a scan as the scan kernel reads it in place: heads, elements between its tokens (the pointer carries a
   // column offset)
   struct Operand { const void* p; int heads; int64_t row; };
-  auto scan_launch = [&](Operand q, Operand k, Operand v, bool reversed, int dk, int dv, const float* g, const float* vs, float* out,
-                         bool accumulate, int pieces = 1, int qk_cols = 0) -> int {
+  // (out_bf16: the output goes out as bf16 in the operands' own time order instead of fp32 in scan order)
+  auto scan_launch = [&](Operand q, Operand k, Operand v, bool reversed, int dk, int dv, const float* g, const float* vs, void* out,
+                         bool accumulate, int pieces = 1, int qk_cols = 0, bool out_bf16 = false) -> int {
     LinArgs la{};
     la.q = q.p; la.k = k.p; la.v = v.p; la.o = out; la.log_decay = g; la.v_scale = vs; la.q_scale = a.q_scale;
     la.B = a.B; la.H = a.H; la.Hq = q.heads; la.Hk = k.heads; la.Hv = v.heads; la.T = a.T; la.Dv = dv;
     la.q_row = q.row; la.k_row = k.row; la.v_row = v.row; la.rev = reversed ? 1 : 0;
-    la.out_f32 = accumulate ? 2 : 1;
+    la.out_f32 = out_bf16 ? 0 : (accumulate ? 2 : 1);
+    la.rev_o = out_bf16 && reversed ? 1 : 0;
     if (pieces > 1) { la.n_pieces = pieces; la.piece_qk = dk; la.piece_o = piece_stride; }
     la.qk_cols = qk_cols;
     return linear_fwd_dispatch(la, dk, 0, scan, scan_ws, stream, nullptr);
@@ -313,9 +315,13 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
     if (const int rc = scan_launch(qs, ks, Operand{k_p, a.Hk, a.Dk}, false, sl.w[s], a.Dk, a.log_decay, a.v_scale, dqh, s > 0, 1, piece_cols(s))) return rc;
   }
 
-  // du (reversed) = LA(R k, R q, R do), contraction over the key columns: the operands are read in reversed time in place
-  if (const int rc = scan_launch(Operand{k_p, a.Hk, a.Dk}, Operand{q_p, a.Hq, a.Dk}, Operand{do_p, a.H, a.Dv}, true, a.Dk, a.Dv, grev, nullptr, du, false))
+  // du (reversed) = LA(R k, R q, R do), contraction over the key columns: the operands are read in reversed time in place.
+  // Without a v_scale dv is du itself, and the scan writes it: bf16, rows back in time order.
+  const bool direct_dv = !a.v_scale && !a.dv_scale;
+  if (const int rc = scan_launch(Operand{k_p, a.Hk, a.Dk}, Operand{q_p, a.Hq, a.Dk}, Operand{do_p, a.H, a.Dv}, true, a.Dk, a.Dv, grev, nullptr,
+                                 direct_dv ? a.dv : (void*)du, false, 1, 0, direct_dv))
     return rc;
+  if (direct_dv) du = nullptr;
 
   // dk (per head, reversed, before its v_scale factor) = LA(R v, R do, R q), contraction over the value columns
   if (side_by_side) {

@@ -24,6 +24,9 @@ struct LinArgs {
   // rest of the Dk-wide contraction is zeros that are never loaded (the tiles' LDS is cleared once, the loads of the missing
   // columns are switched off).
   int qk_cols;
+  // rev_o (general addressing only): the outputs are written in reversed time order (row T-1-t holds the scan's token t), so
+  // that a scan over reversed operands leaves its result in the operands' own order.
+  int rev_o;
   // pieces (general addressing only; 0 or 1: none): the launch runs n_pieces independent scans side by side, piece p with
   // its q and k pointers moved on by p * piece_qk elements (the next slice of the contraction's columns) and its output
   // (fp32) by p * piece_o elements; the caller adds the pieces' outputs up.  Single pass only (no sequence segments).

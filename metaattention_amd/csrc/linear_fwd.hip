@@ -125,7 +125,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
   const int b = bh0 / a.H, h0 = bh0 % a.H;        // (HG divides H, and the heads of a group share hq and hk)
   const int hq = h0 / (a.H / a.Hq), hk = h0 / (a.H / a.Hk);
   const int Tn = a.T;
-  const bool rev = GEN && a.rev != 0;
+  const bool rev = GEN && a.rev != 0, rev_o = GEN && a.rev_o != 0;
   const int64_t q_rb = GEN ? a.q_row * 2 : (int64_t)RBQ, k_rb = GEN ? a.k_row * 2 : (int64_t)RBQ;   // bytes between an operand's rows in memory
   const int64_t v_row_bytes = (GEN ? a.v_row : (int64_t)a.Dv) * 2;
   const int64_t bh0_v = GEN ? (int64_t)b * a.Hv + h0 / (a.H / a.Hv) : (int64_t)bh0;
@@ -547,7 +547,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
           const u32x4 w = ALIAS_OST ? lds_read<u32x4>(vbase + row * RBV + (uint32_t)(((4 * wave + cc) ^ swz_tile<CPRV>(row)) << 4))
                                     : lds_read<u32x4>(lds_ost + row * OROW + cc * 16);
           if (t0 + row < Tn) {
-            f32x4* dst = (f32x4*)(ob32 + (int64_t)(t0 + row) * a.Dv + 16 * half + cc * 4);
+            f32x4* dst = (f32x4*)(ob32 + (int64_t)(rev_o ? Tn - 1 - (t0 + row) : t0 + row) * a.Dv + 16 * half + cc * 4);
             f32x4 val = __builtin_bit_cast(f32x4, w);
             if (a.out_f32 == 2) val += *dst;   // (a contraction cut into pieces: the pieces' outputs add up)
             *dst = val;
@@ -571,7 +571,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
       for (int it = 0; it < 2; it++) {
         const int ci = ln + 64 * it, row = ci >> 2, cc = ci & 3;
         const u32x4 w = ALIAS_OST ? lds_read<u32x4>(ra + 16 * it * RBV) : lds_read<u32x4>(lds_ost + row * OROW + cc * 16);
-        if (t0 + row < Tn) *(u32x4*)(ob + (int64_t)(t0 + row) * a.Dv + cc * 8) = w;
+        if (t0 + row < Tn) *(u32x4*)(ob + (int64_t)(rev_o ? Tn - 1 - (t0 + row) : t0 + row) * a.Dv + cc * 8) = w;
       }
     }
   }
@@ -651,7 +651,7 @@ struct Config {
     args.dv_blocks = a.Dv / (32 * NWH);
     // general operand addressing: defaults for what is left at zero; the row distances must be multiples of the tile
     // rows (the kernel XORs the swizzle of an instruction's first row onto the finished lane offset)
-    const bool gen = a.rev != 0 || a.q_row != 0 || a.k_row != 0 || a.v_row != 0 || (a.Hv != 0 && a.Hv != a.H) || a.qk_cols != 0 || a.n_pieces > 1;
+    const bool gen = a.rev != 0 || a.q_row != 0 || a.k_row != 0 || a.v_row != 0 || (a.Hv != 0 && a.Hv != a.H) || a.qk_cols != 0 || a.n_pieces > 1 || a.rev_o != 0;
     if (gen) {
       if (args.q_row == 0) args.q_row = DK;
       if (args.k_row == 0) args.k_row = DK;
