@@ -59,7 +59,7 @@ __device__ __forceinline__ X8 scale_bf16x8(X8 v, const float (&w)[8]) {
 // minimum waves per SIMD asked of the register allocator: 8 waves of one workgroup need 2; the
 // two-heads-per-workgroup configuration is meant to run three workgroups of 4 waves per CU
 template <int DK, int NWH, int HG>
-constexpr int min_waves_per_simd() { return HG > 1 ? 3 : (NWH == 4 ? 1 : 2); }
+constexpr int min_waves_per_simd() { return HG > 1 ? 3 : (NWH == 4 && DK > 128 ? 1 : 2); }
 
 // GEN: the operands' general addressing (reversed time, row strides, v head broadcast) of LinArgs; without it the
 // addressing is the plain one, with compile-time row sizes.
