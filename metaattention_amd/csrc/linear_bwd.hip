@@ -135,13 +135,39 @@ __global__ __launch_bounds__(256) void grads_shared_kernel(LinBwdArgs a, const f
 #pragma unroll
     for (int i = 0; i < 4; i++) { qv[i] = (float)q4[i]; kv[i] = (float)k4[i]; }
   }
+  // What head j + 1 needs is requested before head j is worked on (the compiler cannot move a load above the stores
+  // of the head before, which it must assume to alias).
+  struct Row { f32x4 gq, gk, gu; bf16x4 vv; float vs; };
+  const int cv0 = 4 * sub;
+  const bool has_v = live && du_rev && cv0 < a.Dv;
+  auto load_row = [&](int j) {
+    Row r{};
+    const int64_t bh = b * a.H + (int64_t)g * G + j, tk = bh * a.T + t, rtok = bh * a.T + (a.T - 1 - t);
+    r.vs = a.v_scale ? a.v_scale[tk] : 1.f;
+    if (has_c) {
+      r.gq = *(const f32x4*)(dqh + tk * a.Dk + c);
+      r.gk = *(const f32x4*)(dkh_rev + rtok * a.Dk + c);
+    }
+    if (has_v) {
+      r.gu = *(const f32x4*)(du_rev + rtok * a.Dv + cv0);
+      r.vv = *(const bf16x4*)((const __bf16*)a.v + tk * a.Dv + cv0);
+    }
+    return r;
+  };
+  constexpr int PF = 3;   // heads ahead
+  Row ring[PF];
+#pragma unroll
+  for (int i = 0; i < PF; i++) ring[i] = i < G ? load_row(i) : Row{};
   for (int j = 0; j < G; j++) {
     const int64_t bh = b * a.H + (int64_t)g * G + j, tk = bh * a.T + t, rtok = bh * a.T + (a.T - 1 - t);
-    const float vs = a.v_scale ? a.v_scale[tk] : 1.f;
+    const Row row = ring[0];
+#pragma unroll
+    for (int i = 0; i + 1 < PF; i++) ring[i] = ring[i + 1];
+    if (j + PF < G) ring[PF - 1] = load_row(j + PF);
+    const float vs = row.vs;
     float acc = 0.f, acc_vs = 0.f;
     if (has_c) {
-      f32x4 gq = *(const f32x4*)(dqh + tk * a.Dk + c);
-      f32x4 gk = *(const f32x4*)(dkh_rev + rtok * a.Dk + c);
+      f32x4 gq = row.gq, gk = row.gk;
       for (int p = 1; p < np; p++) {
         gq += *(const f32x4*)(dqh + p * piece_stride + tk * a.Dk + c);
         gk += *(const f32x4*)(dkh_rev + p * piece_stride + rtok * a.Dk + c);
@@ -154,10 +180,10 @@ __global__ __launch_bounds__(256) void grads_shared_kernel(LinBwdArgs a, const f
         sk[i] += gk[i];
       }
     }
-    if (live && du_rev) {
-      for (int cv = 4 * sub; cv < a.Dv; cv += 4 * LPT) {
-        const f32x4 gu = *(const f32x4*)(du_rev + rtok * a.Dv + cv);
-        const bf16x4 vv = *(const bf16x4*)((const __bf16*)a.v + tk * a.Dv + cv);
+    if (has_v) {
+      for (int cv = cv0; cv < a.Dv; cv += 4 * LPT) {
+        const f32x4 gu = cv == cv0 ? row.gu : *(const f32x4*)(du_rev + rtok * a.Dv + cv);
+        const bf16x4 vv = cv == cv0 ? row.vv : *(const bf16x4*)((const __bf16*)a.v + tk * a.Dv + cv);
         bf16x4 w;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
