@@ -67,6 +67,26 @@ def test_linear_backward(B, Hq, H, T, Dk, Dv, use_vs):
     _check(got, ref, "linear")
 
 
+@pytest.mark.parametrize("B,Hq,H,T,Dk,Dv", [(1, 2, 2, 300, 256, 512), (2, 1, 4, 77, 128, 64), (1, 2, 2, 256, 128, 128)])
+def test_dv_written_by_the_scan_equals_dv_through_the_epilogue(B, Hq, H, T, Dk, Dv):
+    """Without a value scale the du scan writes dv itself (bf16, rows back in time order); with a value scale of ones dv goes
+    through the fp32 workspace and the epilogue kernel.  Both round the same fp32 numbers, so every gradient is the same bit
+    for bit, also with a partial last chunk and with the sequence cut into segments."""
+    hb = _hb()
+    g = torch.Generator().manual_seed(B * T + Dv)
+    q = torch.randn(B, Hq, T, Dk, generator=g).bfloat16().cuda()
+    k = (0.1 * torch.randn(B, Hq, T, Dk, generator=g)).bfloat16().cuda()
+    v = torch.randn(B, H, T, Dv, generator=g).bfloat16().cuda()
+    ld = torch.nn.functional.logsigmoid(torch.randn(B, H, T, generator=g) + 3.0).cuda()
+    dout = (0.5 * torch.randn(B, H, T, Dv, generator=g)).bfloat16().cuda()
+    print(f"dv two ways B{B} H{H}/{Hq} T{T} Dk{Dk} Dv{Dv}", flush=True)
+    direct = hb.linear_bwd(q, k, v, ld, dout, q_scale=Dk ** -0.5)
+    ones = hb.linear_bwd(q, k, v, ld, dout, q_scale=Dk ** -0.5, v_scale=torch.ones(B, H, T, device="cuda"))
+    torch.cuda.synchronize()
+    for name, a, b in zip(("dq", "dk", "dv", "dlog_decay"), direct, ones):
+        assert torch.equal(a, b), f"{name}: {float((a.float() - b.float()).abs().max())}"
+
+
 def test_engine_mamba2_backward():
     """mod(C, B, x, dt, A, dt_bf16) as testing/test.py:198-204 followed by o.backward(do): gradients reach
     C, B, x and, through the eager mods, dt and A."""
