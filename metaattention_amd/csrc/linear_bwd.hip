@@ -239,22 +239,42 @@ __global__ __launch_bounds__(256) void group_sum_kernel(__bf16* __restrict__ dst
   *(bf16x4*)(dst + row * D + c) = w;
 }
 
-// dlog_decay[b, h, t] = sum_{t' >= t} dG[b, h, t']: one wave per (batch, head), blocks of 64 tokens from the end
-__global__ __launch_bounds__(64) void suffix_sum_kernel(float* __restrict__ dst, const float* __restrict__ dG, int T) {
-  const int lane = threadIdx.x;
+// dlog_decay[b, h, t] = sum_{t' >= t} dG[b, h, t']: one workgroup of 256 threads per (batch, head), blocks of 2048 tokens from
+// the end, eight consecutive tokens per thread (its own running sum), the threads' totals scanned through the wave and LDS
+__global__ __launch_bounds__(256) void suffix_sum_kernel(float* __restrict__ dst, const float* __restrict__ dG, int T) {
+  __shared__ float wave_total[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* src = dG + (int64_t)blockIdx.x * T;
   float* out = dst + (int64_t)blockIdx.x * T;
-  float carry = 0.f;
-  for (int t0 = (T - 1) / 64 * 64; t0 >= 0; t0 -= 64) {
-    const int t = t0 + lane;
-    float x = t < T ? src[t] : 0.f;
+  float carry = 0.f;   // sum of everything behind the block
+  for (int t0 = (T - 1) / 2048 * 2048; t0 >= 0; t0 -= 2048) {
+    const int t = t0 + 8 * tid;
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) x[i] = t + i < T ? src[t + i] : 0.f;
+#pragma unroll
+    for (int i = 6; i >= 0; i--) x[i] += x[i + 1];   // x[i] = sum of this thread's tokens i..7
+    // sum of the totals of the later lanes of the wave, then of the later waves
+    float incl = x[0];
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
-      const float y = __shfl_down(x, off, 64);
-      if (lane + off < 64) x += y;
+      const float y = __shfl_down(incl, off, 64);
+      if (lane + off < 64) incl += y;
     }
-    if (t < T) out[t] = x + carry;
-    carry += __shfl(x, 0, 64);
+    if (lane == 0) wave_total[wave] = incl;
+    __syncthreads();
+    float behind = carry + (incl - x[0]);
+    float block_total = 0.f;
+#pragma unroll
+    for (int w = 3; w >= 0; w--) {
+      if (w > wave) behind += wave_total[w];
+      block_total += wave_total[w];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      if (t + i < T) out[t + i] = x[i] + behind;
+    carry += block_total;
+    __syncthreads();
   }
 }
 
@@ -368,7 +388,7 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
     else
       hipLaunchKernelGGL(grads_shared_kernel<32>, dim3((unsigned)((n_tok + 7) / 8)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh,
                          (const float*)du, dG, np, piece_stride);
-    hipLaunchKernelGGL(suffix_sum_kernel, dim3((unsigned)(a.B * a.H)), dim3(64), 0, stream, a.dlog_decay, (const float*)dG, a.T);
+    hipLaunchKernelGGL(suffix_sum_kernel, dim3((unsigned)(a.B * a.H)), dim3(256), 0, stream, a.dlog_decay, (const float*)dG, a.T);
     return launch_status();
   }
   if ((a.Dk > a.Dv ? a.Dk : a.Dv) >= 256)
@@ -387,7 +407,7 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
     hipLaunchKernelGGL(group_sum_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, (__bf16*)a.dk, (const float*)dkh, a.v_scale, a.H, a.Hk,
                        a.T, a.Dk, 1, n4, np, piece_stride);
   }
-  hipLaunchKernelGGL(suffix_sum_kernel, dim3((unsigned)(a.B * a.H)), dim3(64), 0, stream, a.dlog_decay, (const float*)dG, a.T);
+  hipLaunchKernelGGL(suffix_sum_kernel, dim3((unsigned)(a.B * a.H)), dim3(256), 0, stream, a.dlog_decay, (const float*)dG, a.T);
   return launch_status();
 }
 
