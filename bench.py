@@ -63,8 +63,8 @@ RAMP_MS = 80.0
 
 def time_gpu(fn, steps, warmup, flush=None):
     """Average milliseconds per call over `steps` calls, HIP events on the launch stream.
-    With `flush`, the caches are overwritten before every call and each call is
-    timed on its own (for the HBM-bound workload)."""
+    With `flush`, that callable runs before every call (it replaces what the caches hold) and each
+    call is timed on its own (for the HBM-bound workloads)."""
     import torch
     t0 = time.perf_counter()
     while (time.perf_counter() - t0) * 1e3 < RAMP_MS:
@@ -92,6 +92,18 @@ def time_gpu(fn, steps, warmup, flush=None):
         torch.cuda.synchronize()
         total += e0.elapsed_time(e1)
     return total / steps
+
+
+COLD_NOTE = ("ms: 1 GiB of other data is READ through the caches before every timed call, so the call starts with cold caches that "
+             "hold clean lines; ms_after_cache_overwrite: the same with that buffer WRITTEN instead -- the timed call then also "
+             "pays for the write-back of the buffer's dirty lines (L2 and the last-level cache), which is the flush's traffic, not the "
+             "kernel's; ms_without_cache_flush: calls back to back")
+
+
+def _junk():
+    """1 GiB of int32 ones: more than L2 and the 256 MB last-level cache together."""
+    import torch
+    return torch.ones(2 ** 28, dtype=torch.int32, device="cuda")
 
 
 def _mfma_entry(ms, flops, note=None, **extra):
@@ -189,15 +201,16 @@ def bench_decode(steps, warmup, B=64, H=32, Hkv=8, Skv=4096, D=128):
     o = torch.empty_like(q)
     qv, ov = q.view(B, Hkv, grp, D).transpose(1, 2), o.view(B, Hkv, grp, D).transpose(1, 2)
     ws = torch.empty(1 << 26, dtype=torch.uint8, device="cuda")
-    junk = torch.empty(512 * 2 ** 20, dtype=torch.uint8, device="cuda")
+    junk = _junk()
     fn = lambda: hb.attn_fwd(qv, k, v, family=hb.MA_ATTN_SOFTMAX, causal=False, scale=1 / math.sqrt(D), out=ov, workspace=ws)
-    ms = time_gpu(fn, steps, warmup, flush=lambda: junk.fill_(1))
     ms_warm = time_gpu(fn, steps, warmup)
+    ms_dirty = time_gpu(fn, steps, warmup, flush=lambda: junk.fill_(1))
+    ms = time_gpu(fn, steps, warmup, flush=lambda: junk.sum())   # (last: a kernel trace's last `steps` dispatches are these)
     nbytes = 2.0 * (k.numel() + v.numel() + q.numel() + o.numel())
     gbs = nbytes / ms / 1e6
     return dict(ms=round(ms, 4), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / PEAK_HBM_GBS, 4), algorithmic_bytes=nbytes,
-                ms_without_cache_flush=round(ms_warm, 4), shape=dict(B=B, H=H, Hkv=Hkv, Sq=1, Skv=Skv, D=D),
-                note="split-KV kernel + combine kernel per call; caches overwritten before every timed call")
+                ms_after_cache_overwrite=round(ms_dirty, 4), ms_without_cache_flush=round(ms_warm, 4),
+                shape=dict(B=B, H=H, Hkv=Hkv, Sq=1, Skv=Skv, D=D), note="split-KV kernel + combine kernel per call; " + COLD_NOTE)
 
 
 def bench_retnet_chunked(steps, warmup, backward=False):
@@ -301,16 +314,17 @@ def bench_mla(steps, warmup):
     k_pe = torch.randn(B, Skv, 1, Dpe, device="cuda", dtype=torch.bfloat16, generator=g)
     o = torch.empty_like(q)
     ws = torch.empty(max(hb.mla_workspace_bytes(B, Hq, Skv), 16), dtype=torch.uint8, device="cuda")
-    junk = torch.empty(512 * 2 ** 20, dtype=torch.uint8, device="cuda")   # larger than L2 + the 256 MB last-level cache
+    junk = _junk()
     fn = lambda: hb.mla_decode(q, q_pe, kv, k_pe, scale=1 / math.sqrt(D + Dpe), out=o, workspace=ws)
-    ms = time_gpu(fn, steps, warmup, flush=lambda: junk.fill_(1))
     ms_warm = time_gpu(fn, steps, warmup)
+    ms_dirty = time_gpu(fn, steps, warmup, flush=lambda: junk.fill_(1))
+    ms = time_gpu(fn, steps, warmup, flush=lambda: junk.sum())   # (last: a kernel trace's last `steps` dispatches are these)
     nbytes = 2.0 * (kv.numel() + k_pe.numel() + q.numel() + q_pe.numel() + o.numel())
     flops = 2.0 * B * Hq * Skv * (D + Dpe + D)
     gbs = nbytes / ms / 1e6
     return dict(ms=round(ms, 4), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / PEAK_HBM_GBS, 4), algorithmic_bytes=nbytes,
-                tflops=round(flops / ms / 1e9, 1), ms_without_cache_flush=round(ms_warm, 4),
-                note="split-KV kernel + combine kernel per call; caches overwritten before every timed call")
+                tflops=round(flops / ms / 1e9, 1), ms_after_cache_overwrite=round(ms_dirty, 4), ms_without_cache_flush=round(ms_warm, 4),
+                note="split-KV kernel + combine kernel per call; " + COLD_NOTE)
 
 
 def cpu_baseline_softmax():
