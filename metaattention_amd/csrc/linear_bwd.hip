@@ -301,7 +301,7 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   const int64_t BHT = (int64_t)a.B * a.H * a.T;
   const Slices sl(a.Dv);   // contraction of the dq and dk scans
 
-  // workspace: fp32 scan outputs, dG, reversed log decay, packed operands, the scan kernel's own workspace
+  // workspace: fp32 scan outputs, dG, reversed log decay, the scan kernel's own workspace
   size_t off = 0;
   auto take = [&](size_t bytes) { const size_t o = off; off += align256(bytes); return o; };
   // (a contraction of equal pieces that are all read in place runs its pieces side by side, each with an output of its own)
