@@ -403,62 +403,6 @@ def cpu_baseline_mla():
                 sample=f"B=64 of 64, Hq={Hq}, KV={Skv}, d={D}+{Dpe}, fp32 oracle, {dt:.1f} s; algorithmic bytes of the bf16 tensors over the time")
 
 
-def run_probes():
-    """Ceilings measured on this box with the probe kernels of csrc/probe/ceilings.hip (their own small library).
-
-    `attention_step`: 8 waves per CU run the per-step work of the 128/128 forward kernel (16 MFMAs of 32x32x16 per wave and
-    32-key sub-tile) in a loop, with more and more of what surrounds the MFMAs in the real kernel switched on, once with
-    constant and once with pseudo-random operands.  `tflops` is what the same step rate would mean for the whole chip.
-    `stream_to_lds`: direct-to-LDS streaming rate of the whole chip from windows that fit L2 / the last-level cache / HBM.
-    `issue_hold`: cycles a direct-to-LDS instruction holds its wave at issue, by how many waves of the CU issue at once."""
-    import ctypes
-    lib_path = os.path.join(ROOT, "metaattention_amd", "lib", "libmetaattention_probe.so")
-    if not os.path.exists(lib_path):
-        raise RuntimeError(f"{lib_path} is not built (python -m metaattention_amd.build)")
-    lib = ctypes.CDLL(lib_path)
-    lib.ma_probe_attention_step.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
-    lib.ma_probe_stream_to_lds.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
-    names = {0: "mfma only", 1: "+ vector work", 2: "+ LDS fragment reads", 3: "+ vector work + LDS reads",
-             7: "+ vector + LDS + barrier per step", 15: "+ vector + LDS + barrier + direct-to-LDS loads",
-             31: "the same with the two loads behind the 3rd and 6th MFMA pair instead of at the start of the step"}
-    flop_per_step = 256 * 8 * 16 * 2 * 32 * 32 * 16        # CUs x waves x MFMAs x flop of one 32x32x16
-    steps = []
-    for mode, name in names.items():
-        row = {"what": name}
-        for rnd in (0, 1):
-            ns, cyc = ctypes.c_double(), ctypes.c_double()
-            rc = lib.ma_probe_attention_step(mode, rnd, 4000, ctypes.byref(ns), ctypes.byref(cyc))
-            if rc != 0:
-                raise RuntimeError(f"ma_probe_attention_step({mode}, {rnd}) returned {rc}")
-            key = "random_operands" if rnd else "constant_operands"
-            row[key] = {"ns_per_step": round(ns.value, 1), "cycles_per_step_wave0": round(cyc.value, 1),
-                        "tflops": round(flop_per_step / ns.value / 1e3, 1), "frac_of_bf16_peak": round(flop_per_step / ns.value / 1e3 / PEAK_BF16_TFLOPS, 4)}
-        steps.append(row)
-    streams = []
-    for region_mb, what in ((16, "fits L2 (8 x 4 MB)"), (128, "fits the last-level cache (256 MB)"), (2048, "HBM")):
-        for depth in (2, 6):
-            gbs = ctypes.c_double()
-            rc = lib.ma_probe_stream_to_lds(region_mb << 20, depth, 400, ctypes.byref(gbs))
-            if rc != 0:
-                raise RuntimeError(f"ma_probe_stream_to_lds({region_mb} MB, {depth}) returned {rc}")
-            streams.append({"region_mb": region_mb, "region": what, "kb_in_flight_per_cu": 8 * depth, "gb_per_s": round(gbs.value, 1),
-                            "frac_of_hbm_peak": round(gbs.value / PEAK_HBM_GBS, 4)})
-    lib.ma_probe_issue_hold.argtypes = [ctypes.c_int, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
-    holds = []
-    kinds = {0: "global_load_lds_dwordx4 (1 KB)", 1: "global_load_lds_dword (256 B)", 2: "global_load_dwordx4 to registers (1 KB)"}
-    for kind, kname in kinds.items():
-        for region_mb, what in ((16, "L2"), (2048, "HBM")):
-            for nwaves, per_round in ((1, 1), (1, 8), (8, 1), (8, 2), (8, 4), (8, 8)):
-                ci, ct = ctypes.c_double(), ctypes.c_double()
-                rc = lib.ma_probe_issue_hold(kind, region_mb << 20, nwaves, per_round, ctypes.byref(ci), ctypes.byref(ct))
-                if rc != 0:
-                    raise RuntimeError(f"ma_probe_issue_hold({kind}, {region_mb} MB, {nwaves}, {per_round}) returned {rc}")
-                holds.append({"instruction": kname, "from": what, "waves_issuing_per_cu": nwaves, "instructions_per_burst": per_round,
-                              "kb_per_burst_and_cu": nwaves * per_round * (0.25 if kind == 1 else 1.0),
-                              "issue_cycles_per_instruction": round(ci.value, 1), "cycles_per_instruction_with_wait": round(ct.value, 1)})
-    return {"probe": "ceilings", "attention_step": steps, "stream_to_lds": streams, "issue_hold": holds}
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -471,9 +415,6 @@ def main():
                     help="run 5 plain device-to-device copies of 1 GiB and exit (reference point for rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--only", default="", help="comma list limiting the other workloads (e.g. 'mla'); 'none' skips them")
-    ap.add_argument("--probe", action="store_true",
-                    help="instead of the benchmark, run the ceiling probes (what the forward kernel's instruction mix and the "
-                         "global-to-LDS path reach on this box) and print them as one JSON line")
     args = ap.parse_args()
     globals()["RAMP_MS"] = max(args.ramp_ms, 0.0)
     if args.gpus != 1:
@@ -493,10 +434,6 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"calibration": "5 device-to-device copies", "bytes_read_per_copy": 2 ** 30, "bytes_written_per_copy": 2 ** 30}))
-        return
-
-    if args.probe:
-        print(json.dumps(run_probes()))
         return
 
     main_res = bench_softmax(args.steps, args.warmup, "softmax")

@@ -16,9 +16,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmetaattention_hip.so")
-# ceiling probes for bench.py --probe: their own small library, not part of the operator library
-PROBE_SRC = os.path.join(CSRC, "probe", "ceilings.hip")
-PROBE_LIB_PATH = os.path.join(LIB_DIR, "libmetaattention_probe.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32
@@ -59,12 +56,6 @@ def build_library(verbose: bool = False, jobs: int = 8) -> str:
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-shared", PROBE_SRC, "-o", PROBE_LIB_PATH]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed for {PROBE_SRC}:\n{res.stdout}\n{res.stderr}")
     return LIB_PATH
 
 
