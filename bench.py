@@ -16,9 +16,11 @@ cores over a bounded sample as "cpu_baseline"):
   c2_softmax_causal_bwd  backward of the headline workload (dq, dk, dv)
   c3_retnet_chunked   RetNet retention, chunked operator, B8 H16 S2048 Dqk256 Dv512
   c3_retnet_parallel  same shape, normalised parallel operator with a [1,H,S,S] decay mask
+  c3_retnet_parallel_operator  the same through the operator AttentionEngine returns, mod(q, k, v, mask): it recognises the decay mask
   c3_retnet_parallel_generated_mask  the same operator told the mask is gamma_h^(i-j) (decay_gamma): no mask tensor is read
   c3_retnet_parallel_bwd  backward of that operator (dq, dk, dv; the row scale held constant, as the reference defines it)
   c4_mamba2_ssd       Mamba2 SSD, B8 H64 S2048 P64 N128, one B/C group
+  c3_retnet_chunked_operator / c4_mamba2_ssd_operator / c5_mla_decode_operator  those three through the operators the engines return
   c5_mla_decode       absorbed MLA decode, B64 Hq128 KV4096 d512+64 (HBM bound)
   gqa_decode          grouped-query softmax decode, B64 H32 Hkv8 KV4096 D128 (HBM bound)
 """
@@ -94,16 +96,28 @@ def time_gpu(fn, steps, warmup, flush=None):
     return total / steps
 
 
-COLD_NOTE = ("ms: 1 GiB of other data is READ through the caches before every timed call, so the call starts with cold caches that "
-             "hold clean lines; ms_after_cache_overwrite: the same with that buffer WRITTEN instead -- the timed call then also "
-             "pays for the write-back of the buffer's dirty lines (L2 and the last-level cache), which is the flush's traffic, not the "
-             "kernel's; ms_without_cache_flush: calls back to back")
+COLD_NOTE = ("ms / frac_of_hbm_peak_clean_read: 1 GiB of other data is READ through the caches before every timed call, so the call "
+             "starts with cold caches that hold clean lines; ms_after_cache_overwrite / frac_of_hbm_peak: the same with that buffer "
+             "WRITTEN instead -- the timed call then also pays for the write-back of the buffer's dirty lines (L2 and the "
+             "last-level cache); ms_without_cache_flush: calls back to back")
 
 
 def _junk():
     """1 GiB of int32 ones: more than L2 and the 256 MB last-level cache together."""
     import torch
     return torch.ones(2 ** 28, dtype=torch.int32, device="cuda")
+
+
+def _hbm_entry(ms_clean, ms_dirty, ms_warm, nbytes):
+    """An HBM-bound workload timed call by call in three cache states.  `frac_of_hbm_peak` is the figure after the
+    OVERWRITING flush (a 1 GiB buffer written before every timed call: caches hold none of the workload, and the call also
+    pays for the write-back of that buffer's dirty lines); `frac_of_hbm_peak_clean_read` after the same buffer was READ
+    (cold caches holding clean lines: what a decode step meets in a serving loop); both against 8 TB/s."""
+    gbs_dirty, gbs_clean = nbytes / ms_dirty / 1e6, nbytes / ms_clean / 1e6
+    return dict(ms=round(ms_clean, 4), ms_after_cache_overwrite=round(ms_dirty, 4), ms_without_cache_flush=round(ms_warm, 4),
+                gb_per_s=round(gbs_dirty, 1), frac_of_hbm_peak=round(gbs_dirty / PEAK_HBM_GBS, 4),
+                gb_per_s_clean_read=round(gbs_clean, 1), frac_of_hbm_peak_clean_read=round(gbs_clean / PEAK_HBM_GBS, 4),
+                algorithmic_bytes=nbytes)
 
 
 def _mfma_entry(ms, flops, note=None, **extra):
@@ -172,6 +186,131 @@ def bench_softmax_operator(steps, warmup):
     return _mfma_entry(ms, 0.5 * 4.0 * B * H * S * S * D, "the headline workload through the AttentionEngine operator (allocates o and lse per call)")
 
 
+def bench_linear_operators(steps, warmup, which):
+    """The chunked RetNet / Mamba2 workloads through the operator LinearAttentionEngine returns (reference call sites:
+    testing/test.py:198-200 mod(C, B, x, dt, A, dt_bf16) and :776 mod(q, k, v, decay)): with the eager decay_mod / v_mod
+    tensor work around the kernel, the output allocation and the workspace the operator keeps."""
+    import torch
+    from attn_engine import LinearAttentionEngine
+    from core import CustomIO, meta_tensor
+    g = torch.Generator(device="cuda").manual_seed(0)
+    if which == "retnet":
+        B, H, T, Dk, Dv = 8, 16, 2048, 256, 512
+        meta = (meta_tensor(B, H, T, Dk, dtype=torch.bfloat16), meta_tensor(B, H, T, Dk, dtype=torch.bfloat16), meta_tensor(B, H, T, Dv, dtype=torch.bfloat16))
+        mod = LinearAttentionEngine(meta, q_mod=lambda q, io: q * (Dk ** -0.5), decay_mod=lambda decay, io: decay.log(), custom_io=CustomIO({}))
+        q = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 16).bfloat16()
+        k = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 16).bfloat16()
+        v = torch.randn(B, H, T, Dv, device="cuda", generator=g).bfloat16()
+        decay = (1 - torch.exp2(-5 - torch.arange(H, device="cuda").float())).view(1, H, 1).expand(B, H, T).contiguous()
+        with torch.no_grad():
+            ms = time_gpu(lambda: mod(q, k, v, decay), steps, warmup)
+        flops = B * H * (2.0 * T * 64 * (Dk + Dv) + 4.0 * T * Dk * Dv)
+        return _mfma_entry(ms, flops, "c3_retnet_chunked through the LinearAttentionEngine operator (eager log of the decay, output allocation)")
+    B, H, T, P, N = 8, 64, 2048, 64, 128
+    meta = (meta_tensor(B, 1, T, N, dtype=torch.bfloat16), meta_tensor(B, 1, T, N, dtype=torch.bfloat16), meta_tensor(B, H, T, P, dtype=torch.bfloat16))
+    io = CustomIO({"A": (1, "heads"), "dt": ("batch", "heads", "seq_len")})
+    mod = LinearAttentionEngine(meta, decay_mod=lambda decay, io: decay * io.input_tensors["A"], v_mod=lambda v, io: v * io.input_tensors["dt"], custom_io=io)
+    Cm = (torch.randn(B, 1, T, N, device="cuda", generator=g) / math.sqrt(N)).bfloat16()
+    Bm = (torch.randn(B, 1, T, N, device="cuda", generator=g) / math.sqrt(N)).bfloat16()
+    x = torch.randn(B, H, T, P, device="cuda", generator=g).bfloat16()
+    dt = torch.nn.functional.softplus(torch.randn(B, H, T, device="cuda", generator=g) - 2)
+    A = -torch.exp(torch.rand(1, H, device="cuda", generator=g) * math.log(16))
+    dt16 = dt.bfloat16()
+    with torch.no_grad():
+        ms = time_gpu(lambda: mod(Cm, Bm, x, dt, A, dt16), steps, warmup)
+    flops = B * H * (2.0 * T * 256 * N + 2.0 * T * 256 * P + 4.0 * T * N * P)
+    return _mfma_entry(ms, flops, "c4_mamba2_ssd through the LinearAttentionEngine operator (eager dt * A, output allocation)")
+
+
+def bench_retention_operator(steps, warmup):
+    """c3_retnet_parallel through the operator AttentionEngine returns for the spec of examples/retention_parallel.py:25-111,
+    called as testing/benchmark_h100.py:794-801 does: mod(q, k, v, mask) with the [1,H,S,S] bf16 decay mask.  The operator
+    checks once per mask tensor (on the device) whether it is gamma_h^(i-j) below the diagonal, and then lets the kernel
+    generate it."""
+    import torch
+    from attn_engine import AttentionEngine, OnlineFunc
+    from core import CustomIO, SymbolScalar, Var, meta_tensor
+    B, H, S, D, DV = 8, 16, 2048, 256, 512
+
+    class OnlineRetention(OnlineFunc):   # examples/retention_parallel.py:36-86
+        def __init__(self):
+            super().__init__({"r_wo_clamp": SymbolScalar("r_wo_clamp", Var("0.0")), "r": SymbolScalar("r", Var("0.0"))},
+                             {"r": SymbolScalar("r", Var("0.0"))}, CustomIO())
+
+        @staticmethod
+        def online_fwd(scores, rs, b, h, q_idx):
+            r_wo_clamp = rs["r_wo_clamp"] + scores.get_reduce("abssum")
+            r_new = r_wo_clamp.max(1.0)
+            return scores / r_new, {"r_wo_clamp": r_wo_clamp, "r": r_new}, rs["r"] / r_new
+
+        @staticmethod
+        def online_fwd_epilogue(o, rs, b, h, q_idx):
+            return o, {"r": rs["r"]}
+
+    meta = (meta_tensor(B, H, S, D, dtype=torch.bfloat16), meta_tensor(B, H, S, D, dtype=torch.bfloat16), meta_tensor(B, H, S, DV, dtype=torch.bfloat16))
+    mod = AttentionEngine(meta, CustomIO({"mask": (1, "heads", "seq_len", "seq_len_kv")}),
+                          score_mod=lambda s, io, b, h, qi, ki: s * io.input_tensors["mask"], mask_mod=lambda b, h, qi, ki: qi >= ki,
+                          online_func=OnlineRetention(), mask_value="0")
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q = (torch.randn(B, S, H, D, device="cuda", generator=g) / 16).bfloat16()
+    k = (torch.randn(B, S, H, D, device="cuda", generator=g) / 16).bfloat16()
+    v = torch.randn(B, S, H, DV, device="cuda", generator=g).bfloat16()
+    idx = torch.arange(S, device="cuda", dtype=torch.float32)
+    gam = 1 - torch.exp2(-5 - torch.arange(H, device="cuda").float())
+    diff = (idx.view(S, 1) - idx.view(1, S))
+    mask = (torch.exp2(diff.clamp(min=0).unsqueeze(0) * torch.log2(gam).view(H, 1, 1)) * (diff >= 0)).unsqueeze(0).bfloat16()
+    with torch.no_grad():
+        ms = time_gpu(lambda: mod(q, k, v, mask), steps, warmup)
+    generated = any(gm is not None for gm in getattr(mod, "_gamma_cache", {}).values())
+    return _mfma_entry(ms, 0.5 * 2.0 * B * H * S * S * (D + DV),
+                       "c3_retnet_parallel through the AttentionEngine operator, mod(q, k, v, mask) with the [1,H,S,S] bf16 decay mask; "
+                       "the operator found the mask to be gamma_h^(i-j) and the kernel generates it" if generated else
+                       "c3_retnet_parallel through the AttentionEngine operator, mod(q, k, v, mask): the mask tensor is read")
+
+
+def bench_mla_operator(steps, warmup):
+    """c5_mla_decode through the operator AttentionEngine(kv_shared=True) returns (reference call site testing/test.py:842-848):
+    mod(q, q_pe, kv, k_pe), with its output and workspace handling; cold, clean caches as for the C-ABI figure."""
+    import torch
+    from attn_engine import AttentionEngine, OnlineFunc
+    from core import CustomIO, SymbolScalar, Var, meta_tensor
+    B, Hq, Skv, D, Dpe = 64, 128, 4096, 512, 64
+
+    class Online(OnlineFunc):   # (the MLA path takes the template's own softmax: lower_decode_mla.py:25-38)
+        def __init__(self):
+            super().__init__({"m": SymbolScalar("m", Var("-inf")), "r": SymbolScalar("r", Var("0.0"))},
+                             {"lse": SymbolScalar("lse", Var("0.0"))}, CustomIO())
+
+        @staticmethod
+        def online_fwd(scores, rs, b, h, q_idx):
+            m_new = rs["m"].max(scores.get_reduce("max"))
+            c = (rs["m"] - m_new).exp()
+            p = (scores - m_new).exp()
+            return p, {"m": m_new, "r": rs["r"] * c + p.get_reduce("sum")}, c
+
+        @staticmethod
+        def online_fwd_epilogue(o, rs, b, h, q_idx):
+            return o / rs["r"], {"lse": rs["r"].log() + rs["m"]}
+
+    meta = (meta_tensor(B, Hq, 1, D + Dpe, dtype=torch.bfloat16), meta_tensor(B, 1, Skv, D + Dpe, dtype=torch.bfloat16),
+            meta_tensor(B, 1, Skv, D, dtype=torch.bfloat16))
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=lambda s, io, b, h, qi, ki: s * ((D + Dpe) ** -0.5), mask_mod=None,
+                          online_func=Online(), kv_shared=True)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q = torch.randn(B, 1, Hq, D, device="cuda", dtype=torch.bfloat16, generator=g)
+    q_pe = torch.randn(B, 1, Hq, Dpe, device="cuda", dtype=torch.bfloat16, generator=g)
+    kv = torch.randn(B, Skv, 1, D, device="cuda", dtype=torch.bfloat16, generator=g)
+    k_pe = torch.randn(B, Skv, 1, Dpe, device="cuda", dtype=torch.bfloat16, generator=g)
+    junk = _junk()
+    with torch.no_grad():
+        fn = lambda: mod(q, q_pe, kv, k_pe)
+        ms_warm = time_gpu(fn, steps, warmup)
+        ms_dirty = time_gpu(fn, steps, warmup, flush=lambda: junk.fill_(1))
+        ms = time_gpu(fn, steps, warmup, flush=lambda: junk.sum())
+    nbytes = 2.0 * (kv.numel() + k_pe.numel() + q.numel() + q_pe.numel() + q.numel())
+    return dict(**_hbm_entry(ms, ms_dirty, ms_warm, nbytes), note="c5_mla_decode through the AttentionEngine(kv_shared=True) operator; " + COLD_NOTE)
+
+
 def bench_softmax_bwd(steps, warmup):
     """Backward of the headline workload (dq, dk, dv given o, lse, do).  FLOPs by the usual convention:
     5 tile products against the forward's 2, causal at one half."""
@@ -207,9 +346,7 @@ def bench_decode(steps, warmup, B=64, H=32, Hkv=8, Skv=4096, D=128):
     ms_dirty = time_gpu(fn, steps, warmup, flush=lambda: junk.fill_(1))
     ms = time_gpu(fn, steps, warmup, flush=lambda: junk.sum())   # (last: a kernel trace's last `steps` dispatches are these)
     nbytes = 2.0 * (k.numel() + v.numel() + q.numel() + o.numel())
-    gbs = nbytes / ms / 1e6
-    return dict(ms=round(ms, 4), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / PEAK_HBM_GBS, 4), algorithmic_bytes=nbytes,
-                ms_after_cache_overwrite=round(ms_dirty, 4), ms_without_cache_flush=round(ms_warm, 4),
+    return dict(**_hbm_entry(ms, ms_dirty, ms_warm, nbytes),
                 shape=dict(B=B, H=H, Hkv=Hkv, Sq=1, Skv=Skv, D=D), note="split-KV kernel + combine kernel per call; " + COLD_NOTE)
 
 
@@ -321,9 +458,7 @@ def bench_mla(steps, warmup):
     ms = time_gpu(fn, steps, warmup, flush=lambda: junk.sum())   # (last: a kernel trace's last `steps` dispatches are these)
     nbytes = 2.0 * (kv.numel() + k_pe.numel() + q.numel() + q_pe.numel() + o.numel())
     flops = 2.0 * B * Hq * Skv * (D + Dpe + D)
-    gbs = nbytes / ms / 1e6
-    return dict(ms=round(ms, 4), gb_per_s=round(gbs, 1), frac_of_hbm_peak=round(gbs / PEAK_HBM_GBS, 4), algorithmic_bytes=nbytes,
-                tflops=round(flops / ms / 1e9, 1), ms_after_cache_overwrite=round(ms_dirty, 4), ms_without_cache_flush=round(ms_warm, 4),
+    return dict(**_hbm_entry(ms, ms_dirty, ms_warm, nbytes), tflops=round(flops / ms / 1e9, 1),
                 note="split-KV kernel + combine kernel per call; " + COLD_NOTE)
 
 
@@ -437,6 +572,10 @@ def main():
         return
 
     main_res = bench_softmax(args.steps, args.warmup, "softmax")
+    ramp = RAMP_MS
+    globals()["RAMP_MS"] = 0.0
+    ms_no_ramp = bench_softmax(args.steps, args.warmup, "softmax")["ms"]   # the same launches right after the warm-up steps, no clock ramp
+    globals()["RAMP_MS"] = ramp
     others = {}
     want = [w for w in args.only.split(",") if w]
     table = [("c2_sigmoid_causal", "sigmoid", lambda: (lambda r: _mfma_entry(r["ms"], r["flops"]))(bench_softmax(args.steps, args.warmup, "sigmoid"))),
@@ -450,11 +589,15 @@ def main():
              ("c3_retnet_chunked", "retnet", lambda: bench_retnet_chunked(args.steps, args.warmup)),
              ("c3_retnet_chunked_bwd", "retnet_bwd", lambda: bench_retnet_chunked(args.steps, args.warmup, backward=True)),
              ("c3_retnet_parallel", "retention", lambda: bench_retnet_parallel(args.steps, args.warmup)),
+             ("c3_retnet_parallel_operator", "retention_operator", lambda: bench_retention_operator(args.steps, args.warmup)),
              ("c3_retnet_parallel_generated_mask", "retention_gamma", lambda: bench_retnet_parallel(args.steps, args.warmup, generated_mask=True)),
              ("c3_retnet_parallel_bwd", "retention_bwd", lambda: bench_retnet_parallel(args.steps, args.warmup, backward=True)),
              ("c4_mamba2_ssd", "mamba", lambda: bench_mamba2(args.steps, args.warmup)),
              ("c4_mamba2_bwd", "mamba_bwd", lambda: bench_mamba2(args.steps, args.warmup, backward=True)),
+             ("c3_retnet_chunked_operator", "retnet_operator", lambda: bench_linear_operators(args.steps, args.warmup, "retnet")),
+             ("c4_mamba2_ssd_operator", "mamba_operator", lambda: bench_linear_operators(args.steps, args.warmup, "mamba")),
              ("c5_mla_decode", "mla", lambda: bench_mla(args.steps, args.warmup)),
+             ("c5_mla_decode_operator", "mla_operator", lambda: bench_mla_operator(args.steps, args.warmup)),
              ("gqa_decode", "decode", lambda: bench_decode(args.steps, args.warmup))]
     cpu_legs = {"c3_retnet_chunked": cpu_baseline_retnet_chunked, "c3_retnet_parallel": cpu_baseline_retention_parallel,
                 "c4_mamba2_ssd": cpu_baseline_mamba2, "c5_mla_decode": cpu_baseline_mla}
@@ -474,6 +617,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "clock_ramp_ms": RAMP_MS,   # device kept busy with the workload for this long before the warm-up steps (see time_gpu)
         "ms_per_step": round(main_res["ms"], 4),
+        "ms_per_step_no_ramp": round(ms_no_ramp, 4),   # timed right after the warm-up launches, without the clock ramp (comparable with figures taken before the ramp existed)
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "causal softmax MHA forward, bf16 in / fp32 accumulate, B=8 H=32 S=4096 D=128",

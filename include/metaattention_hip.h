@@ -129,7 +129,8 @@ typedef struct ma_attn_params {
  * (ma_attn_bwd_workspace_bytes: fp32 [B,H,Sq]) carries delta = sum_d dout*o between the two kernels.  Sequence
  * strides of q, k, v and dout must be non-negative and below 2^26 elements (MA_ERR_UNSUPPORTED otherwise). */
 typedef struct ma_attn_bwd_params {
-  int32_t family; /* ma_attn_family: SOFTMAX, SIGMOID, RELU or RETENTION (Dqk 256, Dv 512) */
+  int32_t family; /* ma_attn_family: SOFTMAX, SIGMOID, RELU or RETENTION; head sizes (dim_qk / dim_v) 128/128, 64/64, 128/256,
+                   * 256/256 and 256/512 for every family, others MA_ERR_UNSUPPORTED */
   int32_t dtype;
   int32_t mask;   /* ma_mask_kind */
   int32_t batch, heads, heads_kv /* 0 = heads */, seqlen_q, seqlen_kv, dim_qk, dim_v;
@@ -193,7 +194,7 @@ typedef struct ma_linear_params {
  * Tensors as in ma_linear_params (bf16, BHSD, contiguous, 16-byte aligned); dout [B,H,T,Dv] bf16; dq, dk, dv are bf16
  * with the shapes of q, k, v (heads that share a q / k head have their gradients summed, :1300-1303); dlog_decay fp32
  * [B,H,T]; dv_scale fp32 [B,H,T], written when v_scale is given (may then still be NULL to skip it).  dim_k 128 or 256,
- * dim_v a multiple of 64.  The workspace (ma_linear_bwd_workspace_bytes, 256-byte aligned) holds the fp32 per-head
+ * dim_v a multiple of 64, at most 4096.  The workspace (ma_linear_bwd_workspace_bytes, 256-byte aligned) holds the fp32 per-head
  * gradients the decay gradient is formed from, and is required. */
 typedef struct ma_linear_bwd_params {
   int32_t dtype;

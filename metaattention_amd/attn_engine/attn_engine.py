@@ -222,6 +222,9 @@ class AttentionEngine:
         if block_mask is not None and block_mask.dim() != 3:
             raise NotImplementedError("block masks are [batch, heads_kv, kv blocks] (decode) or [batch, heads, q blocks, kv blocks] (prefill)")
 
+        # (decided here: inside an autograd function's forward, gradient mode is off)
+        needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
+
         def run(q, k, v):
             B, Sq, H, D = q.shape
             Hkv, Dv = k.shape[2], v.shape[-1]
@@ -256,7 +259,16 @@ class AttentionEngine:
             mask_t = given[form.mask_tensor] if form.mask_tensor else None
             if mask_t is not None and mask_t.dtype != q.dtype:
                 mask_t = mask_t.to(q.dtype)
-            out = attn_fwd(q, k, v, score_mask=mask_t, row_scale=rs, **kw)
+            gamma = None
+            if (mask_t is not None and self.family == "retention" and kw["causal"] and (D, Dv) == (256, 512) and Sq == k.shape[1]
+                    and not needs_grad):
+                gamma = self._decay_gamma_of(given[form.mask_tensor], H, Sq)
+            if gamma is not None:
+                # the multiplier is gamma_h^(i - j) [i >= j]: the kernel generates it instead of reading the tensor once per
+                # batch entry and column half (the row function sees fp32 factors where the tensor holds rounded ones)
+                out = attn_fwd(q, k, v, decay_gamma=gamma, row_scale=rs, **kw)
+            else:
+                out = attn_fwd(q, k, v, score_mask=mask_t, row_scale=rs, **kw)
             self.final_rowscales = rs     # kept for a backward pass, not returned (attn_tl.py:661-667)
             return out
 
@@ -417,6 +429,37 @@ class AttentionEngine:
             # the paged interface of the reference's second MLA backend (attn_engine.py:196-224): mod(q [B,1,Hq,576],
             # k_cache [B * Skv / 64, 64, 1, 576]) -> (out, lse), every sequence full, pages in order
             self.attention = self._call_mla_paged
+
+    def _decay_gamma_of(self, mask, H, S):
+        """fp32 [H] gamma if the retention operator's multiplier tensor `mask` [1, H, S, S] is a per-head exponential decay
+        gamma_h^(i - j) for j <= i (whatever lies above the diagonal is never read under the causal mask), else None.
+        Decided on the device, once per tensor (data pointer, version counter, shape): log2 gamma_h is fitted to the first
+        column, the whole lower triangle is then compared with the regenerated mask to two units in the last place of the
+        tensor's dtype.  examples/retention_parallel.py:25-111 builds exactly such a mask."""
+        key = (mask.data_ptr(), mask._version, tuple(mask.shape), mask.dtype)
+        cache = self.__dict__.setdefault("_gamma_cache", {})
+        if key in cache:
+            return cache[key]
+        gamma = None
+        if mask.dim() == 4 and tuple(mask.shape) == (1, H, S, S) and S >= 2:
+            m = mask[0].float()                                         # [H, S, S]
+            col = m[:, :, 0]                                            # gamma_h^i
+            i = torch.arange(S, device=mask.device, dtype=torch.float32)
+            ok = col > 1e-30
+            lg = torch.log2(col.clamp_min(1e-30))
+            w = torch.where(ok, i, torch.zeros_like(i))                 # least squares through the origin: sum i lg / sum i^2
+            l2g = (w * lg).sum(dim=1) / (w * i).sum(dim=1).clamp_min(1.0)
+            if bool(ok[:, :2].all()) and bool((l2g <= 0).all()) and bool(torch.isfinite(l2g).all()):
+                diff = (i.view(S, 1) - i.view(1, S)).clamp_min(0.0)
+                want = torch.exp2(diff.unsqueeze(0) * l2g.view(H, 1, 1))
+                eps = 2.0 ** (-7 if mask.dtype == torch.bfloat16 else -10)    # two units in the last place
+                lower = (i.view(S, 1) >= i.view(1, S)).unsqueeze(0)
+                if bool((((m - want).abs() <= eps * want + 1e-30) | ~lower).all()):
+                    gamma = torch.exp2(l2g).contiguous()
+        if len(cache) > 8:
+            cache.clear()
+        cache[key] = gamma
+        return gamma
 
     def _call_mla_paged(self, q, k_cache):
         from hip_backend import flash_mla_with_kvcache

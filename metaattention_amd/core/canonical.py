@@ -487,9 +487,10 @@ class _IndexWasRead(Exception):
     pass
 
 
-# a mask_mod that reads its batch / head index is compared over every (batch, head) pair when the whole mask has at
-# most this many elements; beyond that it is taken to depend on them
-_MASK_COMPARE_LIMIT = 1 << 30
+# a mask_mod that reads its batch / head index is compared over every (batch, head) pair (stopping at the first pair that
+# differs) when the whole mask has at most this many elements -- about a second of construction time; beyond that it is
+# taken to depend on them
+_MASK_COMPARE_LIMIT = 1 << 28
 
 
 def classify_mask(mask_mod, B, H, Sq, Skv, block_M=128, block_N=128) -> str:
@@ -503,7 +504,7 @@ def classify_mask(mask_mod, B, H, Sq, Skv, block_M=128, block_N=128) -> str:
     Whether the pattern depends on (batch, head) is decided, not sampled: a mask_mod that never touches
     its b and h arguments (found by calling it with stand-ins that raise on any use) is evaluated once;
     one that does is evaluated for every pair and compared with the first, and where that would be more
-    than 2^30 elements it counts as depending on them (always correct, possibly a larger keep mask than
+    than 2^28 elements it counts as depending on them (always correct, possibly a larger keep mask than
     needed)."""
     if mask_mod is None:
         return "none"
@@ -518,8 +519,8 @@ def classify_mask(mask_mod, B, H, Sq, Skv, block_M=128, block_N=128) -> str:
     try:
         first = dense(_IndexNotToBeRead(), _IndexNotToBeRead())
         reads_bh = False
-    except Exception:   # the stand-in was used (or handed to something that refuses it)
-        first = dense(torch.tensor(0), torch.tensor(0))
+    except (_IndexWasRead, TypeError, RuntimeError):   # the stand-in was used, or handed to something that refuses it;
+        first = dense(torch.tensor(0), torch.tensor(0))  # any other error is the mask_mod's own and is raised here, the first time
         reads_bh = True
     if reads_bh and B * H > 1:
         if B * H * Sq * Skv > _MASK_COMPARE_LIMIT:

@@ -425,13 +425,16 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
 // address, until the process ends.  In host code the array's name is only a handle for hipGetSymbolAddress (passing it to
 // a kernel would hand the kernel a host-side address): the device address is looked up once per device, with that
 // device current, and everything else uses the looked-up pointer.
+// Footprint: the 40 MiB belong to the library's code object, so EVERY process that loads the library holds them on every
+// GPU it initialises, whether or not it ever calls the entry point (16 processes sharing one GPU: 640 MiB of it).
 #define MA_MLA_SCRATCH_BYTES (40u << 20)
+#define MA_MAX_DEVICES 64
 static __device__ __align__(256) unsigned char scratch[MA_MLA_SCRATCH_BYTES];
-static std::atomic<void*> g_scratch_ptr[64];   // by device ordinal
+static std::atomic<void*> g_scratch_ptr[MA_MAX_DEVICES];   // by device ordinal
 
 static void* scratch_of_current_device() {
   const int dev = ma::current_device();
-  if (dev < 0 || dev >= 64) return nullptr;
+  if (dev < 0 || dev >= MA_MAX_DEVICES) return nullptr;   // (the caller has checked the ordinal)
   void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
   if (ptr) return ptr;
   if (ma::hip_check(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) != 0 || !ptr) return nullptr;
@@ -455,6 +458,10 @@ int ma_mla_decode_noalloc(const ma_mla_params* p, ma_stream_t stream) {
   q.workspace = nullptr;
   q.workspace_bytes = 0;
   if (need > 0) {
+    const int dev = ma::current_device();
+    if (dev < 0 || dev >= MA_MAX_DEVICES)
+      return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode_noalloc: device ordinal %d is outside the %d the scratch table covers: use ma_mla_decode "
+                  "with a workspace of the caller's", dev, MA_MAX_DEVICES);
     void* s = scratch_of_current_device();
     if (!s) return fail(MA_ERR_LAUNCH, "ma_mla_decode_noalloc: no address for the scratch array: %s", hipGetErrorString(ma::t_hip_error));
     q.workspace = s;

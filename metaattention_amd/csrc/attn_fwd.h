@@ -12,14 +12,16 @@ struct AttnArgs {
   int64_t qsb, qss, qsh, ksb, kss, ksh, vsb, vss, vsh, osb, oss, osh, msb, msh, msq;
   int B, H, Sq, Skv, num_m_blocks;
   int kv_group;   // query heads per kv head (1 unless grouped-query)
-  // decode-style kv selection (attn_wide_fwd_kernel only): per-batch cache length and a per-(batch, kv head)
+  // The fields from here on are read by attn_wide_fwd_kernel only; a call at 128/128 that sets one of them is routed to
+  // that kernel's 128/128 instantiation by the dispatcher instead of to attn_fwd_kernel.
+  // decode-style kv selection: per-batch cache length and a per-(batch, kv head)
   // mask over blocks of kv_block keys (a multiple of 32)
   const int32_t* kv_lens;
   const uint8_t* kv_block_mask;
   int64_t kbm_sb, kbm_sh, kbm_sq;   // (kbm_sq: stride between blocks of 128 query rows; 0 for the decode form)
   int kv_block;
   int kbm_by_query_head;            // the mask's head axis counts query heads (prefill form) instead of kv heads
-  // element-wise keep mask (attn_wide_fwd_kernel only): uint8 [B|1, H|1, Sq, Skv], 0 = the score is masked
+  // element-wise keep mask: uint8 [B|1, H|1, Sq, Skv], 0 = the score is masked
   const uint8_t* elem_mask;
   int64_t em_sb, em_sh, em_sq;
   // split-kv decode (attn_wide_fwd_kernel with one wave per workgroup): n_split kv ranges per (batch, head,
@@ -29,7 +31,7 @@ struct AttnArgs {
   void* o_part;
   float* lse_part;
   float scale, bias;
-  // additive score terms (attn_wide_fwd_kernel only): x = s * scale + bias + add[b, h, q, kv] + slope_q[h] * q + slope_kv[h] * kv,
+  // additive score terms: x = s * scale + bias + add[b, h, q, kv] + slope_q[h] * q + slope_kv[h] * kv,
   // then, with softcap > 0, x = softcap * tanh(x).  add: fp32 or the tensor dtype, element strides (0 broadcasts).
   const void* add;
   int64_t add_sb, add_sh, add_sq, add_sk;

@@ -140,6 +140,12 @@ __device__ __forceinline__ void dma4_so(const void* base_uniform, uint32_t lane_
 // vmcnt(0), other counters untouched.  The builtin (rather than asm) also tells the
 // compiler's own wait-count bookkeeping that no vector-memory load is pending any more.
 __device__ __forceinline__ void wait_dma() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// vmcnt(N): at most the N most recent vector-memory instructions of this wave are still in flight (they complete in order)
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
 
 // XOR swizzle (in 16-byte chunks) of a row-major LDS tile with >= 16 chunks per row:
 // a bijection on the low 4 row bits, so 128-bit reads of 16 consecutive rows at one

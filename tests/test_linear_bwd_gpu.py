@@ -67,6 +67,58 @@ def test_linear_backward(B, Hq, H, T, Dk, Dv, use_vs):
     _check(got, ref, "linear")
 
 
+@pytest.mark.parametrize("B,Hq,Hk,H,T,Dk,Dv", [
+    (1, 4, 1, 4, 77, 128, 64),     # every head its own q, all heads one k: dk is a group sum (time-reversed scan, weighted by v_scale), dq is not
+    (1, 1, 4, 4, 77, 128, 64),     # the other way round: dq is the group sum
+    (2, 2, 1, 4, 100, 256, 128),   # q shared by pairs, k by all
+])
+def test_linear_backward_with_unequal_q_and_k_head_counts(B, Hq, Hk, H, T, Dk, Dv):
+    """Hq != Hk (linear_tl.py:137-138, 1300-1303: the gradients of the heads that share a q or k head are summed, each side
+    over its own groups), with a value scale and a partial last chunk."""
+    hb = _hb()
+    g = torch.Generator().manual_seed(17 * Hq + Hk + T)
+    q = torch.randn(B, Hq, T, Dk, generator=g).bfloat16()
+    k = (0.1 * torch.randn(B, Hk, T, Dk, generator=g)).bfloat16()
+    v = torch.randn(B, H, T, Dv, generator=g).bfloat16()
+    ld = torch.nn.functional.logsigmoid(torch.randn(B, H, T, generator=g) + 3.0)
+    vs = torch.rand(B, H, T, generator=g) + 0.5
+    dout = (0.5 * torch.randn(B, H, T, Dv, generator=g)).bfloat16()
+    q_scale = Dk ** -0.5
+    print(f"linear bwd B{B} H{H} Hq{Hq} Hk{Hk} T{T} Dk{Dk} Dv{Dv}", flush=True)
+    got = hb.linear_bwd(q.cuda(), k.cuda(), v.cuda(), ld.cuda(), dout.cuda(), q_scale=q_scale, v_scale=vs.cuda())
+    torch.cuda.synchronize()
+    assert got[0].shape == q.shape and got[1].shape == k.shape
+    ref = oracle.linear_attention_grads(q, k, v, ld, dout, q_scale=q_scale, v_scale=vs)
+    _check(got, ref, f"Hq{Hq} Hk{Hk}")
+
+
+def test_mamba2_backward_full_size():
+    """The Mamba2 benchmark shape (B8 H64 T2048 P64 N128, one B / C head for all 64 heads, value scale dt) through
+    ma_linear_bwd: the gradients are linear in dout; and one batch entry against the gradient oracle
+    (testing/test.py:364-385 checks dq, dk, dv of this operator) -- dC and dB, which are sums over the 64 heads of the
+    group, two heads of dx, and the per-token gradients of log decay and dt scale to 3 % of their largest magnitude."""
+    hb = _hb()
+    B, H, T, P, N = 8, 64, 2048, 64, 128
+    Cm, Bm, x, dt, A = inputs.mamba2_inputs(B, H, T, P, N, seed=11)
+    ld = (dt * A.view(1, H, 1)).contiguous()
+    dout = (0.5 * torch.randn(B, H, T, P, generator=torch.Generator().manual_seed(2))).bfloat16()
+    print("linear bwd full size Mamba2 B8 H64 T2048 P64 N128", flush=True)
+    args = [t.cuda() for t in (Cm, Bm, x, ld, dout)]
+    dq, dk, dv, dld, dvs = hb.linear_bwd(*args, v_scale=dt.cuda())
+    dq2, dk2, dv2, dld2, dvs2 = hb.linear_bwd(*args[:4], (dout.float() * 2).bfloat16().cuda(), v_scale=dt.cuda())
+    torch.cuda.synchronize()
+    for a, b2 in ((dq, dq2), (dk, dk2), (dv, dv2)):
+        assert torch.isfinite(a.float()).all()
+        torch.testing.assert_close(b2.float(), 2 * a.float(), rtol=1e-2, atol=2e-3 * float(a.float().abs().max()))   # (bf16 rounding of the doubled result)
+    torch.testing.assert_close(dld2, 2 * dld, rtol=1e-3, atol=1e-3 * float(dld.abs().max()))
+    torch.testing.assert_close(dvs2, 2 * dvs, rtol=1e-3, atol=1e-3 * float(dvs.abs().max()))
+    b = 5
+    ref = oracle.linear_attention_grads(Cm[b:b + 1], Bm[b:b + 1], x[b:b + 1], ld[b:b + 1], dout[b:b + 1], v_scale=dt[b:b + 1], chunk=64)
+    heads = [0, 41]
+    got = (dq[b:b + 1], dk[b:b + 1], dv[b:b + 1, heads], dld[b:b + 1], dvs[b:b + 1])
+    _check(got, (ref[0], ref[1], ref[2][:, heads], ref[3], ref[4]), "mamba2 full size")
+
+
 @pytest.mark.parametrize("B,Hq,H,T,Dk,Dv", [(1, 2, 2, 300, 256, 512), (2, 1, 4, 77, 128, 64), (1, 2, 2, 256, 128, 128)])
 def test_dv_written_by_the_scan_equals_dv_through_the_epilogue(B, Hq, H, T, Dk, Dv):
     """Without a value scale the du scan writes dv itself (bf16, rows back in time order); with a value scale of ones dv goes

@@ -92,6 +92,41 @@ def test_engine_retention_parallel():
     torch.testing.assert_close(mod.final_rowscales.cpu(), r_ref, rtol=1e-3, atol=1e-3)
 
 
+def test_engine_takes_the_generated_mask_path_only_for_exponential_decay_masks():
+    """The operator verifies on the device, once per mask tensor, whether the multiplier is gamma_h^(i - j) below the
+    diagonal; only then does the kernel generate it (examples/retention_parallel.py:25-111 builds such a mask).  Any other
+    multiplier -- here the same mask with one entry changed in place -- runs through the tensor path, bit for bit."""
+    hb = _hb()
+    B, H, S, D, DV = 2, 4, 256, 256, 512
+    mod = specs.retention_parallel(B, H, S, D, DV)
+    q, k, v, mask = _inputs(B, H, S, D, DV, seed=4)
+    qc, kc, vc, mc = q.cuda(), k.cuda(), v.cuda(), mask.cuda()
+    with torch.no_grad():
+        o = mod(qc, kc, vc, mc)
+    torch.cuda.synchronize()
+    found = [g for g in mod._gamma_cache.values() if g is not None]
+    assert len(found) == 1
+    gamma_ref = 1.0 - torch.exp2(-5.0 - torch.arange(H, dtype=torch.float64))
+    torch.testing.assert_close(found[0].cpu().double(), gamma_ref, rtol=2e-5, atol=0)
+    ref, r_ref = oracle.retention_parallel(q, k, v, mask, return_r=True)
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(mod.final_rowscales.cpu(), r_ref, rtol=2e-3, atol=2e-3)   # (fp32 factors against the rounded tensor's)
+    # not an exponential decay any more: the tensor is read
+    mc[0, 1, 200, 17] = 0.5
+    with torch.no_grad():
+        o2 = mod(qc, kc, vc, mc)
+    direct = hb.attn_fwd(qc, kc, vc, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mc)
+    torch.cuda.synchronize()
+    assert any(g is None for g in mod._gamma_cache.values())
+    assert torch.equal(o2, direct)
+    # gradients are asked for: the tensor path (the backward kernels read the tensor)
+    mask2 = mask.cuda()
+    qg = qc.clone().requires_grad_(True)
+    o3 = mod(qg, kc, vc, mask2)
+    torch.cuda.synchronize()
+    assert torch.equal(o3.detach(), hb.attn_fwd(qc, kc, vc, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mask2))
+
+
 def _check_grads(got, ref, what):
     for name, a, b in zip(("dq", "dk", "dv"), got, ref):
         oracle.assert_close(a.float().cpu(), b.float(), rtol=RTOL, atol=ATOL, mismatch_ratio=1e-3, msg=f"{what}:{name}")
@@ -162,3 +197,34 @@ def test_parallel_and_chunked_forms_agree_at_full_size():
     assert float(rs.min()) == 1.0 and float(rs.max()) > 1.0
     # the mask tensor is bf16-rounded gamma^(i-j); the chunked form uses fp32 decays
     torch.testing.assert_close(o_par.transpose(1, 2).float() * rs.unsqueeze(-1), o_chk.float(), rtol=3e-2, atol=4e-3)
+
+
+@pytest.mark.parametrize("generated", [False, True], ids=["mask_tensor", "decay_gamma"])
+def test_retention_full_size_slices_against_the_oracle(generated):
+    """B=8 H=16 S=2048 Dqk=256 Dv=512 (the benchmark shape): three (batch, head) slices of the parallel operator against
+    oracle.retention_parallel (bench_utils.py:1158-1163 restated) at atol 2e-2 / rtol 1e-2, the row scale r at 1e-3 --
+    with the [1,H,S,S] multiplier tensor the reference's operator takes, and with the kernel generating it from gamma."""
+    hb = _hb()
+    B, H, S, D, DV = 8, 16, 2048, 256, 512
+    q, k, v, _ = inputs.retnet_inputs(B, H, S, D, DV, seed=3, layout="bshd")
+    q = (q.float() * 4.0).bfloat16()          # row sums straddle the clamp at 1
+    mask32 = oracle.retention_decay_mask(H, S)                  # fp32 gamma_h^(i - j) [i >= j]
+    rs = torch.full((B, H, S), float("nan"), device="cuda")
+    print(f"retention full size, generated={generated}", flush=True)
+    if generated:
+        gamma = (1.0 - torch.exp2(-5.0 - torch.arange(H, dtype=torch.float64))).float()
+        o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, decay_gamma=gamma.cuda(),
+                        row_scale=rs)
+        ref_mask = mask32                                        # the kernel's factors are fp32
+    else:
+        o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0,
+                        score_mask=mask32.bfloat16().cuda(), row_scale=rs)
+        ref_mask = mask32.bfloat16()                             # the operator reads the rounded tensor
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(rs).all()
+    assert float(rs.min()) == 1.0 and float(rs.max()) > 1.0     # both sides of the clamp occur
+    for b, h in [(0, 0), (7, 15), (3, 9)]:
+        ref, r_ref = oracle.retention_parallel(q[b:b + 1, :, h:h + 1], k[b:b + 1, :, h:h + 1], v[b:b + 1, :, h:h + 1],
+                                               ref_mask[:, h:h + 1], return_r=True)
+        oracle.assert_close(o[b:b + 1, :, h:h + 1].float().cpu(), ref, rtol=RTOL, atol=ATOL)
+        torch.testing.assert_close(rs[b:b + 1, h:h + 1].cpu(), r_ref, rtol=1e-3, atol=1e-3)
