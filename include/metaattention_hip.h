@@ -166,6 +166,14 @@ typedef struct ma_attn_bwd_params {
    * kernels; strides in elements, batch stride 0 broadcasts, rows 8-byte aligned (multiples of 4 elements). */
   const void* score_mask;   int64_t sm_stride_b, sm_stride_h, sm_stride_q;
   const void* score_mask_t; int64_t smt_stride_b, smt_stride_h, smt_stride_k;
+  /* SOFTMAX: the additive score terms and the soft-capping of ma_attn_params, exactly as given to the forward pass (the
+   * reference differentiates whatever score_mod was traced, core/transform/core.py:119-199, core/lower/lower.py:510-525):
+   * the scores are recomputed as x = s * scale + bias + score_add[b, h, q, kv] + pos_slope_q[h] * q + pos_slope_kv[h] * kv
+   * and, with softcap > 0, softcap * tanh(x), whose derivative softcap * (1 - tanh^2 x) multiplies ds.  No gradient is
+   * formed for score_add or the slopes (custom inputs get none in the reference either, attn_tl.py:669-692). */
+  const void* score_add; int64_t sa_stride_b, sa_stride_h, sa_stride_q, sa_stride_kv; int32_t score_add_fp32;
+  const float* pos_slope_q; const float* pos_slope_kv;
+  float softcap;
 } ma_attn_bwd_params;
 
 /* Chunked linear / stateful attention forward.  Replaces the three launches

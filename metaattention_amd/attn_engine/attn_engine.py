@@ -91,10 +91,11 @@ class _Attention(torch.autograd.Function):
     (dq, dk, dv) and None for every custom input."""
 
     @staticmethod
-    def forward(ctx, engine, run, fam_code, bias_t, call_masks, score_mask, q, k, v):
+    def forward(ctx, engine, run, fam_code, bias_t, call_masks, score_mask, extras, q, k, v):
         out = run(q, k, v)
         lse = engine.final_rowscales
         ctx.engine, ctx.fam_code, ctx.bias_t, ctx.call_masks, ctx.score_mask = engine, fam_code, bias_t, call_masks, score_mask
+        ctx.extras = extras
         ctx.save_for_backward(q, k, v, out, *([lse] if lse is not None else []))
         return out
 
@@ -115,8 +116,8 @@ class _Attention(torch.autograd.Function):
             # retention: the multiplier tensor in both orientations (the dk / dv kernels walk down its columns)
             masks = dict(score_mask=ctx.score_mask, score_mask_t=ctx.score_mask.transpose(2, 3).contiguous())
         dq, dk, dv = attn_bwd(q, k, v, out, dout, rest[0] if rest else None, family=ctx.fam_code,
-                              causal=causal, scale=form.scale, bias=form.bias, bias_tensor=ctx.bias_t, **masks)
-        return None, None, None, None, None, None, dq, dk, dv
+                              causal=causal, scale=form.scale, bias=form.bias, bias_tensor=ctx.bias_t, **masks, **ctx.extras)
+        return None, None, None, None, None, None, None, dq, dk, dv
 
 
 class AttentionEngine:
@@ -278,9 +279,13 @@ class AttentionEngine:
             return run(q, k, v).squeeze(1)
 
         if any(t.requires_grad for t in (q, k, v)):
+            extras = {}
             if form.extra or form.softcap is not None:
-                # (the backward kernels take the score as s * scale + bias: additive inputs and soft-capping are forward only)
-                return _ForwardOnly.apply(run, q, k, v)
+                # the softmax backward kernels recompute the score with its additive terms and soft-capping (the custom
+                # inputs themselves get no gradient, as in the reference, attn_tl.py:692); the other families' do not
+                if self.family != "softmax":
+                    return _ForwardOnly.apply(run, q, k, v)
+                extras = self._additive_inputs(given, q.shape[2], q.dtype, q.device)
             score_mask = None
             if self.family == "retention":
                 # head sizes the backward kernels of the retention operator are built for (256 / 512 is its own,
@@ -294,7 +299,7 @@ class AttentionEngine:
             if prefill_blocks is not None:
                 shape = (q.shape[0], q.shape[2], q.shape[1], k.shape[1], q.device)
                 call_masks = lambda: self._block_mask_backward_masks(prefill_blocks, *shape)
-            return _Attention.apply(self, run, fam_code, bias_t, call_masks, score_mask, q, k, v)
+            return _Attention.apply(self, run, fam_code, bias_t, call_masks, score_mask, extras, q, k, v)
         return run(q, k, v)
 
     def _additive_inputs(self, given, H, dtype, device):

@@ -113,7 +113,8 @@ class SymbolScalar:
     def maxbwd(self, a, b): return self.op(G.MaxBwd, [a, b])
 
     def backward(self, grad=None):
-        raise NotImplementedError("symbolic differentiation belongs to the backward kernels, which are not built")
+        raise NotImplementedError("a traced score is not differentiated symbolically here: the gradients of the canonical score "
+                                  "forms come from the library's backward kernels, through the engine's autograd function")
 
 
 class SymbolicArray(SymbolScalar):

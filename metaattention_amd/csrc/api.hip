@@ -180,6 +180,13 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
     for (int64_t x : ms)
       if (x % 4 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: elem_mask rows must be 4-byte aligned");
   }
+  if (p->score_add || p->pos_slope_q || p->pos_slope_kv || p->softcap != 0.f) {
+    if (p->family != MA_ATTN_SOFTMAX)
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: score_add / pos_slope / softcap have backward kernels in the softmax family only");
+    if (p->softcap < 0.f) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: softcap must be >= 0");
+    if (p->score_add && (uintptr_t)p->score_add % (p->score_add_fp32 ? 4 : 2) != 0)
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: score_add must be aligned to its element size");
+  }
   if ((p->kv_block_mask != nullptr) != (p->q_block_mask != nullptr))
     return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: kv_block_mask and q_block_mask go together");
   if (p->kv_block_mask && !p->elem_mask)
@@ -198,6 +205,10 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
   a.dvsb = p->dv_stride_b; a.dvss = p->dv_stride_s; a.dvsh = p->dv_stride_h;
   a.B = p->batch; a.H = p->heads; a.Hkv = hkv; a.Sq = p->seqlen_q; a.Skv = p->seqlen_kv;
   a.kv_group = p->heads / hkv;
+  a.add = p->score_add; a.add_sb = p->sa_stride_b; a.add_sh = p->sa_stride_h; a.add_sq = p->sa_stride_q; a.add_sk = p->sa_stride_kv;
+  a.add_f32 = p->score_add_fp32 != 0;
+  a.slope_q = p->pos_slope_q; a.slope_kv = p->pos_slope_kv;
+  a.softcap = p->softcap;
   a.scale = p->scale; a.bias = p->bias;
   a.elem_mask = p->elem_mask; a.em_sb = p->em_stride_b; a.em_sh = p->em_stride_h; a.em_sq = p->em_stride_q;
   a.elem_mask_t = p->elem_mask_t; a.emt_sb = p->emt_stride_b; a.emt_sh = p->emt_stride_h; a.emt_sk = p->emt_stride_k;

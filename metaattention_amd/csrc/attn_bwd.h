@@ -30,6 +30,15 @@ struct AttnBwdArgs {
   // rows are 8-byte aligned.  `lse` then holds the forward's row scale r.
   const void* smask; int64_t sm_sb, sm_sh, sm_sq;
   const void* smask_t; int64_t smt_sb, smt_sh, smt_sk;
+  // softmax family: additive score terms and soft-capping as in the forward pass (AttnArgs): x = s * scale + bias +
+  // add[b, h, q, kv] + slope_q[h] * q + slope_kv[h] * kv, then softcap * tanh(x) when softcap > 0; add in fp32 or the
+  // tensor dtype, element strides (0 broadcasts).  Any of them set selects the kernels' EXTRA instantiations.
+  const void* add;
+  int64_t add_sb, add_sh, add_sq, add_sk;
+  int add_f32;
+  const float* slope_q;
+  const float* slope_kv;
+  float softcap;
 };
 
 int attn_bwd_dispatch(const AttnBwdArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream);

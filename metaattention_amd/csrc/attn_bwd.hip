@@ -77,6 +77,22 @@ __device__ __forceinline__ float row_ds(float p, float dp, float delta) {
   else return p > 0.f ? dp : 0.f;
 }
 
+// EXTRA instantiations (softmax): the additive terms and the soft-capping of the forward pass, applied to the recomputed
+// raw scores.  `extra` is (add + slope_q q + slope_kv kv) of the element; the scores stay in units of 1 / scale, so that
+// everything behind sees s * scale + bias as before.  With softcap > 0, x = s * scale + bias becomes softcap * tanh(x) and
+// `cap_grad` the derivative softcap * (1 - tanh^2 x), which multiplies ds; tanh(x) = 1 - 2 / (1 + e^(2x)) as in the forward.
+__device__ __forceinline__ float apply_extra(float s, float extra, float scale, float inv_scale, float bias, float softcap, float& cap_grad) {
+  s += extra * inv_scale;
+  cap_grad = 1.f;
+  if (softcap > 0.f) {
+    const float x = s * scale + bias;
+    const float th = 1.f - 2.f * fast_rcp(1.f + fast_exp2(x * (2.f * kLog2e)));
+    s = (softcap * th - bias) * inv_scale;
+    cap_grad = softcap * (1.f - th * th);
+  }
+  return s;
+}
+
 // DMA of a [32 x ROWB bytes] tile whose rows are `row_stride` bytes apart in memory: each instruction
 // moves 1 KB; lane i fetches the 16-byte chunk that belongs at physical position i of that KB.  Rows
 // beyond `limit` are clamped to the last one (whatever is computed from them is masked).
@@ -211,7 +227,7 @@ __device__ __forceinline__ void store_rows(const f32x16 (&acc)[DIM / 32], float 
 // ------------------------------------------------------------------------------------------------
 // dq (and delta)
 // ------------------------------------------------------------------------------------------------
-template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL, bool EXTRA = false>
 __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_kernel(const AttnBwdArgs a) {
   using E = Elem<T>;
   using x8 = typename E::x8;
@@ -357,9 +373,22 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
         }
       }
     }
-    const f32x16 s = mm_rows<T, DQK>(kbase, r, g, qf);     // S^T: lane = row m_lane, element jj = key n0 + 8(jj/4) + 4g + jj%4
+    f32x16 s = mm_rows<T, DQK>(kbase, r, g, qf);           // S^T: lane = row m_lane, element jj = key n0 + 8(jj/4) + 4g + jj%4
     const f32x16 dp = mm_rows<T, DV>(vbase, r, g, dof);   // dP^T, same layout
     x8 dsf[2];
+    float cap_grad[16];
+    if constexpr (EXTRA) {
+      const float inv_scale = 1.f / a.scale;
+      const float sl_q = a.slope_q ? a.slope_q[h] * (float)m_ld : 0.f, sl_kv = a.slope_kv ? a.slope_kv[h] : 0.f;
+      const int64_t add_row = (int64_t)b * a.add_sb + (int64_t)h * a.add_sh + (int64_t)m_ld * a.add_sq;
+#pragma unroll
+      for (int jj = 0; jj < 16; jj++) {
+        const int n = min(n0 + 8 * (jj >> 2) + 4 * g + (jj & 3), a.Skv - 1);
+        float e = sl_q + sl_kv * (float)n;
+        if (a.add) e += a.add_f32 ? ((const float*)a.add)[add_row + (int64_t)n * a.add_sk] : (float)((const T*)a.add)[add_row + (int64_t)n * a.add_sk];
+        s[jj] = apply_extra(s[jj], e, a.scale, inv_scale, bias, a.softcap, cap_grad[jj]);
+      }
+    }
     float mr[16];   // retention: multiplier / r per element
     if constexpr (FAMILY == BF_RETENTION) {
 #pragma unroll
@@ -394,6 +423,7 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
         const bool masked = (CAUSAL && n > m_lane) || n >= a.Skv || ((keep[jj >> 2] >> (8 * (jj & 3))) & 0xffu) == 0;
         float p, ds;
         row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, FAMILY == BF_RETENTION ? mr[jj] : lse2, delta, p, ds);
+        if constexpr (EXTRA) ds *= cap_grad[jj];
         dsf[jj >> 3][jj & 7] = (T)ds;
       }
     } else {
@@ -401,6 +431,7 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
       for (int jj = 0; jj < 16; jj++) {
         float p, ds;
         row_fn_bwd<FAMILY>(s[jj], dp[jj], false, c_scale, c_bias, a.scale, bias, FAMILY == BF_RETENTION ? mr[jj] : lse2, delta, p, ds);
+        if constexpr (EXTRA) ds *= cap_grad[jj];
         dsf[jj >> 3][jj & 7] = (T)ds;
       }
     }
@@ -420,7 +451,7 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
 // fragments take 192 registers at 128/128, which leaves one wave per SIMD (forcing two makes the compiler
 // spill the fragments and is slower); computing dv and dk in two launches (the scores are then computed once
 // more) lets each run two waves per SIMD.
-template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL, int WHAT>
+template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL, int WHAT, bool EXTRA = false>
 __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK + DV >= 512 ? 1 : 2))) void attn_bwd_dkv_kernel(const AttnBwdArgs a) {
   constexpr bool DO_DV = (WHAT & 1) != 0, DO_DK = (WHAT & 2) != 0;
   using E = Elem<T>;
@@ -593,7 +624,20 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
         }
       }
     }
-    const f32x16 s = mm_rows<T, DQK>(qbase, r, g, kf);     // S: lane = key n_lane, element jj = row m0 + 8(jj/4) + 4g + jj%4
+    f32x16 s = mm_rows<T, DQK>(qbase, r, g, kf);           // S: lane = key n_lane, element jj = row m0 + 8(jj/4) + 4g + jj%4
+    float cap_grad[16];
+    if constexpr (EXTRA) {
+      const float inv_scale = 1.f / a.scale;
+      const float sl_q = a.slope_q ? a.slope_q[h] : 0.f, sl_kv = a.slope_kv ? a.slope_kv[h] * (float)n_ld : 0.f;
+      const int64_t add_col = (int64_t)b * a.add_sb + (int64_t)h * a.add_sh + (int64_t)n_ld * a.add_sk;
+#pragma unroll
+      for (int jj = 0; jj < 16; jj++) {
+        const int m = min(m0 + 8 * (jj >> 2) + 4 * g + (jj & 3), a.Sq - 1);
+        float e = sl_q * (float)m + sl_kv;
+        if (a.add) e += a.add_f32 ? ((const float*)a.add)[add_col + (int64_t)m * a.add_sq] : (float)((const T*)a.add)[add_col + (int64_t)m * a.add_sq];
+        s[jj] = apply_extra(s[jj], e, a.scale, inv_scale, bias, a.softcap, cap_grad[jj]);
+      }
+    }
     f32x16 dp;
     if constexpr (DO_DK) dp = mm_rows<T, DV>(dobase, r, g, vf);   // dP, same layout
     else
@@ -633,6 +677,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
         row_fn_bwd<FAMILY>(s[jj], dp[jj], masked, c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX || FAMILY == BF_RETENTION ? lse2[jj] : 0.f,
                            FAMILY == BF_SOFTMAX ? dl[jj] : 0.f, p, ds);
         if (masked) ds = 0.f;
+        if constexpr (EXTRA) ds *= cap_grad[jj];
         pf[jj >> 3][jj & 7] = (T)p;
         dsf[jj >> 3][jj & 7] = (T)ds;
       }
@@ -642,6 +687,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
         float p, ds;
         row_fn_bwd<FAMILY>(s[jj], dp[jj], false, c_scale, c_bias, a.scale, bias, FAMILY == BF_SOFTMAX || FAMILY == BF_RETENTION ? lse2[jj] : 0.f,
                            FAMILY == BF_SOFTMAX ? dl[jj] : 0.f, p, ds);
+        if constexpr (EXTRA) ds *= cap_grad[jj];
         pf[jj >> 3][jj & 7] = (T)p;
         dsf[jj >> 3][jj & 7] = (T)ds;
       }
@@ -1037,6 +1083,24 @@ static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   static std::atomic<uint64_t> lds_ok{0};
   if (allow_lds(lds_ok, lds, k1, k2, k3) != 0) return -1;
   AttnBwdArgs args = a;
+  if (a.add || a.slope_q || a.slope_kv || a.softcap != 0.f) {
+    // additive score terms / soft-capping: instantiations of their own (softmax family), dk and dv by the two-launch kernels
+    if constexpr (FAMILY == BF_SOFTMAX) {
+      auto e1 = attn_bwd_dq_kernel<T, DQK, DV, FAMILY, CAUSAL, true>;
+      auto e2 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL, SPLIT ? 1 : 3, true>;
+      auto e3 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL, 2, true>;
+      static std::atomic<uint64_t> elds_ok{0};
+      if (allow_lds(elds_ok, lds, e1, e2, e3) != 0) return -1;
+      args.num_blocks = (a.Sq + 127) / 128;
+      hipLaunchKernelGGL(e1, dim3((unsigned)(args.num_blocks * a.B * a.H)), dim3(256), lds, stream, args);
+      args.num_blocks = (a.Skv + 127) / 128;
+      hipLaunchKernelGGL(e2, dim3((unsigned)(args.num_blocks * a.B * a.Hkv)), dim3(256), lds, stream, args);
+      if (SPLIT) hipLaunchKernelGGL(e3, dim3((unsigned)(args.num_blocks * a.B * a.Hkv)), dim3(256), lds, stream, args);
+      return launch_status();
+    } else {
+      return -2;
+    }
+  }
   args.num_blocks = (a.Sq + 127) / 128;
   hipLaunchKernelGGL(k1, dim3((unsigned)(args.num_blocks * a.B * a.H)), dim3(256), lds, stream, args);
   args.num_blocks = (a.Skv + 127) / 128;

@@ -80,6 +80,8 @@ class AttnBwdParams(Structure):
         ("q_block_mask", c_void_p), ("qbm_stride_b", c_int64), ("qbm_stride_h", c_int64), ("qbm_stride_k", c_int64),
         ("score_mask", c_void_p), ("sm_stride_b", c_int64), ("sm_stride_h", c_int64), ("sm_stride_q", c_int64),
         ("score_mask_t", c_void_p), ("smt_stride_b", c_int64), ("smt_stride_h", c_int64), ("smt_stride_k", c_int64),
+        ("score_add", c_void_p), ("sa_stride_b", c_int64), ("sa_stride_h", c_int64), ("sa_stride_q", c_int64), ("sa_stride_kv", c_int64),
+        ("score_add_fp32", c_int32), ("pos_slope_q", c_void_p), ("pos_slope_kv", c_void_p), ("softcap", c_float),
     ]
 
 
@@ -290,7 +292,8 @@ def attn_fwd(q, k, v, *, family: int, causal: bool, scale: float, bias: float = 
 
 
 def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, bias: float = 0.0, bias_tensor=None,
-             elem_mask=None, elem_mask_t=None, kv_block_mask=None, q_block_mask=None, score_mask=None, score_mask_t=None):
+             elem_mask=None, elem_mask_t=None, kv_block_mask=None, q_block_mask=None, score_mask=None, score_mask_t=None,
+             score_add=None, pos_slope_q=None, pos_slope_kv=None, softcap: float = 0.0):
     """Gradients (dq, dk, dv) of the parallel attention forward on BSHD tensors.  ``o`` and ``lse``
     (fp32 [B,H,Sq]) are the forward pass's output and row scale (softmax and retention; None otherwise),
     ``dout`` the gradient of ``o``.  The retention family takes the forward's multiplier tensor ``score_mask``
@@ -298,8 +301,11 @@ def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, 
     row scale as a constant, as the reference's OnlineRetention.backward does.  ``elem_mask`` (the forward pass's keep mask, [1|B, 1|H, Sq, Skv]) comes with
     its transpose ``elem_mask_t`` [1|B, 1|H, Skv, Sq]; both with rows at 4-byte aligned addresses.  Optional tile masks
     for skipping: ``kv_block_mask`` [1|B, 1|H, ceil(Sq/128), ceil(Skv/32)] and ``q_block_mask`` [1|B, 1|H, ceil(Skv/128),
-    ceil(Sq/32)] (a tile is kept when any of its elements is)."""
-    _require_gpu(q, k, v, o, dout, lse, bias_tensor, elem_mask, elem_mask_t, kv_block_mask, q_block_mask, score_mask, score_mask_t)
+    ceil(Sq/32)] (a tile is kept when any of its elements is).  ``score_add``, ``pos_slope_q`` / ``pos_slope_kv`` and
+    ``softcap`` (softmax family) are the forward pass's additive score terms and soft-capping, given again unchanged; they
+    receive no gradients of their own."""
+    _require_gpu(q, k, v, o, dout, lse, bias_tensor, elem_mask, elem_mask_t, kv_block_mask, q_block_mask, score_mask, score_mask_t,
+                 score_add, pos_slope_q, pos_slope_kv)
     B, Sq, H, Dqk = q.shape
     Skv, Hkv, Dv = k.shape[1], k.shape[2], v.shape[-1]
     assert k.shape == (B, Skv, Hkv, Dqk) and v.shape == (B, Skv, Hkv, Dv) and dout.shape == (B, Sq, H, Dv) and H % Hkv == 0
@@ -351,6 +357,18 @@ def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, 
             setattr(p, f"{pre}_stride_b", t.stride(0) if t.shape[0] > 1 else 0)
             setattr(p, f"{pre}_stride_h", t.stride(1))
             setattr(p, f"{pre}_stride_{last}", t.stride(2))
+    if score_add is not None:
+        assert score_add.dim() == 4 and score_add.dtype in (torch.float32, q.dtype)
+        for ax, full in enumerate((B, H, Sq, Skv)):
+            assert score_add.shape[ax] in (1, full), f"score_add {tuple(score_add.shape)} does not broadcast to {(B, H, Sq, Skv)}"
+        st = [score_add.stride(ax) if score_add.shape[ax] > 1 else 0 for ax in range(4)]
+        p.score_add, p.score_add_fp32 = score_add.data_ptr(), int(score_add.dtype == torch.float32)
+        p.sa_stride_b, p.sa_stride_h, p.sa_stride_q, p.sa_stride_kv = st
+    for name, t in (("pos_slope_q", pos_slope_q), ("pos_slope_kv", pos_slope_kv)):
+        if t is not None:
+            assert t.dtype == torch.float32 and t.numel() == H and t.is_contiguous()
+            setattr(p, name, t.data_ptr())
+    p.softcap = float(softcap)
     lib = load_library()
     need = lib.ma_attn_bwd_workspace_bytes(ctypes.byref(p))
     if need:

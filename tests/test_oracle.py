@@ -269,7 +269,11 @@ def test_attention_grads_vs_finite_differences_and_sdpa():
     v = torch.randn(B, S, Hkv, DV, generator=g, dtype=torch.float64)
     dout = torch.randn(B, S, H, DV, generator=g, dtype=torch.float64)
     cases = [(oracle.softmax_attention, dict(causal=True)), (oracle.sigmoid_attention, dict(bias=-0.7, causal=True, softmax_scale=0.3)),
-             (oracle.relu_attention, dict())]
+             (oracle.relu_attention, dict()),
+             # (the additive-term form the backward kernels of the softmax family are checked against)
+             (oracle.biased_attention, dict(add=torch.randn(B, H, S, S, generator=g, dtype=torch.float64), causal=True, softmax_scale=0.3)),
+             (oracle.biased_attention, dict(add=torch.randn(1, H, 1, S, generator=g, dtype=torch.float64), causal=True,
+                                            softmax_scale=0.4, bias=0.2, softcap=1.5))]
     for fwd, kw in cases:
         dq, dk, dv = oracle.attention_grads(fwd, q, k, v, dout, **kw)
         f = lambda q_, k_, v_: float((fwd(q_, k_, v_, compute_dtype=torch.float64, **kw) * dout).sum())
@@ -285,6 +289,15 @@ def test_attention_grads_vs_finite_differences_and_sdpa():
                                                          vs.repeat_interleave(2, dim=2).transpose(1, 2), is_causal=True)
     o.transpose(1, 2).backward(dout)
     dq, dk, dv = oracle.attention_grads(oracle.softmax_attention, q, k, v, dout, causal=True)
+    for a, b in ((dq, qs.grad), (dk, ks.grad), (dv, vs.grad)):
+        torch.testing.assert_close(a, b, rtol=1e-9, atol=1e-9)
+    # an additive tile is SDPA's float attn_mask
+    add = torch.randn(B, H, S, S, generator=g, dtype=torch.float64)
+    qs, ks, vs = (t.clone().requires_grad_(True) for t in (q, k, v))
+    o = torch.nn.functional.scaled_dot_product_attention(qs.transpose(1, 2), ks.repeat_interleave(2, dim=2).transpose(1, 2),
+                                                         vs.repeat_interleave(2, dim=2).transpose(1, 2), attn_mask=add)
+    o.transpose(1, 2).backward(dout)
+    dq, dk, dv = oracle.attention_grads(oracle.biased_attention, q, k, v, dout, add=add)
     for a, b in ((dq, qs.grad), (dk, ks.grad), (dv, vs.grad)):
         torch.testing.assert_close(a, b, rtol=1e-9, atol=1e-9)
 
