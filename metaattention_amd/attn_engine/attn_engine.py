@@ -11,6 +11,7 @@ the current stream.
 from __future__ import annotations
 
 import math
+import weakref
 
 import torch
 
@@ -438,13 +439,14 @@ class AttentionEngine:
     def _decay_gamma_of(self, mask, H, S):
         """fp32 [H] gamma if the retention operator's multiplier tensor `mask` [1, H, S, S] is a per-head exponential decay
         gamma_h^(i - j) for j <= i (whatever lies above the diagonal is never read under the causal mask), else None.
-        Decided on the device, once per tensor (data pointer, version counter, shape): log2 gamma_h is fitted to the first
+        Decided on the device, once per tensor object and version counter: log2 gamma_h is fitted to the first
         column, the whole lower triangle is then compared with the regenerated mask to two units in the last place of the
         tensor's dtype.  examples/retention_parallel.py:25-111 builds exactly such a mask."""
-        key = (mask.data_ptr(), mask._version, tuple(mask.shape), mask.dtype)
-        cache = self.__dict__.setdefault("_gamma_cache", {})
-        if key in cache:
-            return cache[key]
+        # (remembered per tensor OBJECT and version counter: an address alone could be a new tensor in recycled memory)
+        cache = self.__dict__.setdefault("_gamma_cache", [])
+        for ref, version, known in cache:
+            if ref() is mask and version == mask._version:
+                return known
         gamma = None
         if mask.dim() == 4 and tuple(mask.shape) == (1, H, S, S) and S >= 2:
             m = mask[0].float()                                         # [H, S, S]
@@ -461,9 +463,8 @@ class AttentionEngine:
                 lower = (i.view(S, 1) >= i.view(1, S)).unsqueeze(0)
                 if bool((((m - want).abs() <= eps * want + 1e-30) | ~lower).all()):
                     gamma = torch.exp2(l2g).contiguous()
-        if len(cache) > 8:
-            cache.clear()
-        cache[key] = gamma
+        cache[:] = [e for e in cache if e[0]() is not None and e[0]() is not mask][-7:]
+        cache.append((weakref.ref(mask), mask._version, gamma))
         return gamma
 
     def _call_mla_paged(self, q, k_cache):

@@ -104,7 +104,7 @@ def test_engine_takes_the_generated_mask_path_only_for_exponential_decay_masks()
     with torch.no_grad():
         o = mod(qc, kc, vc, mc)
     torch.cuda.synchronize()
-    found = [g for g in mod._gamma_cache.values() if g is not None]
+    found = [g for _, _, g in mod._gamma_cache if g is not None]
     assert len(found) == 1
     gamma_ref = 1.0 - torch.exp2(-5.0 - torch.arange(H, dtype=torch.float64))
     torch.testing.assert_close(found[0].cpu().double(), gamma_ref, rtol=2e-5, atol=0)
@@ -117,8 +117,15 @@ def test_engine_takes_the_generated_mask_path_only_for_exponential_decay_masks()
         o2 = mod(qc, kc, vc, mc)
     direct = hb.attn_fwd(qc, kc, vc, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mc)
     torch.cuda.synchronize()
-    assert any(g is None for g in mod._gamma_cache.values())
+    assert any(g is None for _, _, g in mod._gamma_cache)
     assert torch.equal(o2, direct)
+    # another tensor object is looked at afresh, whatever address it lives at (a new mask may sit in recycled memory)
+    del mc
+    other = torch.tril(torch.rand(1, H, S, S, device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))).bfloat16()
+    with torch.no_grad():
+        o4 = mod(qc, kc, vc, other)
+    torch.cuda.synchronize()
+    assert torch.equal(o4, hb.attn_fwd(qc, kc, vc, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=other))
     # gradients are asked for: the tensor path (the backward kernels read the tensor)
     mask2 = mask.cuda()
     qg = qc.clone().requires_grad_(True)
