@@ -116,7 +116,10 @@ __global__ __launch_bounds__(256) void grads_kernel(LinBwdArgs a, const float* _
 // The same for heads that share their q and k heads in groups of G = H / Hq (Hq == Hk < H): LPT lanes per (batch, shared
 // head, token) walk the G heads of the group, so that dq and dk of the shared head -- the sums over the group
 // (linear_tl.py:1300-1303) -- are formed while the per-head scan outputs pass through once.
-template <int LPT>
+// DKB: the dk scan has left its per-head output as bf16 in time order (dkh_rev then points at [B,H,T,Dk] bf16; the
+// reference rounds its per-head dk to the tensor dtype before the group sum as well), and the k . dk term of the decay
+// gradient comes from the du scan instead, in fp32: k_s . dk_s = sum_{t>=s} A_ts (do_t . u_s) = u_s . du_s = v_scale_s (v_s . du_s).
+template <int LPT, bool DKB = false>
 __global__ __launch_bounds__(256) void grads_shared_kernel(LinBwdArgs a, const float* __restrict__ dqh, const float* __restrict__ dkh_rev,
                                                           const float* __restrict__ du_rev, float* __restrict__ dG, int np, int64_t piece_stride) {
   const int sub = threadIdx.x % LPT;
@@ -146,7 +149,13 @@ __global__ __launch_bounds__(256) void grads_shared_kernel(LinBwdArgs a, const f
     r.vs = a.v_scale ? a.v_scale[tk] : 1.f;
     if (has_c) {
       r.gq = *(const f32x4*)(dqh + tk * a.Dk + c);
-      r.gk = *(const f32x4*)(dkh_rev + rtok * a.Dk + c);
+      if constexpr (DKB) {
+        const bf16x4 g4 = *(const bf16x4*)((const __bf16*)dkh_rev + tk * a.Dk + c);
+#pragma unroll
+        for (int i = 0; i < 4; i++) r.gk[i] = (float)g4[i];
+      } else {
+        r.gk = *(const f32x4*)(dkh_rev + rtok * a.Dk + c);
+      }
     }
     if (has_v) {
       r.gu = *(const f32x4*)(du_rev + rtok * a.Dv + cv0);
@@ -170,12 +179,12 @@ __global__ __launch_bounds__(256) void grads_shared_kernel(LinBwdArgs a, const f
       f32x4 gq = row.gq, gk = row.gk;
       for (int p = 1; p < np; p++) {
         gq += *(const f32x4*)(dqh + p * piece_stride + tk * a.Dk + c);
-        gk += *(const f32x4*)(dkh_rev + p * piece_stride + rtok * a.Dk + c);
+        if constexpr (!DKB) gk += *(const f32x4*)(dkh_rev + p * piece_stride + rtok * a.Dk + c);
       }
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         gk[i] *= vs;
-        acc += qv[i] * gq[i] - kv[i] * gk[i];
+        acc += DKB ? qv[i] * gq[i] : qv[i] * gq[i] - kv[i] * gk[i];
         sq[i] += gq[i];
         sk[i] += gk[i];
       }
@@ -196,7 +205,7 @@ __global__ __launch_bounds__(256) void grads_shared_kernel(LinBwdArgs a, const f
     acc = lanes_sum<LPT>(acc);
     acc_vs = lanes_sum<LPT>(acc_vs);
     if (live && sub == 0) {
-      dG[tk] = acc;
+      dG[tk] = DKB ? acc - vs * acc_vs : acc;
       if (a.dv_scale) a.dv_scale[tk] = acc_vs;
     }
   }
@@ -369,25 +378,33 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
     return rc;
   if (direct_dv) du = nullptr;
 
-  // dk (per head, reversed, before its v_scale factor) = LA(R v, R do, R q), contraction over the value columns
+  // dk (per head, reversed, before its v_scale factor) = LA(R v, R do, R q), contraction over the value columns.
+  // Heads in groups that share q and k, with a v_scale and a contraction of one piece (Mamba2): the scan leaves bf16 in
+  // time order (see grads_shared_kernel).
+  const bool dk_bf16 = a.Hq == a.Hk && a.Hq != a.H && du && sl.n == 1;
   if (side_by_side) {
     if (const int rc = scan_launch(Operand{v_p, a.H, a.Dv}, Operand{do_p, a.H, a.Dv}, Operand{q_p, a.Hq, a.Dk}, true, sl.w[0], a.Dk, grev, nullptr, dkh, false, np))
       return rc;
   }
   for (int s = 0; s < sl.n && !side_by_side; s++) {
     Operand qs{v_p + sl.c0[s], a.H, a.Dv}, ks{do_p + sl.c0[s], a.H, a.Dv};
-    if (const int rc = scan_launch(qs, ks, Operand{q_p, a.Hq, a.Dk}, true, sl.w[s], a.Dk, grev, nullptr, dkh, s > 0, 1, piece_cols(s))) return rc;
+    if (const int rc = scan_launch(qs, ks, Operand{q_p, a.Hq, a.Dk}, true, sl.w[s], a.Dk, grev, nullptr, dkh, s > 0, 1, piece_cols(s), dk_bf16)) return rc;
   }
 
   if (a.Hq == a.Hk && a.Hq != a.H) {
     // heads in groups that share q and k: gradients, group sums and conversions in one pass over the scan outputs
     const int64_t n_tok = (int64_t)a.B * a.Hq * a.T;
-    if (a.Dk > 128)
-      hipLaunchKernelGGL(grads_shared_kernel<64>, dim3((unsigned)((n_tok + 3) / 4)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh,
-                         (const float*)du, dG, np, piece_stride);
+    const dim3 grid64((unsigned)((n_tok + 3) / 4)), grid32((unsigned)((n_tok + 7) / 8));
+    if (a.Dk > 128 && dk_bf16)
+      hipLaunchKernelGGL((grads_shared_kernel<64, true>), grid64, dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh, (const float*)du, dG, np,
+                         piece_stride);
+    else if (a.Dk > 128)
+      hipLaunchKernelGGL(grads_shared_kernel<64>, grid64, dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh, (const float*)du, dG, np, piece_stride);
+    else if (dk_bf16)
+      hipLaunchKernelGGL((grads_shared_kernel<32, true>), grid32, dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh, (const float*)du, dG, np,
+                         piece_stride);
     else
-      hipLaunchKernelGGL(grads_shared_kernel<32>, dim3((unsigned)((n_tok + 7) / 8)), dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh,
-                         (const float*)du, dG, np, piece_stride);
+      hipLaunchKernelGGL(grads_shared_kernel<32>, grid32, dim3(256), 0, stream, a, (const float*)dqh, (const float*)dkh, (const float*)du, dG, np, piece_stride);
     hipLaunchKernelGGL(suffix_sum_kernel, dim3((unsigned)(a.B * a.H)), dim3(256), 0, stream, a.dlog_decay, (const float*)dG, a.T);
     return launch_status();
   }

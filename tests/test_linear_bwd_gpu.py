@@ -122,8 +122,9 @@ def test_mamba2_backward_full_size():
 @pytest.mark.parametrize("B,Hq,H,T,Dk,Dv", [(1, 2, 2, 300, 256, 512), (2, 1, 4, 77, 128, 64), (1, 2, 2, 256, 128, 128)])
 def test_dv_written_by_the_scan_equals_dv_through_the_epilogue(B, Hq, H, T, Dk, Dv):
     """Without a value scale the du scan writes dv itself (bf16, rows back in time order); with a value scale of ones dv goes
-    through the fp32 workspace and the epilogue kernel.  Both round the same fp32 numbers, so every gradient is the same bit
-    for bit, also with a partial last chunk and with the sequence cut into segments."""
+    through the fp32 workspace and the epilogue kernel.  Both round the same fp32 numbers, so dv (and, where every head has
+    its own q and k, every gradient) is the same bit for bit, also with a partial last chunk and with the sequence cut into
+    segments."""
     hb = _hb()
     g = torch.Generator().manual_seed(B * T + Dv)
     q = torch.randn(B, Hq, T, Dk, generator=g).bfloat16().cuda()
@@ -136,7 +137,13 @@ def test_dv_written_by_the_scan_equals_dv_through_the_epilogue(B, Hq, H, T, Dk, 
     ones = hb.linear_bwd(q, k, v, ld, dout, q_scale=Dk ** -0.5, v_scale=torch.ones(B, H, T, device="cuda"))
     torch.cuda.synchronize()
     for name, a, b in zip(("dq", "dk", "dv", "dlog_decay"), direct, ones):
-        assert torch.equal(a, b), f"{name}: {float((a.float() - b.float()).abs().max())}"
+        if Hq < H and name in ("dk", "dlog_decay"):
+            # heads that share q and k, with a value scale: the per-head dk passes through bf16 before the group sum (as in
+            # the reference, linear_tl.py:1300-1303) and the decay gradient takes k . dk from the du scan -- same
+            # quantities, other roundings
+            oracle.assert_close(a.float().cpu(), b.float().cpu(), rtol=2e-2, atol=2e-2 * float(b.float().abs().max()), msg=name)
+        else:
+            assert torch.equal(a, b), f"{name}: {float((a.float() - b.float()).abs().max())}"
 
 
 def test_engine_mamba2_backward():
