@@ -77,3 +77,62 @@ def test_wrong_custom_tensor_count():
     q = torch.zeros(1, 128, 1, 128, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(TypeError):
         mod(q, q, q)
+
+
+def _replay_against_eager(run, statics, fresh_inputs, replays=3):
+    """Captures run() in a HIP graph, then replays it with new contents in the static input tensors, the program's own
+    eager calls and synchronisations between the replays, and compares every replay with the eager result bit for bit."""
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        for _ in range(2):
+            run()                      # warm-up outside capture: first-call set-up (LDS limits, mask analysis) happens here
+    torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = run()
+    for i in range(replays):
+        for dst, src in zip(statics, fresh_inputs(i)):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = run()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {i}"
+        assert torch.isfinite(got.float()).all()
+
+
+def test_operators_replay_in_a_hip_graph():
+    """A serving loop captures its step once and replays it: the forward operators (parallel softmax, chunked RetNet, MLA
+    decode through its workspace and through the allocation-free entry point) enqueue nothing but kernels on the current
+    stream, so a captured call replays to the eager call's bits with new inputs in place."""
+    from metaattention_amd import hip_backend as hb
+    hb.load_library()
+    dev = "cuda"
+    # parallel softmax, causal
+    B, H, S, D = 1, 4, 384, 128
+    mod = specs.softmax_attention(B, H, S, D, D)
+    q, k, v = (t.to(dev) for t in inputs.softmax_inputs(B, H, S, D, D, seed=21))
+    fresh = lambda i: [t.to(dev) for t in inputs.softmax_inputs(B, H, S, D, D, seed=30 + i)]
+    with torch.no_grad():
+        _replay_against_eager(lambda: mod(q, k, v), (q, k, v), fresh)
+    # chunked RetNet
+    Bl, Hl, T, Dk, Dv = 1, 2, 160, 256, 512
+    lin = specs.retnet_recurrent(Bl, Hl, T, Dk, Dv)
+    gen = lambda seed: [torch.randn(Bl, Hl, T, Dk, generator=torch.Generator().manual_seed(seed)).bfloat16().to(dev),
+                        (0.1 * torch.randn(Bl, Hl, T, Dk, generator=torch.Generator().manual_seed(seed + 1))).bfloat16().to(dev),
+                        torch.randn(Bl, Hl, T, Dv, generator=torch.Generator().manual_seed(seed + 2)).bfloat16().to(dev)]
+    ql, kl, vl = gen(40)
+    decay = (1 - torch.exp2(-5 - torch.arange(Hl, dtype=torch.float32)))[None, :, None].expand(Bl, Hl, T).contiguous().to(dev)
+    with torch.no_grad():
+        _replay_against_eager(lambda: lin(ql, kl, vl, decay), (ql, kl, vl), lambda i: gen(50 + 3 * i))
+    # MLA decode with kv splits (workspace from the caching allocator's graph pool) and without any allocation
+    Bm, Hq, Skv = 4, 128, 1024
+    qm, qpe, kv, kpe = (t.to(dev) for t in inputs.mla_inputs(Bm, Hq, Skv, 512, 64, seed=60))
+    fresh_m = lambda i: [t.to(dev) for t in inputs.mla_inputs(Bm, Hq, Skv, 512, 64, seed=61 + i)]
+    scale = 576 ** -0.5
+    _replay_against_eager(lambda: hb.mla_decode(qm, qpe, kv, kpe, scale=scale, num_split=4), (qm, qpe, kv, kpe), fresh_m)
+    out = torch.empty(Bm, 1, Hq, 512, dtype=torch.bfloat16, device=dev)
+    _replay_against_eager(lambda: hb.mla_decode(qm, qpe, kv, kpe, scale=scale, num_split=4, out=out, no_alloc=True), (qm, qpe, kv, kpe), fresh_m)
