@@ -261,7 +261,7 @@ def bench_retention_operator(steps, warmup):
     mask = (torch.exp2(diff.clamp(min=0).unsqueeze(0) * torch.log2(gam).view(H, 1, 1)) * (diff >= 0)).unsqueeze(0).bfloat16()
     with torch.no_grad():
         ms = time_gpu(lambda: mod(q, k, v, mask), steps, warmup)
-    generated = any(gm is not None for gm in getattr(mod, "_gamma_cache", {}).values())
+    generated = bool(getattr(mod, "last_call_generated_mask", False))
     return _mfma_entry(ms, 0.5 * 2.0 * B * H * S * S * (D + DV),
                        "c3_retnet_parallel through the AttentionEngine operator, mod(q, k, v, mask) with the [1,H,S,S] bf16 decay mask; "
                        "the operator found the mask to be gamma_h^(i-j) and the kernel generates it" if generated else
@@ -604,9 +604,13 @@ def main():
     for name, key, fn in table:
         if want and (want == ["none"] or not any(key.startswith(w) or w in name for w in want)):
             continue
-        others[name] = fn()
+        try:
+            others[name] = fn()
+        except Exception as e:     # (a workload that fails is reported in its place; the headline line is still printed)
+            others[name] = {"error": f"{type(e).__name__}: {e}"}
+            print(f"bench.py: workload {name} failed: {e!r}", file=sys.stderr)
         torch.cuda.empty_cache()
-        if name in cpu_legs and not args.no_cpu_baseline:
+        if name in cpu_legs and not args.no_cpu_baseline and "error" not in others[name]:
             others[name]["cpu_baseline"] = cpu_legs[name]()
 
     traffic, traffic_from = profiled_traffic(ATTN_FWD_PROFILE, ATTN_FWD_KERNEL)

@@ -265,6 +265,7 @@ class AttentionEngine:
             if (mask_t is not None and self.family == "retention" and kw["causal"] and (D, Dv) == (256, 512) and Sq == k.shape[1]
                     and not needs_grad):
                 gamma = self._decay_gamma_of(given[form.mask_tensor], H, Sq)
+            self.last_call_generated_mask = gamma is not None     # (which of the two forms the last call took)
             if gamma is not None:
                 # the multiplier is gamma_h^(i - j) [i >= j]: the kernel generates it instead of reading the tensor once per
                 # batch entry and column half (the row function sees fp32 factors where the tensor holds rounded ones)

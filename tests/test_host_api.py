@@ -307,3 +307,13 @@ def test_spec_forward_backward_combine_are_checked_against_the_library():
         with pytest.raises(NotImplementedError) as ei:
             identify_online_func(bad())
         assert word in str(ei.value)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py --gpus N with N > 1 exits with a message (the build uses one GPU); decided before anything touches a GPU."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120, cwd=root)
+    assert r.returncode != 0 and "one gpu" in (r.stderr + r.stdout).lower()
