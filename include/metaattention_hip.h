@@ -166,7 +166,8 @@ typedef struct ma_attn_bwd_params {
    * kernels; strides in elements, batch stride 0 broadcasts, rows 8-byte aligned (multiples of 4 elements). */
   const void* score_mask;   int64_t sm_stride_b, sm_stride_h, sm_stride_q;
   const void* score_mask_t; int64_t smt_stride_b, smt_stride_h, smt_stride_k;
-  /* SOFTMAX: the additive score terms and the soft-capping of ma_attn_params, exactly as given to the forward pass (the
+  /* SOFTMAX, SIGMOID, RELU (softcap: SOFTMAX only, as in the forward): the additive score terms and the soft-capping of
+   * ma_attn_params, exactly as given to the forward pass (the
    * reference differentiates whatever score_mod was traced, core/transform/core.py:119-199, core/lower/lower.py:510-525):
    * the scores are recomputed as x = s * scale + bias + score_add[b, h, q, kv] + pos_slope_q[h] * q + pos_slope_kv[h] * kv
    * and, with softcap > 0, softcap * tanh(x), whose derivative softcap * (1 - tanh^2 x) multiplies ds.  No gradient is

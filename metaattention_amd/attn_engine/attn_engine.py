@@ -283,9 +283,9 @@ class AttentionEngine:
         if any(t.requires_grad for t in (q, k, v)):
             extras = {}
             if form.extra or form.softcap is not None:
-                # the softmax backward kernels recompute the score with its additive terms and soft-capping (the custom
-                # inputs themselves get no gradient, as in the reference, attn_tl.py:692); the other families' do not
-                if self.family != "softmax":
+                # the backward kernels recompute the score with its additive terms and soft-capping (the custom inputs
+                # themselves get no gradient, as in the reference, attn_tl.py:692)
+                if self.family == "retention":
                     return _ForwardOnly.apply(run, q, k, v)
                 extras = self._additive_inputs(given, q.shape[2], q.dtype, q.device)
             score_mask = None

@@ -181,8 +181,10 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
       if (x % 4 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: elem_mask rows must be 4-byte aligned");
   }
   if (p->score_add || p->pos_slope_q || p->pos_slope_kv || p->softcap != 0.f) {
-    if (p->family != MA_ATTN_SOFTMAX)
-      return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: score_add / pos_slope / softcap have backward kernels in the softmax family only");
+    if (p->family == MA_ATTN_RETENTION)
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: score_add / pos_slope / softcap do not go with the retention family");
+    if (p->softcap != 0.f && p->family != MA_ATTN_SOFTMAX)
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: softcap goes with the softmax family only (as in ma_attn_fwd)");
     if (p->softcap < 0.f) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: softcap must be >= 0");
     if (p->score_add && (uintptr_t)p->score_add % (p->score_add_fp32 ? 4 : 2) != 0)
       return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: score_add must be aligned to its element size");

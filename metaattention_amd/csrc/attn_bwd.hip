@@ -77,7 +77,7 @@ __device__ __forceinline__ float row_ds(float p, float dp, float delta) {
   else return p > 0.f ? dp : 0.f;
 }
 
-// EXTRA instantiations (softmax): the additive terms and the soft-capping of the forward pass, applied to the recomputed
+// EXTRA instantiations (softmax, sigmoid, relu): the additive terms and the soft-capping of the forward pass, applied to the recomputed
 // raw scores.  `extra` is (add + slope_q q + slope_kv kv) of the element; the scores stay in units of 1 / scale, so that
 // everything behind sees s * scale + bias as before.  With softcap > 0, x = s * scale + bias becomes softcap * tanh(x) and
 // `cap_grad` the derivative softcap * (1 - tanh^2 x), which multiplies ds; tanh(x) = 1 - 2 / (1 + e^(2x)) as in the forward.
@@ -1084,8 +1084,10 @@ static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   if (allow_lds(lds_ok, lds, k1, k2, k3) != 0) return -1;
   AttnBwdArgs args = a;
   if (a.add || a.slope_q || a.slope_kv || a.softcap != 0.f) {
-    // additive score terms / soft-capping: instantiations of their own (softmax family), dk and dv by the two-launch kernels
-    if constexpr (FAMILY == BF_SOFTMAX) {
+    // additive score terms / soft-capping: instantiations of their own (not for the retention family, whose score function
+    // is the multiplier tensor; soft-capping goes with softmax only, as in the forward), dk and dv by the two-launch kernels
+    if constexpr (FAMILY != BF_RETENTION) {
+      if (a.softcap != 0.f && FAMILY != BF_SOFTMAX) return -2;
       auto e1 = attn_bwd_dq_kernel<T, DQK, DV, FAMILY, CAUSAL, true>;
       auto e2 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL, SPLIT ? 1 : 3, true>;
       auto e3 = attn_bwd_dkv_kernel<T, DQK, DV, FAMILY, CAUSAL, 2, true>;

@@ -302,7 +302,7 @@ def attn_bwd(q, k, v, o, dout, lse, *, family: int, causal: bool, scale: float, 
     its transpose ``elem_mask_t`` [1|B, 1|H, Skv, Sq]; both with rows at 4-byte aligned addresses.  Optional tile masks
     for skipping: ``kv_block_mask`` [1|B, 1|H, ceil(Sq/128), ceil(Skv/32)] and ``q_block_mask`` [1|B, 1|H, ceil(Skv/128),
     ceil(Sq/32)] (a tile is kept when any of its elements is).  ``score_add``, ``pos_slope_q`` / ``pos_slope_kv`` and
-    ``softcap`` (softmax family) are the forward pass's additive score terms and soft-capping, given again unchanged; they
+    ``softcap`` (softmax, sigmoid and relu families; softcap with softmax only) are the forward pass's additive score terms and soft-capping, given again unchanged; they
     receive no gradients of their own."""
     _require_gpu(q, k, v, o, dout, lse, bias_tensor, elem_mask, elem_mask_t, kv_block_mask, q_block_mask, score_mask, score_mask_t,
                  score_add, pos_slope_q, pos_slope_kv)

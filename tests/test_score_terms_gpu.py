@@ -242,21 +242,56 @@ def test_attn_bwd_score_terms_through_the_c_abi(D, DV, H, Hkv, Sq, Skv, causal, 
     _check_grads(got, ref, "c abi")
 
 
-def test_backward_through_additive_terms_of_the_other_families_is_refused():
-    """The sigmoid / relu backward kernels take the score as s * scale + bias only: loud, not silently wrong."""
+def test_backward_through_additive_terms_sigmoid_and_relu():
+    """The sigmoid and relu families differentiate through additive terms as well (the score function sees x = s * scale +
+    bias + added terms): an fp32 key vector and a per-row tensor inside a sigmoid spec through the engine, a tile with
+    relu through the C ABI."""
+    from metaattention_amd import hip_backend as hb
+    hb.load_library()
+    B, H, S, D = 2, 2, 192, 128
+    io = {"colv": ("seq_len_kv",), "rowt": ("batch", "heads", "seq_len"), "b1": (1,)}
+
+    def score_mod(s, c, b, h, q, k):
+        t = c.input_tensors
+        x = (s + t["colv"]) * 0.05 + t["rowt"] + t["b1"]
+        return 1 / (1 + (-x).exp())
+
+    mod = _engine(B, H, S, D, io, score_mod, True, online=specs.OnlineIdentity())
+    q, k, v = inputs.softmax_inputs(B, H, S, D, D, seed=9)
+    g = torch.Generator().manual_seed(2)
+    colv, rowt, b1 = torch.randn(S, generator=g) * 4, torch.randn(B, H, S, generator=g), torch.tensor([-3.0])
+    dout = (0.25 * torch.randn(B, S, H, D, generator=g)).bfloat16()
+    print("bwd sigmoid with additive terms", flush=True)
+    _, got = _engine_grads(mod, q, k, v, dout, colv.cuda(), rowt.cuda(), b1.cuda())
+    add = colv.double().view(1, 1, 1, S) * 0.05 + rowt.double().view(B, H, S, 1)
+    ref = oracle.attention_grads(oracle.biased_attention, q, k, v, dout, add=add, causal=True, family="sigmoid", softmax_scale=0.05, bias=-3.0)
+    _check_grads(got, ref, "sigmoid + terms")
+
+    D2, S2 = 64, 130
+    q, k, v = inputs.softmax_inputs(B, H, S2, D2, D2, seed=14)
+    k, v = (k.float() * 0.5).bfloat16(), (v.float() * 0.5).bfloat16()
+    add = torch.randn(1, H, S2, S2, generator=g)
+    dout = (0.25 * torch.randn(B, S2, H, D2, generator=g)).bfloat16()
+    kw = dict(family=hb.MA_ATTN_RELU, causal=False, scale=D2 ** -0.5, score_add=add.cuda())
+    print("bwd relu with an additive tile", flush=True)
+    o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), **kw)
+    got = hb.attn_bwd(q.cuda(), k.cuda(), v.cuda(), o, dout.cuda(), None, **kw)
+    torch.cuda.synchronize()
+    ref = oracle.attention_grads(oracle.biased_attention, q, k, v, dout, add=add.double(), family="relu", softmax_scale=D2 ** -0.5)
+    for name, a, b in zip(("dq", "dk", "dv"), got, ref):
+        oracle.assert_close(a.float().cpu(), b.float(), rtol=RTOL, atol=ATOL, mismatch_ratio=2e-3, msg=f"relu + tile:{name}")
+
+
+def test_soft_capping_outside_the_softmax_family_is_refused():
+    """cap * tanh(x) goes with the softmax row function only, forward and backward: loud, not silently wrong."""
     from metaattention_amd import hip_backend as hb
     hb.load_library()
     B, H, S, D = 1, 1, 128, 128
-
-    def score_mod(s, c, b, h, q, k):
-        x = s * 0.1 + c.input_tensors["colv"]
-        return 1 / (1 + (-x).exp())
-
-    mod = _engine(B, H, S, D, {"colv": ("seq_len_kv",)}, score_mod, True, online=specs.OnlineIdentity())
-    q, k, v = (t.cuda().requires_grad_(True) for t in inputs.softmax_inputs(B, H, S, D, D, seed=15))
-    o = mod(q, k, v, torch.zeros(S, device="cuda"))
-    with pytest.raises(NotImplementedError):
-        o.float().sum().backward()
-    qd, kd, vd = q.detach(), k.detach(), v.detach()
+    q, k, v = (t.cuda() for t in inputs.softmax_inputs(B, H, S, D, D, seed=15))
     with pytest.raises(hb.MetaAttentionError):
-        hb.attn_bwd(qd, kd, vd, o.detach(), o.detach(), None, family=hb.MA_ATTN_SIGMOID, causal=True, scale=0.1, softcap=2.0)
+        hb.attn_bwd(q, k, v, q, q, None, family=hb.MA_ATTN_SIGMOID, causal=True, scale=0.1, softcap=2.0)
+    lse = torch.zeros(B, H, S, device="cuda")
+    mask = torch.ones(1, H, S, S, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(hb.MetaAttentionError):
+        hb.attn_bwd(q, k, v, q, q, lse, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mask, score_mask_t=mask,
+                    score_add=torch.zeros(1, 1, S, S, device="cuda"))
