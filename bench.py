@@ -23,6 +23,7 @@ cores over a bounded sample as "cpu_baseline"):
   c3_retnet_chunked_operator / c4_mamba2_ssd_operator / c5_mla_decode_operator  those three through the operators the engines return
   c5_mla_decode       absorbed MLA decode, B64 Hq128 KV4096 d512+64 (HBM bound)
   gqa_decode          grouped-query softmax decode, B64 H32 Hkv8 KV4096 D128 (HBM bound)
+  reference_shapes    the MLA / RetNet / Mamba2 shapes whose kernel latencies the reference's tuned_config files record
 """
 from __future__ import annotations
 
@@ -462,6 +463,58 @@ def bench_mla(steps, warmup):
                 note="split-KV kernel + combine kernel per call; " + COLD_NOTE)
 
 
+def bench_reference_shapes(steps, warmup):
+    """The shapes for which the reference's tuned_config files record kernel latencies of its own templates (TileLang
+    autotuner, warmup 10 / rep 10: tl_template/linear/linear_tl.py:229-233, tl_template/attn/mla_decode_tl.py:324-328), timed
+    here back to back as the tuner times them.  `reference_ms` is what those files hold (other hardware: context, not a
+    baseline for `vs_baseline`); for the chunked operators it is the sum of the state kernel (h) and the output kernel (o),
+    which the one kernel here replaces."""
+    import torch
+    from metaattention_amd import hip_backend as hb
+    out = {}
+    g = torch.Generator(device="cuda").manual_seed(0)
+    # MLA decode, fp16 (tuned_config/{H100,MI250}/mla_decode.json)
+    for (B, Skv), ref in (((8, 2048), {"H100": 0.0329, "MI250": 0.1986}), ((1, 2048), {"MI250": 0.1779}), ((1, 4096), {"MI250": 0.2507}),
+                          ((1, 8192), {"MI250": 0.4293}), ((8, 4096), {"MI250": 0.4117}), ((8, 8192), {"MI250": 0.7550})):
+        Hq, D, Dpe = 128, 512, 64
+        q = torch.randn(B, 1, Hq, D, device="cuda", dtype=torch.float16, generator=g)
+        q_pe = torch.randn(B, 1, Hq, Dpe, device="cuda", dtype=torch.float16, generator=g)
+        kv = torch.randn(B, Skv, 1, D, device="cuda", dtype=torch.float16, generator=g)
+        k_pe = torch.randn(B, Skv, 1, Dpe, device="cuda", dtype=torch.float16, generator=g)
+        o = torch.empty_like(q)
+        ws = torch.empty(max(hb.mla_workspace_bytes(B, Hq, Skv), 16), dtype=torch.uint8, device="cuda")
+        ms = time_gpu(lambda: hb.mla_decode(q, q_pe, kv, k_pe, scale=1 / math.sqrt(D + Dpe), out=o, workspace=ws), steps, warmup)
+        out[f"mla_decode_fp16_b{B}_hq128_kv{Skv}"] = dict(ms=round(ms, 4), reference_ms=ref)
+    # RetNet chunked forward, bf16 (tuned_config/{H100,MI250}/retention_linear_{h,o}.json)
+    for (B, T), ref in (((8, 2048), {"H100 chunk 128": 2.44, "H100 chunk 64": 3.07, "MI250 chunk 64": 13.8}), ((1, 2048), {"H100 chunk 128": 0.260}),
+                        ((8, 4096), {"MI250 chunk 64": 27.4})):
+        H, Dk, Dv = 32, 256, 512
+        q = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 16).bfloat16()
+        k = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 16).bfloat16()
+        v = torch.randn(B, H, T, Dv, device="cuda", generator=g).bfloat16()
+        ld = torch.log(1 - torch.exp2(-5 - torch.arange(H, device="cuda").float())).view(1, H, 1).expand(B, H, T).contiguous()
+        o = torch.empty_like(v)
+        ws = torch.empty(max(hb.linear_workspace_bytes(B, H, H, H, T, Dk, Dv), 16), dtype=torch.uint8, device="cuda")
+        ms = time_gpu(lambda: hb.linear_fwd(q, k, v, ld, q_scale=Dk ** -0.5, out=o, workspace=ws), steps, warmup)
+        out[f"retnet_chunked_b{B}_h32_s{T}_256_512"] = dict(ms=round(ms, 4), reference_ms=ref)
+    # Mamba2 SSD forward, bf16, 80 heads sharing one B / C head (tuned_config/{H100,MI250}/mamba2_{h,o}.json)
+    for T, ref in ((2048, {"H100 chunk 128": 0.600, "MI250 chunk 64": 2.87}), (8192, {"H100 chunk 128": 2.25, "MI250 chunk 64": 12.1})):
+        B, H, P, N = 8, 80, 64, 128
+        Cm = (torch.randn(B, 1, T, N, device="cuda", generator=g) / math.sqrt(N)).bfloat16()
+        Bm = (torch.randn(B, 1, T, N, device="cuda", generator=g) / math.sqrt(N)).bfloat16()
+        x = torch.randn(B, H, T, P, device="cuda", generator=g).bfloat16()
+        dt = torch.nn.functional.softplus(torch.randn(B, H, T, device="cuda", generator=g) - 2)
+        A = -torch.exp(torch.rand(1, H, device="cuda", generator=g) * math.log(16))
+        ld = (dt * A.view(1, H, 1)).contiguous()
+        o = torch.empty_like(x)
+        ws = torch.empty(max(hb.linear_workspace_bytes(B, H, 1, 1, T, N, P), 16), dtype=torch.uint8, device="cuda")
+        ms = time_gpu(lambda: hb.linear_fwd(Cm, Bm, x, ld, v_scale=dt, out=o, workspace=ws), steps, warmup)
+        out[f"mamba2_ssd_b8_hv80_s{T}_n128_p64"] = dict(ms=round(ms, 4), reference_ms=ref)
+    out["note"] = ("reference_ms: tuned_latency fields of the reference's tuned_config/<GPU>/*.json, the only measured values in its tree "
+                   "(H100 and MI250; per kernel, h + o summed for the chunked operators); ms: one call here, back to back, same shapes and dtypes")
+    return out
+
+
 def cpu_baseline_softmax():
     """Oracle (restated PyTorch reference, fp32) on the host cores over a bounded
     sample: the whole headline workload once (B=8, H=32, S=4096, D=128, causal), about ten seconds."""
@@ -598,7 +651,8 @@ def main():
              ("c4_mamba2_ssd_operator", "mamba_operator", lambda: bench_linear_operators(args.steps, args.warmup, "mamba")),
              ("c5_mla_decode", "mla", lambda: bench_mla(args.steps, args.warmup)),
              ("c5_mla_decode_operator", "mla_operator", lambda: bench_mla_operator(args.steps, args.warmup)),
-             ("gqa_decode", "decode", lambda: bench_decode(args.steps, args.warmup))]
+             ("gqa_decode", "decode", lambda: bench_decode(args.steps, args.warmup)),
+             ("reference_shapes", "reference_shapes", lambda: bench_reference_shapes(args.steps, args.warmup))]
     cpu_legs = {"c3_retnet_chunked": cpu_baseline_retnet_chunked, "c3_retnet_parallel": cpu_baseline_retention_parallel,
                 "c4_mamba2_ssd": cpu_baseline_mamba2, "c5_mla_decode": cpu_baseline_mla}
     for name, key, fn in table:

@@ -29,6 +29,11 @@ def test_bench_line():
                  "c5_mla_decode", "gqa_decode"):
         assert name in others and "error" not in others[name], (name, others.get(name))
         assert others[name]["ms"] > 0
+    ref = others["reference_shapes"]
+    assert "error" not in ref and len([k for k in ref if k != "note"]) == 11
+    for key, entry in ref.items():
+        if key != "note":
+            assert entry["ms"] > 0 and entry["reference_ms"]
     # the operator recognised the decay mask the workload builds
     assert "generates it" in others["c3_retnet_parallel_operator"]["flop_convention"]
     for name in ("c5_mla_decode", "gqa_decode"):
