@@ -24,6 +24,7 @@ cores over a bounded sample as "cpu_baseline"):
   c5_mla_decode       absorbed MLA decode, B64 Hq128 KV4096 d512+64 (HBM bound)
   gqa_decode          grouped-query softmax decode, B64 H32 Hkv8 KV4096 D128 (HBM bound)
   reference_shapes    the MLA / RetNet / Mamba2 shapes whose kernel latencies the reference's tuned_config files record
+  reference_benchmark_shapes  causal softmax at Dqk 192 / Dv 128 and ReLU attention at 64 / 64 as in testing/benchmark_mi250.py
 """
 from __future__ import annotations
 
@@ -515,6 +516,32 @@ def bench_reference_shapes(steps, warmup):
     return out
 
 
+def bench_reference_benchmark_shapes(steps, warmup):
+    """The two parallel-attention figures of the reference's AMD benchmark that BASELINE's configurations do not cover
+    (testing/benchmark_mi250.py:40-55): causal softmax at the DeepSeek-V2-Lite head sizes (16 heads, Dqk 192, Dv 128, fp16) and
+    ReLU attention at the ViT-S head size (6 heads, 64 / 64, fp16), forward and backward through the C ABI at B = 8 / 64.
+    The reference writes its own timings to CSV files at run time and holds none in the tree."""
+    import torch
+    from metaattention_amd import hip_backend as hb
+    out = {}
+    g = torch.Generator(device="cuda").manual_seed(0)
+    for name, fam, causal, B, H, S, D, DV in (("softmax_causal_deepseek_v2_lite_b8_h16_s4096_192_128_fp16", hb.MA_ATTN_SOFTMAX, True, 8, 16, 4096, 192, 128),
+                                              ("relu_vit_s_b64_h6_s1024_64_64_fp16", hb.MA_ATTN_RELU, False, 64, 6, 1024, 64, 64)):
+        q, k = (torch.randn(B, S, H, D, device="cuda", dtype=torch.float16, generator=g) for _ in range(2))
+        v, do = (torch.randn(B, S, H, DV, device="cuda", dtype=torch.float16, generator=g) for _ in range(2))
+        if fam == hb.MA_ATTN_RELU:
+            k, v = k * 0.5, v * 0.5
+        lse = torch.empty(B, H, S, device="cuda") if fam == hb.MA_ATTN_SOFTMAX else None
+        o = torch.empty(B, S, H, DV, device="cuda", dtype=torch.float16)
+        scale = D ** -0.5
+        ms_f = time_gpu(lambda: hb.attn_fwd(q, k, v, family=fam, causal=causal, scale=scale, out=o, row_scale=lse), steps, warmup)
+        ms_b = time_gpu(lambda: hb.attn_bwd(q, k, v, o, do, lse, family=fam, causal=causal, scale=scale), max(steps // 3, 3), 2)
+        flops = (0.5 if causal else 1.0) * 2.0 * B * H * S * S * (D + DV)
+        out[name] = dict(fwd_ms=round(ms_f, 4), fwd_tflops=round(flops / ms_f / 1e9, 1), bwd_ms=round(ms_b, 4),
+                         bwd_tflops_2p5x=round(2.5 * flops / ms_b / 1e9, 1))
+    return out
+
+
 def cpu_baseline_softmax():
     """Oracle (restated PyTorch reference, fp32) on the host cores over a bounded
     sample: the whole headline workload once (B=8, H=32, S=4096, D=128, causal), about ten seconds."""
@@ -652,7 +679,8 @@ def main():
              ("c5_mla_decode", "mla", lambda: bench_mla(args.steps, args.warmup)),
              ("c5_mla_decode_operator", "mla_operator", lambda: bench_mla_operator(args.steps, args.warmup)),
              ("gqa_decode", "decode", lambda: bench_decode(args.steps, args.warmup)),
-             ("reference_shapes", "reference_shapes", lambda: bench_reference_shapes(args.steps, args.warmup))]
+             ("reference_shapes", "reference_shapes", lambda: bench_reference_shapes(args.steps, args.warmup)),
+             ("reference_benchmark_shapes", "reference_benchmark", lambda: bench_reference_benchmark_shapes(args.steps, args.warmup))]
     cpu_legs = {"c3_retnet_chunked": cpu_baseline_retnet_chunked, "c3_retnet_parallel": cpu_baseline_retention_parallel,
                 "c4_mamba2_ssd": cpu_baseline_mamba2, "c5_mla_decode": cpu_baseline_mla}
     for name, key, fn in table:

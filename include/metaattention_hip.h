@@ -61,7 +61,7 @@ typedef struct ma_attn_params {
   int32_t family; /* ma_attn_family */
   int32_t dtype;  /* ma_dtype of q, k, v, o and of score_mask */
   int32_t mask;   /* ma_mask_kind */
-  int32_t batch, heads, seqlen_q, seqlen_kv, dim_qk, dim_v;
+  int32_t batch, heads, seqlen_q, seqlen_kv, dim_qk, dim_v;   /* head sizes: as listed at ma_attn_bwd_params.family */
   /* q [B,Sq,H,Dqk], k [B,Skv,Hkv,Dqk], v [B,Skv,Hkv,Dv], o [B,Sq,H,Dv]; BSHD is the
    * layout the reference operator takes (attn_tl.py:69-70) but any strides
    * with a contiguous last dimension are accepted (sequence strides of k and v
@@ -130,7 +130,8 @@ typedef struct ma_attn_params {
  * strides of q, k, v and dout must be non-negative and below 2^26 elements (MA_ERR_UNSUPPORTED otherwise). */
 typedef struct ma_attn_bwd_params {
   int32_t family; /* ma_attn_family: SOFTMAX, SIGMOID, RELU or RETENTION; head sizes (dim_qk / dim_v) 128/128, 64/64, 128/256,
-                   * 256/256 and 256/512 for every family, others MA_ERR_UNSUPPORTED */
+                   * 256/256 and 256/512 for every family, 192/128 (DeepSeek-V2-Lite, testing/benchmark_mi250.py:40-46) for
+                   * SOFTMAX, SIGMOID and RELU; others MA_ERR_UNSUPPORTED */
   int32_t dtype;
   int32_t mask;   /* ma_mask_kind */
   int32_t batch, heads, heads_kv /* 0 = heads */, seqlen_q, seqlen_kv, dim_qk, dim_v;

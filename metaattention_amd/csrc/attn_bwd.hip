@@ -96,13 +96,14 @@ __device__ __forceinline__ float apply_extra(float s, float extra, float scale, 
 // DMA of a [32 x ROWB bytes] tile whose rows are `row_stride` bytes apart in memory: each instruction
 // moves 1 KB; lane i fetches the 16-byte chunk that belongs at physical position i of that KB.  Rows
 // beyond `limit` are clamped to the last one (whatever is computed from them is masked).
-template <int ROWB, int NWAVES>
+template <int ROWB, int NWAVES, int USED = ROWB / 16>
 __device__ __forceinline__ void dma_tile(const char* src, int64_t row_stride, int row0, int limit, uint32_t lds_base, int wave, int lane) {
   constexpr int CPR = ROWB / 16, NI = 32 * ROWB / 1024;
   for (int ii = wave; ii < NI; ii += NWAVES) {
     const int row = ii * (1024 / ROWB) + lane / CPR, c = lane % CPR;
     const int grow = min(row0 + row, limit - 1);
-    dma16(src + grow * row_stride + ((c ^ swz_tile<CPR>(row)) << 4), lds_base + ii * 1024);
+    if (USED == CPR || (c ^ swz_tile<CPR>(row)) < USED)   // (chunks beyond the head size do not exist in memory)
+      dma16(src + grow * row_stride + ((c ^ swz_tile<CPR>(row)) << 4), lds_base + ii * 1024);
   }
 }
 
@@ -143,7 +144,7 @@ template <typename T, int DIM>
 __device__ __forceinline__ f32x16 mm_rows(uint32_t tile, int r, int g, const typename Elem<T>::x8 (&bf)[DIM / 16]) {
   using E = Elem<T>;
   using x8 = typename E::x8;
-  constexpr int ROWB = DIM * 2, CPR = DIM / 8, KS = DIM / 16, AH = 2, RING = 3;
+  constexpr int ROWB = pad_width(DIM) * 2, CPR = pad_width(DIM) / 8, KS = DIM / 16, AH = 2, RING = 3;
   // (tile bases and row offsets are multiples of the row size, so the swizzled chunk index has its own address
   // bits: another k-slice is one XOR with a constant away)
   const uint32_t a0 = tile + r * ROWB + (uint32_t)((g ^ swz_tile<CPR>(r)) << 4);
@@ -172,7 +173,7 @@ __device__ __forceinline__ void mm_cols(uint32_t tile, int lane, const typename 
   using E = Elem<T>;
   using x8 = typename E::x8;
   using x4 = typename E::x4;
-  constexpr int ROWB = DIM * 2, CPR = DIM / 8, NB = DIM / 32, PF = NB >= 2 ? 4 : 2;
+  constexpr int ROWB = pad_width(DIM) * 2, CPR = pad_width(DIM) / 8, NB = DIM / 32, PF = NB >= 2 ? 4 : 2;
   const int g = lane >> 5, jr = (lane & 15) >> 2;
   const int lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
   const uint32_t b0 = tile + (4 * g + jr) * ROWB + (lane & 1) * 8 + (uint32_t)((lc ^ swz_tile<CPR>(4 * g + jr)) << 4);
@@ -233,7 +234,7 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
   using x8 = typename E::x8;
   constexpr int BM = 128, BN = 32;
   constexpr int KS = DQK / 16, VS = DV / 16, QB = DQK / 32;
-  constexpr int KROW = DQK * 2, VROW = DV * 2;
+  constexpr int KROW = pad_width(DQK) * 2, VROW = DV * 2;   // (LDS rows; 192-wide keys sit in 256-wide rows)
   constexpr int KTILE = BN * KROW, VTILE = BN * VROW, STAGE = KTILE + VTILE;
 
   extern __shared__ __align__(16) char smem[];
@@ -299,7 +300,7 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
   const bool keep_ok = FAMILY != BF_RETENTION && a.elem_mask && ((a.em_sq | a.em_sb | a.em_sh | (int64_t)(uintptr_t)a.elem_mask) & 15) == 0;
   const uint8_t* bm_full = a.kv_block_mask ? a.kv_block_mask + (int64_t)b * a.kbm_sb + (int64_t)h * a.kbm_sh + (int64_t)mb * a.kbm_sq : nullptr;
   auto tile_full = [&](int jt_) { return bm_full && bm_full[jt_] >= 2; };   // the element-wise mask keeps every score of the tile
-  TileDma<KROW, 4> k_dma;
+  TileDma<KROW, 4, DQK / 8> k_dma;
   TileDma<VROW, 4> v_dma;
   k_dma.init((uint32_t)k_row_bytes, wave, lane);
   v_dma.init((uint32_t)v_row_bytes, wave, lane);
@@ -308,7 +309,7 @@ __global__ __launch_bounds__(256, (DQK + DV >= 512 ? 1 : 2)) void attn_bwd_dq_ke
       k_dma.issue(kb + (int64_t)n0 * k_row_bytes, lds0 + buf * STAGE, wave);
       v_dma.issue(vb + (int64_t)n0 * v_row_bytes, lds0 + buf * STAGE + KTILE, wave);
     } else {
-      dma_tile<KROW, 4>(kb, k_row_bytes, n0, a.Skv, lds0 + buf * STAGE, wave, lane);
+      dma_tile<KROW, 4, DQK / 8>(kb, k_row_bytes, n0, a.Skv, lds0 + buf * STAGE, wave, lane);
       dma_tile<VROW, 4>(vb, v_row_bytes, n0, a.Skv, lds0 + buf * STAGE + KTILE, wave, lane);
     }
     if constexpr (FAMILY == BF_RETENTION) {
@@ -458,7 +459,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
   using x8 = typename E::x8;
   constexpr int BNW = 128, BMT = 32;   // keys per workgroup, query rows per tile
   constexpr int KS = DQK / 16, VS = DV / 16, QB = DQK / 32, VB = DV / 32;
-  constexpr int QROW = DQK * 2, DOROW = DV * 2;
+  constexpr int QROW = pad_width(DQK) * 2, DOROW = DV * 2;   // (LDS rows; 192-wide queries sit in 256-wide rows)
   // a stage: the Q tile and the dO tile; behind both stages, lse and delta of each stage's 32 rows (softmax; 2 x 128
   // bytes per stage -- not inside the stages: the swizzled reads address a tile as base XOR offset, which needs the
   // tile bases aligned to the row size)
@@ -529,7 +530,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
   };
   const bool keep_ok = FAMILY != BF_RETENTION && a.elem_mask_t && ((a.emt_sk | a.emt_sb | a.emt_sh | (int64_t)(uintptr_t)a.elem_mask_t) & 15) == 0;
   const bool mult_ok = FAMILY == BF_RETENTION && (a.smt_sk & 7) == 0 && (a.smt_sb & 7) == 0 && (a.smt_sh & 7) == 0 && ((uintptr_t)a.smask_t & 15) == 0;
-  TileDma<QROW, 4> q_dma;
+  TileDma<QROW, 4, DQK / 8> q_dma;
   TileDma<DOROW, 4> do_dma;
   q_dma.init((uint32_t)q_row_bytes, wave, lane);
   do_dma.init((uint32_t)do_row_bytes, wave, lane);
@@ -541,7 +542,7 @@ __global__ __launch_bounds__(256, (WHAT == 3 ? (DQK + DV >= 256 ? 1 : 2) : (DQK 
       q_dma.issue(qb + (int64_t)m0 * q_row_bytes, lds0 + buf * STAGE, wave);
       do_dma.issue(dob + (int64_t)m0 * do_row_bytes, lds0 + buf * STAGE + QTILE, wave);
     } else {
-      dma_tile<QROW, 4>(qb, q_row_bytes, m0, a.Sq, lds0 + buf * STAGE, wave, lane);
+      dma_tile<QROW, 4, DQK / 8>(qb, q_row_bytes, m0, a.Sq, lds0 + buf * STAGE, wave, lane);
       dma_tile<DOROW, 4>(dob, do_row_bytes, m0, a.Sq, lds0 + buf * STAGE + QTILE, wave, lane);
     }
     if constexpr (FAMILY == BF_SOFTMAX) {
@@ -1072,7 +1073,7 @@ template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL>
 static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   constexpr int DMAX = DQK > DV ? DQK : DV;
   // (+ the row values of the dk / dv kernels' stages and the retention family's multiplier blocks / the keep-mask blocks)
-  constexpr size_t tiles = 2 * (size_t)32 * (DQK + DV) * 2 + 1024 + (FAMILY == BF_RETENTION ? 2 * 4 * 2048 : 2 * 4 * 1024);
+  constexpr size_t tiles = 2 * (size_t)32 * (pad_width(DQK) + DV) * 2 + 1024 + (FAMILY == BF_RETENTION ? 2 * 4 * 2048 : 2 * 4 * 1024);
   constexpr size_t ostage = 4 * 32 * (size_t)(DMAX + 16);
   constexpr size_t lds = tiles > ostage ? tiles : ostage;
   auto k1 = attn_bwd_dq_kernel<T, DQK, DV, FAMILY, CAUSAL>;
@@ -1160,6 +1161,7 @@ static int bwd_dims(const AttnBwdArgs& a, int family, bool causal, int dqk, int 
   if (dqk == 64 && dv == 64) return bwd_family<T, 64, 64>(a, family, causal, stream);
   if (dqk == 128 && dv == 256) return bwd_family<T, 128, 256>(a, family, causal, stream);
   if (dqk == 256 && dv == 256) return bwd_family<T, 256, 256>(a, family, causal, stream);
+  if (dqk == 192 && dv == 128) return bwd_family<T, 192, 128>(a, family, causal, stream);   // (the reference's DeepSeek-V2-Lite benchmark shape)
   if (dqk == 256 && dv == 512) return bwd_family<T, 256, 512>(a, family, causal, stream);
   return -2;
 }

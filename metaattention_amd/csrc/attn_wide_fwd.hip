@@ -45,8 +45,8 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
   using x4 = typename E::x4;
   constexpr int BM = 32 * NW, BN = 32;
   constexpr int KS = DQK / 16, DB = DV / 32;
-  constexpr int KROW = DQK * 2, VROW = DV * 2;
-  constexpr int CPRK = DQK / 8, CPRV = DV / 8;
+  constexpr int KROW = pad_width(DQK) * 2, VROW = DV * 2;   // (LDS rows; 192-wide keys sit in 256-wide rows)
+  constexpr int CPRK = pad_width(DQK) / 8, CPRV = DV / 8, USEDK = DQK / 8;
   constexpr int KTILE = BN * KROW, VTILE = BN * VROW, STAGE = KTILE + VTILE;
   constexpr int NIK = KTILE / 1024, NIV = VTILE / 1024;
   static_assert(CPRK >= 8 && CPRV >= 8 && DQK % 16 == 0 && DV % 64 == 0, "head size");
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
   // DMA of one tile: each instruction moves 1 KB (1024 / row bytes tile rows); lane i fetches the
   // 16-byte chunk that belongs at physical position i of that KB.  Rows beyond the sequence are clamped
   // to its last row (their scores are masked, or multiplied by a zero of M).
-  TileDma<KROW, NW> k_dma;
+  TileDma<KROW, NW, USEDK> k_dma;
   TileDma<VROW, NW> v_dma;
   k_dma.init((uint32_t)k_row_bytes, wave, lane);
   v_dma.init((uint32_t)v_row_bytes, wave, lane);
@@ -164,7 +164,8 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
       if (ii < NIK) {
         const int row = ii * (1024 / KROW) + lane / CPRK, c = lane % CPRK;
         const int nrow = min(n0 + row, skv - 1);
-        dma16(kb + nrow * k_row_bytes + ((c ^ swz_tile<CPRK>(row)) << 4), base + ii * 1024);
+        if (USEDK == CPRK || (c ^ swz_tile<CPRK>(row)) < USEDK)   // (chunks beyond the head size do not exist in memory)
+          dma16(kb + nrow * k_row_bytes + ((c ^ swz_tile<CPRK>(row)) << 4), base + ii * 1024);
       } else {
         const int i2 = ii - NIK;
         const int row = i2 * (1024 / VROW) + lane / CPRV, c = lane % CPRV;
@@ -428,7 +429,7 @@ __global__ __launch_bounds__(256) void attn_split_combine_kernel(const AttnArgs 
 
 template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL, int NW = 4>
 static int launch_wide(const AttnArgs& a, hipStream_t stream) {
-  constexpr size_t tiles = 2 * (size_t)32 * (DQK + DV) * 2;
+  constexpr size_t tiles = 2 * (size_t)32 * (pad_width(DQK) + DV) * 2;
   constexpr size_t ostage = NW * 32 * (size_t)(DV + 16);
   constexpr size_t lds = tiles > ostage ? tiles : ostage;
   auto kern = attn_wide_fwd_kernel<T, DQK, DV, FAMILY, CAUSAL, NW>;
@@ -491,6 +492,7 @@ static int wide_dims(const AttnArgs& a, int family, bool causal, int dqk, int dv
   if (dqk == 64 && dv == 64) return wide_family<T, 64, 64>(a, family, causal, stream);
   if (dqk == 128 && dv == 256) return wide_family<T, 128, 256>(a, family, causal, stream);
   if (dqk == 256 && dv == 256) return wide_family<T, 256, 256>(a, family, causal, stream);
+  if (dqk == 192 && dv == 128) return wide_family<T, 192, 128>(a, family, causal, stream);   // (the reference's DeepSeek-V2-Lite benchmark shape)
   if (dqk == 256 && dv == 512 && family != WF_SOFTMAX) return wide_family<T, 256, 512>(a, family, causal, stream);
   // Softmax at 256/512: rescaling a 256-register accumulator that lives in the MFMA accumulation registers makes the
   // compiler spill it.  Given the probabilities the value columns are independent, so the two halves of V and of the

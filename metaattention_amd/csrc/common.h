@@ -167,13 +167,20 @@ __device__ __forceinline__ int swz_tile(int row) {
 // its wave-uniform first-row address in scalar registers plus those 32-bit offsets: no per-lane 64-bit address
 // arithmetic inside the loops.  The swizzle term repeats every 16 rows, so instructions of a wave that are a multiple
 // of 16 rows apart share an offset and the row distance goes into the scalar base.
-template <int ROWB, int NWAVES>
+// Head sizes that are not powers of two (192) live in LDS rows of the next power of two: the swizzles and the XOR
+// addressing of the k-slices need row sizes that are powers of two.  The columns beyond the head size are neither loaded
+// nor read.
+constexpr int pad_width(int d) { return d <= 64 ? 64 : d <= 128 ? 128 : d <= 256 ? 256 : 512; }
+
+// (USED: the 16-byte chunks of a row that exist in memory; a lane whose chunk lies beyond them sits the instruction out)
+template <int ROWB, int NWAVES, int USED = ROWB / 16>
 struct TileDma {
   static constexpr int CPR = ROWB / 16, RPI = 1024 / ROWB, NI = 32 * ROWB / 1024, NJ = NI / NWAVES;
   static constexpr int RPJ = NWAVES * RPI;   // rows between consecutive instructions of a wave
   static constexpr int NOFF = RPJ % 16 == 0 ? 1 : (16 % RPJ == 0 && 16 / RPJ < NJ ? 16 / RPJ : NJ);
   static_assert(NI % NWAVES == 0, "a tile is a whole number of instructions per wave");
   uint32_t off[NOFF];
+  bool on[USED < CPR ? NOFF : 1];
   uint32_t stride;
   __device__ __forceinline__ void init(uint32_t row_stride, int wave, int lane) {
     stride = row_stride;
@@ -181,12 +188,17 @@ struct TileDma {
     for (int j = 0; j < NOFF; j++) {
       const int row = (wave + NWAVES * j) * RPI + lane / CPR, c = lane % CPR;
       off[j] = (uint32_t)row * row_stride + (uint32_t)((c ^ swz_tile<CPR>(row)) << 4);
+      if constexpr (USED < CPR) on[j] = (c ^ swz_tile<CPR>(row)) < USED;
     }
   }
   __device__ __forceinline__ void issue(const char* first_row, uint32_t lds_base, int wave) const {
 #pragma unroll
-    for (int j = 0; j < NJ; j++)
+    for (int j = 0; j < NJ; j++) {
+      if constexpr (USED < CPR) {
+        if (!on[j % NOFF]) continue;
+      }
       dma16_so(first_row + (uint64_t)((uint32_t)((j / NOFF) * NOFF * RPJ) * stride), off[j % NOFF], lds_base + (wave + NWAVES * j) * 1024);
+    }
   }
 };
 

@@ -46,7 +46,7 @@ def _run(hb, family, q, k, v, dout, causal, scale, bias=0.0):
     return got, ref
 
 
-@pytest.mark.parametrize("D,DV", [(128, 128), (64, 64), (128, 256), (256, 256), (256, 512)])
+@pytest.mark.parametrize("D,DV", [(128, 128), (64, 64), (128, 256), (256, 256), (256, 512), (192, 128)])
 @pytest.mark.parametrize("B,H,Hkv,S,causal", [(1, 2, 2, 256, True), (2, 3, 3, 200, True), (1, 2, 2, 333, False), (1, 4, 2, 129, True), (1, 1, 1, 1, True)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_softmax_backward(D, DV, B, H, Hkv, S, causal, dtype):
@@ -162,6 +162,32 @@ def test_engine_backward_like_the_reference_test():
     torch.cuda.synchronize()
     ref = oracle.attention_grads(oracle.softmax_attention, q, k, v, dout, causal=True)
     _check((qc.grad, kc.grad, vc.grad), ref, "engine softmax")
+
+
+def test_engine_deepseek_v2_lite_head_sizes():
+    """The shape of the reference's own AMD benchmark, testing/benchmark_mi250.py:40-46 (causal softmax, 16 heads, Dqk 192,
+    Dv 128, fp16, forward and o.backward(do)), at a reduced length: 192 is not a power of two, its rows live in 256-wide
+    LDS rows whose last 64 columns are neither loaded nor read."""
+    B, H, S, D, DV = 1, 16, 520, 192, 128
+    mod = specs.softmax_attention(B, H, S, D, DV, dtype=torch.float16)
+    g = torch.Generator().manual_seed(3)
+    q, k = (torch.randn(B, S, H, D, generator=g).half() for _ in range(2))
+    v, dout = (torch.randn(B, S, H, DV, generator=g).half() for _ in range(2))
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = mod(qc, kc, vc)
+    o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    oracle.assert_close(o.float().cpu(), oracle.softmax_attention(q, k, v, causal=True), rtol=RTOL, atol=ATOL)
+    ref = oracle.attention_grads(oracle.softmax_attention, q, k, v, dout, causal=True)
+    _check((qc.grad, kc.grad, vc.grad), ref, "engine softmax 192/128")
+    # columns 192.. of a wider tensor are not touched: q and k as slices of 256-wide storage filled with NaN behind them
+    wide_q = torch.full((B, S, H, 256), float("nan"), dtype=torch.float16, device="cuda")
+    wide_k = torch.full((B, S, H, 256), float("nan"), dtype=torch.float16, device="cuda")
+    wide_q[..., :D], wide_k[..., :D] = q.cuda(), k.cuda()
+    with torch.no_grad():
+        o2 = mod(wide_q[..., :D], wide_k[..., :D], v.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(o2, o.detach())
 
 
 def test_engine_sigmoid_backward_with_bias_tensor():

@@ -21,7 +21,7 @@ def _hb():
     return hb
 
 
-@pytest.mark.parametrize("D,DV", [(64, 64), (128, 256), (256, 256), (256, 512)])
+@pytest.mark.parametrize("D,DV", [(64, 64), (128, 256), (256, 256), (256, 512), (192, 128)])
 @pytest.mark.parametrize("B,H,S,causal", [(1, 2, 256, True), (2, 3, 200, True), (1, 2, 333, False), (1, 1, 1, True), (1, 2, 129, True)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_softmax_other_head_sizes(D, DV, B, H, S, causal, dtype):
@@ -36,7 +36,7 @@ def test_softmax_other_head_sizes(D, DV, B, H, S, causal, dtype):
     torch.testing.assert_close(lse.cpu(), lse_ref, rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("D,DV", [(64, 64), (128, 256), (256, 512)])
+@pytest.mark.parametrize("D,DV", [(64, 64), (128, 256), (256, 512), (192, 128)])
 @pytest.mark.parametrize("S,causal", [(256, True), (200, False), (130, True)])
 def test_sigmoid_other_head_sizes(D, DV, S, causal):
     hb = _hb()
@@ -50,7 +50,7 @@ def test_sigmoid_other_head_sizes(D, DV, S, causal):
     oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
 
 
-@pytest.mark.parametrize("B,H,S,D,DV", [(1, 6, 2048, 64, 64), (1, 2, 130, 64, 64), (1, 2, 256, 256, 512)])
+@pytest.mark.parametrize("B,H,S,D,DV", [(1, 6, 2048, 64, 64), (1, 2, 130, 64, 64), (1, 2, 256, 256, 512), (1, 2, 333, 192, 128)])
 def test_relu_other_head_sizes(B, H, S, D, DV):
     """First case: the reference's own relu test (testing/test.py:62), fp16, inputs scaled as there (:609-610)."""
     hb = _hb()
@@ -79,7 +79,7 @@ def test_reference_softmax_test_shape_128_256():
 def test_causal_mask_is_exact_other_head_sizes():
     """Poisoning keys and values behind the diagonal must not change a row bit for bit."""
     hb = _hb()
-    for D, DV in ((64, 64), (128, 256), (256, 256)):
+    for D, DV in ((64, 64), (128, 256), (256, 256), (192, 128)):
         B, H, S = 1, 2, 256
         q, k, v = (t.cuda() for t in inputs.softmax_inputs(B, H, S, D, DV, seed=D))
         cut = 100
@@ -223,7 +223,7 @@ def test_row_without_any_key_gives_zeros():
     assert float(o.float().abs().max()) == 0.0 and bool(torch.isinf(lse).all())
 
 
-@pytest.mark.parametrize("D,DV", [(128, 128), (64, 64), (128, 256), (256, 256)])
+@pytest.mark.parametrize("D,DV", [(128, 128), (64, 64), (128, 256), (256, 256), (192, 128)])
 @pytest.mark.parametrize("B,H,Hkv,Sq,Skv", [(8, 16, 16, 1, 4096), (2, 8, 2, 1, 1000), (1, 4, 4, 17, 700), (1, 2, 1, 32, 2048)])
 def test_split_kv_decode_matches_unsplit(D, DV, B, H, Hkv, Sq, Skv):
     """Decode shapes through the split-KV path (workspace given: the default of the wrapper) and unsplit: both against

@@ -32,7 +32,7 @@ def test_parallel_forward_random(seed):
     hb = _hb()
     random.seed(seed)
     g = torch.Generator().manual_seed(seed)
-    D, DV = random.choice([(128, 128), (128, 128), (64, 64), (128, 256), (256, 256)])
+    D, DV = random.choice([(128, 128), (128, 128), (64, 64), (128, 256), (256, 256), (192, 128)])
     family = random.choice(["softmax", "softmax", "sigmoid", "relu"])
     dtype = random.choice([torch.bfloat16, torch.float16])
     B, Hkv, grp = random.randint(1, 3), random.randint(1, 3), random.choice([1, 1, 2, 4])
@@ -84,7 +84,7 @@ def test_parallel_backward_random(seed):
     hb = _hb()
     random.seed(100 + seed)
     g = torch.Generator().manual_seed(100 + seed)
-    D, DV = random.choice([(128, 128), (64, 64), (128, 256)])
+    D, DV = random.choice([(128, 128), (64, 64), (128, 256), (192, 128)])
     family = random.choice(["softmax", "softmax", "sigmoid", "relu"])
     dtype = random.choice([torch.bfloat16, torch.float16])
     B, Hkv, grp = random.randint(1, 2), random.randint(1, 2), random.choice([1, 2, 3])
