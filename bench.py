@@ -517,10 +517,10 @@ def bench_reference_shapes(steps, warmup):
 
 
 def bench_reference_benchmark_shapes(steps, warmup):
-    """The two parallel-attention figures of the reference's AMD benchmark that BASELINE's configurations do not cover
-    (testing/benchmark_mi250.py:40-55): causal softmax at the DeepSeek-V2-Lite head sizes (16 heads, Dqk 192, Dv 128, fp16) and
-    ReLU attention at the ViT-S head size (6 heads, 64 / 64, fp16), forward and backward through the C ABI at B = 8 / 64.
-    The reference writes its own timings to CSV files at run time and holds none in the tree."""
+    """Figures of the reference's own benchmarks that BASELINE's configurations do not cover (testing/benchmark_mi250.py:40-55,
+    testing/benchmark_h100.py:112,129): causal softmax at the DeepSeek-V2-Lite head sizes (16 heads, Dqk 192, Dv 128, fp16),
+    ReLU attention at the ViT-S head size (6 heads, 64 / 64, fp16) and gated retention at 64 / 64 and 256 / 256, forward and
+    backward through the C ABI.  The reference writes its own timings to CSV files at run time and holds none in the tree."""
     import torch
     from metaattention_amd import hip_backend as hb
     out = {}
@@ -539,6 +539,20 @@ def bench_reference_benchmark_shapes(steps, warmup):
         flops = (0.5 if causal else 1.0) * 2.0 * B * H * S * S * (D + DV)
         out[name] = dict(fwd_ms=round(ms_f, 4), fwd_tflops=round(flops / ms_f / 1e9, 1), bwd_ms=round(ms_b, 4),
                          bwd_tflops_2p5x=round(2.5 * flops / ms_b / 1e9, 1))
+    # gated retention at the two head sizes of testing/benchmark_h100.py:112,129 (16 heads 64 / 64: the key width runs in the
+    # 128-wide kernel; 40 heads 256 / 256), per-token log decay, forward and backward
+    for H, Dk, Dv in ((16, 64, 64), (40, 256, 256)):
+        B, T = 8, 4096
+        q = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 4).bfloat16()
+        k = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 4).bfloat16()
+        v, do = (torch.randn(B, H, T, Dv, device="cuda", generator=g).bfloat16() for _ in range(2))
+        ld = torch.nn.functional.logsigmoid(torch.randn(B, H, T, device="cuda", generator=g) + 3.0)
+        o = torch.empty_like(v)
+        ws = torch.empty(max(hb.linear_workspace_bytes(B, H, H, H, T, Dk, Dv), 16), dtype=torch.uint8, device="cuda")
+        ms_f = time_gpu(lambda: hb.linear_fwd(q, k, v, ld, q_scale=Dk ** -0.5, out=o, workspace=ws), steps, warmup)
+        wsb = torch.empty(_linear_bwd_workspace(hb, B, H, H, H, T, Dk, Dv), dtype=torch.uint8, device="cuda")
+        ms_b = time_gpu(lambda: hb.linear_bwd(q, k, v, ld, do, q_scale=Dk ** -0.5, workspace=wsb), max(steps // 3, 3), 2)
+        out[f"gated_retention_b8_h{H}_s4096_{Dk}_{Dv}_bf16"] = dict(fwd_ms=round(ms_f, 4), bwd_ms=round(ms_b, 4))
     return out
 
 

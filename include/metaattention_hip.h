@@ -185,7 +185,8 @@ typedef struct ma_attn_bwd_params {
  * q [B,Hq,T,Dk], k [B,Hk,T,Dk], v/o [B,H,T,Dv] (BHSD, contiguous), log_decay
  * fp32 [B,H,T]; head h reads q head h/(H/Hq) and k head h/(H/Hk) (:172,:351-352).
  * v_scale (may be NULL) is fp32 [B,H,T]: the fused per-token v modifier
- * (core/lower/lower_linear.py:211-287). */
+ * (core/lower/lower_linear.py:211-287).  dim_k 64, 128, 192 or 256 (64 and 192 run in the 128- / 256-wide kernel, the rest of
+ * the contraction being zeros that are never loaded), dim_v a multiple of 64. */
 typedef struct ma_linear_params {
   int32_t dtype;
   int32_t batch, heads, heads_q, heads_k, seqlen, dim_k, dim_v, chunk;
@@ -203,7 +204,7 @@ typedef struct ma_linear_params {
  * compute_final_dg :64-76): gradients of ma_linear_fwd's o with respect to q, k, v, log_decay and v_scale, given dout.
  * Tensors as in ma_linear_params (bf16, BHSD, contiguous, 16-byte aligned); dout [B,H,T,Dv] bf16; dq, dk, dv are bf16
  * with the shapes of q, k, v (heads that share a q / k head have their gradients summed, :1300-1303); dlog_decay fp32
- * [B,H,T]; dv_scale fp32 [B,H,T], written when v_scale is given (may then still be NULL to skip it).  dim_k 128 or 256,
+ * [B,H,T]; dv_scale fp32 [B,H,T], written when v_scale is given (may then still be NULL to skip it).  dim_k 64, 128, 192 or 256,
  * dim_v a multiple of 64, at most 4096.  The workspace (ma_linear_bwd_workspace_bytes, 256-byte aligned) holds the fp32 per-head
  * gradients the decay gradient is formed from, and is required. */
 typedef struct ma_linear_bwd_params {

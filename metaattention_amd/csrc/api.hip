@@ -243,8 +243,13 @@ static ma::LinArgs linear_args(const ma_linear_params* p) {
   a.q_scale = p->q_scale;
   a.out_f32 = p->out_fp32 != 0 ? 1 : 0;
   a.B = p->batch; a.H = p->heads; a.Hq = p->heads_q; a.Hk = p->heads_k; a.T = p->seqlen; a.Dv = p->dim_v;
+  // a key width of 64 or 192 runs in the 128- / 256-wide kernel: the operands' rows are read as they are (general operand
+  // addressing) and the rest of the contraction is zeros that are neither loaded nor multiplied
+  if (p->dim_k == 64 || p->dim_k == 192) { a.q_row = a.k_row = p->dim_k; a.qk_cols = p->dim_k; }
   return a;
 }
+// the key width of the kernel that takes dim_k
+static int linear_kernel_dk(int dim_k) { return dim_k == 64 ? 128 : dim_k == 192 ? 256 : dim_k; }
 
 // The state of one sequence stays on chip; a workspace is only used when the sequence is cut into
 // segments that run side by side (few batch x heads): it then holds the segments' fp32 end states.
@@ -255,7 +260,7 @@ size_t ma_linear_workspace_bytes(const ma_linear_params* p) {
       p->heads % p->heads_q != 0 || p->heads % p->heads_k != 0 || p->segments < 0)
     return 0;
   size_t bytes = 0;
-  if (ma::linear_fwd_dispatch(linear_args(p), p->dim_k, p->segments, nullptr, 0, nullptr, &bytes) != 0) return 0;
+  if (ma::linear_fwd_dispatch(linear_args(p), linear_kernel_dk(p->dim_k), p->segments, nullptr, 0, nullptr, &bytes) != 0) return 0;
   return bytes;
 }
 
@@ -267,9 +272,9 @@ int ma_linear_fwd(const ma_linear_params* p, ma_stream_t stream) {
   for (uintptr_t x : ptrs)
     if (x % 16 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: q/k/v/o must be 16-byte aligned");
   const ma::LinArgs a = linear_args(p);
-  const int rc = ma::linear_fwd_dispatch(a, p->dim_k, p->segments, p->workspace, p->workspace_bytes, (hipStream_t)stream, nullptr);
+  const int rc = ma::linear_fwd_dispatch(a, linear_kernel_dk(p->dim_k), p->segments, p->workspace, p->workspace_bytes, (hipStream_t)stream, nullptr);
   if (rc == -2)
-    return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: no kernel for dim_k=%d (128 or 256) / dim_v=%d (multiple of 64)", p->dim_k, p->dim_v);
+    return fail(MA_ERR_UNSUPPORTED, "ma_linear_fwd: no kernel for dim_k=%d (64, 128, 192 or 256) / dim_v=%d (multiple of 64)", p->dim_k, p->dim_v);
   if (rc != 0) return fail(MA_ERR_LAUNCH, "ma_linear_fwd: launch failed: %s", hipGetErrorString(ma::t_hip_error));
   return MA_OK;
 }
@@ -281,8 +286,8 @@ static int check_linear_bwd(const ma_linear_bwd_params* p, const char* who) {
   if (p->dtype != MA_BF16) return fail(MA_ERR_UNSUPPORTED, "%s: only bf16 (the reference's linear kernels are bf16 only)", who);
   if (p->heads % p->heads_q != 0 || p->heads % p->heads_k != 0)
     return fail(MA_ERR_INVALID_ARG, "%s: heads (%d) must be a multiple of heads_q (%d) and heads_k (%d)", who, p->heads, p->heads_q, p->heads_k);
-  if ((p->dim_k != 128 && p->dim_k != 256) || p->dim_v % 64 != 0 || p->dim_v > 4096)
-    return fail(MA_ERR_UNSUPPORTED, "%s: dim_k=%d must be 128 or 256 and dim_v=%d a multiple of 64 (at most 4096)", who, p->dim_k, p->dim_v);
+  if ((p->dim_k != 64 && p->dim_k != 128 && p->dim_k != 192 && p->dim_k != 256) || p->dim_v % 64 != 0 || p->dim_v > 4096)
+    return fail(MA_ERR_UNSUPPORTED, "%s: dim_k=%d must be 64, 128, 192 or 256 and dim_v=%d a multiple of 64 (at most 4096)", who, p->dim_k, p->dim_v);
   if ((int64_t)p->batch * p->heads * p->seqlen * (int64_t)(p->dim_k > p->dim_v ? p->dim_k : p->dim_v) / 8 > 0x7fffffffll * 256)
     return fail(MA_ERR_UNSUPPORTED, "%s: grid too large", who);
   return MA_OK;

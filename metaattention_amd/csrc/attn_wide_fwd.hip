@@ -450,7 +450,7 @@ static int launch_wide(const AttnArgs& a, hipStream_t stream) {
 // so that about four workgroups per CU are in flight, each with at least 8 tiles of 32 keys.
 int attn_decode_splits(int family, bool causal, int B, int H, int Sq, int Skv, int dqk, int dv) {
   if (family != WF_SOFTMAX || causal || Sq > 32) return 1;
-  if (!((dqk == 128 && dv == 128) || (dqk == 64 && dv == 64) || (dqk == 128 && dv == 256) || (dqk == 256 && dv == 256))) return 1;
+  if (!((dqk == 128 && dv == 128) || (dqk == 64 && dv == 64) || (dqk == 128 && dv == 256) || (dqk == 256 && dv == 256) || (dqk == 192 && dv == 128))) return 1;
   const int tiles = (Skv + 31) / 32;
   int n = 1024 / (B * H);
   if (n > tiles / 8) n = tiles / 8;

@@ -306,7 +306,9 @@ struct Slices {
 }  // namespace
 
 int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t stream, size_t* query) {
-  if ((a.Dk != 128 && a.Dk != 256) || a.Dv % 64 != 0 || a.Dv > 16 * 256) return -2;
+  if ((a.Dk != 64 && a.Dk != 128 && a.Dk != 192 && a.Dk != 256) || a.Dv % 64 != 0 || a.Dv > 16 * 256) return -2;
+  // (a key width of 64 or 192 is contracted in the 128- / 256-wide scan kernel: the missing columns are zeros that are never loaded)
+  const int DKP = a.Dk <= 128 ? 128 : 256, dk_cols = a.Dk == DKP ? 0 : a.Dk;
   const int64_t BHT = (int64_t)a.B * a.H * a.T;
   const Slices sl(a.Dv);   // contraction of the dq and dk scans
 
@@ -329,7 +331,9 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
     for (int s = 0; s < sl.n; s++)
       if (linear_fwd_dispatch(la, sl.w[s], 0, nullptr, 0, nullptr, &need) == 0 && need > scan_ws) scan_ws = need;
     la.Hq = a.Hk; la.Hk = a.Hq; la.Dv = a.Dv;
-    if (linear_fwd_dispatch(la, a.Dk, 0, nullptr, 0, nullptr, &need) == 0 && need > scan_ws) scan_ws = need;
+    la.qk_cols = dk_cols;
+    if (dk_cols) la.q_row = la.k_row = a.Dk;
+    if (linear_fwd_dispatch(la, DKP, 0, nullptr, 0, nullptr, &need) == 0 && need > scan_ws) scan_ws = need;
   }
   const size_t o_scan = take(scan_ws);
   if (query) { *query = off; return 0; }
@@ -373,8 +377,8 @@ int linear_bwd_run(const LinBwdArgs& a, void* ws, size_t ws_bytes, hipStream_t s
   // du (reversed) = LA(R k, R q, R do), contraction over the key columns: the operands are read in reversed time in place.
   // Without a v_scale dv is du itself, and the scan writes it: bf16, rows back in time order.
   const bool direct_dv = !a.v_scale && !a.dv_scale;
-  if (const int rc = scan_launch(Operand{k_p, a.Hk, a.Dk}, Operand{q_p, a.Hq, a.Dk}, Operand{do_p, a.H, a.Dv}, true, a.Dk, a.Dv, grev, nullptr,
-                                 direct_dv ? a.dv : (void*)du, false, 1, 0, direct_dv))
+  if (const int rc = scan_launch(Operand{k_p, a.Hk, a.Dk}, Operand{q_p, a.Hq, a.Dk}, Operand{do_p, a.H, a.Dv}, true, DKP, a.Dv, grev, nullptr,
+                                 direct_dv ? a.dv : (void*)du, false, 1, dk_cols, direct_dv))
     return rc;
   if (direct_dv) du = nullptr;
 

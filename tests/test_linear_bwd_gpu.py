@@ -49,6 +49,9 @@ def _check(got, ref, what):
     (1, 2, 2, 50, 256, 192, False),     # 192 value columns as one 256-wide piece
     (1, 2, 2, 130, 256, 768, False),    # three equal pieces side by side in one launch
     (1, 1, 1, 1, 128, 64, False),
+    (1, 2, 2, 150, 64, 64, False),      # key width 64: contracted in the 128-wide scan kernel
+    (2, 1, 4, 77, 64, 64, True),        # the same with heads that share q and k and a value scale
+    (1, 2, 2, 100, 192, 128, False),    # key width 192 in the 256-wide kernel
 ])
 def test_linear_backward(B, Hq, H, T, Dk, Dv, use_vs):
     hb = _hb()

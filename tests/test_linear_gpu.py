@@ -22,6 +22,7 @@ def _hb():
 @pytest.mark.parametrize("B,H,T,Dk,Dv", [
     (1, 2, 64, 256, 256), (1, 2, 256, 256, 512), (2, 3, 100, 128, 64), (1, 2, 128, 128, 128),
     (1, 1, 1, 128, 64), (1, 2, 33, 256, 128), (1, 16, 512, 256, 512),
+    (2, 3, 100, 64, 64), (1, 2, 130, 192, 128), (1, 4, 300, 64, 128),   # key widths 64 and 192: contracted in the 128- / 256-wide kernel
 ])
 def test_retnet_chunked(B, H, T, Dk, Dv):
     hb = _hb()
@@ -92,6 +93,29 @@ def test_engine_gated_retention():
     ref = oracle.simple_gla_chunked(q, k, v, g)
     oracle.assert_close(o.float().cpu(), ref, rtol=1e-1, atol=1e-1)
     oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=1e-3)   # outputs are O(10): bf16 output rounding
+
+
+def test_engine_gated_retention_64_64():
+    """The gated-retention shape of the reference's benchmark (testing/benchmark_h100.py:112: 16 heads, Dk = Dv = 64),
+    forward and backward through the operator."""
+    B, H, T, Dk, Dv = 1, 16, 192, 64, 64
+    mod = specs.gated_retention(B, H, T, Dk, Dv)
+    gen = torch.Generator().manual_seed(8)
+    q = torch.randn(B, H, T, Dk, generator=gen).bfloat16()
+    k = torch.randn(B, H, T, Dk, generator=gen).bfloat16()
+    v = torch.randn(B, H, T, Dv, generator=gen).bfloat16()
+    g = torch.nn.functional.logsigmoid(torch.randn(B, H, T, generator=gen)).clamp_min(-5)
+    dout = (0.25 * torch.randn(B, H, T, Dv, generator=gen)).bfloat16()
+    qc, kc, vc, gc = (t.cuda().requires_grad_(True) for t in (q, k, v, g))
+    o = mod(qc, kc, vc, gc)
+    o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    ref = oracle.simple_gla_chunked(q, k, v, g)
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=1e-3)
+    dq, dk, dv, dg, _ = oracle.linear_attention_grads(q, k, v, g, dout, q_scale=Dk ** -0.5)
+    for name, a, b in (("dq", qc.grad, dq), ("dk", kc.grad, dk), ("dv", vc.grad, dv)):
+        oracle.assert_close(a.float().cpu(), b.float(), rtol=RTOL, atol=ATOL, mismatch_ratio=5e-3, msg=name)
+    assert float((gc.grad.float().cpu() - dg.float()).abs().max()) <= max(0.03 * float(dg.abs().max()), 1e-2)
 
 
 def test_full_size_properties():
