@@ -168,7 +168,8 @@ def test_engine_grouped_query_softmax():
     oracle.assert_close(o.float().cpu(), oracle.softmax_attention(q, k, v, causal=True), rtol=RTOL, atol=ATOL)
 
 
-@pytest.mark.parametrize("B,H,HKV,S,KV,D,DV", [(8, 16, 16, 1, 4096, 128, 128), (2, 32, 4, 1, 1000, 128, 128), (1, 4, 4, 3, 300, 64, 64)])
+@pytest.mark.parametrize("B,H,HKV,S,KV,D,DV", [(8, 16, 16, 1, 4096, 128, 128), (2, 32, 4, 1, 1000, 128, 128), (1, 4, 4, 3, 300, 64, 64),
+                                             (8, 16, 16, 1, 2048, 192, 128)])   # (last: testing/benchmark_h100.py:63)
 def test_engine_dense_decode(B, H, HKV, S, KV, D, DV):
     """Decode operators (first case: testing/test.py:56, reference function :131-148): a short query against a long cache,
     no mask, multi-head and grouped-query."""
