@@ -748,6 +748,14 @@ struct FusedStepRegs {
 // bytes comes with the tile (whole tiles of a 16-byte aligned mask; others are read from global memory), and the
 // masked scores are set to -inf in the same place as for the structural masks.
 constexpr int FUSED_LIST_MAX = 2048;   // steps of a key block that the list holds (the launcher checks)
+// Phase F of a step alternates the k slices of S and dP while both have some left, then finishes the longer contraction:
+// MFMA j of the phase is slice `slice(j)` of S (`is_s(j)`) or of dP.
+template <int KS, int VS>
+struct PhaseF {
+  static constexpr int KMIN = KS < VS ? KS : VS;
+  static constexpr bool is_s(int j) { return j < 2 * KMIN ? j % 2 == 0 : KS > VS; }
+  static constexpr int slice(int j) { return j < 2 * KMIN ? j / 2 : KMIN + (j - 2 * KMIN); }
+};
 template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL, bool MASKS>
 __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBwdArgs a) {
   using E = Elem<T>;
@@ -755,17 +763,17 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBw
   using x4 = typename E::x4;
   constexpr int BNW = 128, BMT = 32;
   constexpr int KS = DQK / 16, VS = DV / 16, QB = DQK / 32, VB = DV / 32;
-  constexpr int QROW = DQK * 2, DOROW = DV * 2;
+  constexpr int QROW = pad_width(DQK) * 2, DOROW = DV * 2;   // (LDS rows; 192-wide queries sit in 256-wide rows)
   // a stage: the Q tile and the dO tile; behind the stages, 512 bytes per stage: lse (first 128) and delta (at 256) of its rows
   constexpr int QTILE = BMT * QROW, DOTILE = BMT * DOROW, STAGE = QTILE + DOTILE;
-  constexpr int NST = MASKS ? 4 : fused_stages(DQK, DV), LA = NST == 8 ? 4 : 3, ROWVALS = NST * STAGE;
+  constexpr int NST = MASKS ? 4 : fused_stages(pad_width(DQK), DV), LA = NST == 8 ? 4 : 3, ROWVALS = NST * STAGE;
   // (MASKS) behind the row values: 1 KB of mask bytes per stage and wave, then the step list and its length
   constexpr int KEEP = ROWVALS + NST * 512, LIST = KEEP + NST * 4 * 1024, LIST_N = LIST + FUSED_LIST_MAX * 4;
   // the MFMAs of a step and the fragment ring
   constexpr int NF = KS + VS, NV = 2 * VB, NK = 2 * QB, NTOT = NF + NV + NK;
   constexpr int RING = 8, AH = NK < 6 ? NK : 6;
   static_assert(NTOT % RING == 0 && AH < RING && AH <= NK && AH <= NF, "fragment ring");
-  static_assert(KS == VS, "phase F alternates the k slices of S and dP");
+  using PhF = PhaseF<KS, VS>;
 
   extern __shared__ __align__(16) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(MA_LDS char*)smem;
@@ -854,11 +862,13 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBw
   auto list_request = [&](int i) { return lds_read<uint32_t>(lds0 + LIST + 4 * (i < n_steps ? i : 0)); };
   auto uniform = [&](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
   const int64_t q_row_bytes = a.qss * 2, do_row_bytes = a.doss * 2;
-  TileDma<QROW, 4> q_dma;
+  TileDma<QROW, 4, DQK / 8> q_dma;
   TileDma<DOROW, 4> do_dma;
   q_dma.init((uint32_t)q_row_bytes, wave, lane);
   do_dma.init((uint32_t)do_row_bytes, wave, lane);
-  constexpr int TILE_DMAS = TileDma<QROW, 4>::NJ + TileDma<DOROW, 4>::NJ;   // what a wave issues per tile at least
+  // what a wave issues per tile at least (with rows wider than the head size a lane may sit out some of its instructions,
+  // a whole wave never does: the chunks of an instruction's rows are spread over all lanes)
+  constexpr int TILE_DMAS = TileDma<QROW, 4>::NJ + TileDma<DOROW, 4>::NJ;
   auto issue_tile = [&](int hg, int t, int st, bool full = true) {
     const int h = hk * a.kv_group + hg, m0 = (t_first + t) * BMT;
     if constexpr (MASKS) {
@@ -873,7 +883,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBw
       q_dma.issue(qb + (int64_t)m0 * q_row_bytes, lds0 + st * STAGE, wave);
       do_dma.issue(dob + (int64_t)m0 * do_row_bytes, lds0 + st * STAGE + QTILE, wave);
     } else {
-      dma_tile<QROW, 4>(qb, q_row_bytes, m0, a.Sq, lds0 + st * STAGE, wave, lane);
+      dma_tile<QROW, 4, DQK / 8>(qb, q_row_bytes, m0, a.Sq, lds0 + st * STAGE, wave, lane);
       dma_tile<DOROW, 4>(dob, do_row_bytes, m0, a.Sq, lds0 + st * STAGE + QTILE, wave, lane);
     }
     if constexpr (FAMILY == BF_SOFTMAX) {
@@ -896,20 +906,20 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBw
 
   // the lane's part of the fragment addresses, relative to a tile: row reads (A operands of S and dP) and
   // transposing reads (A operands of dV^T and dK^T: the tile's columns)
-  const uint32_t aq_l = (uint32_t)(r * QROW) + (uint32_t)((g ^ swz_tile<DQK / 8>(r)) << 4);
+  const uint32_t aq_l = (uint32_t)(r * QROW) + (uint32_t)((g ^ swz_tile<QROW / 16>(r)) << 4);
   const uint32_t ad_l = (uint32_t)(r * DOROW) + (uint32_t)((g ^ swz_tile<DV / 8>(r)) << 4);
   const int jr = (lane & 15) >> 2, lc = (((lane >> 4) & 1) << 1) | ((lane & 3) >> 1);
-  const uint32_t bq_l = (uint32_t)((4 * g + jr) * QROW + (lane & 1) * 8) + (uint32_t)((lc ^ swz_tile<DQK / 8>(4 * g + jr)) << 4);
+  const uint32_t bq_l = (uint32_t)((4 * g + jr) * QROW + (lane & 1) * 8) + (uint32_t)((lc ^ swz_tile<QROW / 16>(4 * g + jr)) << 4);
   const uint32_t bd_l = (uint32_t)((4 * g + jr) * DOROW + (lane & 1) * 8) + (uint32_t)((lc ^ swz_tile<DV / 8>(4 * g + jr)) << 4);
   // the fragment of MFMA j of a step whose current tile sits at `cur` and whose next tile at `nxt` (LDS addresses)
   auto fragment = [&](auto jc, uint32_t cur, uint32_t nxt) __attribute__((always_inline)) -> x8 {
     constexpr int j = decltype(jc)::value;
     // (consecutive MFMAs go to different accumulators: with one wave on the SIMD a dependent MFMA waits for the result
     // of the one before it.  Phase F alternates S and dP; phases V and K walk the column blocks before the k slices)
-    if constexpr (j < NF && j % 2 == 0) {
-      return lds_read<x8>((nxt + aq_l) ^ (uint32_t)((j / 2) * 32));
+    if constexpr (j < NF && PhF::is_s(j)) {
+      return lds_read<x8>((nxt + aq_l) ^ (uint32_t)(PhF::slice(j) * 32));
     } else if constexpr (j < NF) {
-      return lds_read<x8>((nxt + QTILE + ad_l) ^ (uint32_t)((j / 2) * 32));
+      return lds_read<x8>((nxt + QTILE + ad_l) ^ (uint32_t)(PhF::slice(j) * 32));
     } else {
       constexpr bool is_v = j < NF + NV;
       constexpr int idx = is_v ? j - NF : j - NF - NV, db = idx % (is_v ? VB : QB), sl = idx / (is_v ? VB : QB);
@@ -1028,8 +1038,8 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_fused_kernel(const AttnBw
         if constexpr (j + AH < NTOT) fr[(j + AH) % RING] = fragment(IntC<j + AH>(), cur_tile, nxt_tile);
         else fr[(j + AH) % RING] = fragment(IntC<j + AH - NTOT>(), nxt_tile, nn_tile);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (j < NF && j % 2 == 0) nxt.s = E::mfma32(fr[j % RING], kf[j / 2], j == 0 ? zero16 : nxt.s);
-        else if constexpr (j < NF) nxt.dp = E::mfma32(fr[j % RING], vf[j / 2], j == 1 ? zero16 : nxt.dp);
+        if constexpr (j < NF && PhF::is_s(j)) nxt.s = E::mfma32(fr[j % RING], kf[PhF::slice(j)], j == 0 ? zero16 : nxt.s);
+        else if constexpr (j < NF) nxt.dp = E::mfma32(fr[j % RING], vf[PhF::slice(j)], j == 1 ? zero16 : nxt.dp);
         else if constexpr (j < NF + NV) dv[(j - NF) % VB] = E::mfma32(fr[j % RING], pf[(j - NF) / VB], dv[(j - NF) % VB]);
         else dk[(j - NF - NV) % QB] = E::mfma32(fr[j % RING], dsf[(j - NF - NV) / QB], dk[(j - NF - NV) % QB]);
         // vector work behind the MFMA: p of the step's 16 elements in phase F, ds in phase V
@@ -1107,12 +1117,12 @@ static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   args.num_blocks = (a.Sq + 127) / 128;
   hipLaunchKernelGGL(k1, dim3((unsigned)(args.num_blocks * a.B * a.H)), dim3(256), lds, stream, args);
   args.num_blocks = (a.Skv + 127) / 128;
-  if constexpr (FAMILY != BF_RETENTION && DQK + DV <= 256) {
+  if constexpr (FAMILY != BF_RETENTION && (DQK + DV <= 256 || (DQK == 192 && DV == 128))) {
     // dk and dv by the pipelined single launch (with masks: as long as a key block's steps fit its list)
     const bool masks = a.elem_mask_t || a.q_block_mask;
     if (a.scale != 0.f && (!masks || (int64_t)((a.Sq + 31) / 32) * a.kv_group <= FUSED_LIST_MAX)) {
-      constexpr size_t ftiles = fused_stages(DQK, DV) * ((size_t)32 * (DQK + DV) * 2 + 512);
-      constexpr size_t mtiles = 4 * ((size_t)32 * (DQK + DV) * 2 + 512 + 4 * 1024) + FUSED_LIST_MAX * 4 + 16;
+      constexpr size_t ftiles = fused_stages(pad_width(DQK), DV) * ((size_t)32 * (pad_width(DQK) + DV) * 2 + 512);
+      constexpr size_t mtiles = 4 * ((size_t)32 * (pad_width(DQK) + DV) * 2 + 512 + 4 * 1024) + FUSED_LIST_MAX * 4 + 16;
       constexpr size_t fmax = ftiles > mtiles ? ftiles : mtiles, flds = fmax > ostage ? fmax : ostage;
       auto kf = attn_bwd_dkv_fused_kernel<T, DQK, DV, FAMILY, CAUSAL, false>;
       auto km = attn_bwd_dkv_fused_kernel<T, DQK, DV, FAMILY, CAUSAL, true>;
