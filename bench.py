@@ -526,6 +526,7 @@ def bench_reference_benchmark_shapes(steps, warmup):
     out = {}
     g = torch.Generator(device="cuda").manual_seed(0)
     for name, fam, causal, B, H, S, D, DV in (("softmax_causal_deepseek_v2_lite_b8_h16_s4096_192_128_fp16", hb.MA_ATTN_SOFTMAX, True, 8, 16, 4096, 192, 128),
+                                              ("softmax_causal_b8_h12_s4096_128_256_fp16", hb.MA_ATTN_SOFTMAX, True, 8, 12, 4096, 128, 256),   # (benchmark_h100.py:87)
                                               ("relu_vit_s_b64_h6_s1024_64_64_fp16", hb.MA_ATTN_RELU, False, 64, 6, 1024, 64, 64)):
         q, k = (torch.randn(B, S, H, D, device="cuda", dtype=torch.float16, generator=g) for _ in range(2))
         v, do = (torch.randn(B, S, H, DV, device="cuda", dtype=torch.float16, generator=g) for _ in range(2))

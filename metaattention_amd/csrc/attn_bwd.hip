@@ -1117,6 +1117,7 @@ static int launch_bwd(const AttnBwdArgs& a, hipStream_t stream) {
   args.num_blocks = (a.Sq + 127) / 128;
   hipLaunchKernelGGL(k1, dim3((unsigned)(args.num_blocks * a.B * a.H)), dim3(256), lds, stream, args);
   args.num_blocks = (a.Skv + 127) / 128;
+  // (128 / 256 would fit the fused kernel's registers only with 60-90 spilled: measured no faster than its two launches)
   if constexpr (FAMILY != BF_RETENTION && (DQK + DV <= 256 || (DQK == 192 && DV == 128))) {
     // dk and dv by the pipelined single launch (with masks: as long as a key block's steps fit its list)
     const bool masks = a.elem_mask_t || a.q_block_mask;

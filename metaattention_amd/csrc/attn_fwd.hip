@@ -608,6 +608,20 @@ int attn_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, 
     return is_bf16 ? dispatch_family<__bf16, 128, 128>(a, family, causal, stream)
                    : dispatch_family<_Float16, 128, 128>(a, family, causal, stream);
   }
+  // 128 / 256 at prefill lengths: two launches of the 128 / 128 kernel, one per half of the value columns (given the
+  // probabilities the columns are independent; the scores are computed twice, which this kernel still does in less time than
+  // the general kernel needs once: 0.78 against 1.46 ms at B8 H12 S4096).  Both launches write the same row scales.
+  if (family != 3 && dqk == 128 && dv == 256 && a.Sq >= 256 && !a.kv_lens && !a.kv_block_mask && !a.o_part && !a.elem_mask && !a.add &&
+      !a.slope_q && !a.slope_kv && !(a.softcap > 0.f)) {
+    for (int half = 0; half < 2; half++) {
+      AttnArgs h = a;
+      h.v = (const char*)a.v + half * 128 * 2;
+      h.o = (char*)a.o + half * 128 * 2;
+      const int rc = is_bf16 ? dispatch_family<__bf16, 128, 128>(h, family, causal, stream) : dispatch_family<_Float16, 128, 128>(h, family, causal, stream);
+      if (rc != 0) return rc;
+    }
+    return 0;
+  }
   // the retention family, every other head size, per-batch lengths / kv block masks / element-wise masks, split-kv decode
   return attn_wide_fwd_dispatch(a, family, causal, is_bf16, dqk, dv, stream);
 }
