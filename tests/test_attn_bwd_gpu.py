@@ -320,16 +320,18 @@ def test_engine_backward_with_external_block_mask(family, mask, D, S, bq, bk):
     assert torch.count_nonzero(kc.grad[1, :bk, 1]) == 0 and torch.count_nonzero(vc.grad[1, :bk, 1]) == 0
 
 
-def test_masked_backward_through_the_c_abi_matches_causal():
+@pytest.mark.parametrize("D,DV", [(128, 128), (192, 128), (128, 256)])
+def test_masked_backward_through_the_c_abi_matches_causal(D, DV):
     """A lower-triangular keep mask through elem_mask / elem_mask_t gives the gradients of the causal flag (bit for bit:
-    the same tiles, the same masked elements), grouped-query heads included."""
+    the same tiles, the same masked elements), grouped-query heads included; at the head sizes of the fused dk / dv kernel
+    (128 / 128, 192 / 128: its masked form) and of the two-launch kernels (128 / 256)."""
     hb = _hb()
-    B, H, Hkv, S, D = 1, 4, 2, 257, 128
+    B, H, Hkv, S = 1, 4, 2, 257
     g = torch.Generator().manual_seed(11)
     q = torch.randn(B, S, H, D, generator=g).bfloat16().cuda()
     k = torch.randn(B, S, Hkv, D, generator=g).bfloat16().cuda()
-    v = torch.randn(B, S, Hkv, D, generator=g).bfloat16().cuda()
-    dout = torch.randn(B, S, H, D, generator=g).bfloat16().cuda()
+    v = torch.randn(B, S, Hkv, DV, generator=g).bfloat16().cuda()
+    dout = torch.randn(B, S, H, DV, generator=g).bfloat16().cuda()
     lse = torch.empty(B, H, S, device="cuda")
     o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=D ** -0.5, row_scale=lse)
     ref = hb.attn_bwd(q, k, v, o, dout, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=D ** -0.5)

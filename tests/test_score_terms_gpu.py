@@ -212,7 +212,8 @@ def test_backward_through_softcap():
 @pytest.mark.parametrize("D,DV,H,Hkv,Sq,Skv,causal,dtype", [(128, 128, 4, 2, 200, 200, True, torch.bfloat16),
                                                            (64, 64, 2, 2, 70, 333, False, torch.float16),
                                                            (256, 512, 2, 1, 160, 160, True, torch.bfloat16),
-                                                           (128, 256, 2, 2, 1100, 1100, True, torch.bfloat16)])
+                                                           (128, 256, 2, 2, 1100, 1100, True, torch.bfloat16),
+                                                           (192, 128, 2, 1, 300, 300, True, torch.float16)])
 def test_attn_bwd_score_terms_through_the_c_abi(D, DV, H, Hkv, Sq, Skv, causal, dtype):
     """hb.attn_bwd(score_add=..., pos_slope_*=..., softcap=...) directly: every head-size pair of the backward kernels,
     grouped kv heads, unequal lengths, an fp32 tile broadcast over batch (stride 0), all terms at once."""
