@@ -1,0 +1,11 @@
+// Parallel attention backward: the instantiations of attn_bwd_kernels.h for the head sizes 64 / 64
+// (one translation unit per group of head sizes, so that they compile side by side).
+#include "attn_bwd_kernels.h"
+
+namespace ma {
+
+int attn_bwd_64_64(const AttnBwdArgs& a, int family, bool causal, bool is_bf16, hipStream_t stream) {
+  return is_bf16 ? bwd_size<__bf16, 64, 64, true>(a, family, causal, stream) : bwd_size<_Float16, 64, 64, true>(a, family, causal, stream);
+}
+
+}  // namespace ma
