@@ -296,26 +296,40 @@ __global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_
           if (((keep[jj >> 2] >> (8 * (jj & 3))) & 0xff) == 0) s[jj] = -INFINITY;
       }
       if constexpr (FAMILY == WF_SOFTMAX) {
-        float mx = s[0];
+        // Lazy reference: the exponentials are taken relative to row_max, which only moves when some probability of the
+        // tile would exceed 2^8 (exact in fp32, in range for bf16 / fp16; the final division absorbs the offset) -- so
+        // the hot path has no maximum over the scores in front of its exponentials, only one over the probabilities
+        // behind them.  The first tile (row_max = -1e30: infinite probabilities) and growing scores take the cold path,
+        // which moves the reference of the rows concerned to their true maximum; both lanes of a row decide alike.
+        float p[16];
+        float sub = c_bias - row_max;
 #pragma unroll
-        for (int jj = 1; jj < 16; jj++) mx = fmaxf(mx, s[jj]);
-        mx = fmaxf(mx, xhalf(mx)) * c_scale + c_bias;
-        const float m_new = fmaxf(row_max, mx);
-        if (__any(m_new > row_max)) {
+        for (int jj = 0; jj < 16; jj++) p[jj] = fast_exp2(s[jj] * c_scale + sub);
+        const float pm = fmaxf(fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7]))),
+                               fmaxf(fmaxf(fmaxf(p[8], p[9]), fmaxf(p[10], p[11])), fmaxf(fmaxf(p[12], p[13]), fmaxf(p[14], p[15]))));
+        if (__any(pm > 256.f)) {
+          float mx = fmaxf(fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7]))),
+                           fmaxf(fmaxf(fmaxf(s[8], s[9]), fmaxf(s[10], s[11])), fmaxf(fmaxf(s[12], s[13]), fmaxf(s[14], s[15]))));
+          mx = fmaxf(mx, xhalf(mx)) * c_scale + c_bias;
+          // (each row decides for itself, from its own probabilities only: what another row of the wave holds -- keys a
+          // causal mask hides from this one, say -- must not change this row's bits)
+          const bool move = fmaxf(pm, xhalf(pm)) > 256.f;
+          const float m_new = move ? fmaxf(row_max, mx) : row_max;
           const float corr = fast_exp2(row_max - m_new);
           r_part *= corr;
 #pragma unroll
           for (int i = 0; i < DB; i++)
 #pragma unroll
             for (int j = 0; j < 16; j++) o[i][j] *= corr;
+          row_max = m_new;
+          sub = c_bias - row_max;
+#pragma unroll
+          for (int jj = 0; jj < 16; jj++) p[jj] = fast_exp2(s[jj] * c_scale + sub);
         }
-        row_max = m_new;
-        const float sub = c_bias - row_max;
 #pragma unroll
         for (int jj = 0; jj < 16; jj++) {
-          const float p = fast_exp2(s[jj] * c_scale + sub);
-          r_part += p;
-          pf[jj >> 3][jj & 7] = (T)p;
+          r_part += p[jj];
+          pf[jj >> 3][jj & 7] = (T)p[jj];
         }
       } else if constexpr (FAMILY == WF_SIGMOID) {
 #pragma unroll
