@@ -408,3 +408,39 @@ def test_backward_full_size_properties():
     dq2, dk2, dv2 = hb.attn_bwd(q, k, v, o, dout * 2, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale)
     torch.cuda.synchronize()
     assert torch.equal(dq2, dq * 2) and torch.equal(dk2, dk * 2) and torch.equal(dv2, dv * 2)
+
+
+def test_deepseek_v2_lite_full_size():
+    """The reference's AMD benchmark shape (testing/benchmark_mi250.py:40-46: B8 H16 S4096, Dqk 192 / Dv 128, fp16, causal),
+    forward and backward through the C ABI: (batch, head) slices against the oracles, the closed form of the last key's dv,
+    linearity in dout."""
+    hb = _hb()
+    B, H, S, D, DV = 8, 16, 4096, 192, 128
+    scale = 1 / math.sqrt(D)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    q, k = (torch.randn(B, S, H, D, device="cuda", dtype=torch.float16, generator=g) for _ in range(2))
+    v, dout = (torch.randn(B, S, H, DV, device="cuda", dtype=torch.float16, generator=g) for _ in range(2))
+    lse = torch.empty(B, H, S, device="cuda")
+    print("deepseek-v2-lite full size 192/128", flush=True)
+    o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale, row_scale=lse)
+    dq, dk, dv = hb.attn_bwd(q, k, v, o, dout, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale)
+    torch.cuda.synchronize()
+    for t in (o, dq, dk, dv):
+        assert torch.isfinite(t.float()).all()
+    s_last = (q[:, -1].float() * k[:, -1].float()).sum(-1) * scale
+    p_last = torch.exp(s_last - lse[:, :, -1])
+    torch.testing.assert_close(dv[:, -1].float(), p_last.unsqueeze(-1) * dout[:, -1].float(), rtol=2e-2, atol=2e-2)
+    for b, h in [(0, 0), (7, 15), (3, 6)]:
+        sl = lambda t: t[b:b + 1, :, h:h + 1].cpu()
+        ref_o, ref_lse = oracle.softmax_attention(sl(q), sl(k), sl(v), causal=True, softmax_scale=scale, return_lse=True)
+        oracle.assert_close(sl(o).float(), ref_o, rtol=RTOL, atol=ATOL)
+        torch.testing.assert_close(lse[b:b + 1, h:h + 1].cpu(), ref_lse, rtol=1e-3, atol=1e-3)
+        if (b, h) != (3, 6):
+            ref = oracle.attention_grads(oracle.softmax_attention, sl(q), sl(k), sl(v), sl(dout), causal=True, softmax_scale=scale)
+            _check((sl(dq), sl(dk), sl(dv)), ref, f"192/128 full size slice ({b},{h})")
+    dq2, dk2, dv2 = hb.attn_bwd(q, k, v, o, dout * 2, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=scale)
+    torch.cuda.synchronize()
+    # (fp16: not exact as in bf16 -- ds is rounded to the tensor dtype, and where it is subnormal in fp16 a doubling does not
+    # commute with that rounding)
+    for a2, a1 in ((dq2, dq), (dk2, dk), (dv2, dv)):
+        torch.testing.assert_close(a2.float(), 2 * a1.float(), rtol=2e-2, atol=1e-3)
