@@ -37,9 +37,10 @@ def normal(rng, *shape, gain=1.0):
     return bf16_round(rng.standard_normal(shape).astype(np.float32) * gain)
 
 
-def softmax_case(rng, B, H, S, D, causal):
-    (qb, q), (kb, k), (vb, v) = normal(rng, B, S, H, D), normal(rng, B, S, H, D), normal(rng, B, S, H, D)
-    out = np.zeros((B, S, H, D))
+def softmax_case(rng, B, H, S, D, causal, DV=None):
+    DV = DV or D
+    (qb, q), (kb, k), (vb, v) = normal(rng, B, S, H, D), normal(rng, B, S, H, D), normal(rng, B, S, H, DV)
+    out = np.zeros((B, S, H, DV))
     lse = np.zeros((B, H, S))
     for b in range(B):
         for h in range(H):
@@ -155,6 +156,9 @@ CASES = {
     "gated_retention_b1h2t128": lambda r: recurrent_case(r, 1, 2, 2, 128, 128, 128, "gated"),
     "mamba2_b1h4t256": lambda r: recurrent_case(r, 1, 1, 4, 256, 128, 64, "mamba2"),
     "mla_b2h20s200": lambda r: mla_case(r, 2, 20, 200, 512, 64),
+    # DeepSeek-V2-Lite's head sizes (testing/benchmark_mi250.py:40-55) and a 64-wide gated retention (testing/benchmark_h100.py:112)
+    "softmax_causal_b1h2s144d192dv128": lambda r: softmax_case(r, 1, 2, 144, 192, True, DV=128),
+    "gated_retention_b1h2t128dk64": lambda r: recurrent_case(r, 1, 2, 2, 128, 64, 64, "gated"),
 }
 
 

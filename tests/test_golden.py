@@ -79,6 +79,7 @@ ORACLE_CASES = {
     "sigmoid_causal_b1h2s160d128": _o_sigmoid, "relu_b1h2s130d128": _o_relu,
     "retention_parallel_b1h2s136": _o_retention, "retnet_b1h2t160": _o_retnet,
     "gated_retention_b1h2t128": _o_gated, "mamba2_b1h4t256": _o_mamba2, "mla_b2h20s200": _o_mla,
+    "softmax_causal_b1h2s144d192dv128": _o_softmax, "gated_retention_b1h2t128dk64": _o_gated,
 }
 
 
@@ -147,6 +148,7 @@ GPU_CASES = {
     "softmax_causal_b1h2s160d128": _g_softmax, "sigmoid_causal_b1h2s160d128": _g_sigmoid, "relu_b1h2s130d128": _g_relu,
     "retention_parallel_b1h2s136": _g_retention, "retnet_b1h2t160": _g_linear, "gated_retention_b1h2t128": _g_linear,
     "mamba2_b1h4t256": _g_linear, "mla_b2h20s200": _g_mla,
+    "softmax_full_b1h1s96d64": _g_softmax, "softmax_causal_b1h2s144d192dv128": _g_softmax, "gated_retention_b1h2t128dk64": _g_linear,
 }
 
 
