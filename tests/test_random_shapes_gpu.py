@@ -156,3 +156,204 @@ def test_mla_random(seed):
     ref, lse_ref = oracle.mla_decode(q, q_pe, kv, k_pe, return_lse=True)
     oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
     torch.testing.assert_close(lse.cpu(), lse_ref, rtol=1e-4, atol=1e-4)
+
+
+FAMILIES = ("softmax", "softmax", "sigmoid", "relu")
+# Allowed fraction of elements outside atol 2e-2 / rtol 1e-2 in the sweeps below.  The un-normalised families sum hundreds of
+# probabilities that were rounded to the tensor dtype before P V (as the reference's kernel rounds them, attn_tl.py:165-169):
+# a row sum of magnitude 10 - 50 carries an absolute error of a few 1e-2, which the elements near zero cannot hide.  Every
+# case is also held to the reference's own acceptance (testing/test.py:571,623: 1e-1 / 1e-1, 1e-3 of the elements).
+RATIO = {"softmax": 0.0, "sigmoid": 2e-3, "relu": 5e-2}
+
+
+def _fam_code(hb, family):
+    return {"softmax": hb.MA_ATTN_SOFTMAX, "sigmoid": hb.MA_ATTN_SIGMOID, "relu": hb.MA_ATTN_RELU}[family]
+
+
+def _check_out(o, ref, family):
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=RATIO[family], msg="o")
+    oracle.assert_close(o.float().cpu(), ref, rtol=1e-1, atol=1e-1, mismatch_ratio=1e-3, msg="o (reference acceptance)")
+
+
+def _check_grads(got, ref, family, Skv, softcap=0.0):
+    # (a key that hundreds of queries see collects a gradient of magnitude 10 - 50, and cap * tanh(x) multiplies the score
+    # gradients by up to the cap: the same rounding argument as above; in fp16 the same cases are 8 x closer)
+    ratio = 3e-2 if Skv < 32 or family != "softmax" or softcap > 0 else 2e-3
+    for name, a, b in zip(("dq", "dk", "dv"), got, ref):
+        oracle.assert_close(a.float().cpu(), b.float(), rtol=RTOL, atol=ATOL, mismatch_ratio=ratio, msg=name)
+        oracle.assert_close(a.float().cpu(), b.float(), rtol=1e-1, atol=1e-1, mismatch_ratio=1e-3, msg=name + " (reference acceptance)")
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_element_masks_random(seed):
+    """Forward (and, for every other seed, backward) under random element-wise keep masks of four kinds (sliding window,
+    Bernoulli, prefix-LM, documents), per batch / head or broadcast, with and without the tile masks pooled from them
+    (entries 1 = some element kept, 2 = every element kept), lengths that are no multiple of anything."""
+    hb = _hb()
+    random.seed(1000 + seed)
+    g = torch.Generator().manual_seed(1000 + seed)
+    backward = seed % 2 == 1
+    D, DV = random.choice([(128, 128), (64, 64), (128, 256), (192, 128)] + ([] if backward else [(256, 256)]))
+    family = random.choice(FAMILIES)
+    dtype = random.choice([torch.bfloat16, torch.float16])
+    B, Hkv, grp = random.randint(1, 2), random.randint(1, 2), random.choice([1, 2])
+    H = Hkv * grp
+    Sq, Skv = random.randint(1, 400), random.randint(1, 500)
+    q = torch.randn(B, Sq, H, D, generator=g).to(dtype)
+    k = (0.5 * torch.randn(B, Skv, Hkv, D, generator=g)).to(dtype)
+    v = (0.5 * torch.randn(B, Skv, Hkv, DV, generator=g)).to(dtype)
+    kind = random.choice(["window", "random", "prefix", "doc"])
+    i, j = torch.arange(Sq).view(Sq, 1), torch.arange(Skv).view(1, Skv)
+    mb, mh = random.choice([1, B]), random.choice([1, H])
+    keep = torch.zeros(mb, mh, Sq, Skv, dtype=torch.bool)
+    for b in range(mb):
+        for h in range(mh):
+            if kind == "window":
+                keep[b, h] = (i >= j) & (i - j < random.randint(1, 200))
+            elif kind == "random":
+                keep[b, h] = torch.rand(Sq, Skv, generator=g) < random.choice([0.02, 0.5, 0.95])
+            elif kind == "prefix":
+                keep[b, h] = (j < random.randint(0, Skv)) | (i >= j)
+            else:
+                doc = random.randint(8, 150)
+                keep[b, h] = (i // doc == j // doc) & (i >= j)
+
+    def padded(m, rows, cols, fill):      # [.., rows, cols] uint8 holding m in its top left corner
+        out = torch.full((mb, mh, rows, cols), fill, dtype=torch.uint8)
+        out[:, :, :m.shape[2], :m.shape[3]] = m
+        return out
+
+    def pooled(m, with_all):              # tile mask over (128 rows x 32 columns) of m
+        rows, cols = (m.shape[2] + 127) // 128 * 128, (m.shape[3] + 31) // 32 * 32
+        any_ = padded(m, rows, cols, 0).view(mb, mh, rows // 128, 128, cols // 32, 32).amax(dim=(3, 5))
+        all_ = padded(m, rows, cols, 1).view(mb, mh, rows // 128, 128, cols // 32, 32).amin(dim=(3, 5))
+        return (any_ + all_ if with_all else any_).contiguous()
+
+    use_blocks, with_all = random.random() < 0.7, random.random() < 0.5
+    scale, bias = 1 / math.sqrt(D), (-1.0 if family == "sigmoid" else 0.0)
+    print(f"seed {seed}: mask {kind} [{mb},{mh}] {family} D{D}/{DV} B{B} H{H}/{Hkv} Sq{Sq} Skv{Skv} blocks={use_blocks}/{with_all} bwd={backward} {dtype}", flush=True)
+    em = padded(keep, Sq, (Skv + 3) // 4 * 4, 0).cuda()[..., :Skv]       # rows at 4-byte aligned addresses
+    lse = torch.full((B, H, Sq), float("nan"), device="cuda") if family == "softmax" else None
+    kw = dict(family=_fam_code(hb, family), causal=False, scale=scale, bias=bias)
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    o = hb.attn_fwd(qc, kc, vc, row_scale=lse, elem_mask=em, kv_block_mask=pooled(keep, with_all).cuda() if use_blocks else None,
+                    kv_block_size=32 if use_blocks else 0, **kw)
+    torch.cuda.synchronize()
+    okw = dict(keep=keep, family=family, softmax_scale=scale, bias=bias)
+    _check_out(o, oracle.masked_attention(q, k, v, **okw), family)
+    if backward:
+        dout = (0.5 * torch.randn(B, Sq, H, DV, generator=g)).to(dtype)
+        keep_t = keep.transpose(2, 3)
+        em_t = padded(keep_t, Skv, (Sq + 3) // 4 * 4, 0).cuda()[..., :Sq]
+        got = hb.attn_bwd(qc, kc, vc, o, dout.cuda(), lse, elem_mask=em, elem_mask_t=em_t,
+                          kv_block_mask=pooled(keep, with_all).cuda() if use_blocks else None,
+                          q_block_mask=pooled(keep_t, with_all).cuda() if use_blocks else None, **kw)
+        torch.cuda.synchronize()
+        _check_grads(got, oracle.attention_grads(oracle.masked_attention, q, k, v, dout, **okw), family, Skv)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_score_terms_random(seed):
+    """Forward (and, for every other seed, backward) with random additive score terms: a tile, a key vector, a per-row or a
+    per-head tensor in fp32 or the tensor dtype, linear terms in the two indices, tanh soft-capping (softmax), with and
+    without the causal flag."""
+    hb = _hb()
+    random.seed(3000 + seed)
+    g = torch.Generator().manual_seed(3000 + seed)
+    backward = seed % 2 == 1
+    D, DV = random.choice([(128, 128), (64, 64), (128, 256), (192, 128)] + ([] if backward else [(256, 256)]))
+    family = random.choice(FAMILIES)
+    dtype = random.choice([torch.bfloat16, torch.float16])
+    B, Hkv, grp = random.randint(1, 2), random.randint(1, 2), random.choice([1, 2])
+    H = Hkv * grp
+    causal = random.random() < 0.5
+    Sq = random.randint(1, 400)
+    Skv = Sq if causal else random.randint(1, 500)
+    q = torch.randn(B, Sq, H, D, generator=g).to(dtype)
+    k = (0.5 * torch.randn(B, Skv, Hkv, D, generator=g)).to(dtype)
+    v = (0.5 * torch.randn(B, Skv, Hkv, DV, generator=g)).to(dtype)
+    shape = random.choice([(1, H, Sq, Skv), (B, 1, 1, Skv), (B, H, Sq, 1), (1, 1, Sq, Skv), (1, H, 1, 1), None])
+    add = None
+    if shape is not None:
+        add = torch.randn(*shape, generator=g)
+        if random.random() < 0.4:
+            add = add.to(dtype)
+    slopes = random.random() < 0.5
+    slope_q = torch.rand(H, generator=g) * 0.02 if slopes else None
+    slope_kv = -torch.rand(H, generator=g) * 0.02 if slopes else None
+    softcap = random.choice([0.0, 0.0, 5.0, 30.0]) if family == "softmax" else 0.0
+    scale, bias = 1 / math.sqrt(D), (-1.0 if family == "sigmoid" else 0.0)
+    print(f"seed {seed}: terms add={shape} {None if add is None else add.dtype} slopes={slopes} cap={softcap} {family} D{D}/{DV} B{B} H{H}/{Hkv} "
+          f"Sq{Sq} Skv{Skv} causal={causal} bwd={backward} {dtype}", flush=True)
+    total = torch.zeros(B, H, Sq, Skv)
+    if add is not None:
+        total = total + add.float()
+    if slopes:
+        total = total + slope_q.view(1, H, 1, 1) * torch.arange(Sq).view(1, 1, Sq, 1) + slope_kv.view(1, H, 1, 1) * torch.arange(Skv).view(1, 1, 1, Skv)
+    lse = torch.full((B, H, Sq), float("nan"), device="cuda") if family == "softmax" else None
+    kw = dict(family=_fam_code(hb, family), causal=causal, scale=scale, bias=bias, score_add=add.cuda() if add is not None else None,
+              pos_slope_q=slope_q.cuda() if slopes else None, pos_slope_kv=slope_kv.cuda() if slopes else None, softcap=softcap)
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    o = hb.attn_fwd(qc, kc, vc, row_scale=lse, **kw)
+    torch.cuda.synchronize()
+    okw = dict(add=total, causal=causal, family=family, softmax_scale=scale, bias=bias, softcap=softcap if softcap > 0 else None)
+    if family == "softmax":
+        ref, lse_ref = oracle.biased_attention(q, k, v, return_lse=True, **okw)
+        torch.testing.assert_close(lse.cpu(), lse_ref, rtol=1e-3, atol=1e-3)
+    else:
+        ref = oracle.biased_attention(q, k, v, **okw)
+    _check_out(o, ref, family)
+    if backward:
+        dout = (0.5 * torch.randn(B, Sq, H, DV, generator=g)).to(dtype)
+        got = hb.attn_bwd(qc, kc, vc, o, dout.cuda(), lse, **kw)
+        torch.cuda.synchronize()
+        _check_grads(got, oracle.attention_grads(oracle.biased_attention, q, k, v, dout, **okw), family, Skv, softcap)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_linear_backward_random(seed):
+    """ma_linear_bwd at every key width, value widths that run as one, two or three pieces, shared q / k heads, sequence
+    lengths that are no multiple of the chunk, with and without a value scale; tolerances of tests/test_linear_bwd_gpu.py."""
+    import test_linear_bwd_gpu as lin
+    hb = _hb()
+    random.seed(6000 + seed)
+    g = torch.Generator().manual_seed(6000 + seed)
+    Dk, Dv = random.choice([64, 128, 192, 256]), random.choice([64, 128, 192, 256, 384, 512])
+    B, Hq, rep = random.randint(1, 2), random.randint(1, 2), random.choice([1, 1, 2, 4])
+    H, T, use_vs = Hq * rep, random.randint(1, 420), random.random() < 0.5
+    q = torch.randn(B, Hq, T, Dk, generator=g).bfloat16()
+    k = (0.1 * torch.randn(B, Hq, T, Dk, generator=g)).bfloat16()
+    v = torch.randn(B, H, T, Dv, generator=g).bfloat16()
+    ld = torch.nn.functional.logsigmoid(torch.randn(B, H, T, generator=g) + 3.0)
+    vs = torch.rand(B, H, T, generator=g) + 0.5 if use_vs else None
+    dout = (0.5 * torch.randn(B, H, T, Dv, generator=g)).bfloat16()
+    print(f"seed {seed}: linear bwd Dk{Dk} Dv{Dv} B{B} H{H}/{Hq} T{T} v_scale={use_vs}", flush=True)
+    got = hb.linear_bwd(q.cuda(), k.cuda(), v.cuda(), ld.cuda(), dout.cuda(), q_scale=Dk ** -0.5, v_scale=vs.cuda() if use_vs else None)
+    torch.cuda.synchronize()
+    lin._check(got, oracle.linear_attention_grads(q, k, v, ld, dout, q_scale=Dk ** -0.5, v_scale=vs), "linear")
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_mla_cache_lengths_random(seed):
+    """MLA decode with any head count, any cache length and per-entry cache lengths (empty entries included): every
+    entry against the oracle on its own prefix of the cache."""
+    hb = _hb()
+    random.seed(7000 + seed)
+    B, Hq, Skv = random.randint(1, 5), random.randint(1, 140), random.randint(1, 1500)
+    ns = min(random.choice([0, 1, 2, 3, 5, 8]), (Skv + 63) // 64)
+    dtype = random.choice([torch.bfloat16, torch.float16])
+    q, q_pe, kv, k_pe = inputs.mla_inputs(B, Hq, Skv, 512, 64, dtype=dtype, seed=7000 + seed)
+    lens = torch.tensor([random.randint(0, Skv) for _ in range(B)], dtype=torch.int32) if seed % 2 else None
+    print(f"seed {seed}: mla B{B} Hq{Hq} Skv{Skv} ns{ns} lens={None if lens is None else lens.tolist()} {dtype}", flush=True)
+    lse = torch.full((B, Hq), float("nan"), device="cuda")
+    o = hb.mla_decode(q.cuda(), q_pe.cuda(), kv.cuda(), k_pe.cuda(), scale=1 / math.sqrt(576), num_split=ns, lse=lse,
+                      kv_seqlens=lens.cuda() if lens is not None else None)
+    torch.cuda.synchronize()
+    for b in range(B):
+        n = Skv if lens is None else int(lens[b])
+        if n == 0:
+            assert torch.count_nonzero(o[b]) == 0
+            continue
+        ref, lse_ref = oracle.mla_decode(q[b:b + 1], q_pe[b:b + 1], kv[b:b + 1, :n], k_pe[b:b + 1, :n], return_lse=True)
+        oracle.assert_close(o[b:b + 1].float().cpu(), ref, rtol=RTOL, atol=ATOL)
+        torch.testing.assert_close(lse[b:b + 1].cpu(), lse_ref, rtol=1e-4, atol=1e-4)
