@@ -357,3 +357,112 @@ def test_mla_cache_lengths_random(seed):
         ref, lse_ref = oracle.mla_decode(q[b:b + 1], q_pe[b:b + 1], kv[b:b + 1, :n], k_pe[b:b + 1, :n], return_lse=True)
         oracle.assert_close(o[b:b + 1].float().cpu(), ref, rtol=RTOL, atol=ATOL)
         torch.testing.assert_close(lse[b:b + 1].cpu(), lse_ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_decode_random(seed):
+    """One query token over a cache of any length: per-entry cache lengths, a [B, heads_kv, blocks] mask over blocks of 32 /
+    64 / 128 keys, with and without the kv splits, every head size, the query heads of a kv head handed over as rows of
+    that head (a strided view, as the engine does).  Oracle: testing/test.py:654-693 restated."""
+    hb = _hb()
+    random.seed(8000 + seed)
+    g = torch.Generator().manual_seed(8000 + seed)
+    D, DV = random.choice([(128, 128), (64, 64), (128, 256), (256, 256), (192, 128)])
+    dtype = random.choice([torch.bfloat16, torch.float16])
+    B, G, grp = random.randint(1, 6), random.randint(1, 4), random.choice([1, 2, 4, 8, 16])
+    H, S, block = G * grp, random.randint(1, 3000), random.choice([32, 64, 128])
+    q = torch.randn(B, 1, H, D, generator=g).to(dtype)
+    k = torch.randn(B, S, G, D, generator=g).to(dtype)
+    v = torch.randn(B, S, G, DV, generator=g).to(dtype)
+    use_lens, use_bm = random.random() < 0.7, random.random() < 0.6
+    lens = torch.tensor([random.randint(1, S) for _ in range(B)], dtype=torch.int32) if use_lens else None
+    bm = None
+    if use_bm:
+        bm = torch.zeros(B, G, (S + block - 1) // block, dtype=torch.bool)
+        for b in range(B):
+            valid = ((S if lens is None else int(lens[b])) + block - 1) // block
+            keep = max(1, math.ceil(valid * random.choice([0.1, 0.5, 1.0])))
+            for gi in range(G):
+                bm[b, gi, torch.randperm(valid, generator=g)[:keep]] = True
+    split = random.random() < 0.7
+    print(f"seed {seed}: decode D{D}/{DV} B{B} H{H}/{G} S{S} block{block} lens={use_lens} mask={use_bm} split={split} {dtype}", flush=True)
+    qc = q.cuda().view(B, G, grp, D).transpose(1, 2)          # [B, rows = heads of a group, heads_kv, D]
+    o = hb.attn_fwd(qc, k.cuda(), v.cuda(), family=hb.MA_ATTN_SOFTMAX, causal=False, scale=1 / math.sqrt(D),
+                    kv_seqlens=lens.cuda() if use_lens else None, kv_block_mask=bm.to(torch.uint8).cuda() if use_bm else None,
+                    kv_block_size=block if use_bm else 0, split_kv=split)
+    torch.cuda.synchronize()
+    o = o.float().cpu().transpose(1, 2).reshape(B, H, DV)
+    oracle.assert_close(o, oracle.sparse_decode_attention(q, k, v, bm, lens, block_size=block), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_retention_random(seed):
+    """The retention family at its six head sizes, causal or with a full multiplier, a decay mask or any multiplier
+    tensor, query gains that put the row sums on both sides of the clamp; forward with r, and for every other seed
+    backward (gradients of keys reach 20 - 40 with the larger gains: 5e-3 of the elements may leave atol 2e-2 /
+    rtol 1e-2 in bf16; the same cases in fp16 are 8 x closer)."""
+    hb = _hb()
+    random.seed(9000 + seed)
+    g = torch.Generator().manual_seed(9000 + seed)
+    backward = seed % 2 == 1
+    D, DV = random.choice([(256, 512), (256, 512), (128, 128), (64, 64), (128, 256), (256, 256)])
+    dtype = random.choice([torch.bfloat16, torch.float16])
+    B, H, S = random.randint(1, 2), random.randint(1, 4), random.randint(1, 150) * 4      # (mask rows at 8-byte aligned addresses)
+    causal = random.random() < 0.7
+    q, k, v, _ = inputs.retnet_inputs(B, H, S, D, DV, seed=9000 + seed, layout="bshd")
+    q, k, v = (q.float() * random.choice([1.0, 4.0, 8.0])).to(dtype), k.to(dtype), v.to(dtype)
+    mask = oracle.retention_decay_mask(H, S)
+    if not causal:
+        mask = mask + mask.transpose(2, 3)
+    if random.random() < 0.3:
+        mask = mask * (torch.rand(1, H, S, S, generator=g) < 0.8)
+    mask = mask.to(dtype)
+    print(f"seed {seed}: retention D{D}/{DV} B{B} H{H} S{S} causal={causal} bwd={backward} {dtype}", flush=True)
+    rs = torch.full((B, H, S), float("nan"), device="cuda")
+    qc, kc, vc, mc = q.cuda(), k.cuda(), v.cuda(), mask.cuda()
+    o = hb.attn_fwd(qc, kc, vc, family=hb.MA_ATTN_RETENTION, causal=causal, scale=1.0, score_mask=mc, row_scale=rs)
+    torch.cuda.synchronize()
+    ref, r_ref = oracle.retention_parallel(q, k, v, mask, return_r=True)
+    oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(rs.cpu(), r_ref, rtol=1e-3, atol=1e-3)
+    if backward:
+        dout = (0.5 * torch.randn(B, S, H, DV, generator=g)).to(dtype)
+        got = hb.attn_bwd(qc, kc, vc, o, dout.cuda(), rs, family=hb.MA_ATTN_RETENTION, causal=causal, scale=1.0,
+                          score_mask=mc, score_mask_t=mc.transpose(2, 3).contiguous())
+        torch.cuda.synchronize()
+        ref_g = oracle.attention_grads(oracle.retention_parallel, q, k, v, dout, mask=mask, freeze_r=True)
+        for name, a, b_ in zip(("dq", "dk", "dv"), got, ref_g):
+            oracle.assert_close(a.float().cpu(), b_.float(), rtol=RTOL, atol=ATOL, mismatch_ratio=5e-3, msg=name)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_paged_mla_random(seed):
+    """flash_mla_with_kvcache over a shuffled page pool with ragged cache lengths (empty entries included), with the
+    work plan of get_mla_metadata at several part counts or without a plan; every entry against the paged oracle."""
+    hb = _hb()
+    random.seed(10000 + seed)
+    g = torch.Generator().manual_seed(10000 + seed)
+    B, Hq, page = random.randint(1, 12), random.choice([1, 16, 40, 64, 128, 128]), 64
+    maxlen = random.randint(1, 2500)
+    pps = (maxlen + page - 1) // page
+    npg = B * pps + random.randint(0, 5)
+    dtype = random.choice([torch.bfloat16, torch.float16])
+    q = torch.randn(B, 1, Hq, 576, generator=g).to(dtype)
+    cache = torch.randn(npg, page, 1, 576, generator=g).to(dtype)
+    table = torch.randperm(npg, generator=g)[:B * pps].to(torch.int32).view(B, pps)
+    lens = torch.tensor([random.randint(0, maxlen) if random.random() < 0.9 else maxlen for _ in range(B)], dtype=torch.int32)
+    planned, parts = random.random() < 0.6, random.choice([0, 0, 3, 17, 256])
+    print(f"seed {seed}: paged mla B{B} Hq{Hq} maxlen{maxlen} planned={planned} parts={parts} lens={lens.tolist()} {dtype}", flush=True)
+    if planned:
+        meta, splits = hb.get_mla_metadata(lens.cuda(), Hq, 1, num_sm_parts=parts)
+        out, lse = hb.flash_mla_with_kvcache(q.cuda(), cache.cuda(), table.cuda(), lens.cuda(), 512, meta, splits)
+    else:
+        out, lse = hb.flash_mla_with_kvcache(q.cuda(), cache.cuda(), table.cuda(), lens.cuda(), 512)
+    torch.cuda.synchronize()
+    for b in range(B):
+        if int(lens[b]) == 0:
+            assert torch.count_nonzero(out[b]) == 0 and torch.isinf(lse[b]).all()
+            continue
+        ref, lse_ref = oracle.paged_mla_decode(q[b:b + 1], cache, table[b:b + 1], lens[b:b + 1])
+        oracle.assert_close(out[b:b + 1].float().cpu(), ref, rtol=1e-2, atol=2e-2)
+        torch.testing.assert_close(lse[b:b + 1].cpu(), lse_ref, rtol=1e-4, atol=1e-4)
