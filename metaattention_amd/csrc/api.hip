@@ -40,12 +40,21 @@ size_t ma_attn_workspace_bytes(const ma_attn_params* p) {
   return rows * p->dim_v * 2 + rows * sizeof(float);
 }
 
+// The kernels count work items (batch x heads x blocks of rows, kv splits included) and rows in 32-bit integers.
+static bool attn_sizes_too_large(int B, int H, int Sq, int Skv) {
+  const int S = Sq > Skv ? Sq : Skv;
+  return S > (1 << 24) || (int64_t)B * H * ((S + 31) / 32) * 2 > 0x7fffffff;
+}
+
 int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
   if (!p) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: params is NULL");
   if (!p->q || !p->k || !p->v || !p->o) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: q/k/v/o must be non-NULL");
   if (p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->seqlen_kv <= 0 || p->dim_qk <= 0 || p->dim_v <= 0)
     return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: sizes must be positive (B=%d H=%d Sq=%d Skv=%d Dqk=%d Dv=%d)", p->batch,
                 p->heads, p->seqlen_q, p->seqlen_kv, p->dim_qk, p->dim_v);
+  if (attn_sizes_too_large(p->batch, p->heads, p->seqlen_q, p->seqlen_kv))
+    return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: sizes beyond the kernels' 32-bit work indices (B=%d H=%d Sq=%d Skv=%d)", p->batch, p->heads,
+                p->seqlen_q, p->seqlen_kv);
   if (p->dtype != MA_BF16 && p->dtype != MA_FP16) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: dtype %d", p->dtype);
   if (p->mask != MA_MASK_NONE && p->mask != MA_MASK_CAUSAL) return fail(MA_ERR_INVALID_ARG, "ma_attn_fwd: mask kind %d", p->mask);
   if (p->family < MA_ATTN_SOFTMAX || p->family > MA_ATTN_RETENTION)
@@ -139,7 +148,11 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
     return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: q/k/v/dout/dq/dk/dv must be non-NULL");
   if (p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->seqlen_kv <= 0 || p->dim_qk <= 0 || p->dim_v <= 0)
     return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: sizes must be positive");
+  if (attn_sizes_too_large(p->batch, p->heads, p->seqlen_q, p->seqlen_kv))
+    return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: sizes beyond the kernels' 32-bit work indices (B=%d H=%d Sq=%d Skv=%d)", p->batch, p->heads,
+                p->seqlen_q, p->seqlen_kv);
   if (p->dtype != MA_BF16 && p->dtype != MA_FP16) return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: dtype %d", p->dtype);
+  if (p->mask != MA_MASK_NONE && p->mask != MA_MASK_CAUSAL) return fail(MA_ERR_INVALID_ARG, "ma_attn_bwd: mask kind %d", p->mask);
   if (p->family != MA_ATTN_SOFTMAX && p->family != MA_ATTN_SIGMOID && p->family != MA_ATTN_RELU && p->family != MA_ATTN_RETENTION)
     return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: family %d has no backward kernel", p->family);
   if (p->family == MA_ATTN_RETENTION) {
@@ -232,7 +245,9 @@ static int check_linear(const ma_linear_params* p, const char* who) {
   if (p->heads % p->heads_q != 0 || p->heads % p->heads_k != 0)
     return fail(MA_ERR_INVALID_ARG, "%s: heads (%d) must be a multiple of heads_q (%d) and heads_k (%d)", who, p->heads, p->heads_q, p->heads_k);
   if (p->segments < 0) return fail(MA_ERR_INVALID_ARG, "%s: segments must be >= 0", who);
-  if ((int64_t)p->batch * p->heads * ((p->dim_v + 63) / 64) * (p->segments > 8 ? p->segments : 8) > 0x7fffffff)
+  if (p->seqlen > (1 << 30)) return fail(MA_ERR_UNSUPPORTED, "%s: seqlen beyond 2^30", who);
+  const int64_t bh = (int64_t)p->batch * p->heads;     // (compared step by step: the full product does not fit 64 bits for every input)
+  if (bh > 0x7fffffff || bh * ((p->dim_v + 63) / 64) > 0x7fffffff || bh * ((p->dim_v + 63) / 64) * (p->segments > 8 ? p->segments : 8) > 0x7fffffff)
     return fail(MA_ERR_UNSUPPORTED, "%s: grid too large", who);
   return MA_OK;
 }
@@ -288,7 +303,8 @@ static int check_linear_bwd(const ma_linear_bwd_params* p, const char* who) {
     return fail(MA_ERR_INVALID_ARG, "%s: heads (%d) must be a multiple of heads_q (%d) and heads_k (%d)", who, p->heads, p->heads_q, p->heads_k);
   if ((p->dim_k != 64 && p->dim_k != 128 && p->dim_k != 192 && p->dim_k != 256) || p->dim_v % 64 != 0 || p->dim_v > 4096)
     return fail(MA_ERR_UNSUPPORTED, "%s: dim_k=%d must be 64, 128, 192 or 256 and dim_v=%d a multiple of 64 (at most 4096)", who, p->dim_k, p->dim_v);
-  if ((int64_t)p->batch * p->heads * p->seqlen * (int64_t)(p->dim_k > p->dim_v ? p->dim_k : p->dim_v) / 8 > 0x7fffffffll * 256)
+  const int64_t bh = (int64_t)p->batch * p->heads;     // (compared step by step: the full product does not fit 64 bits for every input)
+  if (bh > 0x7fffffff || p->seqlen > (1 << 30) || bh * p->seqlen > (0x7fffffffll * 2048) / (p->dim_k > p->dim_v ? p->dim_k : p->dim_v))
     return fail(MA_ERR_UNSUPPORTED, "%s: grid too large", who);
   return MA_OK;
 }
@@ -332,12 +348,12 @@ int ma_linear_bwd(const ma_linear_bwd_params* p, ma_stream_t stream) {
 // whole number of 64-row tiles, and never more splits than tiles.
 int ma_mla_choose_split(const ma_mla_params* p) {
   if (!p || p->batch <= 0 || p->heads_q <= 0 || p->seqlen_kv <= 0) return 1;
-  const int head_blocks = (p->heads_q + 127) / 128;
-  const int tiles = (p->seqlen_kv + 63) / 64;
+  const int head_blocks = (int)(((int64_t)p->heads_q + 127) / 128);
+  const int tiles = (int)(((int64_t)p->seqlen_kv + 63) / 64);
   int cus = ma::device_cus();
   if (cus <= 0) cus = 256;
-  int split = cus / (p->batch * head_blocks);
-  if (split < 1) split = 1;
+  const int64_t groups = (int64_t)p->batch * head_blocks;
+  int split = groups >= cus ? 1 : (int)(cus / groups);
   if (split > tiles) split = tiles;
   if (split > 64) split = 64;
   return split;
@@ -351,8 +367,8 @@ int ma_mla_num_sm_parts(int heads_q) {
   if (heads_q <= 0) return 0;
   int cus = ma::device_cus();
   if (cus <= 0) cus = 256;
-  const int parts = cus / ((heads_q + 127) / 128);
-  return parts < 1 ? 1 : parts;
+  const int64_t parts = cus / (((int64_t)heads_q + 127) / 128);
+  return parts < 1 ? 1 : (int)parts;
 }
 
 int ma_mla_get_metadata(const int32_t* kv_seqlens, int batch, int num_sm_parts, int32_t* tile_scheduler_metadata, int32_t* num_splits,
@@ -382,6 +398,7 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
   if (p->dtype != MA_BF16 && p->dtype != MA_FP16) return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: dtype %d", p->dtype);
   if (!(p->scale > 0.f)) return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: scale must be > 0");
   if (p->batch > 65535) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: batch > 65535");
+  if (p->seqlen_kv > (1 << 30)) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: seqlen_kv beyond 2^30");
   const int64_t strides[] = {p->q_stride_b, p->q_stride_h, p->qpe_stride_b, p->qpe_stride_h, p->kv_stride_b, p->kv_stride_s,
                              p->kpe_stride_b, p->kpe_stride_s, p->o_stride_b, p->o_stride_h};
   for (int64_t s : strides)
@@ -399,6 +416,8 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
   const int ns = planned ? 1 : mla_split_of(p);
   const int tiles = (p->seqlen_kv + 63) / 64;
   if (ns > tiles || ns > 64) return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: num_split %d exceeds min(kv tiles=%d, 64)", ns, tiles);
+  if ((int64_t)p->batch * p->heads_q > 0x7fffffff || (int64_t)p->batch * ((p->heads_q + 127) / 128) * ns > 0x7fffffff || (planned && (int64_t)p->num_sm_parts * ((p->heads_q + 127) / 128) > 0x7fffffff))
+    return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: grid too large (batch %d x heads_q %d)", p->batch, p->heads_q);
   ma::MlaArgs a{};
   a.q = p->q; a.q_pe = p->q_pe; a.kv = p->kv; a.k_pe = p->k_pe; a.o = p->o; a.lse = p->lse;
   a.qsb = p->q_stride_b; a.qsh = p->q_stride_h; a.qpsb = p->qpe_stride_b; a.qpsh = p->qpe_stride_h;

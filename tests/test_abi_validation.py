@@ -108,6 +108,10 @@ CASES = [
     ("ma_attn_fwd", _attn, {"family": hb.MA_ATTN_RETENTION, "decay_gamma": PTR + 0x50000000}, UNSUPPORTED),   # .. and at 128 / 128
     ("ma_attn_fwd", _attn, {"family": hb.MA_ATTN_SIGMOID, "softcap": 30.0}, UNSUPPORTED), ("ma_attn_fwd", _attn, {"softcap": -1.0}, UNSUPPORTED),
     ("ma_attn_fwd", _attn, {"score_add": PTR + 0x50000002, "score_add_fp32": 1}, UNSUPPORTED),
+    # (sizes whose work-item counts leave 32 bits)
+    ("ma_attn_fwd", _attn, {"batch": (1 << 31) - 1, "heads": (1 << 31) - 1, "heads_kv": (1 << 31) - 1}, UNSUPPORTED),
+    ("ma_attn_fwd", _attn, {"seqlen_q": (1 << 31) - 1, "seqlen_kv": (1 << 31) - 1}, UNSUPPORTED),
+    ("ma_attn_fwd", _attn, {"batch": 1 << 20, "seqlen_q": 1 << 20, "seqlen_kv": 1 << 20}, UNSUPPORTED),
     # ---- ma_attn_bwd
     ("ma_attn_bwd", _attn_bwd, {}, LAUNCH),
     ("ma_attn_bwd", _attn_bwd, {"dout": None}, INVALID), ("ma_attn_bwd", _attn_bwd, {"dk": None}, INVALID), ("ma_attn_bwd", _attn_bwd, {"heads": 0}, INVALID),
@@ -123,6 +127,8 @@ CASES = [
     ("ma_attn_bwd", _attn_bwd, {"family": hb.MA_ATTN_RETENTION}, INVALID),
     ("ma_attn_bwd", _attn_bwd, {"family": hb.MA_ATTN_SIGMOID, "softcap": 5.0}, UNSUPPORTED),
     ("ma_attn_bwd", _attn_bwd, {"dim_qk": 96, "dim_v": 96}, UNSUPPORTED),
+    ("ma_attn_bwd", _attn_bwd, {"mask": 65536}, INVALID),
+    ("ma_attn_bwd", _attn_bwd, {"batch": 1 << 24, "heads": 1 << 10, "heads_kv": 1 << 10, "workspace_bytes": 1 << 62}, UNSUPPORTED),
     # ---- ma_linear_fwd / ma_linear_bwd
     ("ma_linear_fwd", _linear, {}, LAUNCH),
     ("ma_linear_fwd", _linear, {"seqlen": 0}, INVALID), ("ma_linear_fwd", _linear, {"log_decay": None}, INVALID), ("ma_linear_fwd", _linear, {"q": None}, INVALID),
@@ -130,7 +136,10 @@ CASES = [
     ("ma_linear_fwd", _linear, {"segments": -1}, INVALID), ("ma_linear_fwd", _linear, {"dim_k": 96}, UNSUPPORTED),
     ("ma_linear_fwd", _linear, {"dim_v": 96}, UNSUPPORTED), ("ma_linear_fwd", _linear, {"v": PTR + 0x20000002}, UNSUPPORTED),
     ("ma_linear_fwd", _linear, {"batch": 1 << 20, "heads": 1 << 10, "heads_q": 1 << 10, "heads_k": 1 << 10}, UNSUPPORTED),   # grid too large
+    ("ma_linear_fwd", _linear, {"batch": (1 << 31) - 1, "heads": (1 << 31) - 1, "heads_q": (1 << 31) - 1, "heads_k": (1 << 31) - 1, "dim_v": 1 << 30}, UNSUPPORTED),
+    ("ma_linear_fwd", _linear, {"seqlen": (1 << 31) - 1}, UNSUPPORTED),
     ("ma_linear_bwd", _linear_bwd, {}, LAUNCH),
+    ("ma_linear_bwd", _linear_bwd, {"batch": (1 << 31) - 1, "heads": (1 << 31) - 1, "heads_q": (1 << 31) - 1, "heads_k": (1 << 31) - 1, "seqlen": (1 << 31) - 1}, UNSUPPORTED),
     ("ma_linear_bwd", _linear_bwd, {"dlog_decay": None}, INVALID), ("ma_linear_bwd", _linear_bwd, {"heads_k": 3}, INVALID),
     ("ma_linear_bwd", _linear_bwd, {"dim_k": 320}, UNSUPPORTED), ("ma_linear_bwd", _linear_bwd, {"dim_v": 8192}, UNSUPPORTED),
     ("ma_linear_bwd", _linear_bwd, {"workspace": None}, WORKSPACE), ("ma_linear_bwd", _linear_bwd, {"workspace_bytes": 1024}, WORKSPACE),
@@ -144,6 +153,8 @@ CASES = [
     ("ma_mla_decode", _mla, {"num_split": 4}, WORKSPACE),                        # splits without a workspace
     ("ma_mla_decode", _mla, {"num_split": 4, "workspace": PTR + 0x50000000, "workspace_bytes": 4096}, WORKSPACE),
     ("ma_mla_decode", _mla, {"dim": 256, "dim_pe": 32}, UNSUPPORTED),
+    ("ma_mla_decode", _mla, {"batch": 65535, "heads_q": 1 << 24, "num_split": 0}, UNSUPPORTED),      # (batch x blocks of heads leaves 32 bits)
+    ("ma_mla_decode", _mla, {"seqlen_kv": (1 << 31) - 1}, UNSUPPORTED),
     ("ma_mla_decode", _mla, {"block_table": PTR + 0x50000000, "block_table_stride": 16, "page_size": 48}, UNSUPPORTED),
     ("ma_mla_decode", _mla, {"block_table": PTR + 0x50000000, "block_table_stride": 4, "page_size": 64}, INVALID),    # rows do not cover the cache
     ("ma_mla_decode", _mla, {"tile_scheduler_metadata": PTR + 0x50000000}, INVALID),     # a plan without its split table
@@ -166,3 +177,7 @@ def test_workspace_queries_take_bad_arguments():
     assert lib.ma_attn_bwd_workspace_bytes(None) == 0
     assert lib.ma_mla_workspace_bytes(None) == 0
     assert lib.ma_mla_workspace_bytes(ctypes.byref(_mla(num_split=4))) >= 2 * 4 * 128 * 512 * 2
+    # the split choice divides the CUs by batch x blocks of heads: a product beyond 32 bits must not wrap to zero
+    assert lib.ma_mla_choose_split(ctypes.byref(_mla(batch=1 << 20, heads_q=1 << 24, num_split=0))) == 1
+    assert lib.ma_mla_choose_split(ctypes.byref(_mla(batch=65535, heads_q=(1 << 31) - 1, num_split=0))) == 1
+    assert lib.ma_mla_num_sm_parts((1 << 31) - 1) >= 1 and lib.ma_mla_num_sm_parts(0) == 0
