@@ -18,7 +18,10 @@
  *   - return value 0 on success, a negative MA_ERR_* code otherwise, in which
  *     case ma_last_error() (thread local) describes the problem;
  *   - strides are in ELEMENTS of the tensor's dtype; the innermost (feature)
- *     dimension of every tensor must be contiguous.
+ *     dimension of every tensor must be contiguous;
+ *   - tensors may be larger than 4 GiB (bases are 64-bit).  The kernels count work items and rows in 32 bits:
+ *     sequence lengths up to 2^24 (2^30 for the chunked and the MLA operators), batch x heads x ceil(seqlen / 32)
+ *     below 2^30, and whatever else a call's description names; sizes beyond that come back as MA_ERR_UNSUPPORTED.
  */
 #ifndef METAATTENTION_HIP_H
 #define METAATTENTION_HIP_H
