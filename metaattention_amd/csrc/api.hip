@@ -27,23 +27,30 @@ extern "C" {
 int ma_version(void) { return MA_VERSION; }
 const char* ma_last_error(void) { return g_err; }
 
+// Strides beyond this many elements cannot belong to a tensor in device memory; bounding them keeps the kernels' 64-bit
+// address arithmetic (index x stride x element size) from wrapping.
+static constexpr int64_t kMaxStride = (int64_t)1 << 40;
+
+// The kernels count work items (batch x heads x blocks of rows, kv splits included) and rows in 32-bit integers.
+static bool attn_sizes_too_large(int B, int H, int Sq, int Skv) {
+  const int S = Sq > Skv ? Sq : Skv;
+  if (S > (1 << 24) || (int64_t)B * H > 0x7fffffff) return true;      // (step by step: the full product does not fit 64 bits for every input)
+  return (int64_t)B * H * ((S + 31) / 32) * 2 > 0x7fffffff;
+}
+
 static int attn_splits(const ma_attn_params* p) {
   return ma::attn_decode_splits(p->family, p->mask == MA_MASK_CAUSAL, p->batch, p->heads, p->seqlen_q, p->seqlen_kv, p->dim_qk, p->dim_v);
 }
 
 // partial outputs [B, splits, H, Sq, Dv] in the tensor dtype, then their fp32 row scales [B, splits, H, Sq]
 size_t ma_attn_workspace_bytes(const ma_attn_params* p) {
-  if (!p || p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->seqlen_kv <= 0 || p->dim_v <= 0) return 0;
+  if (!p || p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->seqlen_kv <= 0 || p->dim_v <= 0 || p->dim_v > 65536 ||
+      attn_sizes_too_large(p->batch, p->heads, p->seqlen_q, p->seqlen_kv))
+    return 0;
   const int n = attn_splits(p);
   if (n <= 1) return 0;
   const size_t rows = (size_t)p->batch * n * p->heads * p->seqlen_q;
   return rows * p->dim_v * 2 + rows * sizeof(float);
-}
-
-// The kernels count work items (batch x heads x blocks of rows, kv splits included) and rows in 32-bit integers.
-static bool attn_sizes_too_large(int B, int H, int Sq, int Skv) {
-  const int S = Sq > Skv ? Sq : Skv;
-  return S > (1 << 24) || (int64_t)B * H * ((S + 31) / 32) * 2 > 0x7fffffff;
 }
 
 int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
@@ -85,10 +92,16 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
   const int64_t strides[] = {p->q_stride_s, p->q_stride_h, p->k_stride_s, p->k_stride_h, p->v_stride_s, p->v_stride_h,
                              p->o_stride_s, p->o_stride_h, p->q_stride_b, p->k_stride_b, p->v_stride_b, p->o_stride_b};
   for (int64_t s : strides)
-    if (s % 8 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: strides must be multiples of 8 elements (16-byte rows)");
+    if (s % 8 != 0 || s > kMaxStride || s < -kMaxStride)
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: strides must be multiples of 8 elements (16-byte rows) below 2^40");
   const uintptr_t ptrs[] = {(uintptr_t)p->q, (uintptr_t)p->k, (uintptr_t)p->v, (uintptr_t)p->o};
   for (uintptr_t x : ptrs)
     if (x % 16 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: q/k/v/o must be 16-byte aligned");
+
+  const int64_t aux[] = {p->sm_stride_b, p->sm_stride_h, p->sm_stride_q, p->kbm_stride_b, p->kbm_stride_h, p->kbm_stride_q,
+                         p->em_stride_b, p->em_stride_h, p->em_stride_q, p->sa_stride_b, p->sa_stride_h, p->sa_stride_q, p->sa_stride_kv};
+  for (int64_t s : aux)
+    if (s > kMaxStride || s < -kMaxStride) return fail(MA_ERR_UNSUPPORTED, "ma_attn_fwd: mask / score_add strides must stay below 2^40");
 
   ma::AttnArgs a{};
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o;
@@ -138,7 +151,9 @@ int ma_attn_fwd(const ma_attn_params* p, ma_stream_t stream) {
 }
 
 size_t ma_attn_bwd_workspace_bytes(const ma_attn_bwd_params* p) {
-  if (!p || p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->family != MA_ATTN_SOFTMAX) return 0;
+  if (!p || p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->family != MA_ATTN_SOFTMAX ||
+      attn_sizes_too_large(p->batch, p->heads, p->seqlen_q, p->seqlen_q))
+    return 0;
   return (size_t)p->batch * p->heads * p->seqlen_q * sizeof(float);
 }
 
@@ -180,7 +195,14 @@ int ma_attn_bwd(const ma_attn_bwd_params* p, ma_stream_t stream) {
                              p->do_stride_b, p->do_stride_s, p->do_stride_h, p->dq_stride_b, p->dq_stride_s, p->dq_stride_h,
                              p->dk_stride_b, p->dk_stride_s, p->dk_stride_h, p->dv_stride_b, p->dv_stride_s, p->dv_stride_h};
   for (int64_t s : strides)
-    if (s % 8 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: strides must be multiples of 8 elements (16-byte rows)");
+    if (s % 8 != 0 || s > kMaxStride || s < -kMaxStride)
+      return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: strides must be multiples of 8 elements (16-byte rows) below 2^40");
+  const int64_t aux[] = {p->em_stride_b, p->em_stride_h, p->em_stride_q, p->emt_stride_b, p->emt_stride_h, p->emt_stride_k,
+                         p->kbm_stride_b, p->kbm_stride_h, p->kbm_stride_q, p->qbm_stride_b, p->qbm_stride_h, p->qbm_stride_k,
+                         p->sm_stride_b, p->sm_stride_h, p->sm_stride_q, p->smt_stride_b, p->smt_stride_h, p->smt_stride_k,
+                         p->sa_stride_b, p->sa_stride_h, p->sa_stride_q, p->sa_stride_kv};
+  for (int64_t s : aux)
+    if (s > kMaxStride || s < -kMaxStride) return fail(MA_ERR_UNSUPPORTED, "ma_attn_bwd: mask / score_add strides must stay below 2^40");
   const uintptr_t ptrs[] = {(uintptr_t)p->q, (uintptr_t)p->k, (uintptr_t)p->v, (uintptr_t)p->o, (uintptr_t)p->dout,
                             (uintptr_t)p->dq, (uintptr_t)p->dk, (uintptr_t)p->dv};
   for (uintptr_t x : ptrs)
@@ -246,6 +268,7 @@ static int check_linear(const ma_linear_params* p, const char* who) {
     return fail(MA_ERR_INVALID_ARG, "%s: heads (%d) must be a multiple of heads_q (%d) and heads_k (%d)", who, p->heads, p->heads_q, p->heads_k);
   if (p->segments < 0) return fail(MA_ERR_INVALID_ARG, "%s: segments must be >= 0", who);
   if (p->seqlen > (1 << 30)) return fail(MA_ERR_UNSUPPORTED, "%s: seqlen beyond 2^30", who);
+  if (p->dim_k > 65536 || p->dim_v > 65536) return fail(MA_ERR_UNSUPPORTED, "%s: no kernel for dim_k=%d / dim_v=%d", who, p->dim_k, p->dim_v);
   const int64_t bh = (int64_t)p->batch * p->heads;     // (compared step by step: the full product does not fit 64 bits for every input)
   if (bh > 0x7fffffff || bh * ((p->dim_v + 63) / 64) > 0x7fffffff || bh * ((p->dim_v + 63) / 64) * (p->segments > 8 ? p->segments : 8) > 0x7fffffff)
     return fail(MA_ERR_UNSUPPORTED, "%s: grid too large", who);
@@ -271,9 +294,7 @@ static int linear_kernel_dk(int dim_k) { return dim_k == 64 ? 128 : dim_k == 192
 // Without it (or with segments = 1) the forward pass runs as a single pass.  Returns 0 for
 // arguments ma_linear_fwd would refuse and when no device is present.
 size_t ma_linear_workspace_bytes(const ma_linear_params* p) {
-  if (!p || p->batch <= 0 || p->heads <= 0 || p->heads_q <= 0 || p->heads_k <= 0 || p->seqlen <= 0 || p->dim_k <= 0 || p->dim_v <= 0 ||
-      p->heads % p->heads_q != 0 || p->heads % p->heads_k != 0 || p->segments < 0)
-    return 0;
+  if (check_linear(p, "ma_linear_workspace_bytes") != MA_OK) return 0;
   size_t bytes = 0;
   if (ma::linear_fwd_dispatch(linear_args(p), linear_kernel_dk(p->dim_k), p->segments, nullptr, 0, nullptr, &bytes) != 0) return 0;
   return bytes;
@@ -320,9 +341,7 @@ static ma::LinBwdArgs linear_bwd_args(const ma_linear_bwd_params* p) {
 
 // Returns 0 for arguments ma_linear_bwd would refuse.
 size_t ma_linear_bwd_workspace_bytes(const ma_linear_bwd_params* p) {
-  if (!p || p->batch <= 0 || p->heads <= 0 || p->heads_q <= 0 || p->heads_k <= 0 || p->seqlen <= 0 || p->heads % p->heads_q != 0 ||
-      p->heads % p->heads_k != 0)
-    return 0;
+  if (check_linear_bwd(p, "ma_linear_bwd_workspace_bytes") != MA_OK) return 0;
   size_t bytes = 0;
   if (ma::linear_bwd_run(linear_bwd_args(p), nullptr, 0, nullptr, &bytes) != 0) return 0;
   return bytes;
@@ -382,7 +401,9 @@ int ma_mla_get_metadata(const int32_t* kv_seqlens, int batch, int num_sm_parts, 
 }
 
 size_t ma_mla_workspace_bytes(const ma_mla_params* p) {
-  if (!p) return 0;
+  if (!p || p->batch <= 0 || p->batch > 65535 || p->heads_q <= 0 || p->seqlen_kv <= 0 || p->dim <= 0 || p->dim > 65536 || p->num_sm_parts < 0 ||
+      (int64_t)p->batch * p->heads_q > 0x7fffffff)
+    return 0;
   const size_t per_slot = (size_t)p->heads_q * ((size_t)p->dim * 2 + sizeof(float));   // 2-byte partial outputs + fp32 lse
   if (p->tile_scheduler_metadata) return ((size_t)p->batch + (size_t)p->num_sm_parts) * per_slot;   // at most one piece more per part
   const int ns = mla_split_of(p);
@@ -402,7 +423,7 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
   const int64_t strides[] = {p->q_stride_b, p->q_stride_h, p->qpe_stride_b, p->qpe_stride_h, p->kv_stride_b, p->kv_stride_s,
                              p->kpe_stride_b, p->kpe_stride_s, p->o_stride_b, p->o_stride_h};
   for (int64_t s : strides)
-    if (s % 8 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: strides must be multiples of 8 elements");
+    if (s % 8 != 0 || s > kMaxStride || s < -kMaxStride) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: strides must be multiples of 8 elements below 2^40");
   const uintptr_t ptrs[] = {(uintptr_t)p->q, (uintptr_t)p->q_pe, (uintptr_t)p->kv, (uintptr_t)p->k_pe, (uintptr_t)p->o};
   for (uintptr_t x : ptrs)
     if (x % 16 != 0) return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: tensors must be 16-byte aligned");
@@ -430,6 +451,8 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream) {
   if (p->block_table) {
     if (p->page_size < 32 || p->page_size % 32 != 0)
       return fail(MA_ERR_UNSUPPORTED, "ma_mla_decode: page_size must be a positive multiple of 32 (got %d)", p->page_size);
+    if (p->block_table_stride < 0 || p->block_table_stride > 0x7fffffff)
+      return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: block_table_stride %lld", (long long)p->block_table_stride);
     if ((int64_t)p->block_table_stride * p->page_size < p->seqlen_kv)
       return fail(MA_ERR_INVALID_ARG, "ma_mla_decode: block table rows of %lld pages do not cover seqlen_kv=%d", (long long)p->block_table_stride, p->seqlen_kv);
     a.block_table = p->block_table; a.bt_stride = p->block_table_stride; a.page_size = p->page_size;

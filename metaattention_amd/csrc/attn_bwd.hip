@@ -15,7 +15,7 @@ int attn_bwd_256_512(const AttnBwdArgs& a, int family, bool causal, bool is_bf16
 int attn_bwd_dispatch(const AttnBwdArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream) {
   // (the tile DMA addresses a tile's 32 rows with 32-bit byte offsets from its first row)
   for (int64_t row_stride : {a.qss, a.kss, a.vss, a.doss})
-    if (row_stride < 0 || row_stride * 2 * 32 >= ((int64_t)1 << 32)) return -2;
+    if (row_stride < 0 || row_stride >= ((int64_t)1 << 26)) return -2;
   if (dqk == 128 && dv == 128) return attn_bwd_128_128(a, family, causal, is_bf16, stream);
   if (dqk == 64 && dv == 64) return attn_bwd_64_64(a, family, causal, is_bf16, stream);
   if (dqk == 128 && dv == 256) return attn_bwd_128_256(a, family, causal, is_bf16, stream);

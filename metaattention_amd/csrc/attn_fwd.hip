@@ -577,7 +577,9 @@ static int launch(const AttnArgs& a, hipStream_t stream) {
   static std::atomic<uint64_t> lds_ok{0};
   if (allow_lds(lds_ok, lds, kern) != 0) return -1;
   // the kernel addresses K and V rows with 32-bit byte offsets from the (batch, head) plane
-  if ((uint64_t)a.Skv * (uint64_t)a.kss * 2 >= (1ull << 32) || (uint64_t)a.Skv * (uint64_t)a.vss * 2 >= (1ull << 32)) return -2;
+  if (a.kss < 0 || a.vss < 0 || a.kss >= ((int64_t)1 << 31) || a.vss >= ((int64_t)1 << 31) ||
+      (uint64_t)a.Skv * (uint64_t)a.kss * 2 >= (1ull << 32) || (uint64_t)a.Skv * (uint64_t)a.vss * 2 >= (1ull << 32))
+    return -2;
   AttnArgs args = a;
   args.num_m_blocks = (a.Sq + BM - 1) / BM;
   const int num_cus = device_cus();

@@ -527,7 +527,7 @@ static int wide_dims(const AttnArgs& a, int family, bool causal, int dqk, int dv
 int attn_wide_fwd_dispatch(const AttnArgs& a, int family, bool causal, bool is_bf16, int dqk, int dv, hipStream_t stream) {
   // (the tile DMA addresses a tile's 32 rows with 32-bit byte offsets from its first row)
   for (int64_t row_stride : {a.kss, a.vss})
-    if (row_stride < 0 || row_stride * 2 * 32 >= ((int64_t)1 << 32)) return -2;
+    if (row_stride < 0 || row_stride >= ((int64_t)1 << 26)) return -2;
   return is_bf16 ? wide_dims<__bf16>(a, family, causal, dqk, dv, stream) : wide_dims<_Float16>(a, family, causal, dqk, dv, stream);
 }
 

@@ -112,6 +112,8 @@ CASES = [
     ("ma_attn_fwd", _attn, {"batch": (1 << 31) - 1, "heads": (1 << 31) - 1, "heads_kv": (1 << 31) - 1}, UNSUPPORTED),
     ("ma_attn_fwd", _attn, {"seqlen_q": (1 << 31) - 1, "seqlen_kv": (1 << 31) - 1}, UNSUPPORTED),
     ("ma_attn_fwd", _attn, {"batch": 1 << 20, "seqlen_q": 1 << 20, "seqlen_kv": 1 << 20}, UNSUPPORTED),
+    ("ma_attn_fwd", _attn, {"v_stride_s": 1 << 62}, UNSUPPORTED), ("ma_attn_fwd", _attn, {"score_add": PTR + 0x50000000, "v_stride_s": 1 << 62}, UNSUPPORTED),
+    ("ma_attn_fwd", _attn, {"elem_mask": PTR + 0x50000000, "mask": hb.MA_MASK_NONE, "em_stride_b": 1 << 62}, UNSUPPORTED),
     # ---- ma_attn_bwd
     ("ma_attn_bwd", _attn_bwd, {}, LAUNCH),
     ("ma_attn_bwd", _attn_bwd, {"dout": None}, INVALID), ("ma_attn_bwd", _attn_bwd, {"dk": None}, INVALID), ("ma_attn_bwd", _attn_bwd, {"heads": 0}, INVALID),
@@ -137,7 +139,7 @@ CASES = [
     ("ma_linear_fwd", _linear, {"dim_v": 96}, UNSUPPORTED), ("ma_linear_fwd", _linear, {"v": PTR + 0x20000002}, UNSUPPORTED),
     ("ma_linear_fwd", _linear, {"batch": 1 << 20, "heads": 1 << 10, "heads_q": 1 << 10, "heads_k": 1 << 10}, UNSUPPORTED),   # grid too large
     ("ma_linear_fwd", _linear, {"batch": (1 << 31) - 1, "heads": (1 << 31) - 1, "heads_q": (1 << 31) - 1, "heads_k": (1 << 31) - 1, "dim_v": 1 << 30}, UNSUPPORTED),
-    ("ma_linear_fwd", _linear, {"seqlen": (1 << 31) - 1}, UNSUPPORTED),
+    ("ma_linear_fwd", _linear, {"seqlen": (1 << 31) - 1}, UNSUPPORTED), ("ma_linear_fwd", _linear, {"dim_v": (1 << 31) - 1}, UNSUPPORTED),
     ("ma_linear_bwd", _linear_bwd, {}, LAUNCH),
     ("ma_linear_bwd", _linear_bwd, {"batch": (1 << 31) - 1, "heads": (1 << 31) - 1, "heads_q": (1 << 31) - 1, "heads_k": (1 << 31) - 1, "seqlen": (1 << 31) - 1}, UNSUPPORTED),
     ("ma_linear_bwd", _linear_bwd, {"dlog_decay": None}, INVALID), ("ma_linear_bwd", _linear_bwd, {"heads_k": 3}, INVALID),
@@ -154,7 +156,8 @@ CASES = [
     ("ma_mla_decode", _mla, {"num_split": 4, "workspace": PTR + 0x50000000, "workspace_bytes": 4096}, WORKSPACE),
     ("ma_mla_decode", _mla, {"dim": 256, "dim_pe": 32}, UNSUPPORTED),
     ("ma_mla_decode", _mla, {"batch": 65535, "heads_q": 1 << 24, "num_split": 0}, UNSUPPORTED),      # (batch x blocks of heads leaves 32 bits)
-    ("ma_mla_decode", _mla, {"seqlen_kv": (1 << 31) - 1}, UNSUPPORTED),
+    ("ma_mla_decode", _mla, {"seqlen_kv": (1 << 31) - 1}, UNSUPPORTED), ("ma_mla_decode", _mla, {"kv_stride_s": 1 << 62}, UNSUPPORTED),
+    ("ma_mla_decode", _mla, {"block_table": PTR + 0x50000000, "block_table_stride": 1 << 62, "page_size": 64}, INVALID),
     ("ma_mla_decode", _mla, {"block_table": PTR + 0x50000000, "block_table_stride": 16, "page_size": 48}, UNSUPPORTED),
     ("ma_mla_decode", _mla, {"block_table": PTR + 0x50000000, "block_table_stride": 4, "page_size": 64}, INVALID),    # rows do not cover the cache
     ("ma_mla_decode", _mla, {"tile_scheduler_metadata": PTR + 0x50000000}, INVALID),     # a plan without its split table
@@ -181,3 +184,10 @@ def test_workspace_queries_take_bad_arguments():
     assert lib.ma_mla_choose_split(ctypes.byref(_mla(batch=1 << 20, heads_q=1 << 24, num_split=0))) == 1
     assert lib.ma_mla_choose_split(ctypes.byref(_mla(batch=65535, heads_q=(1 << 31) - 1, num_split=0))) == 1
     assert lib.ma_mla_num_sm_parts((1 << 31) - 1) >= 1 and lib.ma_mla_num_sm_parts(0) == 0
+    # sizes whose products leave 64 bits: the queries answer 0 (nothing to allocate for a call that will be refused)
+    big = (1 << 31) - 1
+    assert lib.ma_attn_workspace_bytes(ctypes.byref(_attn(batch=big, heads=big, heads_kv=big))) == 0
+    assert lib.ma_attn_bwd_workspace_bytes(ctypes.byref(_attn_bwd(batch=big, heads=big, heads_kv=big))) == 0
+    assert lib.ma_linear_bwd_workspace_bytes(ctypes.byref(_linear_bwd(batch=big, heads=1 << 24, heads_q=4, heads_k=4, seqlen=65536))) == 0
+    assert lib.ma_linear_workspace_bytes(ctypes.byref(_linear(dim_v=big))) == 0
+    assert lib.ma_mla_workspace_bytes(ctypes.byref(_mla(batch=big, heads_q=big, num_split=4))) == 0
