@@ -97,11 +97,14 @@ def _replay_against_eager(run, statics, fresh_inputs, replays=3):
             dst.copy_(src)
         graph.replay()
         torch.cuda.synchronize()
-        got = out.clone()
+        outs = out if isinstance(out, (tuple, list)) else (out,)
+        got = [t.clone() for t in outs if t is not None]
         want = run()
         torch.cuda.synchronize()
-        assert torch.equal(got, want), f"replay {i}"
-        assert torch.isfinite(got.float()).all()
+        want = [t for t in (want if isinstance(want, (tuple, list)) else (want,)) if t is not None]
+        for j, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), f"replay {i}, output {j}"
+            assert torch.isfinite(a.float()).all()
 
 
 def test_operators_replay_in_a_hip_graph():
@@ -136,3 +139,43 @@ def test_operators_replay_in_a_hip_graph():
     _replay_against_eager(lambda: hb.mla_decode(qm, qpe, kv, kpe, scale=scale, num_split=4), (qm, qpe, kv, kpe), fresh_m)
     out = torch.empty(Bm, 1, Hq, 512, dtype=torch.bfloat16, device=dev)
     _replay_against_eager(lambda: hb.mla_decode(qm, qpe, kv, kpe, scale=scale, num_split=4, out=out, no_alloc=True), (qm, qpe, kv, kpe), fresh_m)
+
+
+def test_backward_and_decode_operators_replay_in_a_hip_graph():
+    """The same for a training step's pieces and the split-KV decode: parallel forward + backward (delta pre-pass, dq and
+    dk / dv kernels, workspace from the graph's pool), the chunked backward (three scans and their epilogue kernels) and the
+    grouped-query decode with kv splits and per-entry cache lengths."""
+    from metaattention_amd import hip_backend as hb
+    hb.load_library()
+    dev = "cuda"
+    B, H, Hkv, S, D, DV = 2, 4, 2, 300, 192, 128
+    gen = lambda seed: [torch.randn(B, S, H, D, generator=torch.Generator().manual_seed(seed)).half().to(dev),
+                        (0.5 * torch.randn(B, S, Hkv, D, generator=torch.Generator().manual_seed(seed + 1))).half().to(dev),
+                        (0.5 * torch.randn(B, S, Hkv, DV, generator=torch.Generator().manual_seed(seed + 2))).half().to(dev),
+                        torch.randn(B, S, H, DV, generator=torch.Generator().manual_seed(seed + 3)).half().to(dev)]
+    q, k, v, do = gen(100)
+
+    def step():
+        lse = torch.empty(B, H, S, device=dev)
+        o = hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=D ** -0.5, row_scale=lse)
+        return (o, lse) + tuple(hb.attn_bwd(q, k, v, o, do, lse, family=hb.MA_ATTN_SOFTMAX, causal=True, scale=D ** -0.5))
+    _replay_against_eager(step, (q, k, v, do), lambda i: gen(110 + 4 * i))
+
+    Bl, Hq, Hl, T, Dk, Dv = 2, 1, 8, 260, 128, 64
+    genl = lambda seed: [(0.1 * torch.randn(Bl, Hq, T, Dk, generator=torch.Generator().manual_seed(seed))).bfloat16().to(dev),
+                         (0.1 * torch.randn(Bl, Hq, T, Dk, generator=torch.Generator().manual_seed(seed + 1))).bfloat16().to(dev),
+                         torch.randn(Bl, Hl, T, Dv, generator=torch.Generator().manual_seed(seed + 2)).bfloat16().to(dev),
+                         torch.randn(Bl, Hl, T, Dv, generator=torch.Generator().manual_seed(seed + 3)).bfloat16().to(dev)]
+    ql, kl, vl, dol = genl(200)
+    ld = torch.nn.functional.logsigmoid(torch.randn(Bl, Hl, T, generator=torch.Generator().manual_seed(7)) + 3.0).to(dev)
+    vs = (torch.rand(Bl, Hl, T, generator=torch.Generator().manual_seed(8)) + 0.5).to(dev)
+    _replay_against_eager(lambda: hb.linear_bwd(ql, kl, vl, ld, dol, q_scale=1.0, v_scale=vs), (ql, kl, vl, dol), lambda i: genl(210 + 4 * i))
+
+    Bd, G, grp, Sk = 3, 2, 4, 2500
+    gend = lambda seed: [torch.randn(Bd, grp, G, 128, generator=torch.Generator().manual_seed(seed)).bfloat16().to(dev),
+                         torch.randn(Bd, Sk, G, 128, generator=torch.Generator().manual_seed(seed + 1)).bfloat16().to(dev),
+                         torch.randn(Bd, Sk, G, 128, generator=torch.Generator().manual_seed(seed + 2)).bfloat16().to(dev)]
+    qd, kd, vd = gend(300)
+    lens = torch.tensor([2500, 40, 1999], dtype=torch.int32, device=dev)
+    _replay_against_eager(lambda: hb.attn_fwd(qd, kd, vd, family=hb.MA_ATTN_SOFTMAX, causal=False, scale=128 ** -0.5, kv_seqlens=lens),
+                          (qd, kd, vd), lambda i: gend(310 + 3 * i))
