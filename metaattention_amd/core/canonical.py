@@ -260,12 +260,14 @@ def canonicalize_score_mod(score_mod, custom_fwd_inputs) -> ScoreForm:
             if toks not in ([], ["heads"]):
                 raise NotImplementedError(f"score_mod: {mono}: an index may be multiplied by a constant, a one-element or a per-head tensor")
     bias_tensor = None
-    if inner.tensors:
-        if len(inner.tensors) > 1:
-            raise NotImplementedError("score_mod: more than one bias tensor")
-        (bias_tensor, coef), = inner.tensors.items()
-        if not _close(coef, 1.0):
-            raise NotImplementedError("score_mod: bias tensor with a coefficient other than 1")
+    if len(inner.tensors) == 1 and _close(next(iter(inner.tensors.values())), 1.0):
+        (bias_tensor, _), = inner.tensors.items()          # the kernels' own bias pointer (examples/sigmoid_attn.py:17-21)
+    elif inner.tensors:
+        # one-element tensors with another coefficient, or several of them: additive terms like any other custom tensor
+        extra = dict(inner.extra)
+        for name, coef in inner.tensors.items():
+            extra[("t:" + name,)] = extra.get(("t:" + name,), 0.0) + coef
+        inner = Affine(inner.a, inner.mask, {}, inner.c, None, extra)
     if act != "identity" and inner.mask is not None:
         raise NotImplementedError("score_mod: activation of a tile-multiplied score")
     if inner.mask is not None and (inner.extra or softcap is not None):

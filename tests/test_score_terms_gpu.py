@@ -60,6 +60,33 @@ def test_kv_vector_and_per_row_tensor_sigmoid():
     oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=2e-3)
 
 
+def test_scaled_and_several_one_element_tensors():
+    """One-element tensors inside the scaling, `(s + t1) * scale - t2`: the kernels' bias pointer carries a lone tensor with
+    coefficient 1 (examples/sigmoid_attn.py:17-21); anything else goes the way of the other additive terms.  Forward and
+    backward through the operator."""
+    B, H, S, D = 2, 2, 160, 128
+    scale = D ** -0.5
+    io = {"t1": (1,), "t2": (1,)}
+    # (under softmax a constant shift cancels: the sigmoid score function keeps it visible)
+    def score_mod(s, c, b, h, q, k):
+        x = (s + c.input_tensors["t1"]) * scale - c.input_tensors["t2"]
+        return 1 / (1 + (-x).exp())
+    mod = _engine(B, H, S, D, io, score_mod, True, online=specs.OnlineIdentity())
+    assert mod.score_form.bias_tensor is None and mod.score_form.extra == {("t:t1",): scale, ("t:t2",): -1.0}
+    q, k, v = inputs.softmax_inputs(B, H, S, D, D, seed=12)
+    t1, t2 = torch.tensor([7.0]), torch.tensor([2.5])
+    qc, kc, vc = (t.cuda().requires_grad_() for t in (q, k, v))
+    o = mod(qc, kc, vc, t1.cuda(), t2.cuda())
+    dout = (0.5 * torch.randn(B, S, H, D, generator=torch.Generator().manual_seed(3))).bfloat16()
+    o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    kw = dict(causal=True, family="sigmoid", softmax_scale=scale, bias=7.0 * scale - 2.5)
+    oracle.assert_close(o.float().cpu(), oracle.biased_attention(q, k, v, **kw), rtol=RTOL, atol=ATOL, mismatch_ratio=2e-3)
+    ref = oracle.attention_grads(oracle.biased_attention, q, k, v, dout, **kw)
+    for name, a, b_ in zip(("dq", "dk", "dv"), (qc.grad, kc.grad, vc.grad), ref):
+        oracle.assert_close(a.float().cpu(), b_.float(), rtol=RTOL, atol=ATOL, mismatch_ratio=5e-3, msg=name)
+
+
 @pytest.mark.parametrize("per_head", [True, False])
 def test_alibi(per_head):
     """score * scale - slope[h] * (q_idx - kv_idx): slopes as a per-head custom tensor, or one constant."""
