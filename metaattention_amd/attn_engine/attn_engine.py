@@ -73,6 +73,12 @@ _FAMILY = {
 }
 
 
+def _kernel_view(t):
+    """t itself when the kernels can read it in place, else a contiguous copy (gradients flow through the copy)."""
+    ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
+    return t if ok else t.contiguous()
+
+
 class _ForwardOnly(torch.autograd.Function):
     """Gives outputs a grad_fn whose backward fails loudly, for the operators whose
     backward kernels are not in the library."""
@@ -226,6 +232,9 @@ class AttentionEngine:
 
         # (decided here: inside an autograd function's forward, gradient mode is off)
         needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
+        # the kernels read strided views in place (rows of 16-byte aligned, 16-byte multiples); any other view is copied once,
+        # as a caller of the reference's operator would have to (its kernels take contiguous tensors: attn_tl.py:69-70)
+        q, k, v = (_kernel_view(t) for t in (q, k, v))
 
         def run(q, k, v):
             B, Sq, H, D = q.shape
@@ -484,7 +493,7 @@ class AttentionEngine:
 
     def _call_mla(self, q, q_pe, kv, k_pe):
         from hip_backend import mla_decode
-        return mla_decode(q, q_pe, kv, k_pe, scale=self.mla_scale)
+        return mla_decode(*(_kernel_view(t) for t in (q, q_pe, kv, k_pe)), scale=self.mla_scale)
 
     def __call__(self, *args, **kargs):
         block_mask, cache_seqlens = kargs.get("block_mask"), kargs.get("cache_seqlens")
