@@ -520,7 +520,8 @@ def bench_reference_benchmark_shapes(steps, warmup):
     """Figures of the reference's own benchmarks that BASELINE's configurations do not cover (testing/benchmark_mi250.py:40-55,
     testing/benchmark_h100.py:112,129): causal softmax at the DeepSeek-V2-Lite head sizes (16 heads, Dqk 192, Dv 128, fp16),
     ReLU attention at the ViT-S head size (6 heads, 64 / 64, fp16) and gated retention at 64 / 64 and 256 / 256, forward and
-    backward through the C ABI.  The reference writes its own timings to CSV files at run time and holds none in the tree."""
+    backward through the C ABI; one query token at the DeepSeek-V2-Lite sizes, the block-sparse grouped-query decode and the
+    parallel retention at 32 heads and S = 4096 (benchmark_h100.py:63-65, 95-99, 151-156), forward.  The reference writes its own timings to CSV files at run time and holds none in the tree."""
     import torch
     from metaattention_amd import hip_backend as hb
     out = {}
@@ -542,8 +543,8 @@ def bench_reference_benchmark_shapes(steps, warmup):
                          bwd_tflops_2p5x=round(2.5 * flops / ms_b / 1e9, 1))
     # gated retention at the two head sizes of testing/benchmark_h100.py:112,129 (16 heads 64 / 64: the key width runs in the
     # 128-wide kernel; 40 heads 256 / 256), per-token log decay, forward and backward
-    for H, Dk, Dv in ((16, 64, 64), (40, 256, 256)):
-        B, T = 8, 4096
+    for B, H, Dk, Dv in ((8, 16, 64, 64), (8, 40, 256, 256), (64, 16, 64, 64)):      # (the last: the batch of benchmark_h100.py:110-113)
+        T = 4096
         q = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 4).bfloat16()
         k = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 4).bfloat16()
         v, do = (torch.randn(B, H, T, Dv, device="cuda", generator=g).bfloat16() for _ in range(2))
@@ -553,7 +554,48 @@ def bench_reference_benchmark_shapes(steps, warmup):
         ms_f = time_gpu(lambda: hb.linear_fwd(q, k, v, ld, q_scale=Dk ** -0.5, out=o, workspace=ws), steps, warmup)
         wsb = torch.empty(_linear_bwd_workspace(hb, B, H, H, H, T, Dk, Dv), dtype=torch.uint8, device="cuda")
         ms_b = time_gpu(lambda: hb.linear_bwd(q, k, v, ld, do, q_scale=Dk ** -0.5, workspace=wsb), max(steps // 3, 3), 2)
-        out[f"gated_retention_b8_h{H}_s4096_{Dk}_{Dv}_bf16"] = dict(fwd_ms=round(ms_f, 4), bwd_ms=round(ms_b, 4))
+        out[f"gated_retention_b{B}_h{H}_s4096_{Dk}_{Dv}_bf16"] = dict(fwd_ms=round(ms_f, 4), bwd_ms=round(ms_b, 4))
+        del q, k, v, do, o, ws, wsb
+    torch.cuda.empty_cache()
+    # one query token against a cache at the DeepSeek-V2-Lite head sizes (benchmark_h100.py:63-65), fp16
+    B, H, Skv, D, DV = 8, 16, 8192, 192, 128
+    q = torch.randn(B, 1, H, D, device="cuda", dtype=torch.float16, generator=g)
+    k = torch.randn(B, Skv, H, D, device="cuda", dtype=torch.float16, generator=g)
+    v = torch.randn(B, Skv, H, DV, device="cuda", dtype=torch.float16, generator=g)
+    o = torch.empty(B, 1, H, DV, device="cuda", dtype=torch.float16)
+    ms = time_gpu(lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_SOFTMAX, causal=False, scale=D ** -0.5, out=o), steps, warmup)
+    out["softmax_decode_deepseek_v2_lite_b8_h16_kv8192_192_128_fp16"] = dict(ms=round(ms, 4), gbytes_per_s=round((k.numel() + v.numel()) * 2 / ms / 1e6, 1))
+    # block-sparse grouped-query decode (benchmark_h100.py:151-156: 32 query heads on 8 kv heads, half of the 32-key blocks kept), fp16
+    B, H, G, Skv, D = 8, 32, 8, 8192, 128
+    q = torch.randn(B, 1, H, D, device="cuda", dtype=torch.float16, generator=g)
+    k, v = (torch.randn(B, Skv, G, D, device="cuda", dtype=torch.float16, generator=g) for _ in range(2))
+    bm = (torch.rand(B, G, Skv // 32, device="cuda", generator=g) < 0.5).to(torch.uint8)
+    lens = torch.full((B,), Skv, dtype=torch.int32, device="cuda")
+    o = torch.empty(B, H // G, G, D, device="cuda", dtype=torch.float16).transpose(1, 2)
+    qv = q.view(B, G, H // G, D).transpose(1, 2)          # the query heads of a kv head as the rows of that head, as the operator passes them
+    ms = time_gpu(lambda: hb.attn_fwd(qv, k, v, family=hb.MA_ATTN_SOFTMAX, causal=False, scale=D ** -0.5, kv_seqlens=lens, kv_block_mask=bm,
+                                      kv_block_size=32), steps, warmup)
+    out["sparse_gqa_decode_b8_h32_g8_kv8192_128_128_fp16"] = dict(ms=round(ms, 4), kept_blocks=round(float(bm.float().mean()), 3))
+    del q, k, v, o
+    torch.cuda.empty_cache()
+    # normalised parallel retention at RetNet-6.7B's 32 heads and S = 4096 (benchmark_h100.py:95-99), bf16: the decay mask as the
+    # [1, H, S, S] tensor the reference's operator takes (1 GiB), and generated by the kernel
+    B, H, S, D, DV = 8, 32, 4096, 256, 512
+    q = (torch.randn(B, S, H, D, device="cuda", generator=g) / 16).bfloat16()
+    k = (torch.randn(B, S, H, D, device="cuda", generator=g) / 16).bfloat16()
+    v = torch.randn(B, S, H, DV, device="cuda", generator=g).bfloat16()
+    o = torch.empty_like(v)
+    gam = 1 - torch.exp2(-5 - torch.arange(H, device="cuda").float())
+    idx = torch.arange(S, device="cuda", dtype=torch.float32)
+    diff = idx.view(S, 1) - idx.view(1, S)
+    mask = torch.empty(1, H, S, S, device="cuda", dtype=torch.bfloat16)
+    for h in range(H):                                     # (head by head: bounds the fp32 temporaries)
+        mask[0, h] = (torch.exp2(diff.clamp(min=0) * torch.log2(gam[h])) * (diff >= 0)).bfloat16()
+    flops = 0.5 * 2.0 * B * H * S * S * (D + DV)
+    ms_t = time_gpu(lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, score_mask=mask, out=o), max(steps // 2, 3), 2)
+    ms_g = time_gpu(lambda: hb.attn_fwd(q, k, v, family=hb.MA_ATTN_RETENTION, causal=True, scale=1.0, decay_gamma=gam, out=o), max(steps // 2, 3), 2)
+    out["retention_parallel_b8_h32_s4096_256_512_bf16"] = dict(ms_mask_tensor=round(ms_t, 4), ms_generated_mask=round(ms_g, 4),
+                                                               tflops_generated_mask=round(flops / ms_g / 1e9, 1))
     return out
 
 

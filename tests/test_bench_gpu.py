@@ -35,7 +35,8 @@ def test_bench_line():
         if key != "note":
             assert entry["ms"] > 0 and entry["reference_ms"]
     rb = others["reference_benchmark_shapes"]
-    assert "error" not in rb and len(rb) == 5 and all(e["fwd_ms"] > 0 and e["bwd_ms"] > 0 for e in rb.values())
+    assert "error" not in rb and len(rb) == 9, rb
+    assert all(min(v for k, v in e.items() if k.endswith("ms") or k.startswith("ms")) > 0 for e in rb.values())
     # the operator recognised the decay mask the workload builds
     assert "generates it" in others["c3_retnet_parallel_operator"]["flop_convention"]
     for name in ("c5_mla_decode", "gqa_decode"):
