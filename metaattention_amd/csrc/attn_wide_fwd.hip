@@ -39,7 +39,7 @@ enum { WF_SOFTMAX = 0, WF_SIGMOID = 1, WF_RELU = 2, WF_RETENTION = 3 };   // = M
 }
 
 template <typename T, int DQK, int DV, int FAMILY, bool CAUSAL, int NW>
-__global__ __launch_bounds__(64 * NW, (DQK + DV >= 512 ? 1 : 2)) void attn_wide_fwd_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(64 * NW, ((DQK + DV >= 512 || (NW == 1 && pad_width(DQK) + DV >= 384)) ? 1 : 2)) void attn_wide_fwd_kernel(const AttnArgs a) {
   using E = Elem<T>;
   using x8 = typename E::x8;
   using x4 = typename E::x4;
@@ -460,16 +460,31 @@ static int launch_wide(const AttnArgs& a, hipStream_t stream) {
   return launch_status();
 }
 
-// Decode shapes: at most 32 query rows per (batch, head), softmax, no structural mask.  Splits are chosen
-// so that about four workgroups per CU are in flight, each with at least 8 tiles of 32 keys.
+// Decode shapes: at most 32 query rows per (batch, head), softmax, no structural mask.  A one-wave workgroup takes one
+// (batch, head, kv split); a CU holds four of them, or as many as their two tile stages fit into its 160 KB of LDS.  The
+// split count is the one with the shortest schedule, counted in tiles: rounds of resident workgroups x (tiles per split +
+// a workgroup's fixed cost), plus the merge, which grows with the splits; every split gets at least 8 tiles of 32 keys.
 int attn_decode_splits(int family, bool causal, int B, int H, int Sq, int Skv, int dqk, int dv) {
   if (family != WF_SOFTMAX || causal || Sq > 32) return 1;
   if (!((dqk == 128 && dv == 128) || (dqk == 64 && dv == 64) || (dqk == 128 && dv == 256) || (dqk == 256 && dv == 256) || (dqk == 192 && dv == 128))) return 1;
   const int tiles = (Skv + 31) / 32;
-  int n = 1024 / (B * H);
-  if (n > tiles / 8) n = tiles / 8;
-  if (n > 64) n = 64;
-  return n < 1 ? 1 : n;
+  const int lds = 2 * 32 * (pad_width(dqk) + dv) * 2;
+  int per_cu = (160 * 1024) / lds;
+  if (per_cu > 4) per_cu = 4;
+  const int64_t slots = (int64_t)per_cu * 256, groups = (int64_t)B * H;
+  int n_max = tiles / 8;
+  if (n_max > 64) n_max = 64;
+  int best = 1;
+  int64_t best_cost = -1;
+  for (int n = 1; n <= n_max || n == 1; n++) {
+    const int64_t rounds = (groups * n + slots - 1) / slots;
+    const int64_t cost = 4 * rounds * ((tiles + n - 1) / n + 3) + n;      // (in quarter tiles)
+    if (best_cost < 0 || cost < best_cost) {
+      best_cost = cost;
+      best = n;
+    }
+  }
+  return best;
 }
 
 template <typename T, int DQK, int DV>
