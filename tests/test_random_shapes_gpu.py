@@ -466,3 +466,52 @@ def test_paged_mla_random(seed):
         ref, lse_ref = oracle.paged_mla_decode(q[b:b + 1], cache, table[b:b + 1], lens[b:b + 1])
         oracle.assert_close(out[b:b + 1].float().cpu(), ref, rtol=1e-2, atol=2e-2)
         torch.testing.assert_close(lse[b:b + 1].cpu(), lse_ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_engine_mask_mods_random(seed):
+    """Through the operators: a random mask_mod out of ten kinds (windows, shifted diagonals, prefix-LM, documents, strided,
+    per-head and per-batch windows, the causal mask, none, the upper triangle), a random family, head size, dtype and length;
+    forward, and for about half of the seeds backward through autograd, against oracle.masked_attention with the mask_mod
+    evaluated densely."""
+    import specs
+    from attn_engine import AttentionEngine
+    from core import CustomIO, meta_tensor
+    rng = random.Random(20000 + seed)
+    g = torch.Generator().manual_seed(20000 + seed)
+    w, s_, p_, d = rng.randint(1, 200), rng.randint(1, 150), rng.randint(0, 200), rng.randint(8, 200)
+    masks = {"window": lambda b, h, q, k: (q >= k) & (q - k < w), "shifted": lambda b, h, q, k: q - s_ >= k,
+             "prefix": lambda b, h, q, k: (q >= k) | (k < p_), "per_head": lambda b, h, q, k: (q >= k) & (q - k < 16 * (h + 1)),
+             "document": lambda b, h, q, k: (q >= k) & ((q // d) == (k // d)), "per_batch": lambda b, h, q, k: (q >= k) & (q - k < 20 * (b + 1)),
+             "strided": lambda b, h, q, k: (q >= k) & ((q - k) % 3 == 0), "causal": lambda b, h, q, k: q >= k, "none": None,
+             "upper": lambda b, h, q, k: q <= k}
+    kind = rng.choice(sorted(masks))
+    mask_mod = masks[kind]
+    family = rng.choice(FAMILIES)
+    D, DV = rng.choice([(128, 128), (64, 64), (128, 256), (192, 128), (256, 256)])
+    dtype = rng.choice([torch.bfloat16, torch.float16])
+    B, H, S = rng.randint(1, 2), rng.randint(1, 3), rng.randint(2, 420)
+    backward = rng.random() < 0.5 and (D, DV) != (256, 256)
+    scale, bias = D ** -0.5, -1.0
+    score_mod = {"softmax": lambda x, io, b, h, q, k: x * scale, "relu": lambda x, io, b, h, q, k: (x * scale).max(0),
+                 "sigmoid": lambda x, io, b, h, q, k: 1 / (1 + (-(x * scale + bias)).exp())}[family]
+    meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, H, S, DV, dtype=dtype))
+    print(f"seed {seed}: engine {kind} {family} D{D}/{DV} B{B} H{H} S{S} bwd={backward} {dtype}", flush=True)
+    mod = AttentionEngine(meta, CustomIO(), score_mod, mask_mod, specs.OnlineSoftmax() if family == "softmax" else specs.OnlineIdentity())
+    q = torch.randn(B, S, H, D, generator=g).to(dtype)
+    k = (0.5 * torch.randn(B, S, H, D, generator=g)).to(dtype)
+    v = (0.5 * torch.randn(B, S, H, DV, generator=g)).to(dtype)
+    dout = (0.5 * torch.randn(B, S, H, DV, generator=g)).to(dtype)
+    qc, kc, vc = (t.cuda().requires_grad_(backward) for t in (q, k, v))
+    o = mod(qc, kc, vc)
+    if backward:
+        o.backward(dout.cuda())
+    torch.cuda.synchronize()
+    keep = None
+    if mask_mod is not None:
+        keep = mask_mod(torch.arange(B).view(B, 1, 1, 1), torch.arange(H).view(1, H, 1, 1), torch.arange(S).view(1, 1, S, 1),
+                        torch.arange(S).view(1, 1, 1, S)).expand(B, H, S, S)
+    okw = dict(keep=keep, family=family, softmax_scale=scale, bias=bias if family == "sigmoid" else 0.0)
+    _check_out(o, oracle.masked_attention(q, k, v, **okw), family)
+    if backward:
+        _check_grads((qc.grad, kc.grad, vc.grad), oracle.attention_grads(oracle.masked_attention, q, k, v, dout, **okw), family, S)
