@@ -34,6 +34,9 @@ struct LinArgs {
   int64_t piece_qk, piece_o;
   float* ws_state;
   float* ws_decay;
+  // head-group range of this launch (a workgroup handles head group bg0 + its own index; bg_n groups in all; bg_n = 0: every
+  // group, from 0).  The workspace of a launch with sequence segments is indexed by the launch's own group index.
+  int bg0, bg_n;
 };
 
 int linear_fwd_dispatch(const LinArgs& a, int dk, int want_segments, void* ws, size_t ws_size, hipStream_t stream, size_t* query);

@@ -101,7 +101,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
   // workgroup -> (head group, value slice, segment); the workgroups of one head group share
   // id % 8 (one XCD, shared L2)
   const int n_seg = MODE == 0 ? 1 : (MODE == 1 ? a.nseg - 1 : a.nseg);
-  const int BG = a.B * a.H / HG;
+  const int BG = a.bg_n > 0 ? a.bg_n : a.B * a.H / HG;     // head groups of this launch
   int bg, dvb, seg;
   {
     int slot;
@@ -120,6 +120,8 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
       bg = slot / a.dv_blocks;
     }
   }
+  const int bg_local = bg;      // (indexes the launch's workspace)
+  bg += a.bg0;
   const int hl = wave / NWH;                      // head of the group this wave works for
   const int bh0 = bg * HG, bh = bh0 + hl;
   const int b = bh0 / a.H, h0 = bh0 % a.H;        // (HG divides H, and the heads of a group share hq and hk)
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
   // this wave's block of the exchanged states: [segment][wave][KB*16 registers][64 lanes]
   float* ws_mine = nullptr;
   if (MODE != 0)
-    ws_mine = a.ws_state + ((((int64_t)bg * a.dv_blocks + dvb) * (a.nseg - 1)) * NW + wave) * (int64_t)(KB * 16 * 64) + lane;
+    ws_mine = a.ws_state + ((((int64_t)bg_local * a.dv_blocks + dvb) * (a.nseg - 1)) * NW + wave) * (int64_t)(KB * 16 * 64) + lane;
   constexpr int64_t WS_SEG = (int64_t)NW * KB * 16 * 64;
 
   // ---- DMA of one chunk: each instruction moves 1 KB (1024/row_bytes tile rows); lane i fetches
@@ -249,7 +251,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
 
   if (MODE == 2 && seg > 0) {
     // entering state: the local end states of the earlier segments, each decayed by the segments between
-    const float* dec = a.ws_decay + (int64_t)bh * (a.nseg - 1);
+    const float* dec = a.ws_decay + (int64_t)(bh - a.bg0 * HG) * (a.nseg - 1);
     float acc_log = 0.f;
     for (int sp = seg - 1; sp >= 0; sp--) {
       const float coef = fast_exp2(acc_log * kLog2e);
@@ -582,7 +584,7 @@ __global__ __launch_bounds__(64 * NWH * HG, (min_waves_per_simd<DK, NWH, HG>()))
     for (int i = 0; i < KB; i++)
 #pragma unroll
       for (int j = 0; j < 16; j++) dst[(i * 16 + j) * 64] = hst[i][j];
-    if (dvb == 0 && wave % NWH == 0 && lane == 0) a.ws_decay[(int64_t)bh * (a.nseg - 1) + seg] = seg_log;
+    if (dvb == 0 && wave % NWH == 0 && lane == 0) a.ws_decay[(int64_t)(bh - a.bg0 * HG) * (a.nseg - 1) + seg] = seg_log;
   }
 }
 
@@ -640,6 +642,33 @@ struct Config {
     return (size_t)((groups * (nseg - 1) * NW * ws_wave_floats + (int64_t)a.B * a.H * (nseg - 1)) * 4);
   }
 
+  // A single pass over more head groups than the device holds at once ends in a round that is mostly empty (320 workgroups
+  // on 256 CUs take as long as 512).  When the last round would be at most half full, the head groups of the full rounds run
+  // the single pass and the rest is cut into sequence segments, as many as fill the device once: tail_bg head groups from
+  // full_bg on, in nseg segments (tail_bg = 0: no such split).
+  struct Tail { int full_bg, tail_bg, nseg, seg_chunks; };
+  static Tail tail_plan(const LinArgs& a, int want, int resident, int cus) {
+    Tail t{0, 0, 1, 0};
+    const int dvb = a.Dv / (32 * NWH), n_chunks = (a.T + L - 1) / L;
+    const int64_t BG = (int64_t)a.B * a.H / HG, per_round = (int64_t)resident * cus / dvb;     // head groups
+    if (want != 0 || a.n_pieces > 1 || per_round < 1 || BG <= per_round) return t;
+    const int64_t tail = BG % per_round;
+    int n = tail > 0 ? (int)(per_round / tail) : 1;
+    if (n > 8) n = 8;
+    if (n > n_chunks / 4) n = n_chunks / 4;
+    if (tail == 0 || tail * 2 > per_round || n < 2) return t;
+    t.full_bg = (int)(BG - tail);
+    t.tail_bg = (int)tail;
+    t.seg_chunks = (n_chunks + n - 1) / n;
+    t.nseg = (n_chunks + t.seg_chunks - 1) / t.seg_chunks;
+    if (t.nseg < 2) t.tail_bg = 0;
+    return t;
+  }
+  static size_t tail_ws_bytes(const Tail& t, int dvb) {
+    if (t.tail_bg <= 0) return 0;
+    return (size_t)(((int64_t)t.tail_bg * dvb * (t.nseg - 1) * NW * ws_wave_floats + (int64_t)t.tail_bg * HG * (t.nseg - 1)) * 4);
+  }
+
   // query != null: only report the workspace the launch would use
   static int run(const LinArgs& a, int want_segments, void* ws, size_t ws_size, hipStream_t stream, size_t* query) {
     int resident = 1, cus = 256;
@@ -666,10 +695,34 @@ struct Config {
     }
     const unsigned pieces = a.n_pieces > 1 ? (unsigned)a.n_pieces : 1u;
     plan(a, want_segments, resident, cus, args.nseg, args.seg_chunks);
-    if (query) { *query = ws_bytes(a, args.nseg); return 0; }
+    const Tail tail = args.nseg <= 1 ? tail_plan(a, want_segments, resident, cus) : Tail{0, 0, 1, 0};
+    if (query) { *query = tail.tail_bg > 0 ? tail_ws_bytes(tail, args.dv_blocks) : ws_bytes(a, args.nseg); return 0; }
     if (args.nseg > 1 && (!ws || ws_size < ws_bytes(a, args.nseg) || ((uintptr_t)ws & 3) != 0)) args.nseg = 1;   // no workspace: single pass
     const unsigned groups = (unsigned)((int64_t)a.B * a.H / HG * args.dv_blocks);
-    if (args.nseg <= 1) {
+    if (args.nseg <= 1 && tail.tail_bg > 0 && ws && ws_size >= tail_ws_bytes(tail, args.dv_blocks) && ((uintptr_t)ws & 3) == 0) {
+      // the full rounds in a single pass, then the tail in segments (see tail_plan)
+      LinArgs full = args;
+      full.nseg = 1;
+      full.bg0 = 0;
+      full.bg_n = tail.full_bg;
+      const unsigned g_full = (unsigned)tail.full_bg * args.dv_blocks, g_tail = (unsigned)tail.tail_bg * args.dv_blocks;
+      if (gen) hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 0, true>), dim3(g_full, pieces), dim3(64 * NW), lds, stream, full);
+      else hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 0>), dim3(g_full), dim3(64 * NW), lds, stream, full);
+      LinArgs rest = args;
+      rest.nseg = tail.nseg;
+      rest.seg_chunks = tail.seg_chunks;
+      rest.bg0 = tail.full_bg;
+      rest.bg_n = tail.tail_bg;
+      rest.ws_state = (float*)ws;
+      rest.ws_decay = rest.ws_state + (int64_t)g_tail * (tail.nseg - 1) * NW * ws_wave_floats;
+      if (gen) {
+        hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 1, true>), dim3(g_tail * (tail.nseg - 1)), dim3(64 * NW), lds, stream, rest);
+        hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 2, true>), dim3(g_tail * tail.nseg), dim3(64 * NW), lds, stream, rest);
+      } else {
+        hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 1>), dim3(g_tail * (tail.nseg - 1)), dim3(64 * NW), lds, stream, rest);
+        hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 2>), dim3(g_tail * tail.nseg), dim3(64 * NW), lds, stream, rest);
+      }
+    } else if (args.nseg <= 1) {
       args.nseg = 1;
       if (gen) hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 0, true>), dim3(groups, pieces), dim3(64 * NW), lds, stream, args);
       else hipLaunchKernelGGL((linear_fwd_kernel<DK, NWH, HG, 0>), dim3(groups), dim3(64 * NW), lds, stream, args);

@@ -232,3 +232,33 @@ def test_linear_rejects_bad_arguments():
     q2 = torch.zeros(1, 2, 64, 128, device="cuda", dtype=torch.float16)
     with pytest.raises(hb.MetaAttentionError):
         hb.linear_fwd(q2, q2, v.half(), ld)
+
+
+def test_last_round_of_a_single_pass_runs_in_sequence_segments():
+    """More head groups than the device holds at once, the last round at most half full (320 workgroups on 256 CUs): the
+    library runs the full rounds as a single pass and the remaining heads in sequence segments.  Same results as the forced
+    single pass up to the rounding of the exchanged states, and oracle slices on both sides of the cut; forward and backward
+    (whose scans take the same route)."""
+    hb = _hb()
+    B, H, T, Dk, Dv = 8, 40, 512, 256, 256
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 4).bfloat16()
+    k = (torch.randn(B, H, T, Dk, device="cuda", generator=g) / 4).bfloat16()
+    v = torch.randn(B, H, T, Dv, device="cuda", generator=g).bfloat16()
+    do = (0.5 * torch.randn(B, H, T, Dv, device="cuda", generator=g)).bfloat16()
+    ld = torch.nn.functional.logsigmoid(torch.randn(B, H, T, device="cuda", generator=g) + 3.0)
+    assert hb.linear_workspace_bytes(B, H, H, H, T, Dk, Dv) > 0 and hb.linear_workspace_bytes(B, H, H, H, T, Dk, Dv, segments=1) == 0
+    o = hb.linear_fwd(q, k, v, ld, q_scale=Dk ** -0.5)
+    o1 = hb.linear_fwd(q, k, v, ld, q_scale=Dk ** -0.5, segments=1)
+    grads = hb.linear_bwd(q, k, v, ld, do, q_scale=Dk ** -0.5)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(o.float(), o1.float(), rtol=1e-2, atol=1e-2)
+    assert torch.equal(o[:6], o1[:6])                      # the first 256 (batch, head) pairs took the single pass
+    for b, h in ((0, 0), (6, 15), (6, 16), (7, 39)):       # (6, 16) is the first head of the segmented tail
+        cut = lambda t: t[b:b + 1, h:h + 1].cpu()
+        ref = oracle.linear_attention_chunked(cut(q), cut(k), cut(v), cut(ld), chunk=64, q_scale=Dk ** -0.5)
+        oracle.assert_close(cut(o).float(), ref, rtol=RTOL, atol=ATOL, mismatch_ratio=1e-3)
+        rq, rk, rv, rg, _ = oracle.linear_attention_grads(cut(q), cut(k), cut(v), cut(ld), cut(do), q_scale=Dk ** -0.5, chunk=64)
+        for name, got, want in zip(("dq", "dk", "dv"), grads, (rq, rk, rv)):
+            oracle.assert_close(cut(got).float(), want.float(), rtol=RTOL, atol=ATOL, mismatch_ratio=5e-3, msg=f"{name} ({b},{h})")
+        assert float((cut(grads[3]).float() - rg.float()).abs().max()) <= max(0.03 * float(rg.abs().max()), 1e-2)
