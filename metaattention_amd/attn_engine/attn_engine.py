@@ -459,8 +459,7 @@ class AttentionEngine:
                 return known
         gamma = None
         if mask.dim() == 4 and tuple(mask.shape) == (1, H, S, S) and S >= 2:
-            m = mask[0].float()                                         # [H, S, S]
-            col = m[:, :, 0]                                            # gamma_h^i
+            col = mask[0, :, :, 0].float()                              # [H, S]: gamma_h^i
             i = torch.arange(S, device=mask.device, dtype=torch.float32)
             ok = col > 1e-30
             lg = torch.log2(col.clamp_min(1e-30))
@@ -468,10 +467,13 @@ class AttentionEngine:
             l2g = (w * lg).sum(dim=1) / (w * i).sum(dim=1).clamp_min(1.0)
             if bool(ok[:, :2].all()) and bool((l2g <= 0).all()) and bool(torch.isfinite(l2g).all()):
                 diff = (i.view(S, 1) - i.view(1, S)).clamp_min(0.0)
-                want = torch.exp2(diff.unsqueeze(0) * l2g.view(H, 1, 1))
+                lower = i.view(S, 1) >= i.view(1, S)
                 eps = 2.0 ** (-7 if mask.dtype == torch.bfloat16 else -10)    # two units in the last place
-                lower = (i.view(S, 1) >= i.view(1, S)).unsqueeze(0)
-                if bool((((m - want).abs() <= eps * want + 1e-30) | ~lower).all()):
+                same = torch.ones((), dtype=torch.bool, device=mask.device)
+                for h in range(H):                                      # (head by head: fp32 temporaries of one [S, S] plane, not of H)
+                    want = torch.exp2(diff * l2g[h])
+                    same &= (((mask[0, h].float() - want).abs() <= eps * want + 1e-30) | ~lower).all()
+                if bool(same):
                     gamma = torch.exp2(l2g).contiguous()
         cache[:] = [e for e in cache if e[0]() is not None and e[0]() is not mask][-7:]
         cache.append((weakref.ref(mask), mask._version, gamma))
