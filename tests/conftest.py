@@ -22,3 +22,11 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_runtest_setup(item):
+    # A kernel fault can end the whole box before pytest reports anything: name the GPU test that is about to run, flushed,
+    # where the tail of the run's output will show it.
+    if "gpu" in item.keywords:
+        sys.stderr.write(f"[gpu test] {item.nodeid}\n")
+        sys.stderr.flush()
