@@ -28,5 +28,8 @@ def pytest_runtest_setup(item):
     # A kernel fault can end the whole box before pytest reports anything: name the GPU test that is about to run, flushed,
     # where the tail of the run's output will show it.
     if "gpu" in item.keywords:
-        sys.stderr.write(f"[gpu test] {item.nodeid}\n")
-        sys.stderr.flush()
+        capman = item.config.pluginmanager.getplugin("capturemanager")
+        if capman is not None:
+            with capman.global_and_fixture_disabled():      # (past pytest's capture: a captured line dies with the process)
+                sys.stderr.write(f"[gpu test] {item.nodeid}\n")
+                sys.stderr.flush()
