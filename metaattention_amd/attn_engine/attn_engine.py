@@ -175,7 +175,12 @@ class AttentionEngine:
     def _init_prefill(self, score_mod, mask_mod, online_func, mask_value):
         m = self.meta
         form = canonicalize_score_mod(score_mod, self.custom_fwd_inputs)
-        row = identify_online_func(online_func)
+        row, inner = identify_online_func(online_func, return_scale=True)
+        if inner != 1.0:
+            # a softmax that scales the scores itself (examples/mha_v2.py:44-69): the library's softmax of inner * score
+            if form.activation != "identity" or form.bias_tensor or form.mask_tensor or form.extra or form.softcap is not None:
+                raise NotImplementedError("an OnlineFunc that scales the scores itself goes with a score_mod of the form a * score + c")
+            form.scale, form.bias = form.scale * inner, form.bias * inner
         fam = _FAMILY.get((form.activation, row))
         if fam is None:
             raise NotImplementedError(f"no library kernel for score activation '{form.activation}' with row function '{row}'")

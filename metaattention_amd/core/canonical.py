@@ -316,8 +316,14 @@ def _random_state(name, M, gen, magnitude=1.0):
     return ()
 
 
-def identify_online_func(online_func) -> str:
-    """Returns the name of the library row function ``online_func`` computes."""
+def identify_online_func(online_func, return_scale: bool = False):
+    """Returns the name of the library row function ``online_func`` computes; with ``return_scale`` the pair
+    (name, inner scale).  The inner scale c is 1 except for a softmax that scales the scores itself,
+    p = exp(c (s - m)) with lse = log r + c m (examples/mha_v2.py:44-69 spells it with exp2 and c log2 e): that is the
+    library's softmax of c s, and the caller folds c into the score function.  ``None`` (examples/sigmoid_attn_v2.py:67,
+    reluattn_v2.py:59) is the identity row function."""
+    if online_func is None:
+        return ("identity", 1.0) if return_scale else "identity"
     idx = [SymbolScalar(n, Var(n)) for n in ("b", "h", "q_idx")]
     state_syms = dict(online_func.online_rowscales)
     names = list(state_syms)
@@ -348,47 +354,71 @@ def identify_online_func(online_func) -> str:
             # perm[i] = index of the user's state variable that plays library role i
             if any(not _same_init(inits[perm[i]], lib_inits[i]) for i in range(len(lib_inits))):
                 continue
-            ok = True
-            for magnitude in (2.0, 0.02, 0.2):
-                s = torch.randn(M, N, generator=gen, dtype=torch.float64) * magnitude
-                st = _random_state(lib_name, M, gen, magnitude)
+
+            def matches(c):
+                # the user's running maximum is in the units of its scores, the library's in those of c * scores
+                ok = True
+                for magnitude in (2.0, 0.02, 0.2):
+                    s = torch.randn(M, N, generator=gen, dtype=torch.float64) * magnitude
+                    st = _random_state(lib_name, M, gen, magnitude)
+                    env = {id(tile_in): s}
+                    for i, j in enumerate(perm):
+                        env[id(state_syms[names[j]])] = st[i]
+                    got = evaluate([tile_out, o_scale] + [state_out[names[j]] for j in perm], env, s)
+                    lib_st = (st[0] * c,) + tuple(st[1:]) if c != 1.0 else st
+                    exp_p, exp_c, exp_st = fn(s * c, lib_st)
+                    if c != 1.0:
+                        got[2] = got[2] * c
+                    ok &= _allclose(got[0], exp_p) and _allclose(got[1], exp_c)
+                    ok &= all(_allclose(g, e) for g, e in zip(got[2:], exp_st))
+                    o = torch.randn(M, DV, generator=gen, dtype=torch.float64)
+                    env = {id(acc_in): o}
+                    for i, j in enumerate(perm):
+                        env[id(state_syms[names[j]])] = st[i]
+                    got = evaluate([acc_out] + list(finals.values()), env, o)
+                    exp_o, exp_final = epi(o, lib_st)
+                    ok &= _allclose(got[0], exp_o)
+                    if exp_final is None:
+                        ok &= len(got) == 1
+                    else:
+                        ok &= len(got) == 2 and _allclose(got[1], exp_final)
+                    if not ok:
+                        break
+                return ok
+
+            inner = 1.0
+            ok = matches(1.0)
+            if not ok and lib_name == "softmax":
+                # a softmax of c * scores: read c off one probability, exp(c (0 - 1)) from an empty state, then compare as above
+                s = torch.tensor([[0.0, 1.0]], dtype=torch.float64)
                 env = {id(tile_in): s}
                 for i, j in enumerate(perm):
-                    env[id(state_syms[names[j]])] = st[i]
-                got = evaluate([tile_out, o_scale] + [state_out[names[j]] for j in perm], env, s)
-                exp_p, exp_c, exp_st = fn(s, st)
-                ok &= _allclose(got[0], exp_p) and _allclose(got[1], exp_c)
-                ok &= all(_allclose(g, e) for g, e in zip(got[2:], exp_st))
-                o = torch.randn(M, DV, generator=gen, dtype=torch.float64)
-                env = {id(acc_in): o}
-                for i, j in enumerate(perm):
-                    env[id(state_syms[names[j]])] = st[i]
-                got = evaluate([acc_out] + list(finals.values()), env, o)
-                exp_o, exp_final = epi(o, st)
-                ok &= _allclose(got[0], exp_o)
-                if exp_final is None:
-                    ok &= len(got) == 1
-                else:
-                    ok &= len(got) == 2 and _allclose(got[1], exp_final)
-                if not ok:
-                    break
+                    env[id(state_syms[names[j]])] = torch.full((1, 1), lib_inits[i], dtype=torch.float64)
+                p0 = float(evaluate([tile_out], env, s)[0][0, 0])
+                if 0.0 < p0 < 1.0:
+                    inner = -math.log(p0)
+                    ok = matches(inner)
             if ok:
-                _check_recompute_and_combine(online_func, lib_name)
-                return lib_name
+                _check_recompute_and_combine(online_func, lib_name, inner)
+                if inner != 1.0 and not return_scale:
+                    raise NotImplementedError("this OnlineFunc scales the scores itself; ask for the scale with return_scale=True")
+                return (lib_name, inner) if return_scale else lib_name
         tried.append(lib_name)
     raise NotImplementedError(
         f"OnlineFunc with row scales {names} (initial values {inits}) matches no library row function "
         f"(softmax, identity, retention); compared against: {tried or 'none with that many row scales'}")
 
 
-def _check_recompute_and_combine(online_func, lib_name: str):
+def _check_recompute_and_combine(online_func, lib_name: str, inner: float = 1.0):
     """The other three methods of the contract, where the spec overrides them: ``forward`` (the probabilities again, from
     the scores and the final row scale), ``backward`` (dscores from dp: both generated into the backward kernel by
     core/lower/lower.py:425-438) and ``combine`` (the weight of every kv split, generated into the split-KV merge by
     core/lower/lower_decode.py:287-313).  The library's backward and combine kernels hold ONE version of each per row
     function; a spec whose traced version computes something else is refused instead of being silently replaced:
         softmax    forward exp(s - lse)   backward (dp - doosum) * p   combine exp(lse_i - logsumexp_i(lse))  (or the same
-                   in base 2, as examples/mha_decode.py:72-80 spells it for its log2-domain lse)
+                   in base 2, as examples/mha_decode.py:72-80 spells it for its log2-domain lse); with an inner scale c:
+                   forward exp(c s - lse), backward (dp - doosum) * p with or without the factor c (examples/mha_v2.py:79-83
+                   leaves it to its template; the kernels compute the gradient of the forward either way)
         identity   forward s              backward dp
         retention  forward s / r          backward dp / r"""
     from attn_engine import OnlineFunc          # (the base class: methods left at its defaults are not looked at)
@@ -417,7 +447,7 @@ def _check_recompute_and_combine(online_func, lib_name: str):
     if lib_name == "retention":
         fin = fin.abs() + 1.0
     sc = torch.randn(M, N, generator=gen, dtype=torch.float64)
-    prob = {"softmax": lambda: torch.exp(sc - fin), "identity": lambda: sc, "retention": lambda: sc / fin}[lib_name]()
+    prob = {"softmax": lambda: torch.exp(sc * inner - fin), "identity": lambda: sc, "retention": lambda: sc / fin}[lib_name]()
 
     if getattr(cls, "forward", None) is not OnlineFunc.forward:
         def build():
@@ -442,7 +472,7 @@ def _check_recompute_and_combine(online_func, lib_name: str):
             except TypeError:
                 out = online_func.backward(dps, ps, fsyms, *idx)
             env = {id(dps): dp, id(ps): prob, id(ds): doosum, **{id(v): fin for v in fsyms.values()}}
-            return out, env, dp, [expect]
+            return out, env, dp, [expect] if inner == 1.0 else [expect, expect * inner]
         run("backward", "score gradient", build)
 
     if getattr(cls, "combine", None) is not OnlineFunc.combine:

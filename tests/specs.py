@@ -55,6 +55,43 @@ class OnlineSoftmaxRespelled(OnlineFunc):
         return o / st["denom"], {"logsum": st["peak"] + st["denom"].log()}
 
 
+def online_softmax_inner_scale(scale):
+    """A softmax that scales the raw scores itself, in base 2 (the spelling of examples/mha_v2.py:26-83): the running
+    maximum is kept in the units of the raw scores, lse = log r + scale * m."""
+    import math
+    sl2 = scale * math.log2(math.e)
+
+    class OnlineSoftmaxInnerScale(OnlineFunc):
+        def __init__(self):
+            super().__init__({"m": SymbolScalar("m", Var("-inf")), "r": SymbolScalar("r", Var("0.0"))},
+                             {"lse": SymbolScalar("lse", Var("0.0"))}, CustomIO())
+
+        @staticmethod
+        def online_fwd(scores, online_rowscales, b, h, q_idx):
+            m, r = online_rowscales["m"], online_rowscales["r"]
+            m_new = m.max(scores.get_reduce("max"))
+            scale_tmp = ((m - m_new) * sl2).exp2()
+            r = r * scale_tmp
+            scores = ((scores - m_new) * sl2).exp2()
+            r = r + scores.get_reduce("sum")
+            return scores, {"m": m_new, "r": r}, scale_tmp
+
+        @staticmethod
+        def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+            lse = online_rowscales["r"].log() + online_rowscales["m"] * scale
+            return o / online_rowscales["r"], {"lse": lse}
+
+        @staticmethod
+        def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
+            return (scores * scale - final_rowscales["lse"]).exp()
+
+        @staticmethod
+        def backward(dp, scores, final_rowscales, doosum_rowscales, b, h, q_idx, kv_idx):
+            return (dp - doosum_rowscales) * scores
+
+    return OnlineSoftmaxInnerScale()
+
+
 class OnlineIdentity(OnlineFunc):
     def __init__(self):
         super().__init__({}, {}, CustomIO())
@@ -102,7 +139,18 @@ def softmax_attention(B, H, S, D, DV, dtype=torch.bfloat16, causal=True, online=
                            tune=tune, tune_file=f"tuned_config/{dev.name}/attn_tl.json", infer_mask=True)
 
 
-def sigmoid_attention(B, H, S, D, DV, dtype=torch.bfloat16, scale=1.0, form="tanh", const_bias=None, causal=True, mask_mod=None):
+def softmax_attention_inner_scale(B, H, S, D, DV, dtype=torch.bfloat16, causal=True, score_mod=None, io=None):
+    """examples/mha_v2.py:15-99: the score_mod returns the raw score, the online function scales it."""
+    if score_mod is None:
+        def score_mod(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
+            return score
+    return AttentionEngine(_meta(B, H, S, D, DV, dtype), io or CustomIO({}), score_mod=score_mod,
+                           mask_mod=causal_mask if causal else None, online_func=online_softmax_inner_scale((1 / D) ** 0.5),
+                           backend="cute_v2")
+
+
+def sigmoid_attention(B, H, S, D, DV, dtype=torch.bfloat16, scale=1.0, form="tanh", const_bias=None, causal=True, mask_mod=None,
+                      online="identity"):
     def score_mod(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
         x = score * scale if scale != 1.0 else score
         x = x + (const_bias if const_bias is not None else custom_fwd_inputs.input_tensors["softmax_bias"])
@@ -112,7 +160,8 @@ def sigmoid_attention(B, H, S, D, DV, dtype=torch.bfloat16, scale=1.0, form="tan
 
     io = CustomIO({} if const_bias is not None else {"softmax_bias": (1,)})
     return AttentionEngine(_meta(B, H, S, D, DV, dtype), io, score_mod=score_mod,
-                           mask_mod=mask_mod if mask_mod is not None else (causal_mask if causal else None), online_func=OnlineIdentity())
+                           mask_mod=mask_mod if mask_mod is not None else (causal_mask if causal else None),
+                           online_func=OnlineIdentity() if online == "identity" else online)
 
 
 def relu_attention(B, H, S, D, DV, dtype=torch.bfloat16):

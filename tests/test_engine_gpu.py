@@ -35,6 +35,41 @@ def test_softmax_operator_fp16_noncausal():
     oracle.assert_close(o.float().cpu(), oracle.softmax_attention(q, k, v, causal=False), rtol=RTOL, atol=ATOL)
 
 
+def test_softmax_that_scales_the_scores_itself():
+    """examples/mha_v2.py:15-99: score_mod returns the raw score, the online function computes exp2((s - m) * scale * log2 e)
+    and lse = log r + scale * m.  The same operator as the usual spelling: output, lse and gradients bit for bit, and the
+    oracle's values."""
+    B, H, S, D = 1, 4, 384, 128
+    mod, usual = specs.softmax_attention_inner_scale(B, H, S, D, D), specs.softmax_attention(B, H, S, D, D)
+    assert mod.score_form.scale == usual.score_form.scale
+    q, k, v = inputs.softmax_inputs(B, H, S, D, D, seed=21)
+    got, exp = [], []
+    for m, out in ((mod, got), (usual, exp)):
+        qq, kk, vv = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        o = m(qq, kk, vv)
+        o.backward(torch.ones_like(o) * 0.25)
+        torch.cuda.synchronize()
+        out += [o.detach(), m.final_rowscales, qq.grad, kk.grad, vv.grad]
+    for a, b in zip(got, exp):
+        assert torch.equal(a, b)
+    ref, lse = oracle.softmax_attention(q, k, v, causal=True, return_lse=True)
+    oracle.assert_close(got[0].float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(got[1].cpu(), lse, rtol=1e-4, atol=1e-4)
+
+
+def test_no_online_function_is_the_identity_row_function():
+    """examples/sigmoid_attn_v2.py:62-68, reluattn_v2.py:54-60 pass online_func=None."""
+    B, H, S, D = 1, 2, 256, 128
+    mod = specs.sigmoid_attention(B, H, S, D, D, online=None)
+    assert mod.family == "sigmoid"
+    q, k, v = inputs.softmax_inputs(B, H, S, D, D, seed=22)
+    q = (q.float() * 0.3).bfloat16()
+    bias = torch.tensor([-4.25])
+    o = mod(q.cuda(), k.cuda(), v.cuda(), bias.cuda())
+    torch.cuda.synchronize()
+    oracle.assert_close(o.float().cpu(), oracle.sigmoid_attention(q, k, v, bias, causal=True), rtol=RTOL, atol=ATOL, mismatch_ratio=2e-3)
+
+
 def test_sigmoid_operator_with_bias_tensor():
     """mod(q, k, v, softmax_bias[1]) as in testing/test.py:552-566."""
     B, H, S, D = 1, 2, 256, 128

@@ -144,6 +144,50 @@ def test_identify_online_funcs():
         identify_online_func(WrongInit())
 
 
+def test_softmax_with_an_inner_scale_and_no_online_function():
+    """The spellings of the reference's second set of examples (examples/mha_v2.py:26-83, sigmoid_attn_v2.py:67): a
+    softmax that scales the raw scores itself is the library's softmax of scale * score; None is the identity."""
+    scale = (1 / 128) ** 0.5
+    name, inner = identify_online_func(specs.online_softmax_inner_scale(scale), return_scale=True)
+    assert name == "softmax" and abs(inner - scale) < 1e-12
+    assert identify_online_func(specs.OnlineSoftmax(), return_scale=True) == ("softmax", 1.0)
+    with pytest.raises(NotImplementedError):          # (a caller that does not ask for the scale must not lose it)
+        identify_online_func(specs.online_softmax_inner_scale(scale))
+    assert identify_online_func(None) == "identity" and identify_online_func(None, return_scale=True) == ("identity", 1.0)
+
+    e = specs.softmax_attention_inner_scale(2, 4, 256, 128, 128)
+    assert (e.family, e.mask_kind) == ("softmax", "causal") and abs(e.score_form.scale - scale) < 1e-12 and e.score_form.bias == 0.0
+    # a constant inside the score function is scaled with it: softmax(scale * (2 s + 3))
+    e = specs.softmax_attention_inner_scale(2, 4, 256, 128, 128, score_mod=lambda s, c, b, h, q, k: s * 2.0 + 3.0)
+    assert abs(e.score_form.scale - 2 * scale) < 1e-12 and abs(e.score_form.bias - 3 * scale) < 1e-12
+    # additive tensors would have to be scaled too: refused, not silently left unscaled
+    io = CustomIO({"rel": (1, "heads", "seq_len", "seq_len_kv")})
+    with pytest.raises(NotImplementedError):
+        specs.softmax_attention_inner_scale(2, 4, 256, 128, 128, io=io,
+                                            score_mod=lambda s, c, b, h, q, k: s + c.input_tensors["rel"])
+
+    # the recomputation must carry the same scale: exp(s - lse) is another function
+    inner_cls = type(specs.online_softmax_inner_scale(scale))
+
+    class ForgetsTheScale(inner_cls):
+        @staticmethod
+        def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
+            return (scores - final_rowscales["lse"]).exp()
+
+    with pytest.raises(NotImplementedError):
+        identify_online_func(ForgetsTheScale(), return_scale=True)
+
+    class InconsistentLse(inner_cls):          # lse without the scale on the maximum
+        @staticmethod
+        def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+            return o / online_rowscales["r"], {"lse": online_rowscales["r"].log() + online_rowscales["m"]}
+
+    with pytest.raises(NotImplementedError):
+        identify_online_func(InconsistentLse(), return_scale=True)
+
+    assert specs.sigmoid_attention(1, 2, 256, 128, 128, online=None).family == "sigmoid"
+
+
 def test_engine_construction_and_dispatch():
     assert get_attn_device().name == "MI355X"
     e = specs.softmax_attention(8, 32, 4096, 128, 128)
