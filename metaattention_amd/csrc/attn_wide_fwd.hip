@@ -12,7 +12,7 @@
 //              element-wise causal mask is applied in forward: with the causal structural mask only kv
 //              tiles above the workgroup's diagonal are skipped and the zeros come from M itself.
 // The head sizes of the reference's own test list are covered (testing/test.py:54-63: 128/256 softmax,
-// 64/64 relu, 256/512 retention) next to 256/256 and, without softmax, 256/512.
+// 64/64 relu, 256/512 retention) next to 256/256 and 256/512.
 //
 // Decode shapes (a few query rows against a long cache, softmax, no mask) run with one wave per
 // workgroup and the kv sequence cut into splits, each writing a normalised partial output and its
@@ -317,10 +317,25 @@ __global__ __launch_bounds__(64 * NW, ((DQK + DV >= 512 || (NW == 1 && pad_width
           const float m_new = move ? fmaxf(row_max, mx) : row_max;
           const float corr = fast_exp2(row_max - m_new);
           r_part *= corr;
+          if constexpr (DQK + DV >= 512) {
+            // one wave per SIMD: the accumulators live in the MFMA accumulation registers and are rescaled there one at a
+            // time through one vector register.  Written as C++ the compiler moves them all to vector registers first: at
+            // Dv 512 it then spills 231 registers, in the loop's hot path as well (12 % of this speed), at 256 / 256 it
+            // holds 438 registers instead of 326 and runs 20 % slower.
 #pragma unroll
-          for (int i = 0; i < DB; i++)
+            for (int i = 0; i < DB; i++)
 #pragma unroll
-            for (int j = 0; j < 16; j++) o[i][j] *= corr;
+              for (int j = 0; j < 16; j++) {
+                float t;
+                asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1" : "+a"(o[i][j]), "=&v"(t) : "v"(corr));
+              }
+            asm volatile("s_nop 4");   // (an accumulation register written by the vector ALU is not read by an MFMA at once)
+          } else {
+#pragma unroll
+            for (int i = 0; i < DB; i++)
+#pragma unroll
+              for (int j = 0; j < 16; j++) o[i][j] *= corr;
+          }
           row_max = m_new;
           sub = c_bias - row_max;
 #pragma unroll
@@ -493,9 +508,8 @@ static int wide_family(const AttnArgs& a, int family, bool causal, hipStream_t s
     case WF_SOFTMAX:
       if constexpr (DV <= 256) {
         if (!causal && a.Sq <= 32 && a.o_part) return launch_wide<T, DQK, DV, WF_SOFTMAX, false, 1>(a, stream);   // decode
-        return causal ? launch_wide<T, DQK, DV, WF_SOFTMAX, true>(a, stream) : launch_wide<T, DQK, DV, WF_SOFTMAX, false>(a, stream);
       }
-      return -2;
+      return causal ? launch_wide<T, DQK, DV, WF_SOFTMAX, true>(a, stream) : launch_wide<T, DQK, DV, WF_SOFTMAX, false>(a, stream);
     case WF_SIGMOID:
       return causal ? launch_wide<T, DQK, DV, WF_SIGMOID, true>(a, stream) : launch_wide<T, DQK, DV, WF_SIGMOID, false>(a, stream);
     case WF_RELU:
@@ -522,11 +536,11 @@ static int wide_dims(const AttnArgs& a, int family, bool causal, int dqk, int dv
   if (dqk == 128 && dv == 256) return wide_family<T, 128, 256>(a, family, causal, stream);
   if (dqk == 256 && dv == 256) return wide_family<T, 256, 256>(a, family, causal, stream);
   if (dqk == 192 && dv == 128) return wide_family<T, 192, 128>(a, family, causal, stream);   // (the reference's DeepSeek-V2-Lite benchmark shape)
-  if (dqk == 256 && dv == 512 && family != WF_SOFTMAX) return wide_family<T, 256, 512>(a, family, causal, stream);
-  // Softmax at 256/512: rescaling a 256-register accumulator that lives in the MFMA accumulation registers makes the
-  // compiler spill it.  Given the probabilities the value columns are independent, so the two halves of V and of the
-  // output go through the 256/256 kernel one after the other (the scores are computed twice; both launches write the
-  // same row scales).
+  if (dqk == 256 && dv == 512 && (family != WF_SOFTMAX || !(a.Sq <= 32 && a.o_part))) return wide_family<T, 256, 512>(a, family, causal, stream);
+  // Softmax decode (split kv, one wave per workgroup) at 256/512: a workgroup's two tile stages would take 96 KB of LDS,
+  // one wave per CU.  Given the probabilities the value columns are independent, so the two halves of V and of the
+  // output go through the 256/256 decode kernel one after the other (the scores are computed twice; both launches write
+  // the same row scales).
   if (dqk == 256 && dv == 512) {
     AttnArgs half = a;
     const int rc = wide_family<T, 256, 256>(half, family, causal, stream);

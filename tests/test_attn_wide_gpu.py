@@ -93,14 +93,17 @@ def test_causal_mask_is_exact_other_head_sizes():
             assert torch.equal(oa[:, :cut], ob[:, :cut]), (D, DV, fam)
 
 
-def test_growing_scores_and_tile_size_independence():
-    """Row maxima that grow along the kv axis exercise the accumulator rescale; a constant key makes the
-    output the running mean of v (closed form)."""
+@pytest.mark.parametrize("D,DV", [(64, 64), (128, 256), (256, 256), (256, 512), (192, 128)])
+def test_growing_scores_and_tile_size_independence(D, DV):
+    """Row maxima that grow along the kv axis exercise the accumulator rescale (at Dv 512 the accumulators are rescaled
+    in the MFMA accumulation registers); a constant key makes the output the running mean of v (closed form)."""
     hb = _hb()
-    B, H, S, D, DV = 1, 2, 300, 64, 64
+    B, H, S = 1, 2, 300
     q, k, v = inputs.softmax_inputs(B, H, S, D, DV, seed=3)
-    ramp = torch.linspace(0.2, 3.0, S).view(1, S, 1, 1)
-    k = (k.float() * ramp).bfloat16()
+    # positive q and k: the scores grow with the key index in every row (about 5 -> 30, the same at every head size), so the
+    # reference of the exponentials moves every few tiles
+    ramp = torch.linspace(0.2, 6.0, S).view(1, S, 1, 1) * (64 / D) ** 0.5
+    q, k = q.abs(), (k.float().abs() * ramp).bfloat16()
     ref = oracle.softmax_attention(q, k, v, causal=True)
     o = hb.attn_fwd(q.cuda(), k.cuda(), v.cuda(), family=hb.MA_ATTN_SOFTMAX, causal=True, scale=1 / math.sqrt(D))
     oracle.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
