@@ -32,7 +32,7 @@ def test_parallel_forward_random(seed):
     hb = _hb()
     random.seed(seed)
     g = torch.Generator().manual_seed(seed)
-    D, DV = random.choice([(128, 128), (128, 128), (64, 64), (128, 256), (256, 256), (192, 128)])
+    D, DV = random.choice([(128, 128), (128, 128), (64, 64), (128, 256), (256, 256), (192, 128), (256, 512)])
     family = random.choice(["softmax", "softmax", "sigmoid", "relu"])
     dtype = random.choice([torch.bfloat16, torch.float16])
     B, Hkv, grp = random.randint(1, 3), random.randint(1, 3), random.choice([1, 1, 2, 4])
@@ -193,7 +193,7 @@ def test_element_masks_random(seed):
     random.seed(1000 + seed)
     g = torch.Generator().manual_seed(1000 + seed)
     backward = seed % 2 == 1
-    D, DV = random.choice([(128, 128), (64, 64), (128, 256), (192, 128)] + ([] if backward else [(256, 256)]))
+    D, DV = random.choice([(128, 128), (64, 64), (128, 256), (192, 128)] + ([] if backward else [(256, 256), (256, 512)]))
     family = random.choice(FAMILIES)
     dtype = random.choice([torch.bfloat16, torch.float16])
     B, Hkv, grp = random.randint(1, 2), random.randint(1, 2), random.choice([1, 2])
@@ -261,7 +261,7 @@ def test_score_terms_random(seed):
     random.seed(3000 + seed)
     g = torch.Generator().manual_seed(3000 + seed)
     backward = seed % 2 == 1
-    D, DV = random.choice([(128, 128), (64, 64), (128, 256), (192, 128)] + ([] if backward else [(256, 256)]))
+    D, DV = random.choice([(128, 128), (64, 64), (128, 256), (192, 128)] + ([] if backward else [(256, 256), (256, 512)]))
     family = random.choice(FAMILIES)
     dtype = random.choice([torch.bfloat16, torch.float16])
     B, Hkv, grp = random.randint(1, 2), random.randint(1, 2), random.choice([1, 2])
