@@ -602,6 +602,37 @@ def bench_reference_benchmark_shapes(steps, warmup):
     return out
 
 
+def bench_head_sizes(steps, warmup):
+    """The parallel kernels at every head size of the tile table (the reference's own list, testing/test.py:54-63,
+    benchmark_h100.py:87,129, benchmark_mi250.py:40-46) x row-function family, causal, B4 H16 S4096 bf16: forward and
+    backward side by side, so that a size which falls behind its neighbours shows."""
+    import torch
+    from metaattention_amd import hip_backend as hb
+    global RAMP_MS
+    B, H, S = 4, 16, 4096
+    fams = {"softmax": hb.MA_ATTN_SOFTMAX, "sigmoid": hb.MA_ATTN_SIGMOID, "relu": hb.MA_ATTN_RELU}
+    g = torch.Generator(device="cuda").manual_seed(0)
+    ramp, out = RAMP_MS, {}
+    RAMP_MS = min(ramp, 20.0)
+    try:
+        for D, DV in ((64, 64), (128, 128), (128, 256), (192, 128), (256, 256), (256, 512)):
+            q, k = (torch.randn(B, S, H, D, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(2))
+            v, do = (0.5 * torch.randn(B, S, H, DV, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(2))
+            o = torch.empty(B, S, H, DV, device="cuda", dtype=torch.bfloat16)
+            flops = 0.5 * 2.0 * B * H * S * S * (D + DV)
+            for name, fam in fams.items():
+                lse = torch.empty(B, H, S, device="cuda") if name == "softmax" else None
+                kw = dict(family=fam, causal=True, scale=D ** -0.5, bias=-3.0 if name == "sigmoid" else 0.0)
+                ms_f = time_gpu(lambda: hb.attn_fwd(q, k, v, out=o, row_scale=lse, **kw), max(steps // 3, 3), 2)
+                ms_b = time_gpu(lambda: hb.attn_bwd(q, k, v, o, do, lse, **kw), max(steps // 5, 3), 1)
+                out[f"{D}/{DV} {name}"] = dict(fwd_ms=round(ms_f, 4), fwd_tflops=round(flops / ms_f / 1e9, 1),
+                                               bwd_ms=round(ms_b, 4), bwd_tflops=round(2.5 * flops / ms_b / 1e9, 1))
+    finally:
+        RAMP_MS = ramp
+    out["note"] = "causal, B4 H16 S4096 bf16; forward: algorithmic FLOPs (causal at one half); backward: 2.5 x the forward's"
+    return out
+
+
 def cpu_baseline_softmax():
     """Oracle (restated PyTorch reference, fp32) on the host cores over a bounded
     sample: the whole headline workload once (B=8, H=32, S=4096, D=128, causal), about ten seconds."""
@@ -740,7 +771,8 @@ def main():
              ("c5_mla_decode_operator", "mla_operator", lambda: bench_mla_operator(args.steps, args.warmup)),
              ("gqa_decode", "decode", lambda: bench_decode(args.steps, args.warmup)),
              ("reference_shapes", "reference_shapes", lambda: bench_reference_shapes(args.steps, args.warmup)),
-             ("reference_benchmark_shapes", "reference_benchmark", lambda: bench_reference_benchmark_shapes(args.steps, args.warmup))]
+             ("reference_benchmark_shapes", "reference_benchmark", lambda: bench_reference_benchmark_shapes(args.steps, args.warmup)),
+             ("head_sizes", "head_sizes", lambda: bench_head_sizes(args.steps, args.warmup))]
     cpu_legs = {"c3_retnet_chunked": cpu_baseline_retnet_chunked, "c3_retnet_parallel": cpu_baseline_retention_parallel,
                 "c4_mamba2_ssd": cpu_baseline_mamba2, "c5_mla_decode": cpu_baseline_mla}
     for name, key, fn in table:

@@ -37,6 +37,9 @@ def test_bench_line():
     rb = others["reference_benchmark_shapes"]
     assert "error" not in rb and len(rb) == 9, rb
     assert all(min(v for k, v in e.items() if k.endswith("ms") or k.startswith("ms")) > 0 for e in rb.values())
+    hs = others["head_sizes"]
+    assert "error" not in hs and len([k for k in hs if k != "note"]) == 18, hs
+    assert all(e["fwd_ms"] > 0 and e["bwd_ms"] > 0 for k, e in hs.items() if k != "note")
     # the operator recognised the decay mask the workload builds
     assert "generates it" in others["c3_retnet_parallel_operator"]["flop_convention"]
     for name in ("c5_mla_decode", "gqa_decode"):
