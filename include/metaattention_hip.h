@@ -297,7 +297,9 @@ int ma_mla_decode(const ma_mla_params* p, ma_stream_t stream);
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose operators
  * allocate their partial results on every call.  Same arguments and results as ma_mla_decode, except that p->workspace is
  * ignored: the partial results of the kv splits go to an array inside the library, ma_mla_noalloc_max_workspace() bytes
- * (40 MiB) per GPU, held until the process ends.  A call whose ma_mla_workspace_bytes(p) exceeds that returns
+ * (40 MiB) per GPU, held until the process ends -- by every process that loads the library and uses that GPU, whether or
+ * not it calls this entry point (the array is part of the code object: 16 processes on one GPU hold 640 MiB); devices
+ * beyond ordinal 63 are refused with MA_ERR_UNSUPPORTED.  A call whose ma_mla_workspace_bytes(p) exceeds that returns
  * MA_ERR_WORKSPACE.  The call itself allocates nothing and synchronises nothing.  All calls on one GPU share the array:
  * calls that overlap on one GPU (different streams, different threads) race; calls on one stream do not.  Every slot a
  * call reads it has written before, so nothing needs clearing between calls.  The first call on a device looks the
