@@ -320,16 +320,22 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   //      and its Q rows are requested before that item's output is written.
   const int nmb = a.num_m_blocks, BH = a.B * a.H, G = (int)gridDim.x;
   const bool paired = CAUSAL && BH * nmb > G;               // (few items: one q block per unit, spread wide)
-  const int upb = paired ? (nmb + 1) >> 1 : nmb;            // units per (batch, head)
   const bool by_xcd = (BH & 7) == 0 && (G & 7) == 0;
-  const int units = by_xcd ? (BH >> 3) * upb : BH * upb;   // units of this workgroup's stream
+  // With an even number of (batch, head) pairs per XCD the two q blocks of a unit come from two pairs: block i of pair 2s,
+  // then block nmb-1-i of pair 2s+1.  Units still weigh the same, so the workgroups of an XCD start their first items
+  // together, at key 0 of the same K/V planes: those are read from HBM once and need no room in L2 beyond the rows in
+  // flight, and only the second items, which start one after the other, need their pair's planes resident (2 MB at
+  // S = 4096 against the XCD's 4 MB; with both q blocks from one pair, two pairs' planes had to stay).
+  const bool cross = paired && by_xcd && ((BH >> 3) & 1) == 0;
+  const int upb = cross ? nmb : paired ? (nmb + 1) >> 1 : nmb;   // units per (batch, head), per two of them if `cross`
+  const int units = cross ? (BH >> 4) * upb : by_xcd ? (BH >> 3) * upb : BH * upb;   // units of this workgroup's stream
   const int first = by_xcd ? (int)blockIdx.x >> 3 : (int)blockIdx.x, stride = by_xcd ? G >> 3 : G;
   // item cursor t = 2 * unit + half; returns the next cursor that names an item (or one past the end)
   int t_next = 0;
   auto next_item = [&](int t) -> int {
     for (;;) {
       t = (t & 1) ? t + 2 * stride - 1 : t + 1;
-      if (t >= 2 * units) return t;
+      if (t >= 2 * units || cross) return t;
       const int k = (t >> 1) % upb;
       if (paired ? !((t & 1) && k == nmb - 1 - k) : !(t & 1)) return t;   // (the middle block of an odd count is its own partner)
     }
@@ -337,6 +343,7 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   // (batch, head) planes of item t
   auto planes_of = [&](int t, const char*& kb, const char*& vb, int& b_, int& h_) __attribute__((always_inline)) {
     int bh = (t >> 1) / upb;
+    if (cross) bh = 2 * bh + (t & 1);
     if (by_xcd) bh = bh * 8 + ((int)blockIdx.x & 7);
     b_ = bh / a.H;
     h_ = bh % a.H;
@@ -346,7 +353,7 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   // decode item t into the per-item variables, request its Q rows, and look up the item after it
   auto open_item = [&](int t) __attribute__((always_inline)) {
     const int k = (t >> 1) % upb;
-    mb = paired ? ((t & 1) ? k : nmb - 1 - k) : (CAUSAL ? nmb - 1 - k : k);
+    mb = cross ? ((t & 1) ? nmb - 1 - k : k) : paired ? ((t & 1) ? k : nmb - 1 - k) : (CAUSAL ? nmb - 1 - k : k);
     planes_of(t, kbase, vbase, b, h);
     // V positions n_sub .. n_sub + 4 of the item before this one (its steps n_sub - 4 .. n_sub) refilled every V slot
     // but the one of its own last sub-tile
