@@ -322,10 +322,11 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   const bool paired = CAUSAL && BH * nmb > G;               // (few items: one q block per unit, spread wide)
   const bool by_xcd = (BH & 7) == 0 && (G & 7) == 0;
   // With an even number of (batch, head) pairs per XCD the two q blocks of a unit come from two pairs: block i of pair 2s,
-  // then block nmb-1-i of pair 2s+1.  Units still weigh the same, so the workgroups of an XCD start their first items
-  // together, at key 0 of the same K/V planes: those are read from HBM once and need no room in L2 beyond the rows in
-  // flight, and only the second items, which start one after the other, need their pair's planes resident (2 MB at
-  // S = 4096 against the XCD's 4 MB; with both q blocks from one pair, two pairs' planes had to stay).
+  // then block nmb-1-i of pair 2s+1.  Units still weigh the same, so the workgroups that share pair 2s start their first
+  // items together, at key 0 of the same K/V planes: those rows are read from HBM once and need no room in L2 beyond the
+  // rows in flight; only the second items, which start one after the other, need their pair's planes resident.  At
+  // S = 4096 (16 q blocks, 2 MB of K/V per pair) the 32 workgroups of an XCD cover two such units of pairs: 4 MB to keep
+  // in the XCD's 4 MB of L2, where both q blocks from one pair made it the planes of four pairs, 8 MB.
   const bool cross = paired && by_xcd && ((BH >> 3) & 1) == 0;
   const int upb = cross ? nmb : paired ? (nmb + 1) >> 1 : nmb;   // units per (batch, head), per two of them if `cross`
   const int units = cross ? (BH >> 4) * upb : by_xcd ? (BH >> 3) * upb : BH * upb;   // units of this workgroup's stream

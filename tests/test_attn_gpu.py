@@ -94,10 +94,13 @@ def test_causal_mask_is_exact():
     assert torch.isfinite(o1.float()).all()
 
 
-@pytest.mark.parametrize("B,H,S,causal", [(8, 16, 768, True), (3, 30, 1280, True), (2, 24, 1536, False)])
+@pytest.mark.parametrize("B,H,S,causal", [(8, 16, 768, True), (3, 30, 1280, True), (2, 24, 1536, False), (16, 16, 768, True), (4, 8, 2304, True),
+                                          (5, 8, 1792, True)])
 def test_softmax_work_distribution(B, H, S, causal):
     """More work items than CUs, odd numbers of q blocks, (batch*head) counts that are and are not
-    multiples of 8: every item must be computed exactly once whatever the item -> workgroup mapping."""
+    multiples of 8 and of 16 (with an even number of pairs per XCD a unit's two q blocks come from two pairs; B16: more
+    than one such unit per workgroup; B5 H8: an odd number per XCD, both blocks from one pair): every item must be computed
+    exactly once whatever the item -> workgroup mapping."""
     hb = _hb()
     D = 128
     g = torch.Generator(device="cuda").manual_seed(S)
