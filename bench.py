@@ -520,7 +520,7 @@ def bench_reference_shapes(steps, warmup):
 
 
 def bench_reference_benchmark_shapes(steps, warmup):
-    """Figures of the reference's own benchmarks that BASELINE's configurations do not cover (testing/benchmark_mi250.py:40-55,
+    """Figures of the reference's own benchmarks that the five headline configurations do not cover (testing/benchmark_mi250.py:40-55,
     testing/benchmark_h100.py:112,129): causal softmax at the DeepSeek-V2-Lite head sizes (16 heads, Dqk 192, Dv 128, fp16),
     ReLU attention at the ViT-S head size (6 heads, 64 / 64, fp16) and gated retention at 64 / 64 and 256 / 256, forward and
     backward through the C ABI; one query token at the DeepSeek-V2-Lite sizes, the block-sparse grouped-query decode and the
