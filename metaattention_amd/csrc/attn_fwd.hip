@@ -326,8 +326,10 @@ __global__ __launch_bounds__(512, 2) void attn_fwd_kernel(const AttnArgs a) {
   // items together, at key 0 of the same K/V planes: those rows are read from HBM once and need no room in L2 beyond the
   // rows in flight; only the second items, which start one after the other, need their pair's planes resident.  At
   // S = 4096 (16 q blocks, 2 MB of K/V per pair) the 32 workgroups of an XCD cover two such units of pairs: 4 MB to keep
-  // in the XCD's 4 MB of L2, where both q blocks from one pair made it the planes of four pairs, 8 MB.
-  const bool cross = paired && by_xcd && ((BH >> 3) & 1) == 0;
+  // in the XCD's 4 MB of L2, where both q blocks from one pair made it the planes of four pairs, 8 MB (HBM reads 0.94
+  // against 1.27 GB per launch at B8 H32).  Longer sequences, whose planes do not fit either way, keep both blocks from one
+  // pair: there the second items of this order, half of them long, re-read more (S = 8192: 1.5 % slower).
+  const bool cross = paired && by_xcd && ((BH >> 3) & 1) == 0 && (int64_t)a.Skv * (DQK + DV) * 2 <= (2 << 20);
   const int upb = cross ? nmb : paired ? (nmb + 1) >> 1 : nmb;   // units per (batch, head), per two of them if `cross`
   const int units = cross ? (BH >> 4) * upb : by_xcd ? (BH >> 3) * upb : BH * upb;   // units of this workgroup's stream
   const int first = by_xcd ? (int)blockIdx.x >> 3 : (int)blockIdx.x, stride = by_xcd ? G >> 3 : G;
